@@ -1,0 +1,66 @@
+// Shared device helpers for the k3q kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "../../include/k3q.h"
+
+namespace k3q {
+
+typedef uint32_t u32;
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef u32 v4u __attribute__((ext_vector_type(4)));
+typedef u32 v2u __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bf16_bits_to_f32(u32 h) { return __uint_as_float(h << 16); }
+
+// float -> bfloat16 bits, round to nearest even (finite inputs; NaN stays NaN).
+__device__ __forceinline__ u32 f32_to_bf16_bits(float f) {
+    u32 u = __float_as_uint(f);
+    u32 r = u + 0x7fffu + ((u >> 16) & 1u);
+    r = ((u & 0x7fffffffu) > 0x7f800000u) ? (u | 0x00400000u) : r;
+    return r >> 16;
+}
+
+// value of f after a round trip through bfloat16
+__device__ __forceinline__ float round_bf16(float f) {
+    return __uint_as_float(f32_to_bf16_bits(f) << 16);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// byte select: result byte i = byte sel[i] of the 8-byte pool {lo: bytes 0-3, hi: bytes 4-7}
+__device__ __forceinline__ u32 byte_perm(u32 hi, u32 lo, u32 sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+inline int launch_status() {
+    return hipGetLastError() == hipSuccess ? K3Q_OK : K3Q_ERR_LAUNCH;
+}
+
+// host-side: value of f after rounding to bfloat16 (nearest even)
+inline float host_round_bf16(float f) {
+    uint32_t u;
+    ::memcpy(&u, &f, 4);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    u &= 0xffff0000u;
+    ::memcpy(&f, &u, 4);
+    return f;
+}
+
+inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+}  // namespace k3q

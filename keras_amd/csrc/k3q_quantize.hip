@@ -1,0 +1,230 @@
+// Row-wise abs-max quantizer: x [rows, cols] (float32 or bfloat16) ->
+// q int8 [rows, cols] + scale [rows].
+//
+// HBM-bound: x is read once, q and scale are written once.  A row is held in
+// registers between the max reduction and the quantisation, so the nine torch
+// passes of the reference collapse into one read and one write.  Every
+// arithmetic step is rounded to the tensor dtype exactly as torch rounds it
+// (for bfloat16: the epsilon, the sum, the quotient and the product are each
+// rounded to bfloat16 before the next step), which is what makes the int8
+// output bit-identical to the reference.
+#include "k3q_common.h"
+
+namespace k3q {
+namespace {
+
+template <int kDtype>
+struct Elem;
+template <>
+struct Elem<K3Q_F32> {
+    static constexpr int kBytes = 4;
+    static constexpr int kPerChunk = 4;  // elements in a 16-byte chunk
+};
+template <>
+struct Elem<K3Q_BF16> {
+    static constexpr int kBytes = 2;
+    static constexpr int kPerChunk = 8;
+};
+
+// unpack one 16-byte chunk into floats
+template <int kDtype>
+__device__ __forceinline__ void chunk_to_floats(const v4u& c, float* f) {
+    if (kDtype == K3Q_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(c[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(c[i] << 16);
+            f[2 * i + 1] = __uint_as_float(c[i] & 0xffff0000u);
+        }
+    }
+}
+
+template <int kDtype>
+__device__ __forceinline__ float scale_from_amax(float amax, float eps, float qhi) {
+    if (kDtype == K3Q_F32) return qhi / (amax + eps);
+    float t = round_bf16(amax + eps);  // eps arrives already rounded to bfloat16
+    return round_bf16(qhi / t);
+}
+
+template <int kDtype>
+__device__ __forceinline__ int quantize_one(float v, float s, float qlo, float qhi) {
+    float p = v * s;
+    if (kDtype == K3Q_BF16) p = round_bf16(p);
+    p = rintf(p);  // round half to even
+    p = fminf(fmaxf(p, qlo), qhi);
+    return (int)p;
+}
+
+// max over the threads that share a row: `kTpr` consecutive threads, kTpr in {64, 256}
+template <int kTpr>
+__device__ __forceinline__ float row_max(float v, float* lds) {
+    v = wave_max(v);
+    if (kTpr == kWave) return v;
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x % kWave) == 0) lds[wave] = v;
+    __syncthreads();
+    float r = lds[0];
+#pragma unroll
+    for (int w = 1; w < kTpr / kWave; ++w) r = fmaxf(r, lds[w]);
+    return r;
+}
+
+// Fast path.  cols % kPerChunk == 0, rows 16-byte aligned.  kTpr threads per row,
+// 256 / kTpr rows per block, each thread keeps up to kChunks 16-byte chunks.
+template <int kDtype, int kTpr, int kChunks>
+__global__ __launch_bounds__(256) void quantize_rows_vec(const char* __restrict__ x, int64_t rows,
+                                                         int64_t chunks_per_row,
+                                                         int64_t x_row_bytes, float eps, float qlo,
+                                                         float qhi, int8_t* __restrict__ q,
+                                                         void* __restrict__ scale) {
+    constexpr int kPer = Elem<kDtype>::kPerChunk;
+    constexpr int kRowsPerBlock = 256 / kTpr;
+    __shared__ float lds[256 / kWave];
+    const int lane = threadIdx.x % kTpr;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kTpr;
+    const bool live = row < rows;
+    const v4u* xr = (const v4u*)(x + (live ? row : 0) * x_row_bytes);
+
+    v4u c[kChunks];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+        int64_t ci = lane + (int64_t)i * kTpr;
+        if (live && ci < chunks_per_row) {
+            c[i] = __builtin_nontemporal_load(xr + ci);
+            float f[kPer];
+            chunk_to_floats<kDtype>(c[i], f);
+#pragma unroll
+            for (int e = 0; e < kPer; ++e) amax = fmaxf(amax, fabsf(f[e]));
+        }
+    }
+    amax = row_max<kTpr>(amax, lds);
+    if (!live) return;
+    const float s = scale_from_amax<kDtype>(amax, eps, qhi);
+    if (lane == 0) {
+        if (kDtype == K3Q_F32)
+            ((float*)scale)[row] = s;
+        else
+            ((uint16_t*)scale)[row] = (uint16_t)(__float_as_uint(s) >> 16);
+    }
+    int8_t* qr = q + row * chunks_per_row * kPer;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+        int64_t ci = lane + (int64_t)i * kTpr;
+        if (ci < chunks_per_row) {
+            float f[kPer];
+            chunk_to_floats<kDtype>(c[i], f);
+            u32 w[kPer / 4];
+#pragma unroll
+            for (int d = 0; d < kPer / 4; ++d) {
+                u32 b0 = (u32)quantize_one<kDtype>(f[4 * d + 0], s, qlo, qhi) & 0xffu;
+                u32 b1 = (u32)quantize_one<kDtype>(f[4 * d + 1], s, qlo, qhi) & 0xffu;
+                u32 b2 = (u32)quantize_one<kDtype>(f[4 * d + 2], s, qlo, qhi) & 0xffu;
+                u32 b3 = (u32)quantize_one<kDtype>(f[4 * d + 3], s, qlo, qhi) & 0xffu;
+                w[d] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            }
+            if (kPer == 4) {
+                __builtin_nontemporal_store(w[0], (u32*)(qr + ci * 4));
+            } else {
+                v2u o = {w[0], w[1]};
+                __builtin_nontemporal_store(o, (v2u*)(qr + ci * 8));
+            }
+        }
+    }
+}
+
+// Any shape / alignment, and rows too long for the register-resident path:
+// one block per row, two passes over the row (the second one hits L2).
+template <int kDtype>
+__global__ __launch_bounds__(256) void quantize_rows_generic(const char* __restrict__ x,
+                                                             int64_t cols, int64_t x_row_stride,
+                                                             float eps, float qlo, float qhi,
+                                                             int8_t* __restrict__ q,
+                                                             void* __restrict__ scale) {
+    __shared__ float lds[256 / kWave];
+    const int64_t row = blockIdx.x;
+    float amax = 0.0f;
+    auto load = [&](int64_t c) -> float {
+        if (kDtype == K3Q_F32) return ((const float*)x)[row * x_row_stride + c];
+        return bf16_bits_to_f32(((const uint16_t*)x)[row * x_row_stride + c]);
+    };
+    for (int64_t c = threadIdx.x; c < cols; c += 256) amax = fmaxf(amax, fabsf(load(c)));
+    amax = row_max<256>(amax, lds);
+    const float s = scale_from_amax<kDtype>(amax, eps, qhi);
+    if (threadIdx.x == 0) {
+        if (kDtype == K3Q_F32)
+            ((float*)scale)[row] = s;
+        else
+            ((uint16_t*)scale)[row] = (uint16_t)(__float_as_uint(s) >> 16);
+    }
+    for (int64_t c = threadIdx.x; c < cols; c += 256)
+        q[row * cols + c] = (int8_t)quantize_one<kDtype>(load(c), s, qlo, qhi);
+}
+
+template <int kDtype, int kTpr, int kChunks>
+void launch_vec(const void* x, int64_t rows, int64_t chunks_per_row, int64_t row_bytes, float eps,
+                float qlo, float qhi, int8_t* q, void* scale, hipStream_t s) {
+    constexpr int kRowsPerBlock = 256 / kTpr;
+    unsigned blocks = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+    quantize_rows_vec<kDtype, kTpr, kChunks><<<blocks, 256, 0, s>>>(
+        (const char*)x, rows, chunks_per_row, row_bytes, eps, qlo, qhi, q, scale);
+}
+
+template <int kDtype>
+int dispatch(const void* x, int64_t rows, int64_t cols, int64_t stride, float eps, float qlo,
+             float qhi, int8_t* q, void* scale, hipStream_t s) {
+    constexpr int kPer = Elem<kDtype>::kPerChunk;
+    constexpr int kBytes = Elem<kDtype>::kBytes;
+    const bool vec_ok = (cols % kPer) == 0 && ((stride * kBytes) % 16) == 0 && aligned_to(x, 16) &&
+                        aligned_to(q, 8);
+    const int64_t cpr = cols / kPer;
+    const int64_t rb = stride * kBytes;
+    if (vec_ok && cpr <= 64 * 4) {
+        if (cpr <= 64)
+            launch_vec<kDtype, 64, 1>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+        else if (cpr <= 128)
+            launch_vec<kDtype, 64, 2>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+        else
+            launch_vec<kDtype, 64, 4>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+    } else if (vec_ok && cpr <= 256 * 16) {
+        if (cpr <= 256 * 2)
+            launch_vec<kDtype, 256, 2>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+        else if (cpr <= 256 * 4)
+            launch_vec<kDtype, 256, 4>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+        else if (cpr <= 256 * 8)
+            launch_vec<kDtype, 256, 8>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+        else
+            launch_vec<kDtype, 256, 16>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+    } else {
+        quantize_rows_generic<kDtype><<<(unsigned)rows, 256, 0, s>>>((const char*)x, cols, stride,
+                                                                     eps, qlo, qhi, q, scale);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace k3q
+
+using namespace k3q;
+
+extern "C" int k3q_absmax_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                                   int64_t x_row_stride, float eps, float qlo, float qhi,
+                                   int8_t* q, void* scale, void* stream) {
+    if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (rows < 0 || cols < 0 || x_row_stride < cols) return K3Q_ERR_SHAPE;
+    if (rows > 0x7fffffff) return K3Q_ERR_SHAPE;
+    if (!(qlo >= -128.0f && qhi <= 127.0f && qlo <= qhi)) return K3Q_ERR_RANGE;
+    if (rows == 0) return K3Q_OK;
+    if (cols == 0) return K3Q_ERR_SHAPE;  // the reference raises on an empty reduction
+    if (!x || !q || !scale) return K3Q_ERR_NULL;
+    if (!aligned_to(x, x_dtype == K3Q_F32 ? 4 : 2) || !aligned_to(scale, x_dtype == K3Q_F32 ? 4 : 2))
+        return K3Q_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    if (x_dtype == K3Q_F32)
+        return dispatch<K3Q_F32>(x, rows, cols, x_row_stride, eps, qlo, qhi, q, scale, s);
+    // torch rounds the epsilon operand to the tensor dtype before the add
+    const float eps_bf16 = host_round_bf16(eps);
+    return dispatch<K3Q_BF16>(x, rows, cols, x_row_stride, eps_bf16, qlo, qhi, q, scale, s);
+}

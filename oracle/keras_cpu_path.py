@@ -1,0 +1,568 @@
+"""CPU restatement of the Keras 3 quantized-inference path (torch-CPU backend).
+
+TEST INFRASTRUCTURE ONLY -- never imported by ``keras_amd``.  Every function
+issues the same torch / numpy primitive sequence that the reference lowers to
+on ``KERAS_BACKEND=torch`` with tensors on the CPU, so integer results are the
+reference's results and float results carry the reference's per-op rounding.
+
+Pinning status (what makes each function trustworthy without importing the
+reference) is listed per function; ``tests/test_oracle_*.py`` holds the checks.
+
+Reference citations are relative to the keras-team/keras 3.16.0 tree.
+"""
+
+import math
+import re
+
+import numpy as np
+import torch
+
+EPSILON = 1e-7  # keras/src/backend/config.py:10 (bound at import in quantizers.py:75)
+
+_TORCH_DTYPES = {
+    "float32": torch.float32,
+    "bfloat16": torch.bfloat16,
+    "float16": torch.float16,
+    "int8": torch.int8,
+    "uint8": torch.uint8,
+    "int32": torch.int32,
+}
+
+
+def _tdtype(name):
+    return name if isinstance(name, torch.dtype) else _TORCH_DTYPES[name]
+
+
+def _scalar_tensor(v):
+    """Python scalar -> 0-dim tensor as `convert_to_tensor` does.
+
+    keras/src/backend/torch/core.py:215-226: int -> int32 (int64 when out of
+    range), float -> floatx (float32).
+    """
+    if isinstance(v, bool):
+        return torch.as_tensor(v, dtype=torch.bool)
+    if isinstance(v, int):
+        dt = torch.int64 if v < -(2**31) or v >= 2**31 else torch.int32
+        return torch.as_tensor(v, dtype=dt)
+    return torch.as_tensor(v, dtype=torch.float32)
+
+
+# --------------------------------------------------------------------------
+# a1 / a2: abs-max quantizer
+# --------------------------------------------------------------------------
+def abs_max_quantize(
+    inputs,
+    axis,
+    value_range=(-127, 127),
+    dtype="int8",
+    epsilon=EPSILON,
+    to_numpy=False,
+):
+    """keras/src/quantizers/quantizers.py:70-120.
+
+    Pinned by: identical primitive sequence; invariants of
+    quantizers_test.py:71-115 (dtype, keepdims scale shape, +-127 range,
+    numpy path == tensor path); closed-form special rows (all-zero row,
+    arg-max element maps to +-127, ties to even); an independent C
+    restatement (oracle/k3q_oracle.c) with explicit bf16 rounding.
+    """
+    if to_numpy:
+        # quantizers.py:95-109 (numpy float math on the host)
+        t = inputs if isinstance(inputs, torch.Tensor) else torch.as_tensor(inputs)
+        original_dtype = t.dtype
+        arr = t.float().numpy() if t.dtype == torch.bfloat16 else t.numpy()
+        if isinstance(axis, list):
+            axis = tuple(axis)
+        scale = np.divide(
+            value_range[1],
+            np.add(np.max(np.abs(arr), axis=axis, keepdims=True), epsilon),
+        )
+        outputs = np.multiply(arr, scale)
+        outputs = np.clip(np.round(outputs), value_range[0], value_range[1])
+        outputs = outputs.astype(dtype)
+        return torch.from_numpy(outputs), torch.from_numpy(
+            np.asarray(scale)
+        ).to(original_dtype)
+
+    x = inputs if isinstance(inputs, torch.Tensor) else torch.as_tensor(inputs)
+    if isinstance(axis, list):
+        axis = tuple(axis)
+    amax = torch.amax(torch.abs(x), dim=axis, keepdim=True)  # numpy.py:298-305
+    denom = torch.add(amax, _scalar_tensor(float(epsilon)))  # numpy.py:68-71
+    scale = torch.divide(value_range[1], denom)  # numpy.py:2192-2197
+    scale = scale.to(x.dtype)
+    outputs = torch.multiply(x, scale)
+    outputs = torch.clip(  # numpy.py:640-653, round :2077-2084
+        torch.round(outputs),
+        min=_scalar_tensor(value_range[0]),
+        max=_scalar_tensor(value_range[1]),
+    )
+    outputs = outputs.to(_tdtype(dtype))
+    return outputs, scale
+
+
+class AbsMaxQuantizer:
+    """keras/src/quantizers/quantizers.py:307-373 (axis precedence only)."""
+
+    def __init__(self, axis=None, value_range=(-127, 127), epsilon=EPSILON,
+                 output_dtype="int8"):
+        if axis is not None and isinstance(axis, int):
+            axis = (axis,)
+        self.axis = None if axis is None else tuple(axis)
+        self.value_range = value_range
+        self.epsilon = epsilon
+        self.output_dtype = output_dtype
+
+    def __call__(self, x, axis=None, to_numpy=False):
+        if axis is None:
+            axis = self.axis
+        if axis is None:
+            axis = -1
+        return abs_max_quantize(
+            x, axis, self.value_range, self.output_dtype, self.epsilon, to_numpy
+        )
+
+
+# --------------------------------------------------------------------------
+# a6: grouped asymmetric quantizer (numpy variant, the one layers use)
+# --------------------------------------------------------------------------
+def abs_max_quantize_grouped_with_zero_point(
+    inputs, block_size, value_range=(-8, 7), dtype="int8", epsilon=EPSILON
+):
+    """keras/src/quantizers/quantizers.py:179-234.
+
+    Pinned by: closed forms checked with a per-(group, column) Python loop;
+    shape / padding cases of quantizers_test.py:790-811; dequantised RMSE
+    bound of quantizers_test.py:754-788.
+    """
+    t = inputs if isinstance(inputs, torch.Tensor) else torch.as_tensor(inputs)
+    original_dtype = t.dtype
+    arr = t.float().numpy() if t.dtype == torch.bfloat16 else t.numpy()
+    input_dim, output_dim = arr.shape
+    n_groups = math.ceil(input_dim / block_size)
+    qmin, qmax = value_range
+    padded = n_groups * block_size
+    if padded > input_dim:
+        arr = np.concatenate(
+            [arr, np.zeros((padded - input_dim, output_dim), dtype=arr.dtype)],
+            axis=0,
+        )
+    g = arr.reshape(n_groups, block_size, output_dim)
+    min_val = np.min(g, axis=1, keepdims=True)
+    max_val = np.max(g, axis=1, keepdims=True)
+    scale = np.divide(np.subtract(max_val, min_val) + epsilon, qmax - qmin)
+    zero = np.round(np.divide(-min_val, scale)) + qmin
+    zero = np.clip(zero, qmin, qmax)
+    q = np.round(np.divide(g, scale)) + zero
+    q = np.clip(q, qmin, qmax).astype(dtype)
+    q = q.reshape(padded, output_dim)[:input_dim, :]
+    scale = np.squeeze(scale, axis=1)
+    zero = np.squeeze(zero, axis=1).astype("int8")
+    return (
+        torch.from_numpy(np.ascontiguousarray(q)),
+        torch.from_numpy(scale).to(original_dtype),
+        torch.from_numpy(zero),
+    )
+
+
+# --------------------------------------------------------------------------
+# a4 / a5: int4 packing
+# --------------------------------------------------------------------------
+def pack_int4(arr, axis=0, dtype="int8"):
+    """keras/src/quantizers/quantizers.py:700-750.
+
+    Pinned by: docstring known-answer vectors (quantizers.py:655-697), the
+    closed form over all 256 (lo, hi) pairs, odd-length padding.
+    """
+    if dtype not in ("int8", "uint8"):
+        raise ValueError(
+            f"Expected dtype to be 'int8' or 'uint8', but got '{dtype}'."
+        )
+    a = arr.numpy() if isinstance(arr, torch.Tensor) else np.asarray(arr)
+    if str(a.dtype) != dtype:
+        raise TypeError(
+            f"Expected {dtype} tensor for packing, got {a.dtype}."
+        )
+    np_dtype = np.dtype(dtype)
+    if axis < 0:
+        axis += a.ndim
+    a = np.moveaxis(a, axis, 0)
+    n = a.shape[0]
+    if n % 2 == 1:
+        a = np.concatenate(
+            [a, np.zeros((1,) + a.shape[1:], dtype=a.dtype)], axis=0
+        )
+    low = a[::2]
+    high = a[1::2]
+    mask = np.array(0x0F, dtype=np_dtype)
+    low_u = np.bitwise_and(low.astype(np_dtype), mask)
+    high_u = np.bitwise_and(high.astype(np_dtype), mask)
+    packed = np.bitwise_or(
+        low_u, np.left_shift(high_u, np.array(4, dtype=np_dtype))
+    ).astype(np_dtype)
+    packed = np.moveaxis(packed, 0, axis)
+    return torch.from_numpy(np.ascontiguousarray(packed)), tuple(packed.shape), n
+
+
+def unpack_int4(packed, orig_len, axis=0, dtype="int8"):
+    """keras/src/quantizers/quantizers.py:830-900 (torch primitive sequence).
+
+    Pinned by: docstring vectors (quantizers.py:786-827), the exhaustive
+    256-byte table, round trips over the 7 scenarios of
+    quantizers_test.py:157-175.
+    """
+    if dtype not in ("int8", "uint8"):
+        raise ValueError(
+            f"Expected dtype to be 'int8' or 'uint8', but got '{dtype}'."
+        )
+    p = packed if isinstance(packed, torch.Tensor) else torch.as_tensor(packed)
+    if p.dtype not in (torch.int8, torch.uint8):
+        raise TypeError(
+            f"Expected int8 or uint8 tensor for unpacking, got {p.dtype}"
+        )
+    out_dtype = _tdtype(dtype)
+    rank = p.dim()
+    if axis < 0:
+        axis += rank
+
+    def to_signed(x):
+        eight = torch.as_tensor(8, dtype=x.dtype)
+        return torch.subtract(torch.bitwise_xor(x, eight), eight)
+
+    perm = [axis] + [i for i in range(rank) if i != axis]
+    inv_perm = [perm.index(i) for i in range(rank)]
+    t = p.permute(perm)
+    mask = torch.as_tensor(0x0F, dtype=p.dtype)
+    low = torch.bitwise_and(t, mask)
+    high = torch.bitwise_and(torch.bitwise_right_shift(t, 4), mask)
+    if dtype == "int8":
+        low = to_signed(low)
+        high = to_signed(high)
+    low = low.to(out_dtype)
+    high = high.to(out_dtype)
+    stacked = torch.stack([low, high], dim=1)
+    unpacked = torch.reshape(stacked, (-1,) + tuple(t.shape[1:]))
+    unpacked = unpacked[:orig_len, ...]
+    return unpacked.permute(inv_perm)
+
+
+# --------------------------------------------------------------------------
+# a7: group de-quantisation
+# --------------------------------------------------------------------------
+def dequantize_with_sz_map(weights_matrix, scale, zero, g_idx, group_axis=-1):
+    """keras/src/quantizers/quantizers.py:1631-1668.
+
+    Pinned by: manual double loop (mirrors quantizers_test.py:1193-1293).
+    """
+    groups = g_idx.to(torch.int32).long()
+    scales_mapped = torch.index_select(scale, group_axis % scale.dim(), groups)
+    zeros_mapped = torch.index_select(zero, group_axis % zero.dim(), groups)
+    zeros_mapped = zeros_mapped.to(scales_mapped.dtype)
+    return torch.multiply(
+        torch.subtract(weights_matrix, zeros_mapped), scales_mapped
+    )
+
+
+# --------------------------------------------------------------------------
+# a9 / a12: backend matmul / einsum on CPU
+# --------------------------------------------------------------------------
+def _result_float(d1, d2):
+    # keras/src/backend/common/dtypes.py:281-324 restricted to the pairs the
+    # path produces: (float, int8) -> the float; (float, float) -> wider.
+    floats = [d for d in (d1, d2) if d.is_floating_point]
+    if not floats:
+        raise TypeError("integer result types other than int8xint8 unused")
+    if len(floats) == 1:
+        return floats[0]
+    if floats[0] == floats[1]:
+        return floats[0]
+    return torch.float32
+
+
+def matmul(x1, x2):
+    """keras/src/backend/torch/numpy.py:101-157, device == 'cpu'.
+
+    int8 x int8 -> int32 exact.  Pinned by numpy int64 brute force.
+    """
+    if x1.dtype == torch.int8 and x2.dtype == torch.int8:
+        return torch.matmul(x1.to(torch.int32), x2.to(torch.int32)).to(
+            torch.int32
+        )
+    rd = _result_float(x1.dtype, x2.dtype)
+    cd = torch.float32 if rd == torch.float16 else rd
+    return torch.matmul(x1.to(cd), x2.to(cd)).to(rd)
+
+
+def einsum(subscripts, *operands):
+    """keras/src/backend/torch/numpy.py:74-87, device == 'cpu'."""
+    if all(o.dtype == torch.int8 for o in operands):
+        ops32 = [o.to(torch.int32) for o in operands]
+        return torch.einsum(subscripts, *ops32).to(torch.int32)
+    return torch.einsum(subscripts, *operands)
+
+
+# --------------------------------------------------------------------------
+# a15: Dense.quantize -- host-side, one-time
+# --------------------------------------------------------------------------
+def dense_quantize_int8(kernel):
+    """keras/src/layers/core/dense.py:1214-1226. -> (int8 [K,N], scale [N])."""
+    q, s = AbsMaxQuantizer(axis=0)(kernel, to_numpy=True)
+    return q, torch.squeeze(s, dim=0)
+
+
+def dense_quantize_int4(kernel, block_size=128):
+    """keras/src/layers/core/dense.py:1227-1275.
+
+    Returns dict(kernel=packed int8 [K, ceil(N/2)], kernel_scale, kernel_zero,
+    g_idx) with absent entries set to None.
+    """
+    K, N = kernel.shape
+    if block_size is None or block_size == -1:
+        q, s = AbsMaxQuantizer(axis=0, value_range=(-8, 7))(kernel, to_numpy=True)
+        s = torch.squeeze(s, dim=0)
+        zero = None
+        g_idx = None
+    else:
+        q, s, zero = abs_max_quantize_grouped_with_zero_point(
+            kernel, block_size=block_size
+        )
+        # dense.py:868-889: float32 floor(arange(K) / block_size)
+        g_idx = torch.floor_divide(
+            torch.arange(K, dtype=torch.float32), block_size
+        )
+    packed, _, _ = pack_int4(q, axis=-1)
+    return dict(kernel=packed, kernel_scale=s, kernel_zero=zero, g_idx=g_idx,
+                unpacked=q)
+
+
+# --------------------------------------------------------------------------
+# a8 / a10: Dense forward
+# --------------------------------------------------------------------------
+def _read_var(v, compute_dtype):
+    """AutocastScope: float variables are read in the compute dtype
+    (keras/src/backend/common/variables.py:245-249, :677-708)."""
+    if v is None:
+        return None
+    if v.dtype.is_floating_point and v.dtype != compute_dtype:
+        return v.to(compute_dtype)
+    return v
+
+
+def dense_int8_call(inputs, kernel, kernel_scale, bias=None,
+                    compute_dtype=None, quantize_inputs=True,
+                    return_intermediates=False):
+    """keras/src/layers/core/dense.py:938-986 (forward only).
+
+    `inputs` must already be in the layer compute dtype
+    (keras/src/layers/layer.py:883-901 casts before `call`).
+    """
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    ks = _read_var(kernel_scale, cd)
+    output_scale = ks
+    q = inputs
+    s_in = None
+    if quantize_inputs:
+        q, s_in = AbsMaxQuantizer()(inputs, axis=-1)
+        output_scale = torch.multiply(output_scale, s_in)
+    acc = matmul(q, kernel)
+    x = acc.to(cd)
+    x = torch.divide(x, output_scale)
+    if bias is not None:
+        x = torch.add(x, _read_var(bias, cd))
+    if return_intermediates:
+        return x, dict(q=q, inputs_scale=s_in, acc=acc)
+    return x
+
+
+def dense_int4_call(inputs, kernel, kernel_scale, orig_output_dim,
+                    kernel_zero=None, g_idx=None, block_size=None, bias=None,
+                    compute_dtype=None, quantize_inputs=False,
+                    return_intermediates=False):
+    """keras/src/layers/core/dense.py:988-1095 (forward only)."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    ks = _read_var(kernel_scale, cd)
+    unpacked = unpack_int4(kernel, orig_output_dim, axis=-1)
+    inter = dict(unpacked=unpacked)
+    if block_size is None or block_size == -1:
+        output_scale = ks
+        xin = inputs
+        if quantize_inputs:
+            xin, s_in = AbsMaxQuantizer()(inputs, axis=-1)
+            output_scale = torch.multiply(output_scale, s_in)
+            inter.update(q=xin, inputs_scale=s_in)
+        x = matmul(xin, unpacked)
+        if quantize_inputs:
+            inter["acc"] = x
+        x = x.to(cd)
+        x = torch.divide(x, output_scale)
+    else:
+        float_kernel = dequantize_with_sz_map(
+            unpacked, ks, kernel_zero, g_idx, group_axis=0
+        )
+        float_kernel = float_kernel.to(cd)
+        x = matmul(inputs, float_kernel)
+    if bias is not None:
+        x = torch.add(x, _read_var(bias, cd))
+    if return_intermediates:
+        return x, inter
+    return x
+
+
+# --------------------------------------------------------------------------
+# a11 / a13: EinsumDense
+# --------------------------------------------------------------------------
+def _einsum_specs(equation, input_rank):
+    """Canonical (input, kernel, output) label strings.
+
+    keras/src/layers/core/einsum_dense.py:1932-1993 (`get_specs`): ellipses
+    are replaced by fresh labels, padded left or right.
+    """
+    eq = equation.replace(" ", "")
+    lhs, out = eq.split("->")
+    a, b = lhs.split(",")
+    if "..." not in eq:
+        return a, b, out
+    used = set(eq) - set(".,->")
+    spare = sorted(set("abcdefghijklmnopqrstuvwxyzABCDEFGHIJKLMNOPQRSTUVWXYZ") - used)
+    if a.startswith("..."):
+        core_in, core_out = a[3:], out[3:]
+        n = input_rank - len(core_in)
+        pad = "".join(spare[:n])
+        return pad + core_in, b, pad + core_out
+    core_in, core_out = a[:-3], out[:-3]
+    n = input_rank - len(core_in)
+    pad = "".join(spare[:n])
+    return core_in + pad, b, core_out + pad
+
+
+def einsum_quantization_info(equation, input_rank):
+    """keras/src/layers/core/einsum_dense.py:1902-2062, restated.
+
+    Returns a dict with the reference's ten fields.  Pinned by: the
+    hand-derived rows for 'btd,dnh->btnh' and 'btnh,nhd->btd'; the
+    mathematical requirement that `inputs_scale * kernel_scale` broadcast
+    against the einsum output so that the de-scaled int8 einsum approximates
+    the float einsum (tests sweep the equations of einsum_dense_test.py).
+    """
+    i_spec, k_spec, o_spec = _einsum_specs(equation, input_rank)
+    info = {}
+    for name, spec in (("input", i_spec), ("kernel", k_spec)):
+        info[name] = dict(
+            reduced=[i for i, c in enumerate(spec) if c not in o_spec],
+            expand=[i for i, c in enumerate(o_spec) if c not in spec],
+            transpose=[spec.index(c) for c in o_spec if c in spec],
+            squeeze=[],
+        )
+    # Reference quirk (:2027-2040): one Python variable `index` is shared by
+    # the label scans and both post-processing loops, so when the expand list
+    # runs dry the last value it held is reused for the transpose insert.  On
+    # entry it holds output_spec.find(<last kernel label>).
+    index = o_spec.find(k_spec[-1])
+    for name in ("input", "kernel"):
+        part = info[name]
+        for ori in part["reduced"]:
+            if part["expand"]:
+                index = part["expand"].pop(0)
+            else:
+                part["squeeze"].append(ori)
+            part["transpose"].insert(index, ori)
+    kt = info["kernel"]["transpose"]
+    info["custom_gradient_equation"] = f"{o_spec},{k_spec}->{i_spec}"
+    info["kernel_reverse_transpose"] = [
+        i for (_, i) in sorted((v, i) for (i, v) in enumerate(kt))
+    ]
+    info["specs"] = (i_spec, k_spec, o_spec)
+    return info
+
+
+def _adjust_scale(scale, part):
+    """einsum_dense.py:1650-1680: transpose, expand_dims, squeeze."""
+    if part["transpose"]:
+        scale = scale.permute(part["transpose"])
+    for a in sorted(part["expand"]):
+        scale = torch.unsqueeze(scale, a)
+    for a in sorted(part["squeeze"], reverse=True):
+        scale = torch.squeeze(scale, a)
+    return scale
+
+
+def einsum_dense_quantize_int8(kernel, equation, input_rank):
+    """keras/src/layers/core/einsum_dense.py:1364-1381."""
+    info = einsum_quantization_info(equation, input_rank)
+    q, s = AbsMaxQuantizer(axis=tuple(info["kernel"]["reduced"]))(
+        kernel, to_numpy=True
+    )
+    s = _adjust_scale(s, info["kernel"])
+    return q, s.contiguous(), info
+
+
+def einsum_dense_int8_call(inputs, kernel, kernel_scale, equation, bias=None,
+                           compute_dtype=None, return_intermediates=False):
+    """keras/src/layers/core/einsum_dense.py:1030-1118 (forward only)."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    info = einsum_quantization_info(equation, inputs.dim())
+    ks = _read_var(kernel_scale, cd)
+    q, s_in = AbsMaxQuantizer()(inputs, axis=tuple(info["input"]["reduced"]))
+    s_adj = _adjust_scale(s_in, info["input"])
+    acc = einsum(equation, q, kernel)
+    x = acc.to(cd)
+    x = torch.divide(x, torch.multiply(s_adj, ks))
+    if bias is not None:
+        x = torch.add(x, _read_var(bias, cd))
+    if return_intermediates:
+        return x, dict(q=q, inputs_scale=s_in, acc=acc)
+    return x
+
+
+def einsum_dense_quantize_int4(kernel, equation, input_rank, block_size=128):
+    """keras/src/layers/core/einsum_dense.py:1382-1430: the kernel is flattened
+    row-major to [rows = prod(reduced dims), cols = prod(kept dims)] and then
+    quantised / packed exactly like a Dense kernel."""
+    info = einsum_quantization_info(equation, input_rank)
+    red = info["kernel"]["reduced"]
+    rows = 1
+    cols = 1
+    for i, d in enumerate(kernel.shape):
+        if i in red:
+            rows *= d
+        else:
+            cols *= d
+    flat = torch.reshape(kernel, (rows, cols))
+    out = dense_quantize_int4(flat, block_size)
+    out.update(rows=rows, cols=cols, info=info,
+               original_kernel_shape=tuple(kernel.shape))
+    return out
+
+
+def einsum_dense_int4_call(inputs, qk, equation, bias=None, compute_dtype=None,
+                           block_size=128):
+    """keras/src/layers/core/einsum_dense.py:1120-1261 (forward, weight-only)."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    ks = _read_var(qk["kernel_scale"], cd)
+    unpacked = unpack_int4(qk["kernel"], qk["cols"], axis=-1)
+    if block_size is None or block_size == -1:
+        float_kernel = torch.divide(unpacked.to(cd), ks)
+    else:
+        float_kernel = dequantize_with_sz_map(
+            unpacked, ks, qk["kernel_zero"], qk["g_idx"], group_axis=0
+        ).to(cd)
+    float_kernel = torch.reshape(float_kernel, qk["original_kernel_shape"])
+    x = torch.einsum(equation, inputs, float_kernel)
+    if bias is not None:
+        x = torch.add(x, _read_var(bias, cd))
+    return x
+
+
+# --------------------------------------------------------------------------
+# helpers shared by tests / bench (input generators named in the configs)
+# --------------------------------------------------------------------------
+def glorot_uniform(fan_in, fan_out, shape=None, generator=None):
+    """U(-L, L), L = sqrt(6 / (fan_in + fan_out))
+    (keras/src/initializers/random_initializers.py:292-318)."""
+    limit = math.sqrt(6.0 / (fan_in + fan_out))
+    shape = shape or (fan_in, fan_out)
+    return (torch.rand(shape, generator=generator) * 2.0 - 1.0) * limit
