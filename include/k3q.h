@@ -75,6 +75,41 @@ int k3q_pack_int4(const void* in, int64_t outer, int64_t len, int64_t inner,
 int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t inner,
                     int64_t orig_len, int is_signed, void* out, void* stream);
 
+/*
+ * Weight-only int4 matmul for decode-sized inputs (any M; tuned for M <= 16):
+ *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)
+ *     grouped     (block_size  > 0):  y = T(x . ((unpack(w) - zero[g]) * scale[g]))  (+ bias),  g = k / block_size
+ * x: [M, K] of x_dtype, contiguous.  w_packed: the layer's int4 kernel as stored,
+ * int8 [K, ceil(N/2)], low nibble = even column.  scale: x_dtype, [N] or
+ * [ceil(K/block_size), N].  zero: int8 [ceil(K/block_size), N] (grouped only).
+ * bias: x_dtype [N] or null.  y: x_dtype [M, N].  The packed kernel is read
+ * once from HBM and is neither unpacked nor de-quantised in memory.
+ * Replaces, per call, unpack_int4 + (dequantize_with_sz_map | cast) + matmul +
+ * divide of Dense._int4_call (keras/src/layers/core/dense.py:988-1095) and the
+ * int4 branch of EinsumDense (keras/src/layers/core/einsum_dense.py:1120-1261).
+ *
+ * workspace: k3q_gemv_w4_workspace_bytes(M, K, N) bytes, 16-byte aligned, whose
+ * first 4096 bytes are ZERO before the first call; the kernel leaves them zero.
+ * It holds split-K partial sums and per-column-block arrival tickets, so two
+ * calls that overlap in time must not share a workspace.
+ */
+int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N);
+int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                const void* w_packed, const void* scale, const void* zero,
+                int64_t block_size, const void* bias, void* y, void* workspace,
+                int64_t workspace_bytes, void* stream);
+
+/*
+ * Same as k3q_gemv_w4 with the launch plan overridden, for tuning sweeps:
+ * plan = {dwords per lane per k row (1|2|4), 16-row steps per chunk (1|2),
+ * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null
+ * `plan` keep the built-in choice.  No counterpart in the reference.
+ */
+int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                     const void* w_packed, const void* scale, const void* zero,
+                     int64_t block_size, const void* bias, void* y, void* workspace,
+                     int64_t workspace_bytes, const int* plan, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

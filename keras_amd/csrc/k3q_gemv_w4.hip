@@ -1,0 +1,595 @@
+// Weight-only int4 skinny matmul (decode sizes): y[M,N] = x[M,K] . W4[K,N].
+//
+// W4 is the Dense int4 kernel exactly as the layer stores it: int8 bytes
+// [K, ceil(N/2)], low nibble = even output column, high nibble = odd column.
+// The kernel is HBM-bound on those bytes, so the design rule is: every packed
+// byte is fetched once, with 16-byte loads that are contiguous along N, goes
+// straight into registers, and is never re-laid-out in memory.
+//
+// How nibbles that are contiguous along N reach a matrix core that wants
+// operands contiguous along K:
+//   v_mfma_f32_16x16x32_bf16 computes D[i,j] = sum_s A[i,s] * B[s,j] over 32
+//   "slots" s.  Lane (i = lane%16, g = lane/16) supplies slots 8g..8g+7 of row
+//   i as four dwords of two bf16 each.  A lane loads 16 bytes (32 columns) of
+//   four consecutive k rows.  For dword q (8 columns) and nibble position p in
+//   0..3, ((w >> 4p) & 0x000F000F) | 0x43004300 is, with no further work, the
+//   bf16 pair (128 + nibble p, 128 + nibble p+4): two DIFFERENT output columns
+//   of the same k.  Those two values are placed in an even and an odd slot, and
+//   the x operand is built so that column j < 8 of B carries x only in even
+//   slots and column j >= 8 only in odd slots.  D[i, j<8] is then the partial
+//   dot product for column (p), D[i, j>=8] the one for column (p + 4), for row
+//   m = j % 8 of x.  Half of the MFMA work multiplies zeros; the matrix core
+//   has >3x headroom over HBM here, so that is free, and the conversion costs
+//   one VALU op per weight.
+//   Nibbles are XOR-ed with 8 first, so the bf16 value is (signed nibble + 136);
+//   an extra MFMA against an all-ones A accumulates sum_k x, and the offset is
+//   removed as acc - 136 * sum_x (grouped: scale * (acc - (136 + zero) * sum_x)
+//   per group, which also folds the zero point).
+//
+// Split-K: wave w of workgroup (nb, ks) owns `klen` consecutive rows of K for
+// the 128 * kVec columns of block nb and walks them in register double-buffered
+// chunks of kSteps * 16 rows.  Waves of a workgroup are reduced through LDS,
+// workgroups through an fp32 scratch in `workspace`; the workgroup that
+// arrives last at a column block (atomic ticket) adds the partials in a fixed
+// order, applies the epilogue and re-arms the ticket.  The result does not
+// depend on arrival order.
+#include "k3q_common.h"
+
+namespace k3q {
+namespace {
+
+constexpr u32 kMagic = 0x43004300u;
+constexpr u32 kNibblePair = 0x000F000Fu;
+constexpr u32 kOnes = 0x3F803F80u;
+constexpr float kOffset = 136.0f;  // 128 (bf16 magic exponent) + 8 (nibble ^ 8)
+constexpr int kMaxWaves = 8;
+constexpr int kLdsBudget = 64 * 1024;
+
+struct GemvParams {
+    const void* x;         // [M, K] bf16 or f32
+    const uint8_t* w;      // [K, row_bytes]
+    const void* scale;     // T [N] or [G, N]
+    const int8_t* zero;    // [G, N] or null
+    const void* bias;      // T [N] or null
+    void* y;               // T [M, N]
+    float* part;           // [KS, M, N] fp32 partials (KS > 1)
+    u32* tickets;          // [n_blocks]
+    int64_t K, N, row_bytes;
+    int M;                 // rows of x in this launch
+    int m0;                // first row of x handled by this launch
+    int block_size;        // rows of K per group (grouped only)
+    int klen;              // rows of K per wave (multiple of the chunk)
+};
+
+__device__ __forceinline__ v8bf as_bf(const v4u& v) { return __builtin_bit_cast(v8bf, v); }
+
+template <bool kBF16>
+__device__ __forceinline__ float load_t(const void* p, int64_t i) {
+    if (kBF16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+    return ((const float*)p)[i];
+}
+
+// epilogue of Dense._int4_call in the layer dtype T
+template <bool kBF16, bool kGrouped>
+__device__ __forceinline__ void finish(const GemvParams& p, int m, int64_t n, float sum) {
+    float v = sum;
+    if (kBF16) {
+        v = round_bf16(v);
+        if (!kGrouped) v = round_bf16(v / load_t<true>(p.scale, n));
+        if (p.bias) v = round_bf16(v + load_t<true>(p.bias, n));
+        ((uint16_t*)p.y)[(int64_t)(p.m0 + m) * p.N + n] = (uint16_t)(__float_as_uint(v) >> 16);
+    } else {
+        if (!kGrouped) v = v / load_t<false>(p.scale, n);
+        if (p.bias) v = v + load_t<false>(p.bias, n);
+        ((float*)p.y)[(int64_t)(p.m0 + m) * p.N + n] = v;
+    }
+}
+
+template <int kVec>
+struct Packed {
+    u32 d[kVec];
+};
+
+template <int kVec>
+__device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
+    Packed<kVec> r;
+    if (kVec == 4) {
+        v4u v = __builtin_nontemporal_load((const v4u*)p);
+#pragma unroll
+        for (int q = 0; q < kVec; ++q) r.d[q] = v[q];
+    } else if (kVec == 2) {
+        v2u v = __builtin_nontemporal_load((const v2u*)p);
+#pragma unroll
+        for (int q = 0; q < kVec; ++q) r.d[q] = v[q];
+    } else {
+        r.d[0] = __builtin_nontemporal_load((const u32*)p);
+    }
+    return r;
+}
+
+// kVec: dwords (8 columns each) a lane loads per k row; the block is 128*kVec columns.
+// kSteps: 16-row K steps per chunk.  kSets: 1 -> up to 8 rows of bf16 x; 2 -> up to 16
+// rows of bf16 x, or up to 8 rows of f32 x split into two bf16 parts.
+template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
+__global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
+    extern __shared__ float red[];  // [waves][M][kNB]
+    constexpr bool kBF16 = !kXF32;
+    constexpr int kAccSets = kXF32 ? 1 : kSets;
+    constexpr int kNB = 128 * kVec;
+    constexpr int kChunk = kSteps * 16;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const int i = lane & 15;
+    const int g = lane >> 4;
+    const int grp = (lane >> 3) & 1;
+    const int mrow = lane & 7;
+    const int64_t nb = (int64_t)blockIdx.x * kNB;
+    const int64_t kw0 = ((int64_t)blockIdx.y * nwaves + wave) * p.klen;
+    const int nchunks = p.klen / kChunk;
+    const int M = p.M;
+
+    Packed<kVec> wreg[2][kSteps][4];
+    v4u xb[2][kSteps][kSets];
+    const int64_t ncol = nb + 8 * kVec * i;
+    const bool ncol_ok = ncol < p.N;
+    const uint8_t* wp = p.w + (ncol >> 1);
+
+    auto load_chunk = [&](int b, int c) {
+        const int64_t kc = kw0 + (int64_t)c * kChunk;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int64_t k = kc + 16 * s + 4 * g + t;
+                Packed<kVec> v;
+#pragma unroll
+                for (int q = 0; q < kVec; ++q) v.d[q] = 0u;
+                if (ncol_ok && k < p.K) v = load_packed<kVec>(wp + k * p.row_bytes);
+                wreg[b][s][t] = v;
+            }
+        }
+        // x operand: B[slot, j] holds x[m(j), k] in even (j<8) or odd (j>=8) slots
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const int64_t k = kc + 16 * s + 4 * g;
+#pragma unroll
+            for (int st = 0; st < kSets; ++st) {
+                u32 h[4] = {0u, 0u, 0u, 0u};  // bf16 bits of the four x values
+                if (kXF32) {
+                    if (mrow < M && k < p.K) {
+                        const v4u f = *(const v4u*)((const float*)p.x + (int64_t)(p.m0 + mrow) * p.K + k);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            const u32 hi = f[t] & 0xffff0000u;
+                            if (st == 0) {
+                                h[t] = hi >> 16;
+                            } else {
+                                const float rem = __uint_as_float(f[t]) - __uint_as_float(hi);
+                                h[t] = f32_to_bf16_bits(rem);
+                            }
+                        }
+                    }
+                } else {
+                    const int m = mrow + 8 * st;
+                    if (m < M && k < p.K) {
+                        const v2u d = *(const v2u*)((const uint16_t*)p.x + (int64_t)(p.m0 + m) * p.K + k);
+                        h[0] = d[0] & 0xffffu;
+                        h[1] = d[0] >> 16;
+                        h[2] = d[1] & 0xffffu;
+                        h[3] = d[1] >> 16;
+                    }
+                }
+                v4u bv;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) bv[t] = grp ? (h[t] << 16) : h[t];
+                xb[b][s][st] = bv;
+            }
+        }
+    };
+
+    v4f acc[kAccSets][kVec][4];
+    v4f accs[kAccSets];
+    v4f tot[kGrouped ? kAccSets : 1][kGrouped ? kVec : 1][kGrouped ? 4 : 1];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int a = 0; a < kAccSets; ++a) {
+            accs[a] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < kVec; ++q)
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) acc[a][q][pp] = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    clear_acc();
+    if (kGrouped) {
+#pragma unroll
+        for (int a = 0; a < kAccSets; ++a)
+#pragma unroll
+            for (int q = 0; q < kVec; ++q)
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) tot[a][q][pp] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    const v4u ones = {kOnes, kOnes, kOnes, kOnes};
+
+    auto compute_chunk = [&](int b) {
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+#pragma unroll
+            for (int st = 0; st < kSets; ++st) {
+                const int a = kXF32 ? 0 : st;
+                accs[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(ones), as_bf(xb[b][s][st]),
+                                                                  accs[a], 0, 0, 0);
+            }
+#pragma unroll
+            for (int q = 0; q < kVec; ++q) {
+                u32 d[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) d[t] = wreg[b][s][t].d[q] ^ 0x88888888u;
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    v4u av;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) av[t] = ((d[t] >> (4 * pp)) & kNibblePair) | kMagic;
+#pragma unroll
+                    for (int st = 0; st < kSets; ++st) {
+                        const int a = kXF32 ? 0 : st;
+                        acc[a][q][pp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            as_bf(av), as_bf(xb[b][s][st]), acc[a][q][pp], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+
+    // lane (j = lane%16, gq = lane/16) holds D[row 4*gq + r][col j]:
+    //   column n_local = 8*kVec*(4*gq + r) + 8*q + pp + 4*grp,  x row m = (j % 8) + 8*set
+    // grouped: fold this group's scale and zero point into the running totals
+    auto flush_group = [&](int64_t gi) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+#pragma unroll
+            for (int q = 0; q < kVec; ++q) {
+                const int64_t n = nb + 8 * kVec * (4 * g + r) + 8 * q + 4 * grp;
+                float sc[4] = {0.f, 0.f, 0.f, 0.f};
+                float zp[4] = {0.f, 0.f, 0.f, 0.f};
+                if (n < p.N) {
+                    const int64_t o = gi * p.N + n;
+                    const u32 z4 = *(const u32*)(p.zero + o);
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp) {
+                        sc[pp] = load_t<kBF16>(p.scale, o + pp);
+                        zp[pp] = (float)(int)(int8_t)(z4 >> (8 * pp));
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < kAccSets; ++a)
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp)
+                        tot[a][q][pp][r] += sc[pp] * (acc[a][q][pp][r] - (kOffset + zp[pp]) * accs[a][r]);
+            }
+        }
+        clear_acc();
+    };
+    auto after_chunk = [&](int c) {
+        if (!kGrouped) return;
+        const int64_t kend = kw0 + (int64_t)(c + 1) * kChunk;  // first row after this chunk
+        if (kend - kChunk >= p.K) return;                       // chunk entirely past K
+        if ((kend % p.block_size) == 0 || c == nchunks - 1 || kend >= p.K)
+            flush_group((kend - 1 < p.K ? kend - 1 : p.K - 1) / p.block_size);
+    };
+
+    load_chunk(0, 0);
+#pragma unroll 1
+    for (int c = 0; c < nchunks; c += 2) {
+        if (c + 1 < nchunks) load_chunk(1, c + 1);
+        compute_chunk(0);
+        after_chunk(c);
+        if (c + 2 < nchunks) load_chunk(0, c + 2);
+        if (c + 1 < nchunks) {
+            compute_chunk(1);
+            after_chunk(c + 1);
+        }
+    }
+
+    // ---- remove the +136 offset (per-channel) and park this wave's partial in LDS ----
+#pragma unroll
+    for (int a = 0; a < kAccSets; ++a) {
+        const int m = mrow + 8 * a;
+        if (m < M) {
+            float* dst = red + ((size_t)wave * M + m) * kNB;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                for (int q = 0; q < kVec; ++q) {
+                    const int nl = 8 * kVec * (4 * g + r) + 8 * q + 4 * grp;
+                    v4f o;
+#pragma unroll
+                    for (int pp = 0; pp < 4; ++pp)
+                        o[pp] = kGrouped ? tot[a][q][pp][r] : acc[a][q][pp][r] - kOffset * accs[a][r];
+                    *(v4f*)(dst + nl) = o;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- reduce the waves of this workgroup ----
+    const int KS = gridDim.y;
+    for (int idx = threadIdx.x; idx < M * kNB; idx += blockDim.x) {
+        const int m = idx / kNB;
+        const int nl = idx % kNB;
+        float sum = 0.f;
+        for (int w = 0; w < nwaves; ++w) sum += red[((size_t)w * M + m) * kNB + nl];
+        const int64_t n = nb + nl;
+        if (n < p.N) {
+            if (KS == 1)
+                finish<kBF16, kGrouped>(p, m, n, sum);
+            else
+                p.part[((int64_t)blockIdx.y * M + m) * p.N + n] = sum;
+        }
+    }
+    if (KS == 1) return;
+
+    // ---- last workgroup to arrive at this column block finishes it ----
+    __shared__ u32 ticket;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) ticket = atomicAdd(p.tickets + blockIdx.x, 1u);
+    __syncthreads();
+    if (ticket != (u32)(KS - 1)) return;
+    __threadfence();
+    for (int idx = threadIdx.x; idx < M * kNB; idx += blockDim.x) {
+        const int m = idx / kNB;
+        const int64_t n = nb + (idx % kNB);
+        if (n < p.N) {
+            float sum = 0.f;
+            for (int ks = 0; ks < KS; ++ks)
+                sum += __builtin_nontemporal_load(p.part + ((int64_t)ks * M + m) * p.N + n);
+            finish<kBF16, kGrouped>(p, m, n, sum);
+        }
+    }
+    if (threadIdx.x == 0) p.tickets[blockIdx.x] = 0u;
+}
+
+// Any shape: one thread per output, fp32 FMA chain over K.  Used when N is not a
+// multiple of 8, K not a multiple of 16, or the group size does not tile.
+template <bool kBF16, bool kGrouped>
+__global__ __launch_bounds__(256) void gemv_w4_generic(GemvParams p) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int m = blockIdx.y;
+    if (n >= p.N) return;
+    const int shift = (n & 1) ? 4 : 0;
+    const uint8_t* wp = p.w + (n >> 1);
+    float total = 0.f;
+    if (kGrouped) {
+        for (int64_t k0 = 0; k0 < p.K; k0 += p.block_size) {
+            const int64_t gi = k0 / p.block_size;
+            const float sc = load_t<kBF16>(p.scale, gi * p.N + n);
+            const float zp = (float)p.zero[gi * p.N + n];
+            float acc = 0.f;
+            const int64_t k1 = (k0 + p.block_size < p.K) ? k0 + p.block_size : p.K;
+            for (int64_t k = k0; k < k1; ++k) {
+                const int u = (wp[k * p.row_bytes] >> shift) & 0xF;
+                const float wv = (float)((u ^ 8) - 8) - zp;
+                acc = fmaf(load_t<kBF16>(p.x, (int64_t)(p.m0 + m) * p.K + k), wv, acc);
+            }
+            total = fmaf(acc, sc, total);
+        }
+    } else {
+        for (int64_t k = 0; k < p.K; ++k) {
+            const int u = (wp[k * p.row_bytes] >> shift) & 0xF;
+            total = fmaf(load_t<kBF16>(p.x, (int64_t)(p.m0 + m) * p.K + k), (float)((u ^ 8) - 8), total);
+        }
+    }
+    finish<kBF16, kGrouped>(p, m, n, total);
+}
+
+struct Plan {
+    bool fast;
+    int vec;     // dwords per lane per k row
+    int steps;   // 16-row steps per chunk
+    int sets;
+    int rows;    // rows of x per launch
+    int waves;   // waves per workgroup
+    int klen;    // rows of K per wave
+    int ks;      // workgroups along K
+};
+
+constexpr int64_t kTicketBytes = 4096;  // room for 1024 column blocks
+constexpr int kTargetWorkgroups = 512;
+
+// plan_override (may be null): {vec, steps, waves, klen}; entries <= 0 keep the heuristic.
+Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
+               const int* plan_override) {
+    Plan pl{};
+    const bool grouped = block_size > 0;
+    pl.fast = (N % 8) == 0 && (K % 16) == 0 && (!grouped || block_size % 16 == 0);
+    if (!pl.fast) return pl;
+    const bool f32 = x_dtype == K3Q_F32;
+    pl.rows = f32 ? 8 : (M > 8 ? 16 : 8);
+    pl.sets = f32 ? 2 : (M > 8 ? 2 : 1);
+    const int rows_used = (int)(M < pl.rows ? M : pl.rows);
+
+    int vec = grouped ? (pl.sets == 2 ? 1 : 2) : (pl.sets == 2 ? 2 : 4);
+    if (plan_override && plan_override[0] > 0) vec = plan_override[0];
+    while (vec > 1 && (N % (8 * vec)) != 0) vec >>= 1;
+    if (vec != 1 && vec != 2 && vec != 4) vec = 1;
+    pl.vec = vec;
+
+    int steps = 2;
+    if (plan_override && plan_override[1] > 0) steps = plan_override[1];
+    if (steps != 1 && steps != 2) steps = 2;
+    if ((K % 32) != 0 || (grouped && (block_size % 32) != 0)) steps = 1;
+    pl.steps = steps;
+    const int chunk = steps * 16;
+
+    const int nb_cols = 128 * vec;
+    const int64_t nblocks = (N + nb_cols - 1) / nb_cols;
+    int waves = kMaxWaves;
+    while (waves > 1 && (int64_t)waves * rows_used * nb_cols * 4 > kLdsBudget) waves >>= 1;
+    if (plan_override && plan_override[2] > 0 && plan_override[2] <= waves) waves = plan_override[2];
+
+    // rows of K per wave: the longest slice that still yields kTargetWorkgroups workgroups
+    const int64_t chunks_total = (K + chunk - 1) / chunk;
+    int64_t want_slices = (kTargetWorkgroups + nblocks - 1) / nblocks * waves;
+    if (want_slices < waves) want_slices = waves;
+    int64_t nch = chunks_total / want_slices;
+    if (nch < 1) nch = 1;
+    int64_t klen = nch * chunk;
+    if (plan_override && plan_override[3] > 0) klen = (plan_override[3] + chunk - 1) / chunk * chunk;
+    pl.klen = (int)klen;
+    const int64_t slices = (K + klen - 1) / klen;
+    while (waves > 1 && waves / 2 >= slices) waves >>= 1;
+    pl.waves = waves;
+    pl.ks = (int)((slices + waves - 1) / waves);
+    if (nblocks > kTicketBytes / 4) pl.fast = false;
+    return pl;
+}
+
+template <int kVec, int kSteps, int kSets, bool kXF32>
+void launch4(const GemvParams& p, bool grouped, dim3 grid, int threads, size_t lds, hipStream_t s) {
+    if (grouped)
+        gemv_w4_mfma<kVec, kSteps, kSets, kXF32, true><<<grid, threads, lds, s>>>(p);
+    else
+        gemv_w4_mfma<kVec, kSteps, kSets, kXF32, false><<<grid, threads, lds, s>>>(p);
+}
+
+template <int kVec, int kSteps>
+void launch2(int sets, bool f32, const GemvParams& p, bool grouped, dim3 grid, int threads,
+             size_t lds, hipStream_t s) {
+    if (f32)
+        launch4<kVec, kSteps, 2, true>(p, grouped, grid, threads, lds, s);
+    else if (sets == 2)
+        launch4<kVec, kSteps, 2, false>(p, grouped, grid, threads, lds, s);
+    else
+        launch4<kVec, kSteps, 1, false>(p, grouped, grid, threads, lds, s);
+}
+
+void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, bool grouped, dim3 grid,
+                 int threads, size_t lds, hipStream_t s) {
+    const int key = pl.vec * 10 + pl.steps;
+    switch (key) {
+        case 42: launch2<4, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
+        case 41: launch2<4, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
+        case 22: launch2<2, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
+        case 21: launch2<2, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
+        case 12: launch2<1, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
+        default: launch2<1, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
+    }
+}
+
+int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* w_packed,
+                const void* scale, const void* zero, int64_t block_size, const void* bias, void* y,
+                void* workspace, int64_t workspace_bytes, const int* plan_override, hipStream_t s) {
+    if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (!x || !w_packed || !scale || !y) return K3Q_ERR_NULL;
+    const bool grouped = block_size > 0;
+    if (grouped && !zero) return K3Q_ERR_NULL;
+    const bool f32 = x_dtype == K3Q_F32;
+    const size_t el = f32 ? 4 : 2;
+    if (!aligned_to(x, el) || !aligned_to(scale, el) || !aligned_to(y, el) ||
+        (bias && !aligned_to(bias, el)))
+        return K3Q_ERR_ALIGN;
+
+    GemvParams p{};
+    p.x = x;
+    p.w = (const uint8_t*)w_packed;
+    p.scale = scale;
+    p.zero = (const int8_t*)zero;
+    p.bias = bias;
+    p.y = y;
+    p.K = K;
+    p.N = N;
+    p.row_bytes = (N + 1) / 2;
+    p.block_size = grouped ? (int)block_size : 0;
+
+    Plan pl = make_plan(x_dtype, M, K, N, block_size, plan_override);
+    // vector loads of x rows, packed rows, scales and zero points
+    if (pl.fast && (!aligned_to(x, 16) || !aligned_to(w_packed, 16) || !aligned_to(scale, 16) ||
+                    (zero && !aligned_to(zero, 4))))
+        pl.fast = false;
+    if (!pl.fast) {
+        for (int64_t m0 = 0; m0 < M; m0 += 65535) {
+            const int rows = (int)((M - m0 < 65535) ? M - m0 : 65535);
+            p.m0 = (int)m0;
+            p.M = rows;
+            dim3 grid((unsigned)((N + 255) / 256), rows);
+            if (f32) {
+                if (grouped)
+                    gemv_w4_generic<false, true><<<grid, 256, 0, s>>>(p);
+                else
+                    gemv_w4_generic<false, false><<<grid, 256, 0, s>>>(p);
+            } else {
+                if (grouped)
+                    gemv_w4_generic<true, true><<<grid, 256, 0, s>>>(p);
+                else
+                    gemv_w4_generic<true, false><<<grid, 256, 0, s>>>(p);
+            }
+        }
+        return launch_status();
+    }
+
+    const int nb_cols = 128 * pl.vec;
+    const int64_t nblocks = (N + nb_cols - 1) / nb_cols;
+    const int rows_max = (int)(M < pl.rows ? M : pl.rows);
+    if (pl.ks > 1) {
+        const int64_t need = kTicketBytes + (int64_t)pl.ks * rows_max * N * 4;
+        if (!workspace || workspace_bytes < need) return K3Q_ERR_WORKSPACE;
+        if (!aligned_to(workspace, 16)) return K3Q_ERR_ALIGN;
+        p.tickets = (u32*)workspace;
+        p.part = (float*)((char*)workspace + kTicketBytes);
+    }
+    p.klen = pl.klen;
+    for (int64_t m0 = 0; m0 < M; m0 += pl.rows) {
+        const int rows = (int)((M - m0 < pl.rows) ? M - m0 : pl.rows);
+        p.m0 = (int)m0;
+        p.M = rows;
+        dim3 grid((unsigned)nblocks, (unsigned)pl.ks);
+        const int threads = pl.waves * 64;
+        const size_t lds = (size_t)pl.waves * rows * nb_cols * sizeof(float);
+        const int sets = (!f32 && rows > 8) ? 2 : (f32 ? 2 : 1);
+        launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace k3q
+
+using namespace k3q;
+
+extern "C" int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+    if (M <= 0 || K <= 0 || N <= 0) return 0;
+    // tickets + the largest partial buffer the built-in plans ask for (the plan depends on
+    // the dtype and on whether the kernel is grouped; take the maximum over those)
+    int64_t part = 0;
+    const int64_t groupings[3] = {-1, 128, 32};
+    for (int dt = 0; dt < 2; ++dt)
+        for (int gi = 0; gi < 3; ++gi) {
+            const Plan pl = make_plan(dt, M, K, N, groupings[gi], nullptr);
+            if (!pl.fast || pl.ks <= 1) continue;
+            const int64_t rows = M < pl.rows ? M : pl.rows;
+            const int64_t b = (int64_t)pl.ks * rows * N * 4;
+            if (b > part) part = b;
+        }
+    return kTicketBytes + part;
+}
+
+extern "C" int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                           const void* w_packed, const void* scale, const void* zero,
+                           int64_t block_size, const void* bias, void* y, void* workspace,
+                           int64_t workspace_bytes, void* stream) {
+    return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
+                       workspace_bytes, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                const void* w_packed, const void* scale, const void* zero,
+                                int64_t block_size, const void* bias, void* y, void* workspace,
+                                int64_t workspace_bytes, const int* plan, void* stream) {
+    return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
+                       workspace_bytes, plan, (hipStream_t)stream);
+}

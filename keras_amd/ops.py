@@ -1,0 +1,89 @@
+"""Tensor-level entry points of the quantized forward (thin wrappers over the C ABI).
+
+These are the calls a `_int8_call` / `_int4_call` makes: they take and return
+torch tensors that live on the HIP device, run on torch's current stream and
+allocate only outputs (plus one cached, zero-initialised scratch buffer per
+device and stream for the split-K kernels).
+"""
+
+import ctypes
+
+import torch
+
+from keras_amd import _lib
+
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    """Scratch for split-K partials and arrival tickets.
+
+    One buffer per (device, stream): calls on one stream are ordered, so they
+    can share it; calls on different streams may overlap and must not.  The
+    buffer starts zeroed and the kernels leave its ticket area zeroed.
+    """
+    stream = torch.cuda.current_stream(device)
+    key = (device.index, stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        size = max(int(nbytes), 1 << 20)
+        ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=None,
+                block_size=None, bias=None, plan=None):
+    """`x[..., K] . W4[K, N]` for a Dense int4 kernel as the layer stores it.
+
+    kernel_packed: int8 [K, ceil(N/2)] (two nibbles per byte along N).
+    kernel_scale:  [N] (per-channel, `block_size` None or -1) or [G, N].
+    kernel_zero:   int8 [G, N] for grouped quantisation.
+    Scales and bias must already be in x.dtype (the layer reads its float
+    variables in the compute dtype).  Returns x.dtype [..., N].
+    Reference: keras/src/layers/core/dense.py:988-1095.
+    """
+    _lib.require_device(x, kernel_packed, kernel_scale, kernel_zero, bias)
+    code = _lib.dtype_code(x.dtype)
+    K = kernel_packed.shape[0]
+    N = int(orig_output_dim)
+    if x.shape[-1] != K:
+        raise ValueError(
+            f"last axis of the input ({x.shape[-1]}) does not match the kernel's input dim ({K})"
+        )
+    if kernel_packed.dtype != torch.int8 or kernel_packed.shape[1] != (N + 1) // 2:
+        raise ValueError("kernel must be int8 of shape [input_dim, ceil(units / 2)]")
+    grouped = block_size is not None and block_size > 0
+    if kernel_scale.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise TypeError("kernel_scale and bias must be read in the input's dtype")
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    kp = kernel_packed if kernel_packed.is_contiguous() else kernel_packed.contiguous()
+    ks = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
+    kz = None
+    if grouped:
+        if kernel_zero is None:
+            raise ValueError("grouped int4 needs kernel_zero")
+        kz = kernel_zero if kernel_zero.is_contiguous() else kernel_zero.contiguous()
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    nbytes = lib.k3q_gemv_w4_workspace_bytes(M, K, N)
+    if plan is not None:
+        # an overridden plan may split K into many more workgroups than the built-in one
+        nbytes = max(nbytes, 4096 + (K // 16 + 1) * min(M, 16) * N * 4)
+    ws = _workspace(x.device, nbytes)
+    args = [
+        _lib.ptr(x2), code, M, K, N, _lib.ptr(kp), _lib.ptr(ks), _lib.ptr(kz),
+        int(block_size) if grouped else -1, _lib.ptr(bias), _lib.ptr(y),
+        _lib.ptr(ws), ws.numel(),
+    ]
+    if plan is None:
+        rc = lib.k3q_gemv_w4(*args, _lib.stream_ptr(x.device))
+    else:
+        arr = (ctypes.c_int * 4)(*[int(v) for v in plan])
+        rc = lib.k3q_gemv_w4_plan(*args, arr, _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemv_w4")
+    return y.reshape(*lead, N)

@@ -1,0 +1,96 @@
+"""GPU parity: weight-only int4 Dense forward (k3q_gemv_w4) against the CPU oracle."""
+
+import pytest
+import torch
+
+from keras_amd import ops as kops
+from oracle import keras_cpu_path as ref
+from tests.helpers import RTOL, c_w4_matmul_f64, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def make_layer(K, N, block_size, seed, with_bias):
+    g = torch.Generator().manual_seed(seed)
+    kernel = ref.glorot_uniform(K, N, generator=g)
+    qk = ref.dense_quantize_int4(kernel, block_size)
+    bias = torch.randn(N, generator=g) * 0.02 if with_bias else None
+    return qk, bias
+
+
+def run_case(dev, M, K, N, block_size, dtype, with_bias, seed=0, plan=None):
+    qk, bias = make_layer(K, N, block_size, seed, with_bias)
+    g = torch.Generator().manual_seed(seed + 1)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    grouped = block_size is not None and block_size > 0
+    want = ref.dense_int4_call(
+        x, qk["kernel"], qk["kernel_scale"], N, kernel_zero=qk["kernel_zero"],
+        g_idx=qk["g_idx"], block_size=block_size, bias=bias, compute_dtype=dtype)
+    scale_t = qk["kernel_scale"].to(dtype)
+    bias_t = bias.to(dtype) if bias is not None else None
+    got = kops.int4_matmul(
+        x.to(dev), qk["kernel"].to(dev), scale_t.to(dev), N,
+        kernel_zero=qk["kernel_zero"].to(dev) if grouped else None,
+        block_size=block_size, bias=bias_t.to(dev) if bias is not None else None, plan=plan)
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and tuple(got.shape) == (M, N)
+    exact = c_w4_matmul_f64(x, qk["kernel"], scale_t, qk["kernel_zero"], block_size, bias_t, N)
+    e_ref = max_rel_err(got, want)
+    e_exact = max_rel_err(got, exact)
+    e_ref_exact = max_rel_err(want, exact)
+    tol = RTOL[dtype]
+    assert e_ref <= tol, f"vs oracle: {e_ref:.3e} > {tol:.0e}"
+    # the kernel must be at least about as close to the true value as the reference path is
+    assert e_exact <= max(2.0 * e_ref_exact, tol / 4), (e_exact, e_ref_exact)
+    return e_ref, e_exact
+
+
+SMALL = [
+    # M, K, N, block_size
+    (1, 16, 8, None), (2, 32, 16, -1), (3, 64, 40, 16), (5, 128, 136, 32), (8, 256, 512, 128),
+    (9, 256, 512, 128), (16, 512, 1024, 64), (1, 100, 30, None), (2, 100, 30, 50),
+    (4, 24, 7, 8), (17, 128, 256, 128), (33, 64, 128, None), (1, 500, 64, 128),
+    (2, 8, 16, None), (7, 4096, 96, 128), (16, 1024, 1536, None),
+]
+
+
+@pytest.mark.parametrize("M,K,N,block_size", SMALL)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_int4_matmul_small(dev, M, K, N, block_size, dtype):
+    run_case(dev, M, K, N, block_size, dtype, with_bias=(M % 2 == 1))
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("block_size", [None, 128])
+def test_int4_decode_config(dev, M, block_size):
+    # BASELINE config 2: K = N = 8192, bf16 inputs, M in {1, 4, 16}
+    run_case(dev, M, 8192, 8192, block_size, torch.bfloat16, with_bias=False)
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 4096, 14336), (8, 14336, 4096), (1, 4096, 32000)])
+def test_int4_llama_shapes_grouped(dev, M, K, N):
+    run_case(dev, M, K, N, 128, torch.bfloat16, with_bias=False)
+
+
+def test_int4_f32_decode(dev):
+    run_case(dev, 4, 4096, 4096, None, torch.float32, with_bias=True)
+    run_case(dev, 8, 4096, 4096, 128, torch.float32, with_bias=True)
+
+
+@pytest.mark.parametrize("plan", [(4, 2, 8, 32), (4, 1, 4, 64), (2, 2, 8, 128), (1, 1, 2, 16),
+                                  (1, 2, 8, 1024), (2, 1, 1, 4096)])
+def test_int4_plans_agree(dev, plan):
+    # every launch plan must give the same answer up to fp32 summation order
+    run_case(dev, 4, 4096, 2048, None, torch.bfloat16, with_bias=True, plan=plan)
+    run_case(dev, 12, 4096, 2048, 128, torch.bfloat16, with_bias=False, plan=plan)
+
+
+def test_int4_repeatable(dev):
+    # tickets are re-armed: repeated calls on one workspace give bit-identical results
+    qk, _ = make_layer(2048, 1024, None, 3, False)
+    x = torch.randn(4, 2048).to(torch.bfloat16).to(dev)
+    args = (x, qk["kernel"].to(dev), qk["kernel_scale"].to(torch.bfloat16).to(dev), 1024)
+    first = kops.int4_matmul(*args)
+    for _ in range(5):
+        again = kops.int4_matmul(*args)
+        assert torch.equal(first, again)
