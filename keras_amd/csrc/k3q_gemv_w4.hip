@@ -38,7 +38,7 @@
 namespace k3q {
 namespace {
 
-constexpr u32 kMagic = 0x43004300u;
+constexpr u32 kMagicFlip = 0x43084308u;  // bf16 128.0 in both halves, nibble bit 3 flipped
 constexpr u32 kNibblePair = 0x000F000Fu;
 constexpr u32 kOnes = 0x3F803F80u;
 constexpr float kOffset = 136.0f;  // 128 (bf16 magic exponent) + 8 (nibble ^ 8)
@@ -59,6 +59,7 @@ struct GemvParams {
     int m0;                // first row of x handled by this launch
     int block_size;        // rows of K per group (grouped only)
     int klen;              // rows of K per wave (multiple of the chunk)
+    int two_pass;          // 1: partials are summed by a second kernel instead of the last workgroup
 };
 
 __device__ __forceinline__ v8bf as_bf(const v4u& v) { return __builtin_bit_cast(v8bf, v); }
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     constexpr int kNB = 128 * kVec;
     constexpr int kChunk = kSteps * 16;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction
     const int nwaves = blockDim.x >> 6;
     const int i = lane & 15;
     const int g = lane >> 4;
@@ -131,34 +132,42 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
 
     Packed<kVec> wreg[2][kSteps][4];
     v4u xb[2][kSteps][kSets];
-    const int64_t ncol = nb + 8 * kVec * i;
-    const bool ncol_ok = ncol < p.N;
-    const uint8_t* wp = p.w + (ncol >> 1);
+    int64_t ncol = nb + 8 * kVec * i;
+    if (ncol >= p.N) ncol = p.N - 8 * kVec;  // N % (8 * kVec) == 0: stays a valid lane column
 
+    // Addressing: a wave-uniform 64-bit row base per 16-row step plus four per-lane 32-bit
+    // byte offsets.  Steps past K (K % 16 == 0) are pointed at the last valid step and get a
+    // zero x operand; lane columns past N were pointed at valid columns and are never stored.
+    u32 loff[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) loff[t] = (u32)((4 * g + t) * p.row_bytes + (ncol >> 1));
+    const int xel = kXF32 ? 4 : 2;
+    u32 xoff[kSets];
+#pragma unroll
+    for (int st = 0; st < kSets; ++st)
+        xoff[st] = (u32)(((kXF32 ? mrow : mrow + 8 * st) * p.K + 4 * g) * xel);
+    const char* xbase = (const char*)p.x + (int64_t)p.m0 * p.K * xel;
     auto load_chunk = [&](int b, int c) {
         const int64_t kc = kw0 + (int64_t)c * kChunk;
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
+            const int64_t ks = kc + 16 * s;
+            const uint8_t* rb = p.w + (ks < p.K ? ks : p.K - 16) * p.row_bytes;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int64_t k = kc + 16 * s + 4 * g + t;
-                Packed<kVec> v;
-#pragma unroll
-                for (int q = 0; q < kVec; ++q) v.d[q] = 0u;
-                if (ncol_ok && k < p.K) v = load_packed<kVec>(wp + k * p.row_bytes);
-                wreg[b][s][t] = v;
-            }
+            for (int t = 0; t < 4; ++t) wreg[b][s][t] = load_packed<kVec>(rb + loff[t]);
         }
         // x operand: B[slot, j] holds x[m(j), k] in even (j<8) or odd (j>=8) slots
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
-            const int64_t k = kc + 16 * s + 4 * g;
+            const int64_t ks = kc + 16 * s;
+            const bool kvalid = ks < p.K;
+            const char* xs = xbase + (kvalid ? ks : 0) * xel;
 #pragma unroll
             for (int st = 0; st < kSets; ++st) {
                 u32 h[4] = {0u, 0u, 0u, 0u};  // bf16 bits of the four x values
                 if (kXF32) {
-                    if (mrow < M && k < p.K) {
-                        const v4u f = *(const v4u*)((const float*)p.x + (int64_t)(p.m0 + mrow) * p.K + k);
+                    if (mrow < M && kvalid) {
+                        const v4u f = *(const v4u*)(xs + xoff[st]);
 #pragma unroll
                         for (int t = 0; t < 4; ++t) {
                             const u32 hi = f[t] & 0xffff0000u;
@@ -172,8 +181,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
                     }
                 } else {
                     const int m = mrow + 8 * st;
-                    if (m < M && k < p.K) {
-                        const v2u d = *(const v2u*)((const uint16_t*)p.x + (int64_t)(p.m0 + m) * p.K + k);
+                    if (m < M && kvalid) {
+                        const v2u d = *(const v2u*)(xs + xoff[st]);
                         h[0] = d[0] & 0xffffu;
                         h[1] = d[0] >> 16;
                         h[2] = d[1] & 0xffffu;
@@ -223,14 +232,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
             }
 #pragma unroll
             for (int q = 0; q < kVec; ++q) {
-                u32 d[4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) d[t] = wreg[b][s][t].d[q] ^ 0x88888888u;
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
                     v4u av;
+                    // (nibble ^ 8) | 0x4300 per half, as one and-xor (v_bitop3_b32)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) av[t] = ((d[t] >> (4 * pp)) & kNibblePair) | kMagic;
+                    for (int t = 0; t < 4; ++t)
+                        av[t] = ((wreg[b][s][t].d[q] >> (4 * pp)) & kNibblePair) ^ kMagicFlip;
 #pragma unroll
                     for (int st = 0; st < kSets; ++st) {
                         const int a = kXF32 ? 0 : st;
@@ -325,31 +333,65 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
         if (n < p.N) {
             if (KS == 1)
                 finish<kBF16, kGrouped>(p, m, n, sum);
-            else
+            else if (p.two_pass & 4)
                 p.part[((int64_t)blockIdx.y * M + m) * p.N + n] = sum;
+            else  // written through to memory so that workgroups on other XCDs can read it
+                __hip_atomic_store(p.part + ((int64_t)blockIdx.y * M + m) * p.N + n, sum,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    if (KS == 1) return;
+    if (KS == 1 || (p.two_pass & 1)) return;
 
     // ---- last workgroup to arrive at this column block finishes it ----
     __shared__ u32 ticket;
-    __threadfence();
+    if (!(p.two_pass & 2)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
-    if (threadIdx.x == 0) ticket = atomicAdd(p.tickets + blockIdx.x, 1u);
+    if (threadIdx.x == 0)
+        ticket = __hip_atomic_fetch_add(p.tickets + blockIdx.x, 1u, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (ticket != (u32)(KS - 1)) return;
-    __threadfence();
     for (int idx = threadIdx.x; idx < M * kNB; idx += blockDim.x) {
         const int m = idx / kNB;
         const int64_t n = nb + (idx % kNB);
         if (n < p.N) {
-            float sum = 0.f;
-            for (int ks = 0; ks < KS; ++ks)
-                sum += __builtin_nontemporal_load(p.part + ((int64_t)ks * M + m) * p.N + n);
-            finish<kBF16, kGrouped>(p, m, n, sum);
+            // agent-scope loads: served from memory, never from a stale L2 line.  Four
+            // independent chains keep the loads in flight; the order of addition is fixed.
+            float s4[4] = {0.f, 0.f, 0.f, 0.f};
+            const float* src = p.part + (int64_t)m * p.N + n;
+            const int64_t stride = (int64_t)M * p.N;
+            int ks = 0;
+            for (; ks + 4 <= KS; ks += 4) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    s4[u] += __hip_atomic_load(src + (ks + u) * stride, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+            }
+            for (; ks < KS; ++ks)
+                s4[0] += __hip_atomic_load(src + ks * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            finish<kBF16, kGrouped>(p, m, n, (s4[0] + s4[1]) + (s4[2] + s4[3]));
         }
     }
-    if (threadIdx.x == 0) p.tickets[blockIdx.x] = 0u;
+    if (threadIdx.x == 0)
+        __hip_atomic_store(p.tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// second pass of the two-pass variant: sum the KS partials of every output and finish it
+template <bool kBF16, bool kGrouped>
+__global__ __launch_bounds__(256) void gemv_w4_reduce(GemvParams p, int KS) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int m = blockIdx.y;
+    if (n >= p.N) return;
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+    const float* src = p.part + (int64_t)m * p.N + n;
+    const int64_t stride = (int64_t)p.M * p.N;
+    int ks = 0;
+    for (; ks + 4 <= KS; ks += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s4[u] += src[(ks + u) * stride];
+    }
+    for (; ks < KS; ++ks) s4[0] += src[ks * stride];
+    finish<kBF16, kGrouped>(p, m, n, (s4[0] + s4[1]) + (s4[2] + s4[3]));
 }
 
 // Any shape: one thread per output, fp32 FMA chain over K.  Used when N is not a
@@ -397,7 +439,8 @@ struct Plan {
 };
 
 constexpr int64_t kTicketBytes = 4096;  // room for 1024 column blocks
-constexpr int kTargetWorkgroups = 512;
+constexpr int kTargetWorkgroups = 256;  // one per CU
+constexpr int kDefaultTwoPass = 1;
 
 // plan_override (may be null): {vec, steps, waves, klen}; entries <= 0 keep the heuristic.
 Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
@@ -411,7 +454,9 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     pl.sets = f32 ? 2 : (M > 8 ? 2 : 1);
     const int rows_used = (int)(M < pl.rows ? M : pl.rows);
 
-    int vec = grouped ? (pl.sets == 2 ? 1 : 2) : (pl.sets == 2 ? 2 : 4);
+    // Measured on MI355X at K = N = 8192: 8 waves per workgroup, 8-byte loads per lane and
+    // one workgroup per CU (256 workgroups) beat wider loads and finer K splits.
+    int vec = (grouped && pl.sets == 2) ? 1 : 2;
     if (plan_override && plan_override[0] > 0) vec = plan_override[0];
     while (vec > 1 && (N % (8 * vec)) != 0) vec >>= 1;
     if (vec != 1 && vec != 2 && vec != 4) vec = 1;
@@ -430,14 +475,12 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     while (waves > 1 && (int64_t)waves * rows_used * nb_cols * 4 > kLdsBudget) waves >>= 1;
     if (plan_override && plan_override[2] > 0 && plan_override[2] <= waves) waves = plan_override[2];
 
-    // rows of K per wave: the longest slice that still yields kTargetWorkgroups workgroups
-    const int64_t chunks_total = (K + chunk - 1) / chunk;
-    int64_t want_slices = (kTargetWorkgroups + nblocks - 1) / nblocks * waves;
-    if (want_slices < waves) want_slices = waves;
-    int64_t nch = chunks_total / want_slices;
-    if (nch < 1) nch = 1;
-    int64_t klen = nch * chunk;
+    // rows of K per wave: the slice length that gives about one workgroup per CU
+    int64_t klen = K * nblocks / ((int64_t)kTargetWorkgroups * waves);
+    klen = klen / chunk * chunk;
+    if (klen < chunk) klen = chunk;
     if (plan_override && plan_override[3] > 0) klen = (plan_override[3] + chunk - 1) / chunk * chunk;
+    if (klen > K) klen = (K + chunk - 1) / chunk * chunk;
     pl.klen = (int)klen;
     const int64_t slices = (K + klen - 1) / klen;
     while (waves > 1 && waves / 2 >= slices) waves >>= 1;
@@ -543,6 +586,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         p.part = (float*)((char*)workspace + kTicketBytes);
     }
     p.klen = pl.klen;
+    p.two_pass = (plan_override && plan_override[4] >= 0) ? plan_override[4] : kDefaultTwoPass;
     for (int64_t m0 = 0; m0 < M; m0 += pl.rows) {
         const int rows = (int)((M - m0 < pl.rows) ? M - m0 : pl.rows);
         p.m0 = (int)m0;
@@ -552,6 +596,20 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         const size_t lds = (size_t)pl.waves * rows * nb_cols * sizeof(float);
         const int sets = (!f32 && rows > 8) ? 2 : (f32 ? 2 : 1);
         launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
+        if (pl.ks > 1 && (p.two_pass & 1)) {
+            dim3 rgrid((unsigned)((N + 255) / 256), rows);
+            if (f32) {
+                if (grouped)
+                    gemv_w4_reduce<false, true><<<rgrid, 256, 0, s>>>(p, pl.ks);
+                else
+                    gemv_w4_reduce<false, false><<<rgrid, 256, 0, s>>>(p, pl.ks);
+            } else {
+                if (grouped)
+                    gemv_w4_reduce<true, true><<<rgrid, 256, 0, s>>>(p, pl.ks);
+                else
+                    gemv_w4_reduce<true, false><<<rgrid, 256, 0, s>>>(p, pl.ks);
+            }
+        }
     }
     return launch_status();
 }
