@@ -76,6 +76,38 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
                     int64_t orig_len, int is_signed, void* out, void* stream);
 
 /*
+ * int8 x int8 -> int32 matmul with the Dense / EinsumDense de-scale fused:
+ *     acc[m,n] = sum_k a[m,k] * b[k,n]                       (exact int32)
+ *     y[m,n]   = T(T(acc[m,n]) / T(b_scale[n] * a_scale[m]))  (+ bias[n])
+ * a: [M,K] int8 (the quantised activations).  b: the layer's int8 kernel, either
+ * as the variable stores it, [K,N] (b_layout 0), or as the [N,K] shadow copy made
+ * by k3q_prepack_kernel_i8 (b_layout 1).  a_scale [M], b_scale [N], bias [N] are
+ * of out_dtype; a null scale counts as 1, a null bias as absent.  y: out_dtype
+ * [M,N] or null.  acc_out: int32 [M,N] or null (the raw accumulators, for
+ * bit-exact checks).  At least one of y / acc_out must be given.
+ * flags bit 0 (K3Q_GEMM_EXACT_EPILOGUE): round after every step exactly as the
+ * reference's op chain does; otherwise y = T(acc * (1/a_scale) * (1/b_scale) + bias)
+ * with one final rounding (differs from the chain by at most the chain's own
+ * intermediate roundings).
+ * The MFMA kernel needs K % 128 == 0, N % 4 == 0 and 16-byte aligned operands;
+ * other shapes run a plain kernel.  With b_layout 0 the MFMA kernel also needs
+ * `workspace` (k3q_gemm_i8_workspace_bytes, 16-byte aligned) to hold the [N,K]
+ * copy it makes on every call; callers that reuse a kernel should prepack once.
+ * Replaces cast, cast, matmul (keras/src/backend/torch/numpy.py:139-157), cast,
+ * multiply, divide, add of Dense._int8_call (keras/src/layers/core/dense.py:961-983)
+ * and the einsum form in EinsumDense._int8_call
+ * (keras/src/layers/core/einsum_dense.py:1072-1084).
+ */
+#define K3Q_GEMM_EXACT_EPILOGUE 1
+int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N, int8_t* prepacked,
+                          void* stream);
+int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64_t N, int64_t K,
+                const void* a_scale, const void* b_scale, const void* bias, int out_dtype,
+                int flags, void* y, int32_t* acc_out, void* workspace, int64_t workspace_bytes,
+                void* stream);
+
+/*
  * Weight-only int4 matmul for decode-sized inputs (any M; tuned for M <= 16):
  *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)
  *     grouped     (block_size  > 0):  y = T(x . ((unpack(w) - zero[g]) * scale[g]))  (+ bias),  g = k / block_size

@@ -40,6 +40,13 @@ SIGNATURES = {
     ),
     "k3q_pack_int4": (_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr]),
     "k3q_unpack_int4": (_int, [_ptr, _i64, _i64, _i64, _i64, _int, _ptr, _ptr]),
+    "k3q_gemm_i8_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "k3q_prepack_kernel_i8": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "k3q_gemm_i8": (
+        _int,
+        [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _int, _int, _ptr, _ptr, _ptr,
+         _i64, _ptr],
+    ),
     "k3q_gemv_w4_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "k3q_gemv_w4": (
         _int,

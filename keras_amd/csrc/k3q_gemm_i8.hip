@@ -1,0 +1,495 @@
+// int8 x int8 -> int32 GEMM with the Dense de-scale epilogue fused:
+//     y[m,n] = T( acc[m,n] / (a_scale[m] * b_scale[n]) ) (+ bias[n]),  acc = sum_k a[m,k] * b[k,n]
+//
+// MFMA-bound kernel for prefill-sized M.  Both operands are consumed K-contiguous:
+// `a` is [M,K] as the activation quantizer writes it, the weight comes as the
+// [N,K] shadow copy that k3q_prepack_kernel_i8 makes once per layer (the layer's
+// own [K,N] variable stays what it is).
+//
+// Workgroup: 512 threads = 8 waves as 4 (N) x 2 (M); tile 256 (M) x 256 (N), 128
+// bytes of K per stage (a full cache line per row and request).  Global -> LDS goes
+// through the LDS-DMA path (global_load_lds_dwordx4: 64 lanes x 16 bytes land
+// lane-linear in LDS, no VGPR staging), two 64 KiB stages.  The LDS tile is
+// [row][128 B] with the eight 16-byte chunks of a row XOR-swizzled by row bits, applied on the global side
+// of the DMA (a lane fetches the chunk that belongs at its LDS position), so the
+// ds_read_b128 fragment reads are bank-conflict free.
+//
+// MFMA: v_mfma_i32_32x32x32_i8.  The weight tile is the first (row) operand and
+// the activation tile the second (column) operand, so a lane ends up with ONE
+// output row m and groups of four consecutive n: stores are 8 or 16 bytes wide.
+#include "k3q_common.h"
+
+namespace k3q {
+namespace {
+
+constexpr int kBM = 256;  // tile rows of a / y
+constexpr int kBN = 256;  // tile rows of the prepacked weight = columns of y
+constexpr int kBK = 128;  // bytes of K per stage: one full 128-byte line per row
+constexpr int kStages = 2;
+constexpr int kKSteps = kBK / 32;  // MFMA K steps per stage
+constexpr int kThreads = 512;
+constexpr int kWavesN = 4;  // waves along N
+constexpr int kWavesM = 2;  // waves along M
+constexpr int kWN = kBN / kWavesN;  // 64 columns per wave
+constexpr int kWM = kBM / kWavesM;  // 128 rows per wave
+constexpr int kNBlk = kWN / 32;     // 2 MFMA blocks along N per wave
+constexpr int kMBlk = kWM / 32;     // 4 MFMA blocks along M per wave
+constexpr int kTileBytes = kBM * kBK;             // 16 KiB per operand tile
+constexpr int kStageBytes = 2 * kTileBytes;       // 32 KiB
+constexpr int kLdsBytes = kStages * kStageBytes;  // 128 KiB
+constexpr int kDmaPerTile = kTileBytes / 1024;                        // 32 DMA instructions per operand tile
+constexpr int kDmaPerWave = (2 * kDmaPerTile) / (kThreads / 64);      // 8 per wave per stage
+constexpr int kRowChunks = kBK / 16;                                  // 16-byte chunks per LDS row
+
+constexpr int kFlagExactEpilogue = 1;
+constexpr int kFlagSkipEpilogue = 1024;  // undocumented timing aid
+
+struct GemmParams {
+    const int8_t* a;        // [M, K]
+    const int8_t* bt;       // [N, K]
+    const void* a_scale;    // T [M] or null
+    const void* b_scale;    // T [N] or null
+    const void* bias;       // T [N] or null
+    void* y;                // T [M, N] or null
+    int32_t* acc_out;       // [M, N] or null
+    int64_t M, N, K;
+    int tiles_m, tiles_n;
+    int flags;
+};
+
+// 16-byte chunk swizzle of a 128-byte LDS row (8 chunks): chunk c of row r lives at chunk
+// c ^ swz(r).  ds_read_b128 of one chunk index over consecutive rows is then bank-conflict
+// free whether the LDS services 8 or 16 lanes per clock.
+__device__ __forceinline__ int swz(int row) {
+    return (row & 6) | ((row ^ (row >> 3)) & 1);
+}
+
+// gfx9 s_waitcnt encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]
+__device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+__device__ __forceinline__ void wait_vmcnt_one_stage() { __builtin_amdgcn_s_waitcnt(0x0F70 | kDmaPerWave); }
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+__device__ __forceinline__ void bare_barrier() {
+    // s_barrier without a fence: a fence would also drain the DMA of the stage in flight
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <bool kBF16>
+__device__ __forceinline__ float load_t(const void* p, int64_t i) {
+    if (kBF16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+    return ((const float*)p)[i];
+}
+
+template <bool kBF16, bool kExact>
+__global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave % kWavesN;
+    const int wm = wave / kWavesN;
+
+    // ---- tile of this workgroup: XCD-aware order ----
+    // Workgroups are dealt round-robin to the 8 XCDs; each XCD walks a contiguous range of
+    // the tile list, and the list is ordered in bands of 4 tile rows so that the 32 tiles an
+    // XCD runs at a time share A rows and B rows in its L2.
+    const int total = p.tiles_m * p.tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (t >= total) return;
+    constexpr int kBand = 4;
+    const int band = t / (kBand * p.tiles_n);
+    const int band_rows = min(kBand, p.tiles_m - band * kBand);
+    const int within = t - band * kBand * p.tiles_n;
+    const int tile_m = band * kBand + within % band_rows;
+    const int tile_n = within / band_rows;
+    const int64_t m0 = (int64_t)tile_m * kBM;
+    const int64_t n0 = (int64_t)tile_n * kBN;
+
+    // ---- DMA source addresses ----
+    // DMA instruction d of this wave fills LDS bytes [(wave * kDmaPerWave + d) * 1024, +1024) of
+    // the stage: 8 rows x 128 B.  Instructions 0..31 of a stage are the A tile, 32..63 the B tile.
+    const char* src[kDmaPerWave];
+#pragma unroll
+    for (int d = 0; d < kDmaPerWave; ++d) {
+        const int inst = wave * kDmaPerWave + d;
+        const bool is_b = inst >= kDmaPerTile;
+        const int row = (inst % kDmaPerTile) * 8 + lane / kRowChunks;
+        const int chunk = (lane & (kRowChunks - 1)) ^ swz(row);
+        int64_t grow = (is_b ? n0 : m0) + row;
+        const int64_t lim = (is_b ? p.N : p.M) - 1;
+        grow = grow < lim ? grow : lim;
+        src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.K + chunk * 16;
+    }
+    auto issue_stage = [&](int kt) {
+        char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
+#pragma unroll
+        for (int d = 0; d < kDmaPerWave; ++d) {
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
+                (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
+        }
+    };
+
+    // ---- fragment reads ----
+    // MFMA operand lane (i = lane % 32, g = lane / 32) holds row i, bytes [16g, 16g+16) of the
+    // 32-byte K step, i.e. logical chunk 2*ks + g of the row.
+    const int fi = lane & 31;
+    const int fg = lane >> 5;
+    int a_row[kMBlk], a_swz[kMBlk], b_row[kNBlk], b_swz[kNBlk];
+#pragma unroll
+    for (int mb = 0; mb < kMBlk; ++mb) {
+        const int row = wm * kWM + mb * 32 + fi;
+        a_row[mb] = row * kBK;
+        a_swz[mb] = swz(row);
+    }
+#pragma unroll
+    for (int nb = 0; nb < kNBlk; ++nb) {
+        const int row = wn * kWN + nb * 32 + fi;
+        b_row[nb] = kTileBytes + row * kBK;
+        b_swz[nb] = swz(row);
+    }
+    v4i af[2][kMBlk], bf[2][kNBlk];
+    auto read_frags = [&](int fb, int stage, int ks) {
+        const char* st = lds + stage * kStageBytes;
+#pragma unroll
+        for (int nb = 0; nb < kNBlk; ++nb)
+            bf[fb][nb] = *(const v4i*)(st + b_row[nb] + (((2 * ks + fg) ^ b_swz[nb]) << 4));
+#pragma unroll
+        for (int mb = 0; mb < kMBlk; ++mb)
+            af[fb][mb] = *(const v4i*)(st + a_row[mb] + (((2 * ks + fg) ^ a_swz[mb]) << 4));
+    };
+
+    v16i acc[kNBlk][kMBlk];
+#pragma unroll
+    for (int nb = 0; nb < kNBlk; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < kMBlk; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0;
+
+    // ---- main loop ----
+    // Two LDS stages.  The fragments of K step ks+1 are read in the middle of the MFMAs of
+    // step ks; the one barrier per stage sits in the middle of the LAST step's MFMAs, so the
+    // matrix core has work queued while waves meet.  At that barrier every wave holds its
+    // last fragments of stage kt in registers, so stage kt+2 may be DMA-ed over stage kt, and
+    // stage kt+1 (whose DMA every wave has waited for) may be read.
+    const int KT = (int)(p.K / kBK);
+    issue_stage(0);
+    if (KT > 1) {
+        issue_stage(1);
+        wait_vmcnt_one_stage();
+    } else {
+        wait_vmcnt0();
+    }
+    bare_barrier();
+    read_frags(0, 0, 0);
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks) {
+            // first half of this step's MFMAs, then the reads for the next step, then the
+            // second half: the reads get half a step of matrix-core time to come back
+            __builtin_amdgcn_sched_barrier(0);
+#ifndef K3Q_GEMM_PROBE_NO_MMA
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb)
+                acc[0][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][0], af[ks & 1][mb],
+                                                                   acc[0][mb], 0, 0, 0);
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+            if (ks + 1 < kKSteps) {
+                read_frags((ks + 1) & 1, cur, ks + 1);
+            } else if (kt + 1 < KT) {
+                wait_vmcnt0();  // own DMA of stage kt+1 has landed (own reads of stage kt are done)
+                bare_barrier();
+#ifndef K3Q_GEMM_PROBE_NO_DMA
+                if (kt + 2 < KT) issue_stage(kt + 2);
+#endif
+                read_frags(0, cur ^ 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#ifndef K3Q_GEMM_PROBE_NO_MMA
+#pragma unroll
+            for (int nb = 1; nb < kNBlk; ++nb)
+#pragma unroll
+                for (int mb = 0; mb < kMBlk; ++mb)
+                    acc[nb][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][nb], af[ks & 1][mb],
+                                                                        acc[nb][mb], 0, 0, 0);
+#else
+            // probe build: consume the fragments so that the reads stay
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] ^= af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1];
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- epilogue ----
+    // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
+    // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: per lane 4 rows of y and 8 groups
+    // of four consecutive columns.  All scale / bias loads are issued before any is used.
+    if (p.flags & kFlagSkipEpilogue) {  // timing aid: main loop only
+        int sink = 0;
+#pragma unroll
+        for (int nb = 0; nb < kNBlk; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sink ^= acc[nb][mb][r];
+        if (sink == 0x7fffffff && p.y) ((char*)p.y)[0] = 1;
+        return;
+    }
+    int64_t mrow[kMBlk];
+    float sa[kMBlk], ra[kMBlk];
+#pragma unroll
+    for (int mb = 0; mb < kMBlk; ++mb) {
+        mrow[mb] = m0 + wm * kWM + mb * 32 + fi;
+        const int64_t mc = mrow[mb] < p.M ? mrow[mb] : p.M - 1;
+        sa[mb] = p.a_scale ? load_t<kBF16>(p.a_scale, mc) : 1.0f;
+    }
+    float sb[kNBlk][4][4], bv[kNBlk][4][4];
+#pragma unroll
+    for (int nb = 0; nb < kNBlk; ++nb)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            int64_t n = n0 + wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+            n = n < p.N ? n : p.N - 4;  // N % 4 == 0 on this path
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                sb[nb][rg][e] = 1.0f;
+                bv[nb][rg][e] = 0.0f;
+            }
+            if (kBF16) {
+                if (p.b_scale) {
+                    const v2u t = *(const v2u*)((const uint16_t*)p.b_scale + n);
+                    sb[nb][rg][0] = __uint_as_float(t[0] << 16);
+                    sb[nb][rg][1] = __uint_as_float(t[0] & 0xffff0000u);
+                    sb[nb][rg][2] = __uint_as_float(t[1] << 16);
+                    sb[nb][rg][3] = __uint_as_float(t[1] & 0xffff0000u);
+                }
+                if (p.bias) {
+                    const v2u t = *(const v2u*)((const uint16_t*)p.bias + n);
+                    bv[nb][rg][0] = __uint_as_float(t[0] << 16);
+                    bv[nb][rg][1] = __uint_as_float(t[0] & 0xffff0000u);
+                    bv[nb][rg][2] = __uint_as_float(t[1] << 16);
+                    bv[nb][rg][3] = __uint_as_float(t[1] & 0xffff0000u);
+                }
+            } else {
+                if (p.b_scale) {
+                    const v4f t = *(const v4f*)((const float*)p.b_scale + n);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sb[nb][rg][e] = t[e];
+                }
+                if (p.bias) {
+                    const v4f t = *(const v4f*)((const float*)p.bias + n);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) bv[nb][rg][e] = t[e];
+                }
+            }
+        }
+    if (!kExact) {
+#pragma unroll
+        for (int mb = 0; mb < kMBlk; ++mb) ra[mb] = 1.0f / sa[mb];
+#pragma unroll
+        for (int nb = 0; nb < kNBlk; ++nb)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sb[nb][rg][e] = 1.0f / sb[nb][rg][e];
+    }
+    const bool has_bias = p.bias != nullptr;
+#pragma unroll
+    for (int mb = 0; mb < kMBlk; ++mb) {
+        const int64_t m = mrow[mb];
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int nb = 0; nb < kNBlk; ++nb) {
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const int64_t n = n0 + wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+                if (n >= p.N) continue;  // all four columns in or out
+                if (p.acc_out) {
+                    v4i o = {acc[nb][mb][4 * rg], acc[nb][mb][4 * rg + 1], acc[nb][mb][4 * rg + 2],
+                             acc[nb][mb][4 * rg + 3]};
+                    *(v4i*)(p.acc_out + m * p.N + n) = o;
+                }
+                if (!p.y) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float accf = (float)acc[nb][mb][4 * rg + e];
+                    float r;
+                    if (kExact) {
+                        // the reference's op sequence, every step rounded to T
+                        if (kBF16) {
+                            const float os = round_bf16(sb[nb][rg][e] * sa[mb]);
+                            r = round_bf16(round_bf16(accf) / os);
+                            if (has_bias) r = round_bf16(r + bv[nb][rg][e]);
+                        } else {
+                            r = accf / (sb[nb][rg][e] * sa[mb]);
+                            if (has_bias) r = r + bv[nb][rg][e];
+                        }
+                    } else {
+                        r = (accf * ra[mb]) * sb[nb][rg][e] + bv[nb][rg][e];
+                    }
+                    v[e] = r;
+                }
+                if (kBF16) {
+                    v2u o;
+                    o[0] = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+                    o[1] = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+                    *(v2u*)((uint16_t*)p.y + m * p.N + n) = o;
+                } else {
+                    v4f o = {v[0], v[1], v[2], v[3]};
+                    *(v4f*)((float*)p.y + m * p.N + n) = o;
+                }
+            }
+        }
+    }
+}
+
+// Any shape: one thread per output.  b is addressed through strides so that both the
+// [K,N] variable layout and the [N,K] shadow copy work.
+template <bool kBF16>
+__global__ __launch_bounds__(256) void gemm_i8_simple(const int8_t* a, const int8_t* b,
+                                                      int64_t b_stride_k, int64_t b_stride_n,
+                                                      GemmParams p) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t m = blockIdx.y;
+    if (n >= p.N) return;
+    int acc = 0;
+    for (int64_t k = 0; k < p.K; ++k) acc += (int)a[m * p.K + k] * (int)b[k * b_stride_k + n * b_stride_n];
+    if (p.acc_out) p.acc_out[m * p.N + n] = acc;
+    if (!p.y) return;
+    const float sa = p.a_scale ? load_t<kBF16>(p.a_scale, m) : 1.0f;
+    const float sb = p.b_scale ? load_t<kBF16>(p.b_scale, n) : 1.0f;
+    float r;
+    if (kBF16) {
+        r = round_bf16(round_bf16((float)acc) / round_bf16(sb * sa));
+        if (p.bias) r = round_bf16(r + load_t<true>(p.bias, n));
+        ((uint16_t*)p.y)[m * p.N + n] = (uint16_t)f32_to_bf16_bits(r);
+    } else {
+        r = (float)acc / (sb * sa);
+        if (p.bias) r = r + load_t<false>(p.bias, n);
+        ((float*)p.y)[m * p.N + n] = r;
+    }
+}
+
+// [K, N] -> [N, K] byte transpose through a padded LDS tile (one-time per layer).
+__global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ in,
+                                                    int8_t* __restrict__ out, int64_t K, int64_t N) {
+    __shared__ int8_t tile[64][64 + 4];
+    const int64_t k0 = (int64_t)blockIdx.y * 64;
+    const int64_t n0 = (int64_t)blockIdx.x * 64;
+    for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+        const int r = e / 64, c = e % 64;
+        int8_t v = 0;
+        if (k0 + r < K && n0 + c < N) v = in[(k0 + r) * N + n0 + c];
+        tile[r][c] = v;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+        const int r = e / 64, c = e % 64;  // r: n within tile, c: k within tile
+        if (n0 + r < N && k0 + c < K) out[(n0 + r) * K + k0 + c] = tile[c][r];
+    }
+}
+
+bool g_lds_attr_set[4] = {false, false, false, false};
+
+template <bool kBF16, bool kExact>
+int launch_mfma(const GemmParams& p, hipStream_t s) {
+    // 128 KiB of dynamic LDS needs the attribute raised once per kernel (idempotent).
+    constexpr int slot = (kBF16 ? 1 : 0) + (kExact ? 2 : 0);
+    if (!g_lds_attr_set[slot]) {
+        if (hipFuncSetAttribute((const void*)gemm_i8_mfma<kBF16, kExact>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+            return K3Q_ERR_LAUNCH;
+        g_lds_attr_set[slot] = true;
+    }
+    const int total = p.tiles_m * p.tiles_n;
+    const int grid = ((total + 7) / 8) * 8;
+    gemm_i8_mfma<kBF16, kExact><<<grid, kThreads, kLdsBytes, s>>>(p);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace k3q
+
+using namespace k3q;
+
+extern "C" int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    (void)M;
+    if (N <= 0 || K <= 0) return 0;
+    return N * K;  // room for the [N,K] copy when the weight is passed in its [K,N] layout
+}
+
+extern "C" int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N, int8_t* prepacked,
+                                     void* stream) {
+    if (K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (!kernel || !prepacked) return K3Q_ERR_NULL;
+    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
+    transpose_i8<<<grid, 256, 0, (hipStream_t)stream>>>(kernel, prepacked, K, N);
+    return launch_status();
+}
+
+extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64_t N,
+                           int64_t K, const void* a_scale, const void* b_scale, const void* bias,
+                           int out_dtype, int flags, void* y, int32_t* acc_out, void* workspace,
+                           int64_t workspace_bytes, void* stream) {
+    if (out_dtype != K3Q_F32 && out_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || N <= 0 || K <= 0) return K3Q_ERR_SHAPE;
+    if (b_layout != 0 && b_layout != 1) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (!a || !b || (!y && !acc_out)) return K3Q_ERR_NULL;
+    hipStream_t s = (hipStream_t)stream;
+    const bool bf16 = out_dtype == K3Q_BF16;
+
+    GemmParams p{};
+    p.a = a;
+    p.a_scale = a_scale;
+    p.b_scale = b_scale;
+    p.bias = bias;
+    p.y = y;
+    p.acc_out = acc_out;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.flags = flags;
+    p.tiles_m = (int)((M + kBM - 1) / kBM);
+    p.tiles_n = (int)((N + kBN - 1) / kBN);
+
+    const size_t el = bf16 ? 2 : 4;
+    bool fast = (K % kBK) == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
+                (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
+                (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&
+                (int64_t)p.tiles_m * p.tiles_n < (1 << 28);
+    if (fast && b_layout == 0) {
+        // needs the [N,K] copy: made here per call when the caller supplies scratch for it
+        if (workspace && workspace_bytes >= N * K && aligned_to(workspace, 16)) {
+            int rc = k3q_prepack_kernel_i8(b, K, N, (int8_t*)workspace, stream);
+            if (rc != K3Q_OK) return rc;
+            p.bt = (const int8_t*)workspace;
+        } else {
+            fast = false;
+        }
+    } else {
+        p.bt = b;
+    }
+    if (fast) {
+        const bool exact = (flags & kFlagExactEpilogue) != 0;
+        if (bf16) return exact ? launch_mfma<true, true>(p, s) : launch_mfma<true, false>(p, s);
+        return exact ? launch_mfma<false, true>(p, s) : launch_mfma<false, false>(p, s);
+    }
+
+    if (M > 65535) return K3Q_ERR_SHAPE;
+    dim3 grid((unsigned)((N + 255) / 256), (unsigned)M);
+    const int64_t sk = b_layout == 0 ? N : 1;
+    const int64_t sn = b_layout == 0 ? 1 : K;
+    if (bf16)
+        gemm_i8_simple<true><<<grid, 256, 0, s>>>(a, b, sk, sn, p);
+    else
+        gemm_i8_simple<false><<<grid, 256, 0, s>>>(a, b, sk, sn, p);
+    return launch_status();
+}

@@ -87,3 +87,69 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
         rc = lib.k3q_gemv_w4_plan(*args, arr, _lib.stream_ptr(x.device))
     _lib.check(rc, "k3q_gemv_w4")
     return y.reshape(*lead, N)
+
+
+GEMM_EXACT_EPILOGUE = 1
+
+
+def prepack_int8_kernel(kernel):
+    """[K, N] int8 kernel -> the [N, K] shadow copy the MFMA GEMM consumes.
+
+    Made once per layer (the layer's own variable keeps its [K, N] layout).
+    """
+    _lib.require_device(kernel)
+    if kernel.dtype != torch.int8 or kernel.dim() != 2:
+        raise TypeError("kernel must be a 2-D int8 tensor")
+    k = kernel if kernel.is_contiguous() else kernel.contiguous()
+    K, N = k.shape
+    out = torch.empty((N, K), dtype=torch.int8, device=k.device)
+    rc = _lib.load().k3q_prepack_kernel_i8(_lib.ptr(k), K, N, _lib.ptr(out),
+                                           _lib.stream_ptr(k.device))
+    _lib.check(rc, "k3q_prepack_kernel_i8")
+    return out
+
+
+def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype=None,
+                prepacked=None, exact_epilogue=False, want_acc=False, want_y=True):
+    """`a[M, K] int8 . kernel[K, N] int8` with the de-scale epilogue fused.
+
+    Returns y (out_dtype [M, N]); with want_acc also the int32 accumulators.
+    `prepacked` is the cached result of `prepack_int8_kernel(kernel)`; without it
+    the [N, K] copy is rebuilt in scratch memory on every call.
+    Reference: keras/src/layers/core/dense.py:961-983.
+    """
+    _lib.require_device(a, kernel, a_scale, kernel_scale, bias, prepacked)
+    if a.dtype != torch.int8 or kernel.dtype != torch.int8:
+        raise TypeError("int8_matmul takes int8 operands")
+    M, K = a.shape
+    if kernel.shape[0] != K:
+        raise ValueError(f"inner dimensions differ: {a.shape} x {kernel.shape}")
+    N = kernel.shape[1]
+    if out_dtype is None:
+        out_dtype = a_scale.dtype if a_scale is not None else torch.float32
+    code = _lib.dtype_code(out_dtype)
+    for t in (a_scale, kernel_scale, bias):
+        if t is not None and t.dtype != out_dtype:
+            raise TypeError("scales and bias must be read in the output dtype")
+    a = a if a.is_contiguous() else a.contiguous()
+    sa = a_scale.reshape(-1).contiguous() if a_scale is not None else None
+    sb = kernel_scale.reshape(-1).contiguous() if kernel_scale is not None else None
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device) if want_y else None
+    acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
+    lib = _lib.load()
+    if prepacked is not None:
+        b, layout, ws, ws_bytes = prepacked, 1, None, 0
+    else:
+        b = kernel if kernel.is_contiguous() else kernel.contiguous()
+        layout = 0
+        ws = _workspace(a.device, lib.k3q_gemm_i8_workspace_bytes(M, N, K))
+        ws_bytes = ws.numel()
+    rc = lib.k3q_gemm_i8(
+        _lib.ptr(a), _lib.ptr(b), layout, M, N, K, _lib.ptr(sa), _lib.ptr(sb), _lib.ptr(bias),
+        code, GEMM_EXACT_EPILOGUE if exact_epilogue else 0, _lib.ptr(y), _lib.ptr(acc),
+        _lib.ptr(ws), ws_bytes, _lib.stream_ptr(a.device),
+    )
+    _lib.check(rc, "k3q_gemm_i8")
+    if want_acc and want_y:
+        return y, acc
+    return acc if want_acc else y

@@ -1,0 +1,109 @@
+"""GPU parity: int8 GEMM + de-scale epilogue (k3q_gemm_i8) against the CPU oracle."""
+
+import pytest
+import torch
+
+from keras_amd import ops as kops
+from keras_amd import quantizers as kq
+from oracle import keras_cpu_path as ref
+from tests.helpers import RTOL, c_gemm_i8, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(M, K, N, dtype, seed, with_bias=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    kernel = ref.glorot_uniform(K, N, generator=g)
+    bias = (torch.randn(N, generator=g) * 0.02) if with_bias else None
+    qkernel, kscale = ref.dense_quantize_int8(kernel)
+    return x, qkernel, kscale, bias
+
+
+def run_dense_int8(dev, M, K, N, dtype, prepack, exact, seed=0, with_bias=True):
+    x, qk, ks, bias = make_case(M, K, N, dtype, seed, with_bias)
+    want, inter = ref.dense_int8_call(x, qk, ks, bias, compute_dtype=dtype, return_intermediates=True)
+    q, s = kq.abs_max_quantize(x.to(dev), axis=-1)
+    assert torch.equal(q.cpu(), inter["q"])
+    qk_d = qk.to(dev)
+    pre = kops.prepack_int8_kernel(qk_d) if prepack else None
+    y, acc = kops.int8_matmul(
+        q, qk_d, a_scale=s, kernel_scale=ks.to(dtype).to(dev),
+        bias=bias.to(dtype).to(dev) if bias is not None else None, out_dtype=dtype,
+        prepacked=pre, exact_epilogue=exact, want_acc=True)
+    torch.cuda.synchronize()
+    assert torch.equal(acc.cpu(), inter["acc"]), "int32 accumulators differ from the reference"
+    if exact:
+        # same op chain, same rounding points: bit-identical
+        assert torch.equal(y.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                           want.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    else:
+        e = max_rel_err(y, want)
+        assert e <= RTOL[dtype], e
+    return y
+
+
+SHAPES = [
+    (1, 128, 4), (3, 128, 12), (16, 4096, 4096), (17, 256, 260), (64, 512, 1000),
+    (255, 384, 256), (256, 1024, 512), (300, 640, 772), (513, 256, 1028),
+    # shapes off the MFMA path (K % 128 != 0 or N % 4 != 0): plain kernel
+    (5, 100, 30), (8, 8, 16), (33, 64, 7), (2, 200, 64),
+]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("prepack", [True, False])
+def test_dense_int8_exact_epilogue(dev, M, K, N, dtype, prepack):
+    run_dense_int8(dev, M, K, N, dtype, prepack, exact=True)
+
+
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 4096), (300, 640, 772), (512, 4096, 4096)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_int8_fast_epilogue(dev, M, K, N, dtype):
+    run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=False)
+
+
+def test_config1_dense_4096(dev):
+    # BASELINE config 1: Dense(4096) on [16, 4096] float32 inputs, bias, seed 0
+    run_dense_int8(dev, 16, 4096, 4096, torch.float32, prepack=True, exact=True, seed=0)
+
+
+def test_gemm_extreme_values(dev):
+    # +-127 everywhere: |acc| = K * 127 * 127 must not overflow or saturate
+    K = 14336
+    a = torch.full((130, K), 127, dtype=torch.int8)
+    a[::2] = -127
+    b = torch.full((K, 260), -127, dtype=torch.int8)
+    acc = kops.int8_matmul(a.to(dev), b.to(dev), want_acc=True, want_y=False,
+                           prepacked=kops.prepack_int8_kernel(b.to(dev)))
+    want = torch.matmul(a.to(torch.int32), b.to(torch.int32))
+    assert torch.equal(acc.cpu(), want)
+    assert want.abs().max().item() == K * 127 * 127
+
+
+@pytest.mark.parametrize("M,K,N", [(4096, 8192, 8192), (2048, 4096, 4096), (512, 8192, 28672)])
+def test_gemm_full_size_accumulators(dev, M, K, N):
+    # full BASELINE sizes: sampled rows against the CPU oracle (bit-exact) plus two
+    # size-independent integer identities over the whole output
+    g = torch.Generator().manual_seed(7)
+    a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (K, N), generator=g, dtype=torch.int8)
+    a_d, b_d = a.to(dev), b.to(dev)
+    acc = kops.int8_matmul(a_d, b_d, want_acc=True, want_y=False,
+                           prepacked=kops.prepack_int8_kernel(b_d))
+    rows = torch.randint(0, M, (24,), generator=g)
+    want_rows = c_gemm_i8(a[rows], b)
+    assert torch.equal(acc[rows.to(dev)].cpu(), want_rows)
+    # sum over rows of acc == (column sums of a) . b ; sum over columns == a . (row sums of b)
+    colsum_a = a.to(torch.int64).sum(0)
+    rowsum_b = b.to(torch.int64).sum(1)
+    assert torch.equal(acc.to(torch.int64).sum(0).cpu(), colsum_a @ b.to(torch.int64))
+    assert torch.equal(acc.to(torch.int64).sum(1).cpu(), a.to(torch.int64) @ rowsum_b)
+
+
+def test_prepack_is_transpose(dev):
+    g = torch.Generator().manual_seed(1)
+    for K, N in [(128, 64), (100, 37), (4096, 4096), (65, 129)]:
+        b = torch.randint(-128, 128, (K, N), generator=g, dtype=torch.int8)
+        assert torch.equal(kops.prepack_int8_kernel(b.to(dev)).cpu(), b.t().contiguous())
