@@ -1,0 +1,525 @@
+"""`EinsumDense` with the int8 / int4 quantized forward on MI355X.
+
+Mirrors the quantization-related surface of `keras.layers.EinsumDense`
+(keras/src/layers/core/einsum_dense.py): equation analysis, variable names and
+shapes (`_kernel`, `kernel_scale` in the reference's broadcast layout,
+`kernel_zero`, `g_idx`), `quantize`, `_int8_call`, `_int4_call`.
+
+The quantized einsum is lowered to the 2-D kernels: every equation whose labels
+split into free (input and output), contracted (input and kernel) and kept
+(kernel and output) sets is a GEMM of the input viewed as [free, contracted]
+with the kernel viewed as [contracted, kept]; the views are free of copies for
+the usual projection equations (`btd,dnh->btnh`, `btnh,nhd->btd`, `ab,bc->ac`).
+"""
+
+import math
+import string
+
+import torch
+
+from keras_amd import dtype_policies, ops as kops, quantizers
+from keras_amd.layers.dense import _ACTIVATIONS, _EXACT_EPILOGUE_MAX_OUTPUTS, glorot_uniform
+from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
+
+
+def _canonical_specs(equation, input_rank):
+    """(input, kernel, output) label strings with `...` replaced by fresh labels.
+
+    Accepts `X,Y->Z`, `...X,Y->...Z` and `X...,Y->Z...`
+    (keras/src/layers/core/einsum_dense.py:1728-1757, :1932-1993).
+    """
+    eq = equation.replace(" ", "")
+    bad = ValueError(
+        f"Invalid einsum equation '{equation}'. Equations must be in the "
+        "form [X],[Y]->[Z], ...[X],[Y]->...[Z], or [X]...,[Y]->[Z]...."
+    )
+    if eq.count("->") != 1 or eq.count(",") != 1:
+        raise bad
+    lhs, out = eq.split("->")
+    a, b = lhs.split(",")
+    if "." in b:
+        raise bad
+    if "..." not in a and "..." not in out:
+        if not (a.isalpha() and b.isalpha() and out.isalpha()):
+            raise bad
+        return a, b, out, 0, False
+    left = a.startswith("...") and out.startswith("...")
+    right = a.endswith("...") and out.endswith("...")
+    if left == right:
+        raise bad
+    core_in = a[3:] if left else a[:-3]
+    core_out = out[3:] if left else out[:-3]
+    if not (core_in.isalpha() and b.isalpha() and core_out.isalpha()):
+        raise bad
+    if right and len(core_in) < 2:
+        raise bad
+    n = input_rank - len(core_in)
+    spare = sorted(set(string.ascii_letters) - set(core_in) - set(b) - set(core_out))
+    pad = "".join(spare[:n])
+    if left:
+        return pad + core_in, b, pad + core_out, n, True
+    return core_in + pad, b, core_out + pad, n, False
+
+
+def analyze_einsum_shapes(equation, bias_axes, input_shape, output_shape):
+    """Kernel shape, bias shape and full output shape of an EinsumDense
+    (keras/src/layers/core/einsum_dense.py:1700-1899)."""
+    i_spec, k_spec, o_spec, elided, left = _canonical_specs(equation, len(input_shape))
+    out_dims = [output_shape] if isinstance(output_shape, int) else list(output_shape)
+    out_dims.insert(0, input_shape[0])
+    if elided > 0 and left:
+        for i in range(1, elided):
+            out_dims.insert(1, input_shape[i])
+    elif elided > 0:
+        for i in range(len(input_shape) - elided, len(input_shape)):
+            out_dims.append(input_shape[i])
+    size_in = {c: input_shape[i] for i, c in enumerate(i_spec)}
+    size_out = {c: out_dims[i] for i, c in enumerate(o_spec)}
+    for c in i_spec:
+        if c in size_out and size_out[c] is not None and size_out[c] != size_in[c]:
+            raise ValueError(
+                "Input shape and output shape do not match at shared "
+                f"dimension '{c}'. Input shape is {size_in[c]}, "
+                f"and output shape is {size_out[c]}."
+            )
+    for c in o_spec:
+        if c not in i_spec and c not in k_spec:
+            raise ValueError(
+                f"Dimension '{c}' was specified in the output '{o_spec}' but has no "
+                f"corresponding dim in the input spec '{i_spec}' or weight spec '{k_spec}'"
+            )
+    kernel_shape = []
+    for c in k_spec:
+        if c in size_out:
+            kernel_shape.append(size_out[c])
+        elif c in size_in:
+            kernel_shape.append(size_in[c])
+        else:
+            raise ValueError(
+                f"Weight dimension '{c}' did not have a match in either "
+                f"the input spec '{i_spec}' or the output spec '{o_spec}'. "
+                "For this layer, the weight must be fully specified."
+            )
+    bias_shape = None
+    if bias_axes is not None:
+        # labels of the user's output spec only (the padded ones never carry a bias)
+        user_o = o_spec[elided:] if left else (o_spec[:-elided] if elided else o_spec)
+        for c in bias_axes:
+            if c not in user_o:
+                raise ValueError(
+                    f"Bias dimension '{c}' was requested, but is not part "
+                    f"of the output spec '{user_o}'"
+                )
+        first = min(user_o.find(c) for c in bias_axes)
+        bias_shape = [size_out[c] if c in bias_axes else 1 for c in user_o[first:]]
+        if not left:
+            bias_shape += [1] * elided
+    return tuple(kernel_shape), (None if bias_shape is None else tuple(bias_shape)), tuple(out_dims)
+
+
+def analyze_quantization_info(equation, input_rank):
+    """Axes bookkeeping for per-axis quantisation of an einsum
+    (keras/src/layers/core/einsum_dense.py:1902-2062).
+
+    For the input and for the kernel: the axes the quantizer reduces, and the
+    transpose / expand_dims / squeeze that turn a keepdims scale into a tensor
+    that broadcasts against the einsum output.  The reference shares one scratch
+    variable between its label scans and both fix-up loops; when an operand has
+    more reduced axes than the output has axes missing from it, the surplus axes
+    are squeezed and inserted at the last position that variable held.  That
+    behaviour decides stored `kernel_scale` shapes, so it is kept.
+    """
+    i_spec, k_spec, o_spec, _, _ = _canonical_specs(equation, input_rank)
+    parts = {}
+    for name, spec in (("input", i_spec), ("kernel", k_spec)):
+        parts[name] = {
+            "reduced": [ax for ax, c in enumerate(spec) if c not in o_spec],
+            "expand": [ax for ax, c in enumerate(o_spec) if c not in spec],
+            "transpose": [spec.index(c) for c in o_spec if c in spec],
+            "squeeze": [],
+        }
+    position = o_spec.find(k_spec[-1])
+    for name in ("input", "kernel"):
+        part = parts[name]
+        for ax in part["reduced"]:
+            if part["expand"]:
+                position = part["expand"].pop(0)
+            else:
+                part["squeeze"].append(ax)
+            part["transpose"].insert(position, ax)
+    parts["specs"] = (i_spec, k_spec, o_spec)
+    parts["custom_gradient_equation"] = f"{o_spec},{k_spec}->{i_spec}"
+    return parts
+
+
+def _adjust_scale(scale, part):
+    """transpose, expand_dims, squeeze (einsum_dense.py:1650-1680)."""
+    if part["transpose"]:
+        scale = scale.permute(part["transpose"])
+    for ax in sorted(part["expand"]):
+        scale = scale.unsqueeze(ax)
+    for ax in sorted(part["squeeze"], reverse=True):
+        if scale.shape[ax] == 1:
+            scale = scale.squeeze(ax)
+    return scale
+
+
+class _GemmView:
+    """How an einsum `X,Y->Z` maps onto `[M, K] x [K, N]`."""
+
+    def __init__(self, i_spec, k_spec, o_spec):
+        si, sk, so = set(i_spec), set(k_spec), set(o_spec)
+        if si & sk & so:
+            raise NotImplementedError(
+                f"labels {sorted(si & sk & so)} appear in the input, the kernel and the output: "
+                "batched-kernel einsums are not lowered to the quantized GEMM"
+            )
+        if (si - sk - so) or (sk - si - so):
+            raise NotImplementedError("einsums that sum a label out of one operand alone are not supported")
+        self.contracted = [c for c in k_spec if c in si]        # kernel order
+        self.kept = [c for c in o_spec if c in sk]              # output order
+        self.free = [c for c in i_spec if c in so]              # input order
+        self.in_perm = [i_spec.index(c) for c in self.free + self.contracted]
+        self.k_perm = [k_spec.index(c) for c in self.contracted + self.kept]
+        gemm_out = self.free + self.kept
+        self.out_perm = [gemm_out.index(c) for c in o_spec]
+        self.in_is_view = self.in_perm == list(range(len(i_spec)))
+        self.k_is_view = self.k_perm == list(range(len(k_spec)))
+        self.out_is_view = self.out_perm == list(range(len(o_spec)))
+        # int4 stores reshape(kernel, [prod(reduced), prod(kept)]) row-major: that is the
+        # [K, N] matrix only when the kernel is already laid out [contracted..., kept...]
+        # with the kept labels in kernel order equal to their output order
+        self.k_plain = self.k_is_view
+
+
+class EinsumDense(Layer):
+    def __init__(self, equation, output_shape, activation=None, bias_axes=None,
+                 kernel_initializer=None, bias_initializer="zeros", dtype=None, name=None,
+                 device=None):
+        super().__init__(dtype=dtype, name=name, device=device)
+        self.equation = equation
+        self.partial_output_shape = (output_shape,) if isinstance(output_shape, int) else tuple(output_shape)
+        self.bias_axes = bias_axes
+        self.activation = activation if callable(activation) else _ACTIVATIONS[activation]
+        self.kernel_initializer = kernel_initializer or glorot_uniform
+        self.bias_initializer = bias_initializer
+        self.lora_enabled = False
+        self.exact_epilogue = None
+        self._cache = {}
+
+    # ---- build ---------------------------------------------------------------
+    def build(self, input_shape):
+        kernel_shape, bias_shape, full_output_shape = analyze_einsum_shapes(
+            self.equation, self.bias_axes, tuple(input_shape), self.partial_output_shape
+        )
+        self.full_output_shape = full_output_shape
+        self.input_rank = len(input_shape)
+        self.original_kernel_shape = kernel_shape
+        if self.quantization_mode is not None:
+            self.quantized_build(kernel_shape, mode=self.quantization_mode)
+        if self.quantization_mode not in ("int8", "int4"):
+            self._kernel = self.add_weight(
+                name="kernel", shape=kernel_shape, initializer=self.kernel_initializer, trainable=True
+            )
+        if bias_shape is not None:
+            self.bias = self.add_weight(
+                name="bias", shape=bias_shape, initializer=self.bias_initializer, trainable=True
+            )
+        else:
+            self.bias = None
+        self.built = True
+
+    @property
+    def kernel(self):
+        if not self.built:
+            raise AttributeError("You must build the layer before accessing `kernel`.")
+        kernel = as_tensor(self._kernel)
+        if self.quantization_mode == "int4":
+            kernel = quantizers.unpack_int4(kernel, self._int4_unpacked_column_size, axis=-1)
+            kernel = kernel.reshape(self.original_kernel_shape)
+        return kernel
+
+    def call(self, inputs, training=None):
+        x = torch.einsum(self.equation, inputs, self.read(self._kernel))
+        if self.bias is not None:
+            x = torch.add(x, self.read(self.bias))
+        if self.activation is not None:
+            x = self.activation(x)
+        return x
+
+    # ---- quantized variables -----------------------------------------------------
+    def _set_quantization_info(self):
+        if hasattr(self, "_quant_info"):
+            return
+        info = analyze_quantization_info(self.equation, self.input_rank)
+        self._quant_info = info
+        self._input_reduced_axes = info["input"]["reduced"]
+        self._kernel_reduced_axes = info["kernel"]["reduced"]
+        self._custom_gradient_equation = info["custom_gradient_equation"]
+        self._gemm = None
+        try:
+            self._gemm = _GemmView(*info["specs"])
+        except NotImplementedError as e:
+            self._gemm_error = e
+
+    def quantized_build(self, kernel_shape, mode, config=None):
+        if mode == "int8":
+            self._int8_build(kernel_shape, config)
+        elif mode == "int4":
+            self._int4_build(kernel_shape, config)
+        else:
+            raise self._quantization_mode_error(mode)
+        self._is_quantized = True
+
+    def _get_kernel_scale_shape(self, kernel_shape):
+        """Per-channel scale shape: the kernel shape with reduced axes set to 1, taken
+        through the kernel's transpose / expand / squeeze (einsum_dense.py:1478-1491)."""
+        probe = torch.empty(
+            [1 if ax in self._kernel_reduced_axes else d for ax, d in enumerate(kernel_shape)],
+            device="meta",
+        )
+        return tuple(_adjust_scale(probe, self._quant_info["kernel"]).shape)
+
+    def _int8_build(self, kernel_shape, config=None):
+        self._set_quantization_info()
+        self.inputs_quantizer = QuantizationConfig.activation_quantizer_or_default(
+            config, quantizers.AbsMaxQuantizer()
+        )
+        self.quantization_axis = tuple(self._input_reduced_axes)
+        self._kernel = self.add_weight(name="kernel", shape=kernel_shape, dtype="int8")
+        self.kernel_scale = self.add_weight(
+            name="kernel_scale", shape=self._get_kernel_scale_shape(kernel_shape), initializer="ones"
+        )
+
+    def _flat_dims(self, kernel_shape):
+        rows = cols = 1
+        for ax, d in enumerate(kernel_shape):
+            if ax in self._kernel_reduced_axes:
+                rows *= d
+            else:
+                cols *= d
+        return rows, cols
+
+    def _int4_build(self, kernel_shape, config=None):
+        self._set_quantization_info()
+        self.inputs_quantizer = QuantizationConfig.activation_quantizer_or_default(config, None)
+        self.quantization_axis = tuple(self._input_reduced_axes)
+        self.original_kernel_shape = tuple(kernel_shape)
+        rows, cols = self._flat_dims(kernel_shape)
+        block_size = get_block_size_for_layer(self, config)
+        use_grouped = block_size is not None and block_size != -1
+        self._int4_block_size = block_size if use_grouped else None
+        self._int4_unpacked_column_size = cols
+        self._int4_rows = rows
+        self._kernel = self.add_weight(name="kernel", shape=(rows, (cols + 1) // 2), dtype="int8")
+        scale_shape = (math.ceil(rows / block_size), cols) if use_grouped else (cols,)
+        self.kernel_scale = self.add_weight(name="kernel_scale", shape=scale_shape, initializer="ones")
+        if use_grouped:
+            self.kernel_zero = self.add_weight(name="kernel_zero", shape=scale_shape, dtype="int8")
+            self.g_idx = self.add_weight(
+                name="g_idx", shape=(rows,), dtype="float32",
+                initializer=lambda shape, dtype: torch.floor_divide(
+                    torch.arange(rows, dtype=dtype), block_size),
+            )
+
+    # ---- quantize ---------------------------------------------------------------------
+    def _quantize(self, mode, config, type_check=True):
+        if type_check and type(self) is not EinsumDense:
+            raise self._not_implemented_error(self.quantize)
+        self.quantization_config = config
+        kernel_shape = self._kernel.shape
+        self._set_quantization_info()
+        kernel_zero = None
+        if mode == "int8":
+            weight_quantizer = QuantizationConfig.weight_quantizer_or_default(
+                config, quantizers.AbsMaxQuantizer(axis=self._kernel_reduced_axes)
+            )
+            kernel_value, kernel_scale = weight_quantizer(as_tensor(self._kernel), to_numpy=True)
+            kernel_scale = _adjust_scale(kernel_scale, self._quant_info["kernel"]).contiguous()
+        elif mode == "int4":
+            block_size = get_block_size_for_layer(self, config)
+            use_grouped = block_size is not None and block_size != -1
+            rows, cols = self._flat_dims(kernel_shape)
+            flat = as_tensor(self._kernel).reshape(rows, cols)
+            if not use_grouped:
+                q4, kernel_scale = quantizers.abs_max_quantize(
+                    flat, axis=0, value_range=(-8, 7), dtype="int8", to_numpy=True
+                )
+                kernel_scale = torch.squeeze(kernel_scale, dim=0)
+            else:
+                q4, kernel_scale, kernel_zero = quantizers.abs_max_quantize_grouped_with_zero_point(
+                    flat, block_size=block_size, to_numpy=True
+                )
+            kernel_value, _, _ = quantizers.pack_int4(q4.to(self.device), axis=-1)
+        else:
+            raise self._quantization_mode_error(mode)
+        self._variables = [v for v in self._variables if v is not self._kernel]
+        del self._kernel
+        self.quantized_build(kernel_shape, mode, config)
+        self._kernel.assign(kernel_value)
+        self.kernel_scale.assign(kernel_scale)
+        if kernel_zero is not None:
+            self.kernel_zero.assign(kernel_zero)
+        if self.dtype_policy.quantization_mode is None:
+            policy_name = mode
+            if mode == "int4":
+                block_size = get_block_size_for_layer(self, config)
+                policy_name = f"int4/{-1 if block_size is None else block_size}"
+            self._dtype_policy = dtype_policies.get(f"{policy_name}_from_{self.dtype_policy.name}")
+        self._cache.clear()
+
+    # ---- helpers ---------------------------------------------------------------------------
+    def _cached(self, key, var, make):
+        if var is None:
+            return None
+        hit = self._cache.get(key)
+        if hit is not None and hit[0] == var.version and hit[1] is var:
+            return hit[2]
+        value = make(as_tensor(var))
+        self._cache[key] = (var.version, var, value)
+        return value
+
+    def _gemm_view(self):
+        if self._gemm is None:
+            raise self._gemm_error
+        return self._gemm
+
+    def _input_rows(self, inputs, gv):
+        x = inputs if gv.in_is_view else inputs.permute(gv.in_perm)
+        k = 1
+        for d in x.shape[len(gv.free):]:
+            k *= d
+        free_shape = tuple(x.shape[:len(gv.free)])
+        return x.reshape(-1, k), free_shape
+
+    def _finish(self, y2, free_shape, gv, fused_bias):
+        kept_shape = tuple(self.full_output_shape_of(c) for c in gv.kept)
+        y = y2.reshape(*free_shape, *kept_shape)
+        if not gv.out_is_view:
+            y = y.permute(gv.out_perm)
+        if self.bias is not None and not fused_bias:
+            y = torch.add(y, self.read(self.bias))
+        if self.activation is not None:
+            y = self.activation(y)
+        return y
+
+    def full_output_shape_of(self, label):
+        k_spec = self._quant_info["specs"][1]
+        return self.original_kernel_shape[k_spec.index(label)]
+
+    def _fusable_bias(self, gv, n):
+        """The bias as an [N] vector when it spans exactly the kept (kernel) axes, which
+        are then the trailing output axes; otherwise None and the bias is added after."""
+        if self.bias is None:
+            return None, True
+        o_spec = self._quant_info["specs"][2]
+        trailing = list(o_spec[len(o_spec) - len(gv.kept):]) == gv.kept
+        kept_shape = tuple(self.full_output_shape_of(c) for c in gv.kept)
+        if trailing and self.bias.shape == kept_shape:
+            cd = to_torch_dtype(self.compute_dtype)
+            return self._cached("bias", self.bias, lambda t: t.to(cd).reshape(-1).contiguous()), True
+        return None, False
+
+    # ---- quantized forward -----------------------------------------------------------------
+    def _int8_call(self, inputs, training=None):
+        """keras/src/layers/core/einsum_dense.py:1030-1118 as quantise-rows + int8 GEMM."""
+        if self.lora_enabled:
+            raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
+        if not self.inputs_quantizer:
+            raise NotImplementedError(
+                "Weight-only int8 (no activation quantizer) is not on the fused path yet."
+            )
+        gv = self._gemm_view()
+        x2, free_shape = self._input_rows(inputs, gv)
+        q, scale = self.inputs_quantizer(x2, axis=-1)
+        cd = to_torch_dtype(self.compute_dtype)
+
+        def kernel_matrix(t):
+            k2 = t if gv.k_is_view else t.permute(gv.k_perm)
+            return k2.reshape(x2.shape[1], -1).contiguous()
+
+        k2 = self._cached("kernel2d", self._kernel, kernel_matrix)
+        n = k2.shape[1]
+        pre = self._cached("prepacked", self._kernel, lambda t: kops.prepack_int8_kernel(kernel_matrix(t)))
+        bias, fused = self._fusable_bias(gv, n)
+        exact = self.exact_epilogue
+        if exact is None:
+            exact = x2.shape[0] * n <= _EXACT_EPILOGUE_MAX_OUTPUTS
+        y2 = kops.int8_matmul(
+            q, k2, a_scale=scale,
+            kernel_scale=self._cached("kernel_scale", self.kernel_scale,
+                                      lambda t: t.to(cd).reshape(-1).contiguous()),
+            bias=bias, out_dtype=cd, prepacked=pre, exact_epilogue=exact,
+        )
+        return self._finish(y2, free_shape, gv, fused)
+
+    def _int4_call(self, inputs, training=None):
+        """keras/src/layers/core/einsum_dense.py:1120-1261, weight-only."""
+        if self.lora_enabled:
+            raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
+        if self.inputs_quantizer:
+            raise NotImplementedError("int4 with an activation quantizer is not on the fused path yet.")
+        gv = self._gemm_view()
+        if not gv.k_plain:
+            raise NotImplementedError(
+                f"equation '{self.equation}': the stored int4 kernel is a row-major reshape of a kernel "
+                "whose contracted axes are not leading, which the fused int4 kernel cannot consume in place"
+            )
+        x2, free_shape = self._input_rows(inputs, gv)
+        cd = to_torch_dtype(self.compute_dtype)
+        block_size = self._int4_block_size
+        grouped = block_size is not None and block_size > 0
+        bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
+        y2 = kops.int4_matmul(
+            x2, as_tensor(self._kernel),
+            self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).contiguous()),
+            self._int4_unpacked_column_size,
+            kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+            block_size=block_size if grouped else None,
+            bias=bias,
+        )
+        return self._finish(y2, free_shape, gv, fused)
+
+    # ---- serialization -------------------------------------------------------------------------
+    @property
+    def variable_serialization_spec(self):
+        """einsum_dense.py:560-610, the modes built here."""
+        return {
+            None: ["kernel", "bias"],
+            "int8": ["kernel", "bias", "kernel_scale"],
+            "int4": ["kernel", "bias", "kernel_scale", "kernel_zero", "g_idx"],
+        }
+
+    def save_own_variables(self, store):
+        if not self.built:
+            return
+        idx = 0
+        for name in self.variable_serialization_spec[self.quantization_mode]:
+            if name == "kernel":
+                value = self._kernel
+            elif name == "bias" and self.bias is None:
+                continue
+            elif name in ("kernel_zero", "g_idx") and not hasattr(self, name):
+                continue
+            else:
+                value = getattr(self, name)
+            store[str(idx)] = as_tensor(value)
+            idx += 1
+
+    def load_own_variables(self, store):
+        if not self.built:
+            return
+        idx = 0
+        for name in self.variable_serialization_spec[self.quantization_mode]:
+            if name == "kernel":
+                target = self._kernel
+            elif name == "bias" and self.bias is None:
+                continue
+            elif name in ("kernel_zero", "g_idx") and not hasattr(self, name):
+                continue
+            else:
+                target = getattr(self, name)
+            target.assign(store[str(idx)])
+            idx += 1
+        self._cache.clear()

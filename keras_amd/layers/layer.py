@@ -1,0 +1,236 @@
+"""Layer plumbing shared by `Dense` and `EinsumDense`.
+
+Only what the quantized forward needs of `keras.layers.Layer` is restated:
+the dtype policy, the cast of inputs to the compute dtype, reading float
+variables in the compute dtype (autocast), the `quantize()` argument checks and
+the dispatch to `_int8_call` / `_int4_call`
+(keras/src/layers/layer.py:243-261, :797-849, :874-1003, :1366-1458).
+"""
+
+import numpy as np
+import torch
+
+from keras_amd import dtype_policies
+from keras_amd.quantization_config import validate_and_resolve_config
+
+_TORCH_DTYPES = {
+    "float32": torch.float32,
+    "bfloat16": torch.bfloat16,
+    "float16": torch.float16,
+    "int8": torch.int8,
+    "uint8": torch.uint8,
+    "int32": torch.int32,
+}
+
+
+def to_torch_dtype(name):
+    if isinstance(name, torch.dtype):
+        return name
+    return _TORCH_DTYPES[name]
+
+
+def default_device():
+    return torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else torch.device("cpu")
+
+
+class Variable:
+    """A named tensor with `assign`, as far as the quantized layers use it."""
+
+    def __init__(self, value, name, trainable=False):
+        self.name = name
+        self.trainable = trainable
+        self._value = value
+        self.version = 0  # bumped by assign(); caches derived from the value key on it
+
+    @property
+    def value(self):
+        return self._value
+
+    @property
+    def shape(self):
+        return tuple(self._value.shape)
+
+    @property
+    def dtype(self):
+        return str(self._value.dtype).replace("torch.", "")
+
+    @property
+    def device(self):
+        return self._value.device
+
+    def assign(self, value):
+        if isinstance(value, Variable):
+            value = value.value
+        if not isinstance(value, torch.Tensor):
+            value = torch.as_tensor(np.asarray(value))
+        if tuple(value.shape) != self.shape:
+            raise ValueError(
+                "The shape of the target variable and the shape of the target value in "
+                f"`variable.assign(value)` must match. variable.shape={self.shape}, "
+                f"Received: value.shape={tuple(value.shape)}. Target variable: {self.name}"
+            )
+        self._value = value.to(device=self._value.device, dtype=self._value.dtype).contiguous()
+        self.version += 1
+
+    def numpy(self):
+        v = self._value.detach().cpu()
+        return (v.float() if v.dtype == torch.bfloat16 else v).numpy()
+
+    def __repr__(self):
+        return f"<Variable {self.name} shape={self.shape} dtype={self.dtype}>"
+
+
+def as_tensor(x):
+    return x.value if isinstance(x, Variable) else x
+
+
+class Layer:
+    def __init__(self, dtype=None, name=None, device=None):
+        self.name = name or type(self).__name__.lower()
+        self._dtype_policy = dtype_policies.get(dtype)
+        self.device = torch.device(device) if device is not None else default_device()
+        self.built = False
+        self._is_quantized = False
+        self.quantization_config = None
+        self._variables = []
+
+    # ---- dtype policy ------------------------------------------------------
+    @property
+    def dtype_policy(self):
+        return self._dtype_policy
+
+    @dtype_policy.setter
+    def dtype_policy(self, value):
+        policy = dtype_policies.get(value)
+        # keras/src/layers/layer.py:797-817: a quantized policy set on a built float layer
+        # converts the layer
+        if policy.quantization_mode is not None and self.built and not self._is_quantized:
+            self.quantize(policy.quantization_mode, type_check=False)
+        self._dtype_policy = policy
+
+    @property
+    def compute_dtype(self):
+        return self._dtype_policy.compute_dtype
+
+    @property
+    def variable_dtype(self):
+        return self._dtype_policy.variable_dtype
+
+    @property
+    def quantization_mode(self):
+        return self._dtype_policy.quantization_mode
+
+    # ---- variables ----------------------------------------------------------
+    def add_weight(self, name, shape, dtype=None, initializer="zeros", trainable=False):
+        tdtype = to_torch_dtype(dtype or self.variable_dtype)
+        if callable(initializer):
+            value = initializer(tuple(shape), tdtype)
+            if not isinstance(value, torch.Tensor):
+                value = torch.as_tensor(np.asarray(value))
+            value = value.to(device=self.device, dtype=tdtype)
+        elif initializer == "ones":
+            value = torch.ones(tuple(shape), dtype=tdtype, device=self.device)
+        elif initializer == "zeros":
+            value = torch.zeros(tuple(shape), dtype=tdtype, device=self.device)
+        else:
+            raise ValueError(f"Unknown initializer: {initializer}")
+        var = Variable(value, name=f"{self.name}/{name}", trainable=trainable)
+        self._variables.append(var)
+        return var
+
+    def read(self, var):
+        """Value of a variable as `call` sees it: float variables are read in the compute
+        dtype under a mixed policy (AutocastScope,
+        keras/src/backend/common/variables.py:245-249, :677-708)."""
+        if var is None:
+            return None
+        t = as_tensor(var)
+        cd = to_torch_dtype(self.compute_dtype)
+        if t.dtype.is_floating_point and t.dtype != cd:
+            return t.to(cd)
+        return t
+
+    # ---- call ---------------------------------------------------------------
+    def __call__(self, inputs, training=None):
+        if not isinstance(inputs, torch.Tensor):
+            inputs = torch.as_tensor(np.asarray(inputs))
+        if not self.built:
+            self.build(tuple(inputs.shape))
+        if inputs.device != self.device:
+            inputs = inputs.to(self.device)
+        cd = to_torch_dtype(self.compute_dtype)
+        if inputs.dtype.is_floating_point and inputs.dtype != cd:
+            inputs = inputs.to(cd)
+        if self.quantization_mode is not None:
+            return self.quantized_call(inputs, training=training)
+        return self.call(inputs, training=training)
+
+    def quantized_call(self, *args, **kwargs):
+        mode = self.quantization_mode
+        if mode == "int8":
+            return self._int8_call(*args, **kwargs)
+        if mode == "int4":
+            return self._int4_call(*args, **kwargs)
+        raise self._quantization_mode_error(mode)
+
+    def _int8_call(self, *args, **kwargs):
+        raise self._not_implemented_error(self._int8_call)
+
+    def _int4_call(self, *args, **kwargs):
+        raise self._not_implemented_error(self._int4_call)
+
+    # ---- quantize -----------------------------------------------------------
+    def quantize(self, mode=None, config=None, **kwargs):
+        """Argument checks of `quantize_wrapper`, then the layer's own conversion."""
+        config = validate_and_resolve_config(mode, config)
+        mode = config.mode
+        self._check_quantize_args(mode, self.compute_dtype)
+        return self._quantize(mode=mode, config=config, **kwargs)
+
+    def _quantize(self, mode, config, type_check=True):
+        raise self._not_implemented_error(self.quantize)
+
+    def _check_quantize_args(self, mode, compute_dtype):
+        if not self.built:
+            raise ValueError(
+                "Cannot quantize a layer that isn't yet built. "
+                f"Layer '{self.name}' (of type '{self.__class__.__name__}') "
+                "is not built yet."
+            )
+        if getattr(self, "_is_quantized", False):
+            raise ValueError(
+                f"Layer '{self.name}' is already quantized with "
+                f"dtype_policy='{self.dtype_policy.name}'. "
+                f"Received: mode={mode}"
+            )
+        if mode not in dtype_policies.QUANTIZATION_MODES:
+            raise ValueError(
+                "Invalid quantization mode. "
+                f"Expected one of {dtype_policies.QUANTIZATION_MODES}. "
+                f"Received: mode={mode}"
+            )
+        if mode == "int8" and compute_dtype == "float16":
+            raise ValueError(
+                f"Quantization mode='{mode}' doesn't work well with "
+                "compute_dtype='float16'. Consider loading model/layer with "
+                "another dtype policy such as 'mixed_bfloat16' or "
+                "'mixed_float16' before calling `quantize()`."
+            )
+
+    def _not_implemented_error(self, attr, msg=None):
+        if callable(attr):
+            attr_name, attr_type = attr.__name__, "method"
+        else:
+            attr_name, attr_type = str(attr), "attribute"
+        msg = f" {msg}" if msg is not None else ""
+        return NotImplementedError(
+            f"Layer {self.__class__.__name__} does not have a `{attr_name}` "
+            f"{attr_type} implemented.{msg}"
+        )
+
+    def _quantization_mode_error(self, mode):
+        return NotImplementedError(
+            "Invalid quantization mode. Expected one of "
+            f"{dtype_policies.QUANTIZATION_MODES}. "
+            f"Received: quantization_mode={mode}"
+        )

@@ -1,0 +1,211 @@
+"""GPU parity: Dense / EinsumDense quantized layers end to end against the CPU oracle."""
+
+import pytest
+import torch
+
+import keras_amd as ka
+from keras_amd.layers import Dense, EinsumDense
+from oracle import keras_cpu_path as ref
+from tests.helpers import RTOL, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def bits(t):
+    return t.view(torch.int16) if t.dtype == torch.bfloat16 else t.view(torch.int32)
+
+
+def build_dense(dev, K, N, policy, seed, use_bias=True):
+    g = torch.Generator().manual_seed(seed)
+    layer = Dense(N, use_bias=use_bias, dtype=policy, device=dev,
+                  kernel_initializer=lambda s, d: ref.glorot_uniform(s[0], s[1], generator=g).to(d),
+                  bias_initializer=lambda s, d: (torch.randn(s, generator=g) * 0.02).to(d))
+    layer.build((None, K))
+    return layer
+
+
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16", "bfloat16"])
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 4096), (5, 128, 48), (300, 256, 512), (2, 100, 30)])
+def test_dense_int8_layer(dev, policy, M, K, N):
+    layer = build_dense(dev, K, N, policy, seed=0)
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(1))
+    y_float = layer(x)
+    layer.quantize("int8")
+    assert layer.dtype_policy.name == f"int8_from_{policy}"
+    assert layer._kernel.dtype == "int8" and layer.kernel_scale.dtype == layer.variable_dtype
+    qk, ks = ref.dense_quantize_int8(kernel_f)
+    assert torch.equal(layer._kernel.value.cpu(), qk)
+    assert torch.equal(bits(layer.kernel_scale.value.cpu()), bits(ks))
+    layer.exact_epilogue = True
+    y = layer(x)
+    want = ref.dense_int8_call(x.to(cd), qk, ks, bias_f, compute_dtype=cd)
+    assert y.dtype == cd
+    assert torch.equal(bits(y.cpu()), bits(want))
+    layer.exact_epilogue = False
+    assert max_rel_err(layer(x), want) <= RTOL[cd]
+    # the reference's own (weak) check: dense_test.py:438-463
+    mse = (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item()
+    mse_ref = (y_float.float().cpu() - want.float()).pow(2).mean().item()
+    assert mse <= 1.25 * mse_ref + 1e-5
+
+
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+@pytest.mark.parametrize("block_size", [128, 64, None, -1])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 512), (16, 512, 384), (7, 300, 64), (40, 256, 96)])
+def test_dense_int4_layer(dev, policy, block_size, M, K, N):
+    layer = build_dense(dev, K, N, policy, seed=2)
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(3))
+    y_float = layer(x)
+    layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=block_size))
+    per_channel = block_size is None or block_size == -1
+    assert layer.dtype_policy.name == f"int4/{-1 if per_channel else block_size}_from_{policy}"
+    qk = ref.dense_quantize_int4(kernel_f, block_size)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    assert torch.equal(layer.kernel_scale.value.cpu(), qk["kernel_scale"])
+    assert torch.equal(layer.kernel.cpu(), qk["unpacked"])
+    if per_channel:
+        assert not hasattr(layer, "kernel_zero")
+    else:
+        assert torch.equal(layer.kernel_zero.value.cpu(), qk["kernel_zero"])
+        assert torch.equal(layer.g_idx.value.cpu(), qk["g_idx"])
+    y = layer(x)
+    want = ref.dense_int4_call(
+        x.to(cd), qk["kernel"], qk["kernel_scale"], N, kernel_zero=qk["kernel_zero"],
+        g_idx=qk["g_idx"], block_size=block_size, bias=bias_f, compute_dtype=cd)
+    assert y.dtype == cd and tuple(y.shape) == (M, N)
+    assert max_rel_err(y, want) <= RTOL[cd]
+    # quantisation noise must be the reference's, not more (its own weak test bounds the MSE
+    # of an 8 -> 16 layer, dense_test.py:438-463; the bound does not carry to other sizes)
+    mse = (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item()
+    mse_ref = (y_float.float().cpu() - want.float()).pow(2).mean().item()
+    assert mse <= 1.25 * mse_ref + 1e-5
+
+
+def test_dense_leading_axes_and_activation(dev):
+    layer = Dense(64, activation="relu", device=dev)
+    layer.build((None, None, 256))
+    x = torch.randn(2, 3, 256)
+    layer.quantize("int8")
+    y = layer(x)
+    assert tuple(y.shape) == (2, 3, 64) and (y >= 0).all()
+    flat = layer(x.reshape(6, 256)).reshape(2, 3, 64)
+    assert torch.equal(y, flat)
+
+
+def test_variables_reload_round_trip(dev):
+    a = build_dense(dev, 512, 256, "float32", seed=5)
+    a.quantize("int4")
+    store = {}
+    a.save_own_variables(store)
+    assert list(store) == ["0", "1", "2", "3", "4"]
+    b = Dense(256, dtype="int4/128_from_float32", device=dev)
+    b.build((None, 512))
+    b.load_own_variables({k: v.cpu() for k, v in store.items()})
+    x = torch.randn(3, 512)
+    assert torch.equal(a(x), b(x))
+
+
+EQUATIONS = [
+    # equation, output_shape, input_shape  (einsum_dense_test.py:556-691 and BASELINE config 4 shapes, scaled)
+    ("btnh,nhd->btd", (None, 8), (1, 2, 2, 4)),
+    ("btd,ndh->btnh", (None, 2, 8), (1, 2, 4)),
+    ("btd,df->btf", (None, 4), (1, 2, 4)),
+    ("ab,bcd->acd", (8, 32), (2, 3)),
+    ("btd,dnh->btnh", (None, 4, 32), (3, 5, 256)),
+    ("btnh,nhd->btd", (None, 256), (3, 5, 4, 64)),
+    ("...b,bc->...c", (24,), (2, 3, 128)),
+]
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape", EQUATIONS)
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_einsum_dense_int8(dev, equation, output_shape, input_shape, policy):
+    g = torch.Generator().manual_seed(1337)
+    layer = EinsumDense(equation, output_shape, dtype=policy, device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    x = torch.rand(input_shape, generator=g)
+    y_float = layer(x)
+    layer.quantize("int8")
+    qk, ks, _ = ref.einsum_dense_quantize_int8(kernel_f, equation, len(input_shape))
+    assert torch.equal(layer._kernel.value.cpu(), qk)
+    assert tuple(layer.kernel_scale.shape) == tuple(ks.shape)
+    assert torch.equal(layer.kernel_scale.value.cpu(), ks)
+    layer.exact_epilogue = True
+    y = layer(x)
+    want = ref.einsum_dense_int8_call(x.to(cd), qk, ks, equation, compute_dtype=cd)
+    assert tuple(y.shape) == tuple(want.shape)
+    assert torch.equal(bits(y.cpu().contiguous()), bits(want.contiguous()))
+    assert (y_float.float() - y.float()).pow(2).mean().item() < 2e-2
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape", [EQUATIONS[0], EQUATIONS[2], EQUATIONS[4], EQUATIONS[5]])
+@pytest.mark.parametrize("block_size", [128, None])
+def test_einsum_dense_int4(dev, equation, output_shape, input_shape, block_size):
+    g = torch.Generator().manual_seed(1337)
+    layer = EinsumDense(equation, output_shape, dtype="mixed_bfloat16", device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d))
+    layer.build(input_shape)
+    kernel_f = layer._kernel.value.cpu()
+    x = torch.rand(input_shape, generator=g)
+    y_float = layer(x)
+    layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=block_size))
+    qk = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), block_size)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    assert torch.equal(layer.kernel_scale.value.cpu(), qk["kernel_scale"])
+    y = layer(x)
+    want = ref.einsum_dense_int4_call(x.to(torch.bfloat16), qk, equation, compute_dtype=torch.bfloat16,
+                                      block_size=block_size)
+    assert max_rel_err(y, want) <= RTOL[torch.bfloat16]
+    mse = (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item()
+    mse_ref = (y_float.float().cpu() - want.float()).pow(2).mean().item()
+    assert mse <= 1.25 * mse_ref + 1e-5
+
+
+@pytest.mark.parametrize("t", [1, 512])
+def test_config4_attention_projections(dev, t):
+    # BASELINE config 4: d_model 4096, 32 heads x 128, batch 8, bf16
+    g = torch.Generator().manual_seed(4)
+    for equation, out_shape, in_shape in [
+        ("btd,dnh->btnh", (None, 32, 128), (8, t, 4096)),
+        ("btnh,nhd->btd", (None, 4096), (8, t, 32, 128)),
+    ]:
+        layer = EinsumDense(equation, out_shape, dtype="mixed_bfloat16", device=dev,
+                            kernel_initializer=lambda s, d: ref.glorot_uniform(4096, 4096, shape=s, generator=g).to(d))
+        layer.build(in_shape)
+        kernel_f = layer._kernel.value.cpu()
+        x = torch.randn(in_shape, generator=g).to(torch.bfloat16)
+        layer.quantize("int8")
+        layer.exact_epilogue = True
+        y = layer(x)
+        qk, ks, _ = ref.einsum_dense_quantize_int8(kernel_f, equation, len(in_shape))
+        ts = slice(0, min(t, 16))
+        want = ref.einsum_dense_int8_call(x[3:4, ts], qk, ks, equation, compute_dtype=torch.bfloat16)
+        assert torch.equal(bits(y[3:4, ts].cpu().contiguous()), bits(want.contiguous()))
+
+
+def test_unsupported_paths_raise(dev):
+    layer = Dense(16, device=dev)
+    with pytest.raises(ValueError):
+        layer.quantize("int8")  # not built
+    layer.build((None, 32))
+    with pytest.raises(ValueError):
+        layer.quantize("int5")
+    layer.quantize("int8")
+    with pytest.raises(ValueError):
+        layer.quantize("int8")  # already quantized
+    cpu_layer = Dense(16, device="cpu")
+    cpu_layer.build((None, 32))
+    cpu_layer.quantize("int8")
+    with pytest.raises(RuntimeError):
+        cpu_layer(torch.randn(2, 32))  # no CPU fallback
