@@ -1,0 +1,234 @@
+"""Benchmark of the quantized Dense hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one forward pass of an int8-quantized Dense layer over one batch:
+the fused abs-max activation quantizer followed by the int8 MFMA GEMM with the
+de-scale epilogue, at BASELINE's target shape M=4096, K=N=8192, bfloat16
+activations (inputs and weights already resident in HBM).  `value` is
+2*M*N*K / step time in TOP/s.  The int4 decode GEMV (K=N=8192, M in {1,4,16}),
+the second half of BASELINE's metric, is reported under `int4_gemv` with its own
+HBM roofline.  The CPU oracle (a restatement of the reference's torch-CPU op
+sequence) is timed on the host cores on a bounded sample as `cpu_baseline`.
+
+Prints ONE JSON line.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+INT8_PEAK_TOPS = 5000.0  # MI355X dense int8, published (5.0 POP/s)
+HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
+
+# HBM bytes per GEMM launch measured with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`
+# (see profiles/gemm_i8_mfma_M4096_K8192_N8192.md); None until measured.
+GEMM_HBM_TRAFFIC_BYTES = None
+GEMV_HBM_TRAFFIC_BYTES = None
+
+
+def gemv_algorithmic_bytes(M, K, N, grouped, block=128):
+    scales = 5 * (K // block) * N if grouped else 4 * N
+    return K * (N // 2) + scales + 2 * M * K + 2 * M * N
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the quantized Dense path has no multi-GPU leg "
+                 f"(got --gpus {args.gpus}); its column-sharded form needs no exchange step")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a HIP device; none is visible")
+
+    from keras_amd import _lib, ops as kops, quantizers as kq
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    g = torch.Generator().manual_seed(0)
+
+    # ------------------------------------------------------------------ int8 Dense forward
+    M, K, N = 4096, 8192, 8192
+    limit = (6.0 / (K + N)) ** 0.5
+    kernel_f = (torch.rand(K, N, generator=g) * 2 - 1) * limit  # glorot uniform
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    wq, wscale = kq.abs_max_quantize(kernel_f, axis=0, to_numpy=True)  # one-time, host side
+    wq = wq.to(dev)
+    wscale_t = wscale.reshape(-1).to(torch.bfloat16).to(dev)
+    prepacked = kops.prepack_int8_kernel(wq)  # one-time [N,K] shadow copy of the int8 kernel
+    del kernel_f
+
+    def step():
+        q, s = kq.abs_max_quantize(x, axis=-1)
+        return kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
+                                prepacked=prepacked)
+
+    # W untimed warm-up steps, then exactly K timed steps.  The K steps are recorded once
+    # into a HIP graph and replayed, so that the clock sees the kernels and not the Python
+    # interpreter between them (the layer's forward is two launches).
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        step()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(args.steps):
+                step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    del graph
+    ops_per_step = 2.0 * M * N * K
+    value = ops_per_step / (ms_per_step * 1e-3) / 1e12
+
+    # dominant kernel alone, HIP events on the stream it is launched on
+    q, s = kq.abs_max_quantize(x, axis=-1)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * args.steps)]
+    for i in range(args.steps):
+        ev[2 * i].record()
+        kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
+                         prepacked=prepacked)
+        ev[2 * i + 1].record()
+    torch.cuda.synchronize()
+    gemm_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
+    gemm_tops = ops_per_step / (gemm_ms * 1e-3) / 1e12
+    for i in range(args.steps):
+        ev[2 * i].record()
+        kq.abs_max_quantize(x, axis=-1)
+        ev[2 * i + 1].record()
+    torch.cuda.synchronize()
+    quant_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
+    quant_bytes = M * K * 2 + M * K + M * 2
+
+    # ------------------------------------------------------------------ int4 decode GEMV
+    Kg = Ng = 8192
+    n_rot = 12  # 12 x 32 MiB packed kernels: more than the 256 MiB last-level cache
+    packs = [torch.randint(-128, 128, (Kg, Ng // 2), generator=g, dtype=torch.int8).to(dev)
+             for _ in range(n_rot)]
+    pc_scale = (torch.rand(Ng, generator=g) + 0.5).to(torch.bfloat16).to(dev)
+    gr_scale = (torch.rand(Kg // 128, Ng, generator=g) * 0.01 + 0.001).to(torch.bfloat16).to(dev)
+    gr_zero = torch.randint(-8, 8, (Kg // 128, Ng), generator=g, dtype=torch.int8).to(dev)
+    gemv = []
+    for Mg in (1, 4, 16):
+        xg = torch.randn(Mg, Kg, generator=g).to(torch.bfloat16).to(dev)
+        for grouped in (False, True):
+            def call(i):
+                if grouped:
+                    return kops.int4_matmul(xg, packs[i % n_rot], gr_scale, Ng, kernel_zero=gr_zero,
+                                            block_size=128)
+                return kops.int4_matmul(xg, packs[i % n_rot], pc_scale, Ng)
+
+            # a HIP graph of back-to-back calls: decode loops are launch-bound from Python
+            reps = 4 * n_rot
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                for i in range(n_rot):
+                    call(i)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(reps):
+                        call(i)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / (3 * reps) * 1e3
+            nbytes = gemv_algorithmic_bytes(Mg, Kg, Ng, grouped)
+            gbs = nbytes / (us * 1e-6) / 1e9
+            gemv.append({
+                "M": Mg, "K": Kg, "N": Ng,
+                "scheme": "grouped/128+zero" if grouped else "per-channel",
+                "us_per_call": round(us, 2), "algorithmic_bytes": nbytes,
+                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                             "traffic": GEMV_HBM_TRAFFIC_BYTES},
+            })
+            del graph
+        del xg
+
+    # ------------------------------------------------------------------ CPU baseline (oracle)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import keras_cpu_path as ref
+
+        Mc = 2048  # bounded sample (about 10 s): 2048 rows of the same K = N = 8192 layer
+        xc = x[:Mc].cpu()
+        wq_c, ws_c = wq.cpu(), wscale.reshape(-1)
+        ref.dense_int8_call(xc[:8], wq_c, ws_c, None, compute_dtype=torch.bfloat16)  # warm up
+        t0 = time.perf_counter()
+        ref.dense_int8_call(xc, wq_c, ws_c, None, compute_dtype=torch.bfloat16)
+        cpu_s = time.perf_counter() - t0
+        cpu = {
+            "value": round(2.0 * Mc * N * K / cpu_s / 1e12, 5), "unit": "TOP/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle Dense int8 forward (torch-CPU op sequence of the reference), "
+                      f"{Mc} of {M} rows, K=N={K}, one pass, {cpu_s:.1f} s; host has {os.cpu_count()} cpus",
+        }
+        # int4 decode GEMV on the host: unpack + float matmul per call, as the reference does
+        w4 = packs[0].cpu()
+        x1 = torch.randn(1, Kg, generator=g).to(torch.bfloat16)
+        ref.dense_int4_call(x1, w4, pc_scale.cpu().float(), Ng, compute_dtype=torch.bfloat16)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            ref.dense_int4_call(x1, w4, pc_scale.cpu().float(), Ng, compute_dtype=torch.bfloat16)
+        g_s = (time.perf_counter() - t0) / 3
+        cpu["int4_gemv"] = {"value": round(gemv_algorithmic_bytes(1, Kg, Ng, False) / g_s / 1e9, 3),
+                            "unit": "GB/s", "sample": f"oracle Dense int4 per-channel, M=1, K=N={Kg}, 3 passes"}
+
+    out = {
+        "metric": "int8 GEMM TOPS (Dense int8 forward: quantize + GEMM + de-scale)",
+        "value": round(value, 1),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": f"Dense int8 forward M={M} K={K} N={N}, bf16 activations ~N(0,1), "
+                               "glorot-uniform kernel quantized per channel, kernel prepacked once"},
+        "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": INT8_PEAK_TOPS,
+                     "unit": "TFLOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 4),
+                     "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "gemm_i8_mfma",
+                     "avg_launch_us": round(gemm_ms * 1e3, 1), "ops_per_launch": ops_per_step,
+                     "note": "int8 multiply-accumulate counted as 2 ops; peak is the published dense int8 figure"},
+        "quantizer": {"kernel": "quantize_rows_vec", "avg_launch_us": round(quant_ms * 1e3, 1),
+                      "roofline": {"bound": "hbm", "achieved": round(quant_bytes / (quant_ms * 1e-3) / 1e9, 1),
+                                   "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(quant_bytes / (quant_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                   "traffic": None}},
+        "int4_gemv": gemv,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,272 @@
+"""Pins the CPU oracle: reference known-answer vectors, closed forms, brute force and the
+cross-check between the torch restatement and the independent C restatement."""
+
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import keras_cpu_path as ref
+from tests.helpers import c_gemm_i8, c_oracle, c_w4_matmul_f64
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+# ---------------------------------------------------------------- pack / unpack
+def test_pack_docstring_vectors():
+    data = json.load(open(os.path.join(HERE, "golden", "pack_int4_docstring_vectors.json")))
+    for case in data["cases"]:
+        arr = torch.tensor(case["input"], dtype=torch.int8)
+        packed, shape, n = ref.pack_int4(arr, axis=case["axis"])
+        assert packed.tolist() == case["packed"]
+        assert n == case["orig_len"] and shape == tuple(packed.shape)
+        back = ref.unpack_int4(packed, n, axis=case["axis"])
+        assert back.tolist() == case["input"]
+
+
+def test_pack_closed_form_all_pairs():
+    lo = torch.arange(-8, 8, dtype=torch.int8).repeat(16)
+    hi = torch.arange(-8, 8, dtype=torch.int8).repeat_interleave(16)
+    arr = torch.stack([lo, hi], dim=0)  # pack along axis 0: one byte per column
+    packed, _, _ = ref.pack_int4(arr, axis=0)
+    want = ((lo.to(torch.int32) & 15) | ((hi.to(torch.int32) & 15) << 4)).to(torch.uint8).view(torch.int8)
+    assert torch.equal(packed[0], want)
+
+
+def test_unpack_exhaustive_bytes():
+    b = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    got = ref.unpack_int4(b.view(torch.int8).reshape(1, 256), 2, axis=0)
+    v = b.to(torch.int32)
+    assert torch.equal(got[0].to(torch.int32), ((v & 15) ^ 8) - 8)
+    assert torch.equal(got[1].to(torch.int32), (((v >> 4) & 15) ^ 8) - 8)
+    gotu = ref.unpack_int4(b.reshape(1, 256), 2, axis=0, dtype="uint8")
+    assert torch.equal(gotu[0].to(torch.int32), v & 15)
+    assert torch.equal(gotu[1].to(torch.int32), (v >> 4) & 15)
+
+
+SCENARIOS = [((8, 8), 0), ((8, 8), 1), ((5, 8), 0), ((8, 5), 1), ((4, 6, 8), 1), ((4, 6, 5), -1),
+             ((2, 3, 4, 5), 2)]  # quantizers_test.py:157-175
+
+
+@pytest.mark.parametrize("shape,axis", SCENARIOS)
+@pytest.mark.parametrize("dtype", ["int8", "uint8"])
+def test_pack_round_trip_scenarios(shape, axis, dtype):
+    g = torch.Generator().manual_seed(0)
+    if dtype == "int8":
+        arr = torch.randint(-8, 8, shape, generator=g, dtype=torch.int8)
+    else:
+        arr = torch.randint(0, 16, shape, generator=g, dtype=torch.uint8)
+    packed, pshape, n = ref.pack_int4(arr, axis=axis, dtype=dtype)
+    ax = axis % len(shape)
+    assert pshape[ax] == math.ceil(shape[ax] / 2) and n == shape[ax]
+    assert torch.equal(ref.unpack_int4(packed, n, axis=axis, dtype=dtype), arr)
+    # C restatement agrees byte for byte
+    outer = int(np.prod(shape[:ax])) if ax else 1
+    inner = int(np.prod(shape[ax + 1:])) if ax + 1 < len(shape) else 1
+    cp = torch.empty(pshape, dtype=arr.dtype)
+    c_oracle().k3q_oracle_pack_int4(arr.contiguous().data_ptr(), outer, shape[ax], inner, cp.data_ptr())
+    assert torch.equal(cp, packed)
+    cu = torch.empty(shape, dtype=arr.dtype)
+    c_oracle().k3q_oracle_unpack_int4(cp.data_ptr(), outer, pshape[ax], inner, n,
+                                      1 if dtype == "int8" else 0, cu.data_ptr())
+    assert torch.equal(cu, arr)
+
+
+def test_pack_errors():
+    with pytest.raises(ValueError):
+        ref.pack_int4(torch.zeros(2, 2, dtype=torch.int8), dtype="int16")
+    with pytest.raises(TypeError):
+        ref.pack_int4(torch.zeros(2, 2, dtype=torch.uint8), dtype="int8")
+    with pytest.raises(TypeError):
+        ref.unpack_int4(torch.zeros(2, 2, dtype=torch.int32), 4)
+
+
+# ---------------------------------------------------------------- abs-max quantizer
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_abs_max_invariants(dtype):
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(3, 4, 5, generator=g) * 2).to(dtype)
+    q, s = ref.abs_max_quantize(x, axis=-1)
+    assert q.dtype == torch.int8 and s.dtype == dtype and tuple(s.shape) == (3, 4, 1)
+    assert q.min() >= -127 and q.max() <= 127
+    # the arg-max element of every row maps to +-127
+    idx = x.abs().float().argmax(-1, keepdim=True)
+    assert (q.gather(-1, idx).abs() >= 126).all()
+    deq = q.float() / s.float()
+    assert (deq - x.float()).pow(2).mean().sqrt() < 0.1
+    # numpy path == tensor path in float32 (quantizers_test.py:106-115)
+    if dtype == torch.float32:
+        qn, sn = ref.abs_max_quantize(x, axis=-1, to_numpy=True)
+        assert torch.equal(qn, q) and torch.allclose(sn, s, rtol=1e-6, atol=0)
+
+
+def test_abs_max_closed_form_rows():
+    x = torch.zeros(4, 8)
+    x[1] = torch.tensor([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, 63.5, -127.0])  # scale ~ 1: ties to even
+    x[2] = 2.0 ** torch.arange(-4, 4).float()
+    q, s = ref.abs_max_quantize(x, axis=-1)
+    assert torch.equal(q[0], torch.zeros(8, dtype=torch.int8))
+    assert s[0, 0].item() == pytest.approx(127.0 / 1e-7, rel=1e-6)
+    # 127 / (127 + 1e-7) rounds to exactly 1.0 in float32
+    assert s[1, 0].item() == 1.0
+    assert q[1].tolist() == [127, 0, 2, 2, 0, -2, 64, -127]
+    assert q[2].tolist() == [round(v) for v in (x[2] * s[2, 0]).tolist()]
+
+
+@pytest.mark.parametrize("dtype_code,dtype", [(0, torch.float32), (1, torch.bfloat16)])
+def test_abs_max_c_restatement_agrees(dtype_code, dtype):
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(64, 1000, generator=g) * 3).to(dtype)
+    x[5] = 0
+    x[6, 3] = 1e-6
+    q, s = ref.abs_max_quantize(x, axis=-1)
+    cq = torch.empty_like(q)
+    cs = torch.empty(64, dtype=dtype)
+    c_oracle().k3q_oracle_absmax_quantize(x.data_ptr(), dtype_code, 64, 1000, 1e-7, -127.0, 127.0,
+                                          cq.data_ptr(), cs.data_ptr())
+    assert torch.equal(cs.float(), s.flatten().float())
+    assert torch.equal(cq, q)
+
+
+def test_bf16_epsilon_is_rounded_before_the_add():
+    # torch casts the 0-dim float32 epsilon to bfloat16 before adding: distinguishes the two
+    # candidate semantics on rows whose max is tiny
+    bitsv = torch.arange(0x2000, 0x3800, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    x = bitsv.reshape(-1, 1)
+    _, s = ref.abs_max_quantize(x, axis=-1)
+    eps_bf = torch.tensor(1e-7).to(torch.bfloat16).float()
+    want = (127.0 / (x.float() + eps_bf).to(torch.bfloat16).float()).to(torch.bfloat16)
+    assert torch.equal(s, want)
+
+
+# ---------------------------------------------------------------- grouped quantizer
+def test_grouped_quantizer_against_loops():
+    g = torch.Generator().manual_seed(42)
+    w = torch.randn(500, 6, generator=g)  # 500 rows / block 128: last group is zero padded
+    q, s, z = ref.abs_max_quantize_grouped_with_zero_point(w, block_size=128)
+    assert tuple(q.shape) == (500, 6) and tuple(s.shape) == (4, 6) and tuple(z.shape) == (4, 6)
+    assert z.dtype == torch.int8 and q.min() >= -8 and q.max() <= 7
+    wn = w.numpy()
+    for gi in range(4):
+        rows = wn[gi * 128:(gi + 1) * 128]
+        if rows.shape[0] < 128:
+            rows = np.concatenate([rows, np.zeros((128 - rows.shape[0], 6), np.float32)])
+        for n in range(6):
+            lo, hi = rows[:, n].min(), rows[:, n].max()
+            sc = np.float32((hi - lo + np.float32(1e-7)) / np.float32(15))
+            zp = np.clip(np.round(-lo / sc) + -8, -8, 7)
+            assert s[gi, n].item() == pytest.approx(float(sc), rel=1e-6)
+            assert z[gi, n].item() == int(zp)
+            for r in range(min(128, 500 - gi * 128)):
+                want = int(np.clip(np.round(np.float32(rows[r, n]) / sc) + zp, -8, 7))
+                assert q[gi * 128 + r, n].item() == want
+    # de-quantised error bound of quantizers_test.py:754-788
+    g_idx = torch.floor_divide(torch.arange(500, dtype=torch.float32), 128)
+    deq = ref.dequantize_with_sz_map(q, s, z, g_idx, group_axis=0)
+    assert (deq - w).pow(2).mean().sqrt() < 0.15
+
+
+def test_dequantize_with_sz_map_double_loop():
+    g = torch.Generator().manual_seed(3)
+    q = torch.randint(-8, 8, (12, 5), generator=g, dtype=torch.int8)
+    s = torch.rand(3, 5, generator=g) + 0.1
+    z = torch.randint(-8, 8, (3, 5), generator=g, dtype=torch.int8)
+    g_idx = torch.tensor([0, 0, 0, 0, 1, 1, 1, 1, 2, 2, 2, 2], dtype=torch.float32)
+    got = ref.dequantize_with_sz_map(q, s, z, g_idx, group_axis=0)
+    for k in range(12):
+        for n in range(5):
+            gi = int(g_idx[k])
+            assert got[k, n].item() == pytest.approx((q[k, n].item() - z[gi, n].item()) * s[gi, n].item(), rel=1e-6)
+
+
+# ---------------------------------------------------------------- integer matmul / epilogue
+def test_int8_matmul_brute_force():
+    g = torch.Generator().manual_seed(0)
+    a = torch.randint(-128, 128, (7, 33), generator=g, dtype=torch.int8)
+    b = torch.randint(-128, 128, (33, 5), generator=g, dtype=torch.int8)
+    got = ref.matmul(a, b)
+    assert got.dtype == torch.int32
+    want = a.numpy().astype(np.int64) @ b.numpy().astype(np.int64)
+    assert np.array_equal(got.numpy().astype(np.int64), want)
+    assert torch.equal(c_gemm_i8(a, b), got)
+    e = ref.einsum("ab,bc->ac", a, b)
+    assert torch.equal(e, got)
+
+
+def test_int8_matmul_no_overflow_at_max_k():
+    a = torch.full((2, 14336), 127, dtype=torch.int8)
+    b = torch.full((14336, 3), -127, dtype=torch.int8)
+    assert ref.matmul(a, b)[0, 0].item() == -14336 * 127 * 127
+    assert c_gemm_i8(a, b)[1, 2].item() == -14336 * 127 * 127
+
+
+@pytest.mark.parametrize("dtype_code,dtype", [(0, torch.float32), (1, torch.bfloat16)])
+def test_dense_int8_call_matches_c_restatement(dtype_code, dtype):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(9, 256, generator=g).to(dtype)
+    kernel = ref.glorot_uniform(256, 40, generator=g)
+    bias = torch.randn(40, generator=g) * 0.02
+    qk, ks = ref.dense_quantize_int8(kernel)
+    y, inter = ref.dense_int8_call(x, qk, ks, bias, compute_dtype=dtype, return_intermediates=True)
+    assert torch.equal(inter["acc"], c_gemm_i8(inter["q"], qk))
+    cy = torch.empty(9, 40, dtype=dtype)
+    # keep the operands alive across the call: data_ptr() of a temporary dangles
+    acc_c, si_c = inter["acc"].contiguous(), inter["inputs_scale"].contiguous()
+    ks_c, bias_c = ks.to(dtype).contiguous(), bias.to(dtype).contiguous()
+    c_oracle().k3q_oracle_descale(acc_c.data_ptr(), 9, 40, dtype_code, si_c.data_ptr(),
+                                  ks_c.data_ptr(), bias_c.data_ptr(), cy.data_ptr())
+    assert torch.equal(cy.float(), y.float())
+    # closed form in float64 within the stated tolerance
+    exact = inter["acc"].double() / (ks.double() * inter["inputs_scale"].double()) + bias.double()
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    assert ((y.double() - exact).abs().max() / exact.abs().max()).item() < tol
+
+
+@pytest.mark.parametrize("block_size", [None, 32])
+def test_dense_int4_call_against_f64(block_size):
+    g = torch.Generator().manual_seed(6)
+    kernel = ref.glorot_uniform(128, 24, generator=g)
+    qk = ref.dense_quantize_int4(kernel, block_size)
+    x = torch.randn(5, 128, generator=g)
+    y = ref.dense_int4_call(x, qk["kernel"], qk["kernel_scale"], 24, kernel_zero=qk["kernel_zero"],
+                            g_idx=qk["g_idx"], block_size=block_size)
+    exact = c_w4_matmul_f64(x, qk["kernel"], qk["kernel_scale"], qk["kernel_zero"], block_size, None, 24)
+    assert ((y.double() - exact).abs().max() / exact.abs().max()).item() < 1e-5
+    # and the weight-only result approximates the float layer
+    assert (y - x @ kernel).pow(2).mean().item() < 2e-2
+
+
+# ---------------------------------------------------------------- EinsumDense bookkeeping
+def test_einsum_info_hand_derived_rows():
+    a = ref.einsum_quantization_info("btd,dnh->btnh", 3)
+    assert a["input"]["reduced"] == [2] and a["kernel"]["reduced"] == [0]
+    b = ref.einsum_quantization_info("btnh,nhd->btd", 4)
+    assert b["input"]["reduced"] == [2, 3] and b["input"]["transpose"] == [0, 1, 3, 2]
+    assert b["input"]["squeeze"] == [3] and b["kernel"]["reduced"] == [0, 1]
+    k = torch.randn(4096 // 64, 4, 8)  # stand-in for [d, n, h]
+    _, s, _ = ref.einsum_dense_quantize_int8(k, "btd,dnh->btnh", 3)
+    assert tuple(s.shape) == (1, 1, 4, 8)
+    k2 = torch.randn(4, 8, 16)
+    _, s2, _ = ref.einsum_dense_quantize_int8(k2, "btnh,nhd->btd", 4)
+    assert tuple(s2.shape) == (1, 1, 16)
+
+
+@pytest.mark.parametrize("equation,kshape,xshape", [
+    ("btnh,nhd->btd", (2, 4, 8), (1, 2, 2, 4)), ("btd,ndh->btnh", (2, 4, 8), (1, 2, 4)),
+    ("btd,df->btf", (4, 4), (1, 2, 4)), ("ab,bcd->acd", (3, 8, 32), (2, 3)),
+    ("...b,bc->...c", (7, 5), (2, 3, 7)), ("abc,cd->abd", (6, 9), (2, 3, 6)),
+])
+def test_einsum_int8_descale_approximates_float(equation, kshape, xshape):
+    # the scales must broadcast against the einsum output such that the de-scaled integer
+    # einsum approximates the float einsum: a wrong axis, transpose or squeeze breaks this
+    g = torch.Generator().manual_seed(1337)
+    kernel = torch.rand(kshape, generator=g) - 0.5
+    x = torch.rand(xshape, generator=g)
+    qk, ks, _ = ref.einsum_dense_quantize_int8(kernel, equation, len(xshape))
+    y = ref.einsum_dense_int8_call(x, qk, ks, equation)
+    want = torch.einsum(equation, x, kernel)
+    assert tuple(y.shape) == tuple(want.shape)
+    assert (y - want).pow(2).mean().item() < 1e-3
