@@ -120,10 +120,9 @@ int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64
  * divide of Dense._int4_call (keras/src/layers/core/dense.py:988-1095) and the
  * int4 branch of EinsumDense (keras/src/layers/core/einsum_dense.py:1120-1261).
  *
- * workspace: k3q_gemv_w4_workspace_bytes(M, K, N) bytes, 16-byte aligned, whose
- * first 4096 bytes are ZERO before the first call; the kernel leaves them zero.
- * It holds split-K partial sums and per-column-block arrival tickets, so two
- * calls that overlap in time must not share a workspace.
+ * workspace: k3q_gemv_w4_workspace_bytes(M, K, N) bytes, 16-byte aligned, contents
+ * irrelevant.  It holds the fp32 partial sums of the K split between the two
+ * kernels of a call, so two calls that overlap in time must not share one.
  */
 int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
@@ -135,7 +134,8 @@ int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
  * Same as k3q_gemv_w4 with the launch plan overridden, for tuning sweeps:
  * plan = {dwords per lane per k row (1|2|4), 16-row steps per chunk (1|2),
  * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null
- * `plan` keep the built-in choice.  No counterpart in the reference.
+ * `plan` keep the built-in choice.  The workspace must then hold
+ * ceil(K / (waves * rows per wave)) * min(M, 16) * N floats.  No counterpart in the reference.
  */
 int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
                      const void* w_packed, const void* scale, const void* zero,

@@ -84,6 +84,10 @@ __device__ __forceinline__ float load_t(const void* p, int64_t i) {
 template <bool kBF16, bool kExact>
 __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
+#ifdef K3Q_GEMM_PROBE_CLOCK
+    const uint64_t clk0 = __builtin_readcyclecounter();
+    const uint64_t rt0 = __builtin_amdgcn_s_memrealtime();
+#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -226,6 +230,14 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
         }
     }
 
+#ifdef K3Q_GEMM_PROBE_CLOCK
+    if (p.acc_out && tid == 0 && blockIdx.x < 64) {
+        uint64_t* d = (uint64_t*)p.acc_out + 2 * blockIdx.x;
+        d[0] = __builtin_readcyclecounter() - clk0;
+        d[1] = __builtin_amdgcn_s_memrealtime() - rt0;
+    }
+    if (p.acc_out) return;
+#endif
     // ---- epilogue ----
     // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
     // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: per lane 4 rows of y and 8 groups

@@ -29,10 +29,12 @@
 // Split-K: wave w of workgroup (nb, ks) owns `klen` consecutive rows of K for
 // the 128 * kVec columns of block nb and walks them in register double-buffered
 // chunks of kSteps * 16 rows.  Waves of a workgroup are reduced through LDS,
-// workgroups through an fp32 scratch in `workspace`; the workgroup that
-// arrives last at a column block (atomic ticket) adds the partials in a fixed
-// order, applies the epilogue and re-arms the ticket.  The result does not
-// depend on arrival order.
+// workgroups through fp32 partials in `workspace` that a second, tiny kernel
+// adds in a fixed order before applying the epilogue: the result does not
+// depend on scheduling.  (A single-kernel variant in which the last workgroup
+// to arrive sums the partials needs a device-scope release/acquire per
+// workgroup, which on this multi-XCD part means an L2 write-back and
+// invalidate each: measured 2-5x slower than the second launch.)
 #include "k3q_common.h"
 
 namespace k3q {
@@ -53,13 +55,11 @@ struct GemvParams {
     const void* bias;      // T [N] or null
     void* y;               // T [M, N]
     float* part;           // [KS, M, N] fp32 partials (KS > 1)
-    u32* tickets;          // [n_blocks]
     int64_t K, N, row_bytes;
     int M;                 // rows of x in this launch
     int m0;                // first row of x handled by this launch
     int block_size;        // rows of K per group (grouped only)
     int klen;              // rows of K per wave (multiple of the chunk)
-    int two_pass;          // 1: partials are summed by a second kernel instead of the last workgroup
 };
 
 __device__ __forceinline__ v8bf as_bf(const v4u& v) { return __builtin_bit_cast(v8bf, v); }
@@ -114,6 +114,9 @@ __device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
 template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     extern __shared__ float red[];  // [waves][M][kNB]
+#ifdef K3Q_GEMV_PROBE
+    const uint64_t ts0 = __builtin_amdgcn_s_memrealtime();
+#endif
     constexpr bool kBF16 = !kXF32;
     constexpr int kAccSets = kXF32 ? 1 : kSets;
     constexpr int kNB = 128 * kVec;
@@ -131,7 +134,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     const int M = p.M;
 
     Packed<kVec> wreg[2][kSteps][4];
-    v4u xb[2][kSteps][kSets];
+    constexpr int kRaw = kXF32 ? 1 : kSets;  // raw x loads per step
+    v4u xraw[2][kSteps][kRaw];
     int64_t ncol = nb + 8 * kVec * i;
     if (ncol >= p.N) ncol = p.N - 8 * kVec;  // N % (8 * kVec) == 0: stays a valid lane column
 
@@ -142,10 +146,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) loff[t] = (u32)((4 * g + t) * p.row_bytes + (ncol >> 1));
     const int xel = kXF32 ? 4 : 2;
-    u32 xoff[kSets];
+    u32 xoff[kRaw], xmask[kRaw];
 #pragma unroll
-    for (int st = 0; st < kSets; ++st)
-        xoff[st] = (u32)(((kXF32 ? mrow : mrow + 8 * st) * p.K + 4 * g) * xel);
+    for (int r = 0; r < kRaw; ++r) {
+        const int m = mrow + 8 * r;
+        xmask[r] = m < M ? 0xffffffffu : 0u;
+        xoff[r] = (u32)(((m < M ? m : M - 1) * p.K + 4 * g) * xel);  // clamped, masked later
+    }
     const char* xbase = (const char*)p.x + (int64_t)p.m0 * p.K * xel;
     auto load_chunk = [&](int b, int c) {
         const int64_t kc = kw0 + (int64_t)c * kChunk;
@@ -156,45 +163,54 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) wreg[b][s][t] = load_packed<kVec>(rb + loff[t]);
         }
-        // x operand: B[slot, j] holds x[m(j), k] in even (j<8) or odd (j>=8) slots
+        // raw x values for the same rows; turned into MFMA operands at compute time so that
+        // nothing here waits on memory
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
             const int64_t ks = kc + 16 * s;
-            const bool kvalid = ks < p.K;
-            const char* xs = xbase + (kvalid ? ks : 0) * xel;
+            const char* xs = xbase + (ks < p.K ? ks : 0) * xel;
 #pragma unroll
-            for (int st = 0; st < kSets; ++st) {
-                u32 h[4] = {0u, 0u, 0u, 0u};  // bf16 bits of the four x values
+            for (int r = 0; r < kRaw; ++r) {
                 if (kXF32) {
-                    if (mrow < M && kvalid) {
-                        const v4u f = *(const v4u*)(xs + xoff[st]);
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) {
-                            const u32 hi = f[t] & 0xffff0000u;
-                            if (st == 0) {
-                                h[t] = hi >> 16;
-                            } else {
-                                const float rem = __uint_as_float(f[t]) - __uint_as_float(hi);
-                                h[t] = f32_to_bf16_bits(rem);
-                            }
-                        }
-                    }
+                    xraw[b][s][r] = *(const v4u*)(xs + xoff[r]);
                 } else {
-                    const int m = mrow + 8 * st;
-                    if (m < M && kvalid) {
-                        const v2u d = *(const v2u*)(xs + xoff[st]);
-                        h[0] = d[0] & 0xffffu;
-                        h[1] = d[0] >> 16;
-                        h[2] = d[1] & 0xffffu;
-                        h[3] = d[1] >> 16;
-                    }
+                    const v2u d = *(const v2u*)(xs + xoff[r]);
+                    xraw[b][s][r] = v4u{d[0], d[1], 0u, 0u};
                 }
-                v4u bv;
-#pragma unroll
-                for (int t = 0; t < 4; ++t) bv[t] = grp ? (h[t] << 16) : h[t];
-                xb[b][s][st] = bv;
             }
         }
+    };
+
+    // B[slot, j] holds x[m(j), k] in even (j < 8) or odd (j >= 8) slots; rows of x past M and
+    // steps past K contribute zeros
+    auto x_operand = [&](int b, int c, int s, int st) -> v4u {
+        const bool kvalid = kw0 + (int64_t)c * kChunk + 16 * s < p.K;
+        u32 h[4];
+        if (kXF32) {
+            const u32 mask = kvalid ? xmask[0] : 0u;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const u32 f = xraw[b][s][0][t] & mask;
+                const u32 hi = f & 0xffff0000u;
+                if (st == 0) {
+                    h[t] = hi >> 16;
+                } else {
+                    const float rem = __uint_as_float(f) - __uint_as_float(hi);
+                    h[t] = f32_to_bf16_bits(rem);
+                }
+            }
+        } else {
+            const u32 mask = kvalid ? xmask[st] : 0u;
+            const u32 d0 = xraw[b][s][st][0] & mask, d1 = xraw[b][s][st][1] & mask;
+            h[0] = d0 & 0xffffu;
+            h[1] = d0 >> 16;
+            h[2] = d1 & 0xffffu;
+            h[3] = d1 >> 16;
+        }
+        v4u bv;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) bv[t] = grp ? (h[t] << 16) : h[t];
+        return bv;
     };
 
     v4f acc[kAccSets][kVec][4];
@@ -221,13 +237,16 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     }
     const v4u ones = {kOnes, kOnes, kOnes, kOnes};
 
-    auto compute_chunk = [&](int b) {
+    auto compute_chunk = [&](int b, int c) {
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
+            v4u xb[kSets];
+#pragma unroll
+            for (int st = 0; st < kSets; ++st) xb[st] = x_operand(b, c, s, st);
 #pragma unroll
             for (int st = 0; st < kSets; ++st) {
                 const int a = kXF32 ? 0 : st;
-                accs[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(ones), as_bf(xb[b][s][st]),
+                accs[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(ones), as_bf(xb[st]),
                                                                   accs[a], 0, 0, 0);
             }
 #pragma unroll
@@ -243,7 +262,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
                     for (int st = 0; st < kSets; ++st) {
                         const int a = kXF32 ? 0 : st;
                         acc[a][q][pp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            as_bf(av), as_bf(xb[b][s][st]), acc[a][q][pp], 0, 0, 0);
+                            as_bf(av), as_bf(xb[st]), acc[a][q][pp], 0, 0, 0);
                     }
                 }
             }
@@ -288,18 +307,24 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     };
 
     load_chunk(0, 0);
+#ifdef K3Q_GEMV_PROBE
+    const uint64_t ts1 = __builtin_amdgcn_s_memrealtime();
+#endif
 #pragma unroll 1
     for (int c = 0; c < nchunks; c += 2) {
         if (c + 1 < nchunks) load_chunk(1, c + 1);
-        compute_chunk(0);
+        compute_chunk(0, c);
         after_chunk(c);
         if (c + 2 < nchunks) load_chunk(0, c + 2);
         if (c + 1 < nchunks) {
-            compute_chunk(1);
+            compute_chunk(1, c + 1);
             after_chunk(c + 1);
         }
     }
 
+#ifdef K3Q_GEMV_PROBE
+    const uint64_t ts2 = __builtin_amdgcn_s_memrealtime();
+#endif
     // ---- remove the +136 offset (per-channel) and park this wave's partial in LDS ----
 #pragma unroll
     for (int a = 0; a < kAccSets; ++a) {
@@ -322,76 +347,53 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     }
     __syncthreads();
 
-    // ---- reduce the waves of this workgroup ----
+    // ---- reduce the waves of this workgroup, four columns per thread ----
     const int KS = gridDim.y;
-    for (int idx = threadIdx.x; idx < M * kNB; idx += blockDim.x) {
-        const int m = idx / kNB;
-        const int nl = idx % kNB;
-        float sum = 0.f;
-        for (int w = 0; w < nwaves; ++w) sum += red[((size_t)w * M + m) * kNB + nl];
+    for (int idx = threadIdx.x; idx < M * (kNB / 4); idx += blockDim.x) {
+        const int m = idx / (kNB / 4);
+        const int nl = (idx % (kNB / 4)) * 4;
+        v4f sum = {0.f, 0.f, 0.f, 0.f};
+        for (int w = 0; w < nwaves; ++w) sum += *(const v4f*)(red + ((size_t)w * M + m) * kNB + nl);
         const int64_t n = nb + nl;
-        if (n < p.N) {
-            if (KS == 1)
-                finish<kBF16, kGrouped>(p, m, n, sum);
-            else if (p.two_pass & 4)
-                p.part[((int64_t)blockIdx.y * M + m) * p.N + n] = sum;
-            else  // written through to memory so that workgroups on other XCDs can read it
-                __hip_atomic_store(p.part + ((int64_t)blockIdx.y * M + m) * p.N + n, sum,
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    if (KS == 1 || (p.two_pass & 1)) return;
-
-    // ---- last workgroup to arrive at this column block finishes it ----
-    __shared__ u32 ticket;
-    if (!(p.two_pass & 2)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __syncthreads();
-    if (threadIdx.x == 0)
-        ticket = __hip_atomic_fetch_add(p.tickets + blockIdx.x, 1u, __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (ticket != (u32)(KS - 1)) return;
-    for (int idx = threadIdx.x; idx < M * kNB; idx += blockDim.x) {
-        const int m = idx / kNB;
-        const int64_t n = nb + (idx % kNB);
-        if (n < p.N) {
-            // agent-scope loads: served from memory, never from a stale L2 line.  Four
-            // independent chains keep the loads in flight; the order of addition is fixed.
-            float s4[4] = {0.f, 0.f, 0.f, 0.f};
-            const float* src = p.part + (int64_t)m * p.N + n;
-            const int64_t stride = (int64_t)M * p.N;
-            int ks = 0;
-            for (; ks + 4 <= KS; ks += 4) {
+        if (n < p.N) {  // N % 8 == 0 on this path: all four columns in or out
+            if (KS == 1) {
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    s4[u] += __hip_atomic_load(src + (ks + u) * stride, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
+                for (int e = 0; e < 4; ++e) finish<kBF16, kGrouped>(p, m, n + e, sum[e]);
+            } else {
+                *(v4f*)(p.part + ((int64_t)blockIdx.y * M + m) * p.N + n) = sum;
             }
-            for (; ks < KS; ++ks)
-                s4[0] += __hip_atomic_load(src + ks * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            finish<kBF16, kGrouped>(p, m, n, (s4[0] + s4[1]) + (s4[2] + s4[3]));
         }
     }
-    if (threadIdx.x == 0)
-        __hip_atomic_store(p.tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#ifdef K3Q_GEMV_PROBE
+    if (threadIdx.x == 0 && KS > 1) {
+        uint64_t* d = (uint64_t*)(p.part + (int64_t)KS * M * p.N) + 4 * (blockIdx.y * gridDim.x + blockIdx.x);
+        d[0] = ts0; d[1] = ts1; d[2] = ts2; d[3] = __builtin_amdgcn_s_memrealtime();
+    }
+#endif
 }
 
-// second pass of the two-pass variant: sum the KS partials of every output and finish it
+// Second pass when K is split over workgroups: sum the KS partials of every output in a
+// fixed order and apply the epilogue.  A kernel boundary is the cheapest device-wide
+// ordering point between the partial stores and these loads.
 template <bool kBF16, bool kGrouped>
 __global__ __launch_bounds__(256) void gemv_w4_reduce(GemvParams p, int KS) {
-    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const int m = blockIdx.y;
     if (n >= p.N) return;
-    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+    v4f s4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) s4[u] = v4f{0.f, 0.f, 0.f, 0.f};
     const float* src = p.part + (int64_t)m * p.N + n;
     const int64_t stride = (int64_t)p.M * p.N;
     int ks = 0;
     for (; ks + 4 <= KS; ks += 4) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) s4[u] += src[(ks + u) * stride];
+        for (int u = 0; u < 4; ++u) s4[u] += *(const v4f*)(src + (ks + u) * stride);
     }
-    for (; ks < KS; ++ks) s4[0] += src[ks * stride];
-    finish<kBF16, kGrouped>(p, m, n, (s4[0] + s4[1]) + (s4[2] + s4[3]));
+    for (; ks < KS; ++ks) s4[0] += *(const v4f*)(src + ks * stride);
+    const v4f sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) finish<kBF16, kGrouped>(p, m, n + e, sum[e]);
 }
 
 // Any shape: one thread per output, fp32 FMA chain over K.  Used when N is not a
@@ -438,9 +440,8 @@ struct Plan {
     int ks;      // workgroups along K
 };
 
-constexpr int64_t kTicketBytes = 4096;  // room for 1024 column blocks
 constexpr int kTargetWorkgroups = 256;  // one per CU
-constexpr int kDefaultTwoPass = 1;
+
 
 // plan_override (may be null): {vec, steps, waves, klen}; entries <= 0 keep the heuristic.
 Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
@@ -486,7 +487,6 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     while (waves > 1 && waves / 2 >= slices) waves >>= 1;
     pl.waves = waves;
     pl.ks = (int)((slices + waves - 1) / waves);
-    if (nblocks > kTicketBytes / 4) pl.fast = false;
     return pl;
 }
 
@@ -579,14 +579,12 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
     const int64_t nblocks = (N + nb_cols - 1) / nb_cols;
     const int rows_max = (int)(M < pl.rows ? M : pl.rows);
     if (pl.ks > 1) {
-        const int64_t need = kTicketBytes + (int64_t)pl.ks * rows_max * N * 4;
+        const int64_t need = (int64_t)pl.ks * rows_max * N * 4;
         if (!workspace || workspace_bytes < need) return K3Q_ERR_WORKSPACE;
         if (!aligned_to(workspace, 16)) return K3Q_ERR_ALIGN;
-        p.tickets = (u32*)workspace;
-        p.part = (float*)((char*)workspace + kTicketBytes);
+        p.part = (float*)workspace;
     }
     p.klen = pl.klen;
-    p.two_pass = (plan_override && plan_override[4] >= 0) ? plan_override[4] : kDefaultTwoPass;
     for (int64_t m0 = 0; m0 < M; m0 += pl.rows) {
         const int rows = (int)((M - m0 < pl.rows) ? M - m0 : pl.rows);
         p.m0 = (int)m0;
@@ -596,8 +594,8 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         const size_t lds = (size_t)pl.waves * rows * nb_cols * sizeof(float);
         const int sets = (!f32 && rows > 8) ? 2 : (f32 ? 2 : 1);
         launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
-        if (pl.ks > 1 && (p.two_pass & 1)) {
-            dim3 rgrid((unsigned)((N + 255) / 256), rows);
+        if (pl.ks > 1) {
+            dim3 rgrid((unsigned)((N / 4 + 255) / 256), rows);
             if (f32) {
                 if (grouped)
                     gemv_w4_reduce<false, true><<<rgrid, 256, 0, s>>>(p, pl.ks);
@@ -621,7 +619,7 @@ using namespace k3q;
 
 extern "C" int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
-    // tickets + the largest partial buffer the built-in plans ask for (the plan depends on
+    // the largest partial buffer the built-in plans ask for (the plan depends on
     // the dtype and on whether the kernel is grouped; take the maximum over those)
     int64_t part = 0;
     const int64_t groupings[3] = {-1, 128, 32};
@@ -633,7 +631,7 @@ extern "C" int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N) 
             const int64_t b = (int64_t)pl.ks * rows * N * 4;
             if (b > part) part = b;
         }
-    return kTicketBytes + part;
+    return part;
 }
 
 extern "C" int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,

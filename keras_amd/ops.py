@@ -16,11 +16,10 @@ _workspaces = {}
 
 
 def _workspace(device, nbytes):
-    """Scratch for split-K partials and arrival tickets.
+    """Scratch for split-K partial sums and the per-call [N, K] weight copy.
 
     One buffer per (device, stream): calls on one stream are ordered, so they
-    can share it; calls on different streams may overlap and must not.  The
-    buffer starts zeroed and the kernels leave its ticket area zeroed.
+    can share it; calls on different streams may overlap and must not.
     """
     stream = torch.cuda.current_stream(device)
     key = (device.index, stream.cuda_stream)
@@ -73,7 +72,7 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
     nbytes = lib.k3q_gemv_w4_workspace_bytes(M, K, N)
     if plan is not None:
         # an overridden plan may split K into many more workgroups than the built-in one
-        nbytes = max(nbytes, 4096 + (K // 16 + 1) * min(M, 16) * N * 4)
+        nbytes = max(nbytes, (K // 16 + 1) * min(M, 16) * N * 4)
     ws = _workspace(x.device, nbytes)
     args = [
         _lib.ptr(x2), code, M, K, N, _lib.ptr(kp), _lib.ptr(ks), _lib.ptr(kz),
@@ -83,7 +82,7 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
     if plan is None:
         rc = lib.k3q_gemv_w4(*args, _lib.stream_ptr(x.device))
     else:
-        arr = (ctypes.c_int * 5)(*([int(v) for v in plan] + [-1] * (5 - len(plan))))
+        arr = (ctypes.c_int * 4)(*[int(v) for v in plan[:4]])
         rc = lib.k3q_gemv_w4_plan(*args, arr, _lib.stream_ptr(x.device))
     _lib.check(rc, "k3q_gemv_w4")
     return y.reshape(*lead, N)

@@ -55,7 +55,7 @@ def test_argument_validation_without_device():
     assert lib.k3q_gemv_w4(one, 0, 1, 0, 8, one, one, null, -1, null, one, null, 0, null) == -2
     assert lib.k3q_gemv_w4(one, 9, 1, 16, 8, one, one, null, -1, null, one, null, 0, null) == -4
     assert lib.k3q_gemv_w4(one, 0, 1, 16, 8, one, one, null, 128, null, one, null, 0, null) == -1  # zero missing
-    assert lib.k3q_gemv_w4_workspace_bytes(1, 8192, 8192) > 4096
+    assert lib.k3q_gemv_w4_workspace_bytes(1, 8192, 8192) >= 8192 * 4
     assert lib.k3q_gemm_i8_workspace_bytes(16, 256, 128) == 256 * 128
 
 
