@@ -27,10 +27,19 @@ if ROOT not in sys.path:
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8, published (5.0 POP/s)
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
 
-# HBM bytes per GEMM launch measured with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`
-# (see profiles/gemm_i8_mfma_M4096_K8192_N8192.md); None until measured.
-GEMM_HBM_TRAFFIC_BYTES = None
-GEMV_HBM_TRAFFIC_BYTES = None
+# Bytes crossing the L2 <-> memory boundary per launch, from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` (KiB per dispatch), each scaled by what the same counter reads for a plain
+# device copy of known size (FETCH_SIZE reads 0.50x, WRITE_SIZE 1.00x):
+# profiles/bench_dense_int8_M4096_K8192_N8192_and_int4_decode.md
+GEMM_HBM_TRAFFIC_BYTES = int((196835.4 * 2.0 + 83429.4) * 1024)
+QUANT_HBM_TRAFFIC_BYTES = int((32812.2 * 2.0 + 32832.0) * 1024)
+# int4 decode main kernel, keyed by (M > 8, grouped)
+GEMV_HBM_TRAFFIC_BYTES = {
+    (False, False): int((16600.1 * 2.0 + 640.0) * 1024),
+    (False, True): int((17411.1 * 2.0 + 640.0) * 1024),
+    (True, False): int((17472.0 * 2.0 + 4096.0) * 1024),
+    (True, True): int((34648.5 * 2.0 + 2048.0) * 1024),
+}
 
 
 def gemv_algorithmic_bytes(M, K, N, grouped, block=128):
@@ -165,7 +174,7 @@ def main():
                 "us_per_call": round(us, 2), "algorithmic_bytes": nbytes,
                 "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                              "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                             "traffic": GEMV_HBM_TRAFFIC_BYTES},
+                             "traffic": GEMV_HBM_TRAFFIC_BYTES[(Mg > 8, grouped)]},
             })
             del graph
         del xg
@@ -223,7 +232,7 @@ def main():
                       "roofline": {"bound": "hbm", "achieved": round(quant_bytes / (quant_ms * 1e-3) / 1e9, 1),
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(quant_bytes / (quant_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                   "traffic": None}},
+                                   "traffic": QUANT_HBM_TRAFFIC_BYTES}},
         "int4_gemv": gemv,
         "cpu_baseline": cpu,
     }

@@ -128,7 +128,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     const int g = lane >> 4;
     const int grp = (lane >> 3) & 1;
     const int mrow = lane & 7;
-    const int64_t nb = (int64_t)blockIdx.x * kNB;
+    // Workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous range of
+    // column blocks, so that blocks which share a 128-byte line of a packed row (kVec == 1)
+    // meet in one L2 instead of fetching the line twice.
+    const int per_xcd = gridDim.x / 8;
+    const int cb = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int64_t nb = (int64_t)cb * kNB;
+    if (nb >= p.N) return;  // grid.x is padded to a multiple of 8
     const int64_t kw0 = ((int64_t)blockIdx.y * nwaves + wave) * p.klen;
     const int nchunks = p.klen / kChunk;
     const int M = p.M;
@@ -589,7 +595,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         const int rows = (int)((M - m0 < pl.rows) ? M - m0 : pl.rows);
         p.m0 = (int)m0;
         p.M = rows;
-        dim3 grid((unsigned)nblocks, (unsigned)pl.ks);
+        dim3 grid((unsigned)((nblocks + 7) / 8 * 8), (unsigned)pl.ks);
         const int threads = pl.waves * 64;
         const size_t lds = (size_t)pl.waves * rows * nb_cols * sizeof(float);
         const int sets = (!f32 && rows > 8) ? 2 : (f32 ? 2 : 1);
