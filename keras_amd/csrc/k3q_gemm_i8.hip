@@ -18,6 +18,7 @@
 // the activation tile the second (column) operand, so a lane ends up with ONE
 // output row m and groups of four consecutive n: stores are 8 or 16 bytes wide.
 #include "k3q_common.h"
+#include "k3q_gemm_i8_skinny.h"
 
 namespace k3q {
 namespace {
@@ -27,9 +28,13 @@ constexpr int kBN = 256;  // tile rows of the prepacked weight = columns of y
 constexpr int kBK = 128;  // bytes of K per stage: one full 128-byte line per row
 constexpr int kStages = 2;
 constexpr int kKSteps = kBK / 32;  // MFMA K steps per stage
-constexpr int kThreads = 512;
-constexpr int kWavesN = 4;  // waves along N
-constexpr int kWavesM = 2;  // waves along M
+#ifndef K3Q_GEMM_WAVES_N
+#define K3Q_GEMM_WAVES_N 4
+#define K3Q_GEMM_WAVES_M 2
+#endif
+constexpr int kWavesN = K3Q_GEMM_WAVES_N;  // waves along N
+constexpr int kWavesM = K3Q_GEMM_WAVES_M;  // waves along M
+constexpr int kThreads = 64 * kWavesN * kWavesM;
 constexpr int kWN = kBN / kWavesN;  // 64 columns per wave
 constexpr int kWM = kBM / kWavesM;  // 128 rows per wave
 constexpr int kNBlk = kWN / 32;     // 2 MFMA blocks along N per wave
@@ -66,7 +71,9 @@ __device__ __forceinline__ int swz(int row) {
 
 // gfx9 s_waitcnt encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]
 __device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-__device__ __forceinline__ void wait_vmcnt_one_stage() { __builtin_amdgcn_s_waitcnt(0x0F70 | kDmaPerWave); }
+__device__ __forceinline__ void wait_vmcnt_one_stage() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kDmaPerWave & 0xF) | ((kDmaPerWave >> 4) << 14));
+}
 __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 __device__ __forceinline__ void bare_barrier() {
     // s_barrier without a fence: a fence would also drain the DMA of the stage in flight
@@ -198,9 +205,11 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
             __builtin_amdgcn_sched_barrier(0);
 #ifndef K3Q_GEMM_PROBE_NO_MMA
 #pragma unroll
-            for (int mb = 0; mb < kMBlk; ++mb)
-                acc[0][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][0], af[ks & 1][mb],
-                                                                   acc[0][mb], 0, 0, 0);
+            for (int nb = 0; nb < kNBlk / 2; ++nb)
+#pragma unroll
+                for (int mb = 0; mb < kMBlk; ++mb)
+                    acc[nb][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][nb], af[ks & 1][mb],
+                                                                        acc[nb][mb], 0, 0, 0);
 #endif
             __builtin_amdgcn_sched_barrier(0);
             if (ks + 1 < kKSteps) {
@@ -216,7 +225,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
             __builtin_amdgcn_sched_barrier(0);
 #ifndef K3Q_GEMM_PROBE_NO_MMA
 #pragma unroll
-            for (int nb = 1; nb < kNBlk; ++nb)
+            for (int nb = kNBlk / 2; nb < kNBlk; ++nb)
 #pragma unroll
                 for (int mb = 0; mb < kMBlk; ++mb)
                     acc[nb][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][nb], af[ks & 1][mb],
@@ -240,8 +249,8 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
 #endif
     // ---- epilogue ----
     // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
-    // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: per lane 4 rows of y and 8 groups
-    // of four consecutive columns.  All scale / bias loads are issued before any is used.
+    // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: a lane owns one row of y per mb
+    // and groups of four consecutive columns.
     if (p.flags & kFlagSkipEpilogue) {  // timing aid: main loop only
         int sink = 0;
 #pragma unroll
@@ -253,81 +262,44 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
         if (sink == 0x7fffffff && p.y) ((char*)p.y)[0] = 1;
         return;
     }
-    int64_t mrow[kMBlk];
-    float sa[kMBlk], ra[kMBlk];
-#pragma unroll
-    for (int mb = 0; mb < kMBlk; ++mb) {
-        mrow[mb] = m0 + wm * kWM + mb * 32 + fi;
-        const int64_t mc = mrow[mb] < p.M ? mrow[mb] : p.M - 1;
-        sa[mb] = p.a_scale ? load_t<kBF16>(p.a_scale, mc) : 1.0f;
+    // Stage the tile's scales and bias in LDS as floats (the main loop is done with it): the
+    // per-lane reads below are then cheap and need no large register arrays.
+    float* ep = (float*)lds;  // [0,256) b_scale or its reciprocal, [256,512) bias, [512,768) a_scale or reciprocal
+    __syncthreads();
+    for (int t = tid; t < kBN; t += kThreads) {
+        const int64_t n = n0 + t < p.N ? n0 + t : p.N - 1;
+        const float sbv = p.b_scale ? load_t<kBF16>(p.b_scale, n) : 1.0f;
+        ep[t] = kExact ? sbv : 1.0f / sbv;
+        ep[kBN + t] = p.bias ? load_t<kBF16>(p.bias, n) : 0.0f;
     }
-    float sb[kNBlk][4][4], bv[kNBlk][4][4];
-#pragma unroll
-    for (int nb = 0; nb < kNBlk; ++nb)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-            int64_t n = n0 + wn * kWN + nb * 32 + 8 * rg + 4 * fg;
-            n = n < p.N ? n : p.N - 4;  // N % 4 == 0 on this path
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                sb[nb][rg][e] = 1.0f;
-                bv[nb][rg][e] = 0.0f;
-            }
-            if (kBF16) {
-                if (p.b_scale) {
-                    const v2u t = *(const v2u*)((const uint16_t*)p.b_scale + n);
-                    sb[nb][rg][0] = __uint_as_float(t[0] << 16);
-                    sb[nb][rg][1] = __uint_as_float(t[0] & 0xffff0000u);
-                    sb[nb][rg][2] = __uint_as_float(t[1] << 16);
-                    sb[nb][rg][3] = __uint_as_float(t[1] & 0xffff0000u);
-                }
-                if (p.bias) {
-                    const v2u t = *(const v2u*)((const uint16_t*)p.bias + n);
-                    bv[nb][rg][0] = __uint_as_float(t[0] << 16);
-                    bv[nb][rg][1] = __uint_as_float(t[0] & 0xffff0000u);
-                    bv[nb][rg][2] = __uint_as_float(t[1] << 16);
-                    bv[nb][rg][3] = __uint_as_float(t[1] & 0xffff0000u);
-                }
-            } else {
-                if (p.b_scale) {
-                    const v4f t = *(const v4f*)((const float*)p.b_scale + n);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) sb[nb][rg][e] = t[e];
-                }
-                if (p.bias) {
-                    const v4f t = *(const v4f*)((const float*)p.bias + n);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) bv[nb][rg][e] = t[e];
-                }
-            }
-        }
-    if (!kExact) {
-#pragma unroll
-        for (int mb = 0; mb < kMBlk; ++mb) ra[mb] = 1.0f / sa[mb];
-#pragma unroll
-        for (int nb = 0; nb < kNBlk; ++nb)
-#pragma unroll
-            for (int rg = 0; rg < 4; ++rg)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) sb[nb][rg][e] = 1.0f / sb[nb][rg][e];
+    for (int t = tid; t < kBM; t += kThreads) {
+        const int64_t m = m0 + t < p.M ? m0 + t : p.M - 1;
+        const float sav = p.a_scale ? load_t<kBF16>(p.a_scale, m) : 1.0f;
+        ep[2 * kBN + t] = kExact ? sav : 1.0f / sav;
     }
+    __syncthreads();
     const bool has_bias = p.bias != nullptr;
 #pragma unroll
-    for (int mb = 0; mb < kMBlk; ++mb) {
-        const int64_t m = mrow[mb];
-        if (m >= p.M) continue;
+    for (int nb = 0; nb < kNBlk; ++nb) {
 #pragma unroll
-        for (int nb = 0; nb < kNBlk; ++nb) {
+        for (int rg = 0; rg < 4; ++rg) {
+            const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+            const int64_t n = n0 + nl;
+            if (n >= p.N) continue;  // N % 4 == 0 on this path: all four columns in or out
+            const v4f sb = *(const v4f*)(ep + nl);
+            const v4f bv = *(const v4f*)(ep + kBN + nl);
 #pragma unroll
-            for (int rg = 0; rg < 4; ++rg) {
-                const int64_t n = n0 + wn * kWN + nb * 32 + 8 * rg + 4 * fg;
-                if (n >= p.N) continue;  // all four columns in or out
+            for (int mb = 0; mb < kMBlk; ++mb) {
+                const int ml = wm * kWM + mb * 32 + fi;
+                const int64_t m = m0 + ml;
+                if (m >= p.M) continue;
                 if (p.acc_out) {
                     v4i o = {acc[nb][mb][4 * rg], acc[nb][mb][4 * rg + 1], acc[nb][mb][4 * rg + 2],
                              acc[nb][mb][4 * rg + 3]};
                     *(v4i*)(p.acc_out + m * p.N + n) = o;
                 }
                 if (!p.y) continue;
+                const float sa = ep[2 * kBN + ml];
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -336,15 +308,15 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
                     if (kExact) {
                         // the reference's op sequence, every step rounded to T
                         if (kBF16) {
-                            const float os = round_bf16(sb[nb][rg][e] * sa[mb]);
+                            const float os = round_bf16(sb[e] * sa);
                             r = round_bf16(round_bf16(accf) / os);
-                            if (has_bias) r = round_bf16(r + bv[nb][rg][e]);
+                            if (has_bias) r = round_bf16(r + bv[e]);
                         } else {
-                            r = accf / (sb[nb][rg][e] * sa[mb]);
-                            if (has_bias) r = r + bv[nb][rg][e];
+                            r = accf / (sb[e] * sa);
+                            if (has_bias) r = r + bv[e];
                         }
                     } else {
-                        r = (accf * ra[mb]) * sb[nb][rg][e] + bv[nb][rg][e];
+                        r = (accf * sa) * sb[e] + bv[e];  // sa, sb hold reciprocals here
                     }
                     v[e] = r;
                 }
@@ -432,9 +404,12 @@ int launch_mfma(const GemmParams& p, hipStream_t s) {
 using namespace k3q;
 
 extern "C" int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    (void)M;
     if (N <= 0 || K <= 0) return 0;
-    return N * K;  // room for the [N,K] copy when the weight is passed in its [K,N] layout
+    // decode-sized M with the [K,N] kernel: int32 split-K partials; larger M with the [K,N]
+    // kernel: room for the [N,K] copy made per call
+    if (M > 0 && M <= kSkinnyMaxRows && (N % 16) == 0 && (K % 8) == 0)
+        return gemm_i8_skinny_workspace_bytes(M, N, K);
+    return N * K;
 }
 
 extern "C" int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N, int8_t* prepacked,
@@ -473,6 +448,10 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     p.tiles_n = (int)((N + kBN - 1) / kBN);
 
     const size_t el = bf16 ? 2 : 4;
+    // decode-sized M: bandwidth-bound kernel that reads the [K,N] kernel in place
+    if (b_layout == 0 && gemm_i8_skinny_supported(M, N, K, a, b))
+        return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, y, acc_out, workspace,
+                                  workspace_bytes, s);
     bool fast = (K % kBK) == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
                 (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
                 (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&

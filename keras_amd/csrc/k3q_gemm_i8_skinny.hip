@@ -1,0 +1,331 @@
+// int8 x int8 -> int32 matmul for decode-sized M (<= 64 rows), with the Dense de-scale.
+//
+// HBM-bound on the weights, so the int8 kernel is read ONCE, in the [K, N] layout the layer
+// stores (no shadow copy), with 16-byte loads that are contiguous along N.  As in the int4
+// kernel, the matrix core is fed operands whose "K slots" mix k and n:
+//   v_mfma_i32_32x32x32_i8 gives each lane (i = lane%32, g = lane/32) 16 byte-slots of row i.
+//   The lane loads 16 bytes (columns n0+16i .. +15) of four consecutive k rows.  MFMA c
+//   (c = 0..3) takes dword c of each of the four loads: slot (t, b) of row i is
+//   W[k0 + 4g + t][n0 + 16i + 4c + b], i.e. four k values of four different columns.
+//   The activation operand has 32 columns = 4 column groups x 8 rows of x; column (bb, m)
+//   carries xq[m][k0 + 4g + t] in slot (t, bb) and zero elsewhere, so D[i][(bb, m)] is the
+//   exact int32 partial dot product of x row m with column n0 + 16i + 4c + bb.
+// Three quarters of the MFMA multiplies zeros; at <= 64 rows the matrix core has an order of
+// magnitude of headroom over HBM.
+//
+// Split-K: as in the int4 kernel (waves of a workgroup through LDS, workgroups through int32
+// partials and a second kernel).  Integer partial sums make the result exact whatever the
+// split.
+#include "k3q_common.h"
+#include "k3q_gemm_i8_skinny.h"
+
+namespace k3q {
+namespace {
+
+constexpr int kNB = 512;        // columns per workgroup: 32 lanes x 16 bytes
+constexpr int kStepK = 8;       // k rows per MFMA step: 2 lane groups x 4 rows
+constexpr int kMaxWaves = 8;
+constexpr int kRowStride = kNB + 4;  // ints per x row in the LDS slab: the pad spreads rows over banks
+
+struct SkinnyParams {
+    const int8_t* xq;      // [M, K]
+    const int8_t* w;       // [K, N]
+    const void* a_scale;   // T [M] or null
+    const void* b_scale;   // T [N] or null
+    const void* bias;      // T [N] or null
+    void* y;               // T [M, N] or null
+    int32_t* acc_out;      // [M, N] or null
+    int32_t* part;         // [KS, M, N]
+    int64_t K, N;
+    int M;                 // rows in this launch
+    int m0;                // first row of this launch
+    int klen;              // rows of K per wave
+    int exact;
+};
+
+template <bool kBF16>
+__device__ __forceinline__ float load_t(const void* p, int64_t i) {
+    if (kBF16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+    return ((const float*)p)[i];
+}
+
+template <bool kBF16>
+__device__ __forceinline__ void finish(const SkinnyParams& p, int m, int64_t n, int acc) {
+    const int64_t row = p.m0 + m;
+    if (p.acc_out) p.acc_out[row * p.N + n] = acc;
+    if (!p.y) return;
+    const float sa = p.a_scale ? load_t<kBF16>(p.a_scale, row) : 1.0f;
+    const float sb = p.b_scale ? load_t<kBF16>(p.b_scale, n) : 1.0f;
+    float r;
+    if (kBF16) {
+        // decode-sized outputs always take the reference's rounding chain
+        r = round_bf16(round_bf16((float)acc) / round_bf16(sb * sa));
+        if (p.bias) r = round_bf16(r + load_t<true>(p.bias, n));
+        ((uint16_t*)p.y)[row * p.N + n] = (uint16_t)f32_to_bf16_bits(r);
+    } else {
+        r = (float)acc / (sb * sa);
+        if (p.bias) r = r + load_t<false>(p.bias, n);
+        ((float*)p.y)[row * p.N + n] = r;
+    }
+}
+
+// kSteps: 8-row steps per chunk.  kSets: 8-row groups of x handled per pass (1 or 2).
+template <int kSteps, int kSets>
+__global__ __launch_bounds__(kMaxWaves * 64) void gemm_i8_skinny(SkinnyParams p) {
+    extern __shared__ int red[];  // [M][kRowStride], all waves add into it
+    constexpr int kChunk = kSteps * kStepK;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int i = lane & 31;        // weight lane: columns 16i..16i+15; x lane: column (bb, m)
+    const int g = lane >> 5;
+    const int bb = (lane >> 3) & 3;  // column group of this lane's x operand
+    const int mrow = lane & 7;
+    const int per_xcd = gridDim.x / 8;
+    const int cb = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int64_t nb = (int64_t)cb * kNB;
+    if (nb >= p.N) return;  // grid.x is padded to a multiple of 8
+    const int64_t kw0 = ((int64_t)blockIdx.y * nwaves + wave) * p.klen;
+    const int nchunks = p.klen / kChunk;
+    const int M = p.M;
+
+    int64_t ncol = nb + 16 * i;
+    if (ncol >= p.N) ncol = p.N - 16;  // N % 16 == 0; results of these lanes are never stored
+    u32 loff[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) loff[t] = (u32)((4 * g + t) * p.N + ncol);
+    u32 xoff[kSets], xmask[kSets];
+#pragma unroll
+    for (int st = 0; st < kSets; ++st) {
+        const int m = mrow + 8 * st;
+        xmask[st] = m < M ? 0xffffffffu : 0u;
+        xoff[st] = (u32)((m < M ? m : M - 1) * p.K + 4 * g);
+    }
+    const int8_t* xbase = p.xq + (int64_t)p.m0 * p.K;
+
+    v4u wreg[2][kSteps][4];
+    u32 xraw[2][kSteps][kSets];
+    auto load_chunk = [&](int b, int c) {
+        const int64_t kc = kw0 + (int64_t)c * kChunk;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const int64_t ks = kc + kStepK * s;
+            const int64_t kk = ks < p.K ? ks : p.K - kStepK;  // K % 8 == 0
+            const int8_t* rb = p.w + kk * p.N;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) wreg[b][s][t] = __builtin_nontemporal_load((const v4u*)(rb + loff[t]));
+#pragma unroll
+            for (int st = 0; st < kSets; ++st) xraw[b][s][st] = *(const u32*)(xbase + kk + xoff[st]);
+        }
+    };
+
+    v16i acc[kSets][4];
+#pragma unroll
+    for (int st = 0; st < kSets; ++st)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[st][c][r] = 0;
+
+    auto compute_chunk = [&](int b, int c) {
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const bool kvalid = kw0 + (int64_t)c * kChunk + kStepK * s < p.K;
+            v4i xb[kSets];
+#pragma unroll
+            for (int st = 0; st < kSets; ++st) {
+                const u32 d = xraw[b][s][st] & (kvalid ? xmask[st] : 0u);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) xb[st][t] = (int)(((d >> (8 * t)) & 0xffu) << (8 * bb));
+            }
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                const v4i av = {(int)wreg[b][s][0][cc], (int)wreg[b][s][1][cc], (int)wreg[b][s][2][cc],
+                                (int)wreg[b][s][3][cc]};
+#pragma unroll
+                for (int st = 0; st < kSets; ++st)
+                    acc[st][cc] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, xb[st], acc[st][cc], 0, 0, 0);
+            }
+        }
+    };
+
+    load_chunk(0, 0);
+    // the waves of the workgroup meet in one int32 slab through LDS atomic adds: integer sums
+    // do not depend on the order, so this stays deterministic
+    // (bare barrier after an LDS-only wait: a full __syncthreads would also wait for the
+    // loads just issued)
+    for (int idx = threadIdx.x; idx < M * kRowStride; idx += blockDim.x) red[idx] = 0;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll 1
+    for (int c = 0; c < nchunks; c += 2) {
+        if (c + 1 < nchunks) load_chunk(1, c + 1);
+        compute_chunk(0, c);
+        if (c + 2 < nchunks) load_chunk(0, c + 2);
+        if (c + 1 < nchunks) compute_chunk(1, c + 1);
+    }
+
+    // lane (j = lane%32, gq = lane/32) holds D[row 8*(r/4) + 4*gq + r%4][col j]:
+    //   column n_local = 16*row + 4*c + j/8,  x row m = j%8 + 8*set
+#pragma unroll
+    for (int st = 0; st < kSets; ++st) {
+        const int m = mrow + 8 * st;
+        if (m < M) {
+            int* dst = red + m * kRowStride;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = 8 * (r >> 2) + 4 * g + (r & 3);
+                    __hip_atomic_fetch_add(dst + 16 * row + 4 * c + bb, acc[st][c][r], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+        }
+    }
+    __syncthreads();
+
+    const int KS = gridDim.y;
+    for (int idx = threadIdx.x; idx < M * (kNB / 4); idx += blockDim.x) {
+        const int m = idx / (kNB / 4);
+        const int nl = (idx % (kNB / 4)) * 4;
+        const v4i sum = *(const v4i*)(red + m * kRowStride + nl);
+        const int64_t n = nb + nl;
+        if (n < p.N) {  // N % 16 == 0: all four columns in or out
+            if (KS == 1) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (p.exact & 2)
+                        finish<true>(p, m, n + e, sum[e]);
+                    else
+                        finish<false>(p, m, n + e, sum[e]);
+                }
+            } else {
+                *(v4i*)(p.part + ((int64_t)blockIdx.y * M + m) * p.N + n) = sum;
+            }
+        }
+    }
+}
+
+template <bool kBF16>
+__global__ __launch_bounds__(256) void gemm_i8_skinny_reduce(SkinnyParams p, int KS) {
+    const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const int m = blockIdx.y;
+    if (n >= p.N) return;
+    v4i s4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) s4[u] = v4i{0, 0, 0, 0};
+    const int32_t* src = p.part + (int64_t)m * p.N + n;
+    const int64_t stride = (int64_t)p.M * p.N;
+    int ks = 0;
+    for (; ks + 4 <= KS; ks += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s4[u] += *(const v4i*)(src + (ks + u) * stride);
+    }
+    for (; ks < KS; ++ks) s4[0] += *(const v4i*)(src + ks * stride);
+    const v4i sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) finish<kBF16>(p, m, n + e, sum[e]);
+}
+
+struct Plan {
+    int steps, sets, rows, waves, klen, ks;
+};
+
+Plan make_plan(int64_t M, int64_t K, int64_t N) {
+    Plan pl{};
+    pl.sets = M > 8 ? 2 : 1;
+    pl.rows = 8 * pl.sets;
+    const int rows_used = (int)(M < pl.rows ? M : pl.rows);
+    int steps = pl.sets == 2 ? 2 : 4;
+    while (steps > 1 && (K % (steps * kStepK)) != 0) steps >>= 1;
+    pl.steps = steps;
+    const int chunk = steps * kStepK;
+    const int64_t nblocks = (N + kNB - 1) / kNB;
+    int waves = kMaxWaves;
+    (void)rows_used;
+    int64_t klen = K * nblocks / (256 * (int64_t)waves);  // about one workgroup per CU
+    klen = klen / chunk * chunk;
+    if (klen < chunk) klen = chunk;
+    if (klen > K) klen = (K + chunk - 1) / chunk * chunk;
+    pl.klen = (int)klen;
+    const int64_t slices = (K + klen - 1) / klen;
+    while (waves > 1 && waves / 2 >= slices) waves >>= 1;
+    pl.waves = waves;
+    pl.ks = (int)((slices + waves - 1) / waves);
+    return pl;
+}
+
+template <int kSets>
+void launch_steps(int steps, const SkinnyParams& p, dim3 grid, int threads, size_t lds, hipStream_t s) {
+    switch (steps) {
+        case 4: gemm_i8_skinny<4, kSets><<<grid, threads, lds, s>>>(p); break;
+        case 2: gemm_i8_skinny<2, kSets><<<grid, threads, lds, s>>>(p); break;
+        default: gemm_i8_skinny<1, kSets><<<grid, threads, lds, s>>>(p); break;
+    }
+}
+
+}  // namespace
+
+bool gemm_i8_skinny_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* b) {
+    return M > 0 && M <= kSkinnyMaxRows && (N % 16) == 0 && (K % kStepK) == 0 && aligned_to(a, 4) &&
+           aligned_to(b, 16);
+}
+
+int64_t gemm_i8_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || M > kSkinnyMaxRows) return 0;
+    const Plan pl = make_plan(M, K, N);
+    if (pl.ks <= 1) return 0;
+    const int64_t rows = M < pl.rows ? M : pl.rows;
+    return (int64_t)pl.ks * rows * N * 4;
+}
+
+int gemm_i8_skinny_run(const int8_t* a, const int8_t* b, int64_t M, int64_t N, int64_t K,
+                       const void* a_scale, const void* b_scale, const void* bias, bool bf16,
+                       void* y, int32_t* acc_out, void* workspace, int64_t workspace_bytes,
+                       hipStream_t s) {
+    SkinnyParams p{};
+    p.xq = a;
+    p.w = b;
+    p.a_scale = a_scale;
+    p.b_scale = b_scale;
+    p.bias = bias;
+    p.y = y;
+    p.acc_out = acc_out;
+    p.K = K;
+    p.N = N;
+    p.exact = bf16 ? 2 : 0;
+    const Plan pl = make_plan(M, K, N);
+    const int64_t nblocks = (N + kNB - 1) / kNB;
+    const int rows_max = (int)(M < pl.rows ? M : pl.rows);
+    if (pl.ks > 1) {
+        const int64_t need = (int64_t)pl.ks * rows_max * N * 4;
+        if (!workspace || workspace_bytes < need) return K3Q_ERR_WORKSPACE;
+        if (!aligned_to(workspace, 16)) return K3Q_ERR_ALIGN;
+        p.part = (int32_t*)workspace;
+    }
+    p.klen = pl.klen;
+    for (int64_t m0 = 0; m0 < M; m0 += pl.rows) {
+        const int rows = (int)((M - m0 < pl.rows) ? M - m0 : pl.rows);
+        p.m0 = (int)m0;
+        p.M = rows;
+        dim3 grid((unsigned)((nblocks + 7) / 8 * 8), (unsigned)pl.ks);
+        const int threads = pl.waves * 64;
+        const size_t lds = (size_t)rows * kRowStride * sizeof(int);
+        if (rows > 8)
+            launch_steps<2>(pl.steps, p, grid, threads, lds, s);
+        else
+            launch_steps<1>(pl.steps, p, grid, threads, lds, s);
+        if (pl.ks > 1) {
+            dim3 rgrid((unsigned)((N / 4 + 255) / 256), rows);
+            if (bf16)
+                gemm_i8_skinny_reduce<true><<<rgrid, 256, 0, s>>>(p, pl.ks);
+            else
+                gemm_i8_skinny_reduce<false><<<rgrid, 256, 0, s>>>(p, pl.ks);
+        }
+    }
+    return launch_status();
+}
+
+}  // namespace k3q

@@ -89,6 +89,8 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
 
 
 GEMM_EXACT_EPILOGUE = 1
+# up to this many rows the int8 matmul is bandwidth-bound and reads the [K, N] kernel in place
+SKINNY_MAX_ROWS = 64
 
 
 def prepack_int8_kernel(kernel):
@@ -136,7 +138,8 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
     y = torch.empty((M, N), dtype=out_dtype, device=a.device) if want_y else None
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
     lib = _lib.load()
-    if prepacked is not None:
+    skinny = M <= SKINNY_MAX_ROWS and N % 16 == 0 and K % 8 == 0
+    if prepacked is not None and not skinny:
         b, layout, ws, ws_bytes = prepacked, 1, None, 0
     else:
         b = kernel if kernel.is_contiguous() else kernel.contiguous()

@@ -107,3 +107,17 @@ def test_prepack_is_transpose(dev):
     for K, N in [(128, 64), (100, 37), (4096, 4096), (65, 129)]:
         b = torch.randint(-128, 128, (K, N), generator=g, dtype=torch.int8)
         assert torch.equal(kops.prepack_int8_kernel(b.to(dev)).cpu(), b.t().contiguous())
+
+
+DECODE_SHAPES = [(1, 4096, 4096), (8, 4096, 4096), (16, 4096, 4096), (3, 64, 48), (17, 512, 1040),
+                 (33, 256, 512), (64, 1024, 2048), (5, 8, 16), (12, 14336, 4096), (2, 4096, 14336)]
+
+
+@pytest.mark.parametrize("M,K,N", DECODE_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_int8_decode_sizes(dev, M, K, N, dtype):
+    # M <= 64 without a prepacked kernel: the bandwidth-bound kernel that reads [K, N] in place
+    y = run_dense_int8(dev, M, K, N, dtype, prepack=False, exact=True, seed=M + K)
+    # and the layer-level route (prepacked given, still routed by M) agrees bit for bit
+    y2 = run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True, seed=M + K)
+    assert torch.equal(y, y2)
