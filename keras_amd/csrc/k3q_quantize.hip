@@ -71,15 +71,17 @@ __device__ __forceinline__ float row_max(float v, float* lds) {
     return r;
 }
 
-// Fast path.  cols % kPerChunk == 0, rows 16-byte aligned.  kTpr threads per row,
-// 256 / kTpr rows per block, each thread keeps up to kChunks 16-byte chunks.
-template <int kDtype, int kTpr, int kChunks>
+// Fast path.  cols % 16 == 0, rows 16-byte aligned.  A thread owns groups of 16 consecutive
+// elements (32 or 64 bytes of input, one 16-byte store of output); kTpr threads share a row
+// (a wave, or the whole 256-thread block), each keeps up to kGroups groups in registers.
+template <int kDtype, int kTpr, int kGroups>
 __global__ __launch_bounds__(256) void quantize_rows_vec(const char* __restrict__ x, int64_t rows,
-                                                         int64_t chunks_per_row,
+                                                         int64_t groups_per_row,
                                                          int64_t x_row_bytes, float eps, float qlo,
                                                          float qhi, int8_t* __restrict__ q,
                                                          void* __restrict__ scale) {
     constexpr int kPer = Elem<kDtype>::kPerChunk;
+    constexpr int kCpg = 16 / kPer;  // 16-byte chunks per group
     constexpr int kRowsPerBlock = 256 / kTpr;
     __shared__ float lds[256 / kWave];
     const int lane = threadIdx.x % kTpr;
@@ -87,17 +89,27 @@ __global__ __launch_bounds__(256) void quantize_rows_vec(const char* __restrict_
     const bool live = row < rows;
     const v4u* xr = (const v4u*)(x + (live ? row : 0) * x_row_bytes);
 
-    v4u c[kChunks];
+    v4u c[kGroups][kCpg];
     float amax = 0.0f;
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-        int64_t ci = lane + (int64_t)i * kTpr;
-        if (live && ci < chunks_per_row) {
-            c[i] = __builtin_nontemporal_load(xr + ci);
-            float f[kPer];
-            chunk_to_floats<kDtype>(c[i], f);
+    for (int i = 0; i < kGroups; ++i) {
+        const int64_t gi = lane + (int64_t)i * kTpr;
+        if (live && gi < groups_per_row) {
 #pragma unroll
-            for (int e = 0; e < kPer; ++e) amax = fmaxf(amax, fabsf(f[e]));
+            for (int j = 0; j < kCpg; ++j) c[i][j] = __builtin_nontemporal_load(xr + gi * kCpg + j);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kGroups; ++i) {
+        const int64_t gi = lane + (int64_t)i * kTpr;
+        if (live && gi < groups_per_row) {
+#pragma unroll
+            for (int j = 0; j < kCpg; ++j) {
+                float f[kPer];
+                chunk_to_floats<kDtype>(c[i][j], f);
+#pragma unroll
+                for (int e = 0; e < kPer; ++e) amax = fmaxf(amax, fabsf(f[e]));
+            }
         }
     }
     amax = row_max<kTpr>(amax, lds);
@@ -109,28 +121,26 @@ __global__ __launch_bounds__(256) void quantize_rows_vec(const char* __restrict_
         else
             ((uint16_t*)scale)[row] = (uint16_t)(__float_as_uint(s) >> 16);
     }
-    int8_t* qr = q + row * chunks_per_row * kPer;
+    v4u* qr = (v4u*)(q + row * groups_per_row * 16);
 #pragma unroll
-    for (int i = 0; i < kChunks; ++i) {
-        int64_t ci = lane + (int64_t)i * kTpr;
-        if (ci < chunks_per_row) {
-            float f[kPer];
-            chunk_to_floats<kDtype>(c[i], f);
-            u32 w[kPer / 4];
+    for (int i = 0; i < kGroups; ++i) {
+        const int64_t gi = lane + (int64_t)i * kTpr;
+        if (gi < groups_per_row) {
+            v4u o;
 #pragma unroll
-            for (int d = 0; d < kPer / 4; ++d) {
-                u32 b0 = (u32)quantize_one<kDtype>(f[4 * d + 0], s, qlo, qhi) & 0xffu;
-                u32 b1 = (u32)quantize_one<kDtype>(f[4 * d + 1], s, qlo, qhi) & 0xffu;
-                u32 b2 = (u32)quantize_one<kDtype>(f[4 * d + 2], s, qlo, qhi) & 0xffu;
-                u32 b3 = (u32)quantize_one<kDtype>(f[4 * d + 3], s, qlo, qhi) & 0xffu;
-                w[d] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            for (int j = 0; j < kCpg; ++j) {
+                float f[kPer];
+                chunk_to_floats<kDtype>(c[i][j], f);
+#pragma unroll
+                for (int d = 0; d < kPer / 4; ++d) {
+                    u32 b0 = (u32)quantize_one<kDtype>(f[4 * d + 0], s, qlo, qhi) & 0xffu;
+                    u32 b1 = (u32)quantize_one<kDtype>(f[4 * d + 1], s, qlo, qhi) & 0xffu;
+                    u32 b2 = (u32)quantize_one<kDtype>(f[4 * d + 2], s, qlo, qhi) & 0xffu;
+                    u32 b3 = (u32)quantize_one<kDtype>(f[4 * d + 3], s, qlo, qhi) & 0xffu;
+                    o[j * (kPer / 4) + d] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+                }
             }
-            if (kPer == 4) {
-                __builtin_nontemporal_store(w[0], (u32*)(qr + ci * 4));
-            } else {
-                v2u o = {w[0], w[1]};
-                __builtin_nontemporal_store(o, (v2u*)(qr + ci * 8));
-            }
+            __builtin_nontemporal_store(o, qr + gi);
         }
     }
 }
@@ -163,40 +173,44 @@ __global__ __launch_bounds__(256) void quantize_rows_generic(const char* __restr
         q[row * cols + c] = (int8_t)quantize_one<kDtype>(load(c), s, qlo, qhi);
 }
 
-template <int kDtype, int kTpr, int kChunks>
-void launch_vec(const void* x, int64_t rows, int64_t chunks_per_row, int64_t row_bytes, float eps,
+template <int kDtype, int kTpr, int kGroups>
+void launch_vec(const void* x, int64_t rows, int64_t groups_per_row, int64_t row_bytes, float eps,
                 float qlo, float qhi, int8_t* q, void* scale, hipStream_t s) {
     constexpr int kRowsPerBlock = 256 / kTpr;
     unsigned blocks = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
-    quantize_rows_vec<kDtype, kTpr, kChunks><<<blocks, 256, 0, s>>>(
-        (const char*)x, rows, chunks_per_row, row_bytes, eps, qlo, qhi, q, scale);
+    quantize_rows_vec<kDtype, kTpr, kGroups><<<blocks, 256, 0, s>>>(
+        (const char*)x, rows, groups_per_row, row_bytes, eps, qlo, qhi, q, scale);
 }
+
+#ifndef K3Q_QUANT_WAVE_ROW_MIN
+#define K3Q_QUANT_WAVE_ROW_MIN 1024
+#endif
+constexpr int64_t kWaveRowMin = K3Q_QUANT_WAVE_ROW_MIN;
 
 template <int kDtype>
 int dispatch(const void* x, int64_t rows, int64_t cols, int64_t stride, float eps, float qlo,
              float qhi, int8_t* q, void* scale, hipStream_t s) {
-    constexpr int kPer = Elem<kDtype>::kPerChunk;
     constexpr int kBytes = Elem<kDtype>::kBytes;
-    const bool vec_ok = (cols % kPer) == 0 && ((stride * kBytes) % 16) == 0 && aligned_to(x, 16) &&
-                        aligned_to(q, 8);
-    const int64_t cpr = cols / kPer;
-    const int64_t rb = stride * kBytes;
-    if (vec_ok && cpr <= 64 * 4) {
-        if (cpr <= 64)
-            launch_vec<kDtype, 64, 1>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
-        else if (cpr <= 128)
-            launch_vec<kDtype, 64, 2>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+    const bool vec_ok = (cols % 16) == 0 && ((stride * kBytes) % 16) == 0 && aligned_to(x, 16) &&
+                        aligned_to(q, 16);
+    const int64_t gpr = cols / 16;  // 16-element groups per row
+    // A wave per row (no LDS, no barrier) for short rows, where a 256-thread block would idle
+    // most of its lanes; longer rows do better spread over a block (fewer registers per
+    // thread, more rows in flight per CU).
+    if (vec_ok && (gpr <= 64 || (gpr <= 128 && rows >= kWaveRowMin))) {
+        if (gpr <= 64)
+            launch_vec<kDtype, 64, 1>(x, rows, gpr, stride * kBytes, eps, qlo, qhi, q, scale, s);
         else
-            launch_vec<kDtype, 64, 4>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
-    } else if (vec_ok && cpr <= 256 * 16) {
-        if (cpr <= 256 * 2)
-            launch_vec<kDtype, 256, 2>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
-        else if (cpr <= 256 * 4)
-            launch_vec<kDtype, 256, 4>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
-        else if (cpr <= 256 * 8)
-            launch_vec<kDtype, 256, 8>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+            launch_vec<kDtype, 64, 2>(x, rows, gpr, stride * kBytes, eps, qlo, qhi, q, scale, s);
+    } else if (vec_ok && gpr <= 256 * 8) {
+        if (gpr <= 256)
+            launch_vec<kDtype, 256, 1>(x, rows, gpr, stride * kBytes, eps, qlo, qhi, q, scale, s);
+        else if (gpr <= 512)
+            launch_vec<kDtype, 256, 2>(x, rows, gpr, stride * kBytes, eps, qlo, qhi, q, scale, s);
+        else if (gpr <= 1024)
+            launch_vec<kDtype, 256, 4>(x, rows, gpr, stride * kBytes, eps, qlo, qhi, q, scale, s);
         else
-            launch_vec<kDtype, 256, 16>(x, rows, cpr, rb, eps, qlo, qhi, q, scale, s);
+            launch_vec<kDtype, 256, 8>(x, rows, gpr, stride * kBytes, eps, qlo, qhi, q, scale, s);
     } else {
         quantize_rows_generic<kDtype><<<(unsigned)rows, 256, 0, s>>>((const char*)x, cols, stride,
                                                                      eps, qlo, qhi, q, scale);

@@ -56,7 +56,9 @@ def test_argument_validation_without_device():
     assert lib.k3q_gemv_w4(one, 9, 1, 16, 8, one, one, null, -1, null, one, null, 0, null) == -4
     assert lib.k3q_gemv_w4(one, 0, 1, 16, 8, one, one, null, 128, null, one, null, 0, null) == -1  # zero missing
     assert lib.k3q_gemv_w4_workspace_bytes(1, 8192, 8192) >= 8192 * 4
-    assert lib.k3q_gemm_i8_workspace_bytes(16, 256, 128) == 256 * 128
+    assert lib.k3q_gemm_i8_workspace_bytes(4096, 256, 128) == 256 * 128  # room for the [N,K] copy
+    assert lib.k3q_gemm_i8_workspace_bytes(1, 8192, 8192) >= 8192 * 4  # decode size: split-K partials
+    assert lib.k3q_gemm_i8_workspace_bytes(16, 0, 128) == 0
 
 
 def test_error_codes_become_python_exceptions():
