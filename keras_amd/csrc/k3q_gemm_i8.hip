@@ -279,27 +279,29 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
     }
     __syncthreads();
     const bool has_bias = p.bias != nullptr;
+    // Row-major store order: the eight 8-byte (16-byte for float32) pieces that make up one
+    // 128-byte line of a row of y leave back to back, so that the L2 can merge them.
 #pragma unroll
-    for (int nb = 0; nb < kNBlk; ++nb) {
+    for (int mb = 0; mb < kMBlk; ++mb) {
+        const int ml = wm * kWM + mb * 32 + fi;
+        const int64_t m = m0 + ml;
+        if (m >= p.M) continue;
+        const float sa = ep[2 * kBN + ml];
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-            const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
-            const int64_t n = n0 + nl;
-            if (n >= p.N) continue;  // N % 4 == 0 on this path: all four columns in or out
-            const v4f sb = *(const v4f*)(ep + nl);
-            const v4f bv = *(const v4f*)(ep + kBN + nl);
+        for (int nb = 0; nb < kNBlk; ++nb) {
 #pragma unroll
-            for (int mb = 0; mb < kMBlk; ++mb) {
-                const int ml = wm * kWM + mb * 32 + fi;
-                const int64_t m = m0 + ml;
-                if (m >= p.M) continue;
+            for (int rg = 0; rg < 4; ++rg) {
+                const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+                const int64_t n = n0 + nl;
+                if (n >= p.N) continue;  // N % 4 == 0 on this path: all four columns in or out
                 if (p.acc_out) {
                     v4i o = {acc[nb][mb][4 * rg], acc[nb][mb][4 * rg + 1], acc[nb][mb][4 * rg + 2],
                              acc[nb][mb][4 * rg + 3]};
                     *(v4i*)(p.acc_out + m * p.N + n) = o;
                 }
                 if (!p.y) continue;
-                const float sa = ep[2 * kBN + ml];
+                const v4f sb = *(const v4f*)(ep + nl);
+                const v4f bv = *(const v4f*)(ep + kBN + nl);
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
