@@ -45,7 +45,7 @@ constexpr u32 kNibblePair = 0x000F000Fu;
 constexpr u32 kOnes = 0x3F803F80u;
 constexpr float kOffset = 136.0f;  // 128 (bf16 magic exponent) + 8 (nibble ^ 8)
 constexpr int kMaxWaves = 8;
-constexpr int kLdsBudget = 64 * 1024;
+constexpr int kLdsBudget = 128 * 1024;  // of the CU's 160 KiB; one workgroup per CU by design
 
 struct GemvParams {
     const void* x;         // [M, K] bf16 or f32
@@ -498,6 +498,17 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
 
 template <int kVec, int kSteps, int kSets, bool kXF32>
 void launch4(const GemvParams& p, bool grouped, dim3 grid, int threads, size_t lds, hipStream_t s) {
+    // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+    static const bool raised = [] {
+        bool ok = hipFuncSetAttribute((const void*)gemv_w4_mfma<kVec, kSteps, kSets, kXF32, true>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      kLdsBudget) == hipSuccess;
+        ok = hipFuncSetAttribute((const void*)gemv_w4_mfma<kVec, kSteps, kSets, kXF32, false>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 kLdsBudget) == hipSuccess && ok;
+        return ok;
+    }();
+    (void)raised;
     if (grouped)
         gemv_w4_mfma<kVec, kSteps, kSets, kXF32, true><<<grid, threads, lds, s>>>(p);
     else
