@@ -45,7 +45,8 @@ constexpr u32 kNibblePair = 0x000F000Fu;
 constexpr u32 kOnes = 0x3F803F80u;
 constexpr float kOffset = 136.0f;  // 128 (bf16 magic exponent) + 8 (nibble ^ 8)
 constexpr int kMaxWaves = 8;
-constexpr int kLdsBudget = 128 * 1024;  // of the CU's 160 KiB; one workgroup per CU by design
+constexpr int kRedPad = 8;
+constexpr int kLdsBudget = 144 * 1024;  // of the 160 KiB a workgroup may use
 
 struct GemvParams {
     const void* x;         // [M, K] bf16 or f32
@@ -113,13 +114,16 @@ __device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
 // rows of bf16 x, or up to 8 rows of f32 x split into two bf16 parts.
 template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
-    extern __shared__ float red[];  // [waves][M][kNB]
+    extern __shared__ float red[];  // [waves][M][kNB + kRedPad]
 #ifdef K3Q_GEMV_PROBE
     const uint64_t ts0 = __builtin_amdgcn_s_memrealtime();
 #endif
     constexpr bool kBF16 = !kXF32;
     constexpr int kAccSets = kXF32 ? 1 : kSets;
     constexpr int kNB = 128 * kVec;
+    // LDS row of partial sums: 8 floats of padding put the rows m, m+1, ... that the 16 lanes
+    // of a quarter wave store together on disjoint banks (m * 8 + grp * 4 + 0..3)
+    constexpr int kRedStride = kNB + kRedPad;
     constexpr int kChunk = kSteps * 16;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction
@@ -336,7 +340,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     for (int a = 0; a < kAccSets; ++a) {
         const int m = mrow + 8 * a;
         if (m < M) {
-            float* dst = red + ((size_t)wave * M + m) * kNB;
+            float* dst = red + ((size_t)wave * M + m) * kRedStride;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
 #pragma unroll
@@ -351,7 +355,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
             }
         }
     }
+#ifdef K3Q_GEMV_PROBE
+    const uint64_t ts2b = __builtin_amdgcn_s_memrealtime();
+#endif
     __syncthreads();
+#ifdef K3Q_GEMV_PROBE
+    const uint64_t ts2c = __builtin_amdgcn_s_memrealtime();
+#endif
 
     // ---- reduce the waves of this workgroup, four columns per thread ----
     const int KS = gridDim.y;
@@ -359,7 +369,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
         const int m = idx / (kNB / 4);
         const int nl = (idx % (kNB / 4)) * 4;
         v4f sum = {0.f, 0.f, 0.f, 0.f};
-        for (int w = 0; w < nwaves; ++w) sum += *(const v4f*)(red + ((size_t)w * M + m) * kNB + nl);
+        for (int w = 0; w < nwaves; ++w) sum += *(const v4f*)(red + ((size_t)w * M + m) * kRedStride + nl);
         const int64_t n = nb + nl;
         if (n < p.N) {  // N % 8 == 0 on this path: all four columns in or out
             if (KS == 1) {
@@ -372,8 +382,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     }
 #ifdef K3Q_GEMV_PROBE
     if (threadIdx.x == 0 && KS > 1) {
-        uint64_t* d = (uint64_t*)(p.part + (int64_t)KS * M * p.N) + 4 * (blockIdx.y * gridDim.x + blockIdx.x);
+        uint64_t* d = (uint64_t*)(p.part + (int64_t)KS * M * p.N) + 8 * (blockIdx.y * gridDim.x + blockIdx.x);
         d[0] = ts0; d[1] = ts1; d[2] = ts2; d[3] = __builtin_amdgcn_s_memrealtime();
+        d[4] = ts2b; d[5] = ts2c;
     }
 #endif
 }
@@ -462,7 +473,7 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     const int rows_used = (int)(M < pl.rows ? M : pl.rows);
 
     // Measured on MI355X at K = N = 8192: 8 waves per workgroup, 8-byte loads per lane and
-    // one workgroup per CU (256 workgroups) beat wider loads and finer K splits.
+    // one or two workgroups per CU beat wider loads and finer K splits.
     int vec = (grouped && pl.sets == 2) ? 1 : 2;
     if (plan_override && plan_override[0] > 0) vec = plan_override[0];
     while (vec > 1 && (N % (8 * vec)) != 0) vec >>= 1;
@@ -479,11 +490,14 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     const int nb_cols = 128 * vec;
     const int64_t nblocks = (N + nb_cols - 1) / nb_cols;
     int waves = kMaxWaves;
-    while (waves > 1 && (int64_t)waves * rows_used * nb_cols * 4 > kLdsBudget) waves >>= 1;
+    while (waves > 1 && (int64_t)waves * rows_used * (nb_cols + kRedPad) * 4 > kLdsBudget) waves >>= 1;
     if (plan_override && plan_override[2] > 0 && plan_override[2] <= waves) waves = plan_override[2];
 
     // rows of K per wave: the slice length that gives about one workgroup per CU
-    int64_t klen = K * nblocks / ((int64_t)kTargetWorkgroups * waves);
+    // Per-channel scales and one row set: two workgroups per CU, so that one workgroup's
+    // cross-wave reduction overlaps the other's loads (11.4 vs 12.8 us at M = 1).
+    const int target = (!grouped && pl.sets == 1) ? 2 * kTargetWorkgroups : kTargetWorkgroups;
+    int64_t klen = K * nblocks / ((int64_t)target * waves);
     klen = klen / chunk * chunk;
     if (klen < chunk) klen = chunk;
     if (plan_override && plan_override[3] > 0) klen = (plan_override[3] + chunk - 1) / chunk * chunk;
@@ -608,7 +622,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         p.M = rows;
         dim3 grid((unsigned)((nblocks + 7) / 8 * 8), (unsigned)pl.ks);
         const int threads = pl.waves * 64;
-        const size_t lds = (size_t)pl.waves * rows * nb_cols * sizeof(float);
+        const size_t lds = (size_t)pl.waves * rows * (nb_cols + kRedPad) * sizeof(float);
         const int sets = (!f32 && rows > 8) ? 2 : (f32 ? 2 : 1);
         launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
         if (pl.ks > 1) {
