@@ -281,23 +281,50 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
 
     // lane (j = lane%16, gq = lane/16) holds D[row 4*gq + r][col j]:
     //   column n_local = 8*kVec*(4*gq + r) + 8*q + pp + 4*grp,  x row m = (j % 8) + 8*set
-    // grouped: fold this group's scale and zero point into the running totals
+    // grouped: the scales and zero points of the current group are fetched ahead of time (at
+    // kernel start / right after the previous flush), so that the flush finds them in
+    // registers instead of waiting on memory once per group.
+    constexpr int kGq = kGrouped ? kVec : 1;
+    constexpr int kGr = kGrouped ? 4 : 1;
+    v4u gsc[kGr][kGq];  // four scales: 8 bytes (bf16) or 16 bytes (f32)
+    u32 gzp[kGr][kGq];  // four int8 zero points
+    const int64_t ngroups = kGrouped ? (p.K + p.block_size - 1) / p.block_size : 1;
+    auto load_group = [&](int64_t gi) {
+        if (!kGrouped) return;
+        if (gi > ngroups - 1) gi = ngroups - 1;
+#pragma unroll
+        for (int r = 0; r < kGr; ++r) {
+#pragma unroll
+            for (int q = 0; q < kGq; ++q) {
+                int64_t n = nb + 8 * kVec * (4 * g + r) + 8 * q + 4 * grp;
+                if (n >= p.N) n = p.N - 4;  // N % 8 == 0: a valid, aligned stand-in, never stored
+                const int64_t o = gi * p.N + n;
+                gzp[r][q] = *(const u32*)(p.zero + o);
+                if (kBF16) {
+                    const v2u t = *(const v2u*)((const uint16_t*)p.scale + o);
+                    gsc[r][q] = v4u{t[0], t[1], 0u, 0u};
+                } else {
+                    gsc[r][q] = *(const v4u*)((const float*)p.scale + o);
+                }
+            }
+        }
+    };
+    // fold this group's scale and zero point into the running totals
     auto flush_group = [&](int64_t gi) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < kGr; ++r) {
 #pragma unroll
-            for (int q = 0; q < kVec; ++q) {
-                const int64_t n = nb + 8 * kVec * (4 * g + r) + 8 * q + 4 * grp;
-                float sc[4] = {0.f, 0.f, 0.f, 0.f};
-                float zp[4] = {0.f, 0.f, 0.f, 0.f};
-                if (n < p.N) {
-                    const int64_t o = gi * p.N + n;
-                    const u32 z4 = *(const u32*)(p.zero + o);
+            for (int q = 0; q < kGq; ++q) {
+                float sc[4], zp[4];
 #pragma unroll
-                    for (int pp = 0; pp < 4; ++pp) {
-                        sc[pp] = load_t<kBF16>(p.scale, o + pp);
-                        zp[pp] = (float)(int)(int8_t)(z4 >> (8 * pp));
+                for (int pp = 0; pp < 4; ++pp) {
+                    if (kBF16) {
+                        const u32 w = gsc[r][q][pp >> 1];
+                        sc[pp] = __uint_as_float((pp & 1) ? (w & 0xffff0000u) : (w << 16));
+                    } else {
+                        sc[pp] = __uint_as_float(gsc[r][q][pp]);
                     }
+                    zp[pp] = (float)(int)(int8_t)(gzp[r][q] >> (8 * pp));
                 }
 #pragma unroll
                 for (int a = 0; a < kAccSets; ++a)
@@ -307,6 +334,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
             }
         }
         clear_acc();
+        load_group(gi + 1);
     };
     auto after_chunk = [&](int c) {
         if (!kGrouped) return;
@@ -317,6 +345,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     };
 
     load_chunk(0, 0);
+    if (kGrouped) load_group((kw0 < p.K ? kw0 : p.K - 1) / p.block_size);
 #ifdef K3Q_GEMV_PROBE
     const uint64_t ts1 = __builtin_amdgcn_s_memrealtime();
 #endif
