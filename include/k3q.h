@@ -10,7 +10,7 @@
  *     the call returns without synchronising;
  *   - the return value is K3Q_OK or a negative K3Q_ERR_* code; nothing is
  *     launched when an argument is rejected;
- *   - dtype codes: K3Q_F32 = 0, K3Q_BF16 = 1.
+ *   - dtype codes: K3Q_F32 = 0, K3Q_BF16 = 1; index dtypes K3Q_I32 = 2, K3Q_I64 = 3.
  *
  * The reference (keras-team/keras 3.16.0) has no FFI: these entry points
  * replace chains of torch ops, and each comment cites the chain it replaces.
@@ -27,6 +27,8 @@ extern "C" {
 
 #define K3Q_F32 0
 #define K3Q_BF16 1
+#define K3Q_I32 2
+#define K3Q_I64 3
 
 #define K3Q_OK 0
 #define K3Q_ERR_NULL (-1)      /* a required pointer is null                    */
@@ -93,12 +95,23 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  * other shapes run a plain kernel.  With b_layout 0 the MFMA kernel also needs
  * `workspace` (k3q_gemm_i8_workspace_bytes, 16-byte aligned) to hold the [N,K]
  * copy it makes on every call; callers that reuse a kernel should prepack once.
+ * flags bit 1 (K3Q_GEMM_ROUND_ACC_BF16, float32 output only): acc is cast to bfloat16
+ * before the division, which is what a bfloat16-compute layer with float32 scales
+ * computes (ReversibleEmbedding reads its scale without autocast).
+ * Decode sizes (M <= 64) run bandwidth-bound kernels that read b once, in either
+ * layout (b_layout 0: N % 16 == 0, K % 8 == 0; b_layout 1, e.g. a tied int8
+ * embedding table used as the LM head: K % 64 == 0), always with the exact
+ * epilogue; they may split K and then need `workspace` for int32 partials.
+ * The reverse projection of ReversibleEmbedding._int8_call
+ * (keras/src/layers/core/reversible_embedding.py:272-296) is this call with
+ * b = the [vocab, dim] table as stored, b_layout 1 and no bias.
  * Replaces cast, cast, matmul (keras/src/backend/torch/numpy.py:139-157), cast,
  * multiply, divide, add of Dense._int8_call (keras/src/layers/core/dense.py:961-983)
  * and the einsum form in EinsumDense._int8_call
  * (keras/src/layers/core/einsum_dense.py:1072-1084).
  */
 #define K3Q_GEMM_EXACT_EPILOGUE 1
+#define K3Q_GEMM_ROUND_ACC_BF16 2
 int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N, int8_t* prepacked,
                           void* stream);
@@ -141,6 +154,28 @@ int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N
                      const void* w_packed, const void* scale, const void* zero,
                      int64_t block_size, const void* bias, void* y, void* workspace,
                      int64_t workspace_bytes, const int* plan, void* stream);
+
+/*
+ * Quantized embedding lookup: out[t, :] = dequantise(table[ids[t], :]), t < count.
+ * Replaces the take + cast + divide chain of Embedding._int8_call
+ * (keras/src/layers/core/embedding.py:521-541) and the unpack_int4 + take +
+ * (divide | dequantize_with_sz_map) chain of Embedding._int4_call (:543-582,
+ * keras/src/quantizers/quantizers.py:1631-1668).
+ *   bits = 8: table [vocab, dim] int8, scale [vocab];      out = T(q) / scale[row]
+ *   bits = 4: table [vocab, ceil(dim/2)] int8, low nibble = even column;
+ *     block_size <= 0: scale [vocab];                        out = T(q) / scale[row]
+ *     block_size  > 0: scale, zero [vocab, ceil(dim/block)]; out = (T(q) - zero) * scale
+ * ids: int32 or int64 (ids_dtype); negative ids wrap once by `vocab`
+ * (keras/src/backend/torch/numpy.py:2005-2017).  An id still outside [0, vocab)
+ * gives a row of zeros and sets *oob_flag (may be null) to 1 -- the reference
+ * raises there; the host mirror turns the flag into the same IndexError.
+ * out_dtype follows the reference's promotion: bfloat16 only with bfloat16
+ * scales, else float32 (K3Q_ERR_DTYPE otherwise).
+ */
+int k3q_embedding_lookup(const void* ids, int ids_dtype, int64_t count, const int8_t* table,
+                         int64_t vocab, int64_t dim, int bits, const void* scale,
+                         int scale_dtype, const int8_t* zero, int64_t block_size, int out_dtype,
+                         void* out, int* oob_flag, void* stream);
 
 #ifdef __cplusplus
 }

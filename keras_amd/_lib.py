@@ -14,6 +14,8 @@ LIB_PATH = os.path.join(_HERE, "libk3q.so")
 
 K3Q_F32 = 0
 K3Q_BF16 = 1
+K3Q_I32 = 2
+K3Q_I64 = 3
 
 _ERRORS = {
     -1: ValueError,
@@ -46,6 +48,10 @@ SIGNATURES = {
         _int,
         [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _int, _int, _ptr, _ptr, _ptr,
          _i64, _ptr],
+    ),
+    "k3q_embedding_lookup": (
+        _int,
+        [_ptr, _int, _i64, _ptr, _i64, _i64, _int, _ptr, _int, _ptr, _i64, _int, _ptr, _ptr, _ptr],
     ),
     "k3q_gemv_w4_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "k3q_gemv_w4": (

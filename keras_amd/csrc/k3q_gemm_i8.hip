@@ -47,6 +47,7 @@ constexpr int kDmaPerWave = (2 * kDmaPerTile) / (kThreads / 64);      // 8 per w
 constexpr int kRowChunks = kBK / 16;                                  // 16-byte chunks per LDS row
 
 constexpr int kFlagExactEpilogue = 1;
+constexpr int kFlagRoundAccBF16 = 2;   // float32 output of a bfloat16 layer: acc is cast to bfloat16 first
 constexpr int kFlagSkipEpilogue = 1024;  // undocumented timing aid
 
 struct GemmParams {
@@ -279,6 +280,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
     }
     __syncthreads();
     const bool has_bias = p.bias != nullptr;
+    const bool round_acc = (p.flags & kFlagRoundAccBF16) != 0;
     // Row-major store order: the eight 8-byte (16-byte for float32) pieces that make up one
     // 128-byte line of a row of y leave back to back, so that the L2 can merge them.
 #pragma unroll
@@ -305,7 +307,8 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float accf = (float)acc[nb][mb][4 * rg + e];
+                    float accf = (float)acc[nb][mb][4 * rg + e];
+                    if (!kBF16 && round_acc) accf = round_bf16(accf);
                     float r;
                     if (kExact) {
                         // the reference's op sequence, every step rounded to T
@@ -357,7 +360,8 @@ __global__ __launch_bounds__(256) void gemm_i8_simple(const int8_t* a, const int
         if (p.bias) r = round_bf16(r + load_t<true>(p.bias, n));
         ((uint16_t*)p.y)[m * p.N + n] = (uint16_t)f32_to_bf16_bits(r);
     } else {
-        r = (float)acc / (sb * sa);
+        const float accf = (p.flags & kFlagRoundAccBF16) ? round_bf16((float)acc) : (float)acc;
+        r = accf / (sb * sa);
         if (p.bias) r = r + load_t<false>(p.bias, n);
         ((float*)p.y)[m * p.N + n] = r;
     }
@@ -409,8 +413,12 @@ extern "C" int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K) 
     if (N <= 0 || K <= 0) return 0;
     // decode-sized M with the [K,N] kernel: int32 split-K partials; larger M with the [K,N]
     // kernel: room for the [N,K] copy made per call
-    if (M > 0 && M <= kSkinnyMaxRows && (N % 16) == 0 && (K % 8) == 0)
-        return gemm_i8_skinny_workspace_bytes(M, N, K);
+    if (M > 0 && M <= kSkinnyMaxRows) {
+        // either kernel layout may be passed: room for the larger of the two partial buffers
+        const int64_t kn = ((N % 16) == 0 && (K % 8) == 0) ? gemm_i8_skinny_workspace_bytes(M, N, K) : N * K;
+        const int64_t nk = gemm_i8_skinny_nk_workspace_bytes(M, N, K);
+        return kn > nk ? kn : nk;
+    }
     return N * K;
 }
 
@@ -452,8 +460,11 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     const size_t el = bf16 ? 2 : 4;
     // decode-sized M: bandwidth-bound kernel that reads the [K,N] kernel in place
     if (b_layout == 0 && gemm_i8_skinny_supported(M, N, K, a, b))
-        return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, y, acc_out, workspace,
-                                  workspace_bytes, s);
+        return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
+                                  workspace, workspace_bytes, s);
+    if (b_layout == 1 && gemm_i8_skinny_nk_supported(M, N, K, a, b))
+        return gemm_i8_skinny_nk_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
+                                     workspace, workspace_bytes, s);
     bool fast = (K % kBK) == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
                 (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
                 (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&

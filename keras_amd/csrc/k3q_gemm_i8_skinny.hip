@@ -40,7 +40,7 @@ struct SkinnyParams {
     int M;                 // rows in this launch
     int m0;                // first row of this launch
     int klen;              // rows of K per wave
-    int exact;
+    int exact;             // bit 1: bfloat16 output; bit 2: round the accumulator to bfloat16 first
 };
 
 template <bool kBF16>
@@ -63,7 +63,8 @@ __device__ __forceinline__ void finish(const SkinnyParams& p, int m, int64_t n, 
         if (p.bias) r = round_bf16(r + load_t<true>(p.bias, n));
         ((uint16_t*)p.y)[row * p.N + n] = (uint16_t)f32_to_bf16_bits(r);
     } else {
-        r = (float)acc / (sb * sa);
+        const float accf = (p.exact & 4) ? round_bf16((float)acc) : (float)acc;
+        r = accf / (sb * sa);
         if (p.bias) r = r + load_t<false>(p.bias, n);
         ((float*)p.y)[row * p.N + n] = r;
     }
@@ -229,6 +230,114 @@ __global__ __launch_bounds__(256) void gemm_i8_skinny_reduce(SkinnyParams p, int
     for (int e = 0; e < 4; ++e) finish<kBF16>(p, m, n + e, sum[e]);
 }
 
+// ---- [N, K] kernel layout (K contiguous): tied embedding tables, prepacked kernels ----
+//
+// v_mfma_i32_16x16x64_i8 takes this layout as it is: lane (i = lane%16, c = lane/16) supplies
+// 16 consecutive k bytes (chunk c of a 64-byte step) of weight row n0 + i as the first
+// operand and of x row i as the second; D[4c + r][i] is then the int32 dot product of
+// weight row n0 + 4c + r with x row i.  A wave owns kTiles tiles of 16 weight rows and walks
+// its K slice in batches of kUnroll steps whose loads are all issued before the first MFMA;
+// waves never talk to each other (no LDS, no barrier).  K is split over blockIdx.y only when
+// N alone gives too few waves; partials are int32 and summed by gemm_i8_skinny_reduce.
+constexpr int kNkUnroll = 8;
+
+template <int kTiles>
+__global__ __launch_bounds__(256) void gemm_i8_skinny_nk(SkinnyParams p) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15;
+    const int c = lane >> 4;
+    const int M = p.M;
+    const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * (16 * kTiles);
+    if (n0 >= p.N) return;
+    const int64_t k_begin = (int64_t)blockIdx.y * p.klen;
+    int64_t k_end = k_begin + p.klen;
+    if (k_end > p.K) k_end = p.K;
+
+    const int8_t* wrow[kTiles];
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t) {
+        int64_t n = n0 + 16 * t + i;
+        if (n >= p.N) n = p.N - 1;  // loads stay in bounds; these rows are never stored
+        wrow[t] = p.w + n * p.K + 16 * c;
+    }
+    const int8_t* xrow = p.xq + (int64_t)(p.m0 + (i < M ? i : M - 1)) * p.K + 16 * c;
+    const u32 xmask = i < M ? 0xffffffffu : 0u;
+
+    v4i acc[kTiles];
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t) acc[t] = v4i{0, 0, 0, 0};
+
+    for (int64_t k0 = k_begin; k0 < k_end; k0 += 64 * kNkUnroll) {
+        v4u wv[kNkUnroll][kTiles], xv[kNkUnroll];
+#pragma unroll
+        for (int u = 0; u < kNkUnroll; ++u) {
+            // steps past the slice end re-read the last valid step and meet a zero x operand
+            const int64_t k = k0 + 64 * u < k_end ? k0 + 64 * u : k_end - 64;
+#pragma unroll
+            for (int t = 0; t < kTiles; ++t)
+                wv[u][t] = __builtin_nontemporal_load((const v4u*)(wrow[t] + k));
+            xv[u] = *(const v4u*)(xrow + k);
+        }
+#pragma unroll
+        for (int u = 0; u < kNkUnroll; ++u) {
+            const u32 m = k0 + 64 * u < k_end ? xmask : 0u;
+            const v4u xm = {xv[u][0] & m, xv[u][1] & m, xv[u][2] & m, xv[u][3] & m};
+#pragma unroll
+            for (int t = 0; t < kTiles; ++t)
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wv[u][t]),
+                                                               __builtin_bit_cast(v4i, xm), acc[t],
+                                                               0, 0, 0);
+        }
+    }
+
+    // lane holds rows n0 + 16t + 4c + r (r = 0..3) of x row i
+    if (i >= M) return;
+    const int KS = gridDim.y;
+#pragma unroll
+    for (int t = 0; t < kTiles; ++t) {
+        const int64_t n = n0 + 16 * t + 4 * c;
+        if (KS > 1) {
+            if (n + 3 < p.N) {
+                *(v4i*)(p.part + ((int64_t)blockIdx.y * M + i) * p.N + n) = acc[t];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < p.N) p.part[((int64_t)blockIdx.y * M + i) * p.N + n + r] = acc[t][r];
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (n + r >= p.N) continue;
+                if (p.exact & 2)
+                    finish<true>(p, i, n + r, acc[t][r]);
+                else
+                    finish<false>(p, i, n + r, acc[t][r]);
+            }
+        }
+    }
+}
+
+struct NkPlan {
+    int tiles;    // 16-row tiles per wave
+    int ks;       // K slices (blockIdx.y)
+    int64_t klen; // bytes of K per slice, a multiple of 64
+};
+
+NkPlan make_nk_plan(int64_t N, int64_t K) {
+    NkPlan pl{};
+    pl.tiles = N >= 16384 ? 2 : 1;
+    const int64_t waves = (N + 16 * pl.tiles - 1) / (16 * pl.tiles);
+    int64_t ks = 1;
+    // aim at >= 2048 waves (8 per CU), keep at least 512 bytes of K per slice
+    // (the reduction kernel works on groups of four columns)
+    while ((N % 4) == 0 && waves * ks < 2048 && K / (ks * 2) >= 512) ks *= 2;
+    int64_t klen = (K / ks + 63) / 64 * 64;
+    pl.ks = (int)((K + klen - 1) / klen);
+    pl.klen = klen;
+    return pl;
+}
+
 struct Plan {
     int steps, sets, rows, waves, klen, ks;
 };
@@ -281,8 +390,64 @@ int64_t gemm_i8_skinny_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return (int64_t)pl.ks * rows * N * 4;
 }
 
+bool gemm_i8_skinny_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* b) {
+    return M > 0 && M <= kSkinnyMaxRows && N > 0 && (K % 64) == 0 && aligned_to(a, 16) &&
+           aligned_to(b, 16);
+}
+
+int64_t gemm_i8_skinny_nk_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || M > kSkinnyMaxRows || (K % 64) != 0) return 0;
+    const NkPlan pl = make_nk_plan(N, K);
+    if (pl.ks <= 1) return 0;
+    return (int64_t)pl.ks * (M < 16 ? M : 16) * N * 4;
+}
+
+int gemm_i8_skinny_nk_run(const int8_t* a, const int8_t* b, int64_t M, int64_t N, int64_t K,
+                          const void* a_scale, const void* b_scale, const void* bias, bool bf16, int flags,
+                          void* y, int32_t* acc_out, void* workspace, int64_t workspace_bytes,
+                          hipStream_t s) {
+    SkinnyParams p{};
+    p.xq = a;
+    p.w = b;
+    p.a_scale = a_scale;
+    p.b_scale = b_scale;
+    p.bias = bias;
+    p.y = y;
+    p.acc_out = acc_out;
+    p.K = K;
+    p.N = N;
+    p.exact = (bf16 ? 2 : 0) | ((flags & 2) ? 4 : 0);
+    const NkPlan pl = make_nk_plan(N, K);
+    if (pl.ks > 1) {
+        const int64_t need = (int64_t)pl.ks * (M < 16 ? M : 16) * N * 4;
+        if (!workspace || workspace_bytes < need) return K3Q_ERR_WORKSPACE;
+        if (!aligned_to(workspace, 16)) return K3Q_ERR_ALIGN;
+        p.part = (int32_t*)workspace;
+    }
+    p.klen = (int)pl.klen;
+    const int64_t waves = (N + 16 * pl.tiles - 1) / (16 * pl.tiles);
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int rows = (int)((M - m0 < 16) ? M - m0 : 16);
+        p.m0 = (int)m0;
+        p.M = rows;
+        dim3 grid((unsigned)((waves + 3) / 4), (unsigned)pl.ks);
+        if (pl.tiles == 2)
+            gemm_i8_skinny_nk<2><<<grid, 256, 0, s>>>(p);
+        else
+            gemm_i8_skinny_nk<1><<<grid, 256, 0, s>>>(p);
+        if (pl.ks > 1) {
+            dim3 rgrid((unsigned)((N / 4 + 255) / 256), rows);
+            if (bf16)
+                gemm_i8_skinny_reduce<true><<<rgrid, 256, 0, s>>>(p, pl.ks);
+            else
+                gemm_i8_skinny_reduce<false><<<rgrid, 256, 0, s>>>(p, pl.ks);
+        }
+    }
+    return launch_status();
+}
+
 int gemm_i8_skinny_run(const int8_t* a, const int8_t* b, int64_t M, int64_t N, int64_t K,
-                       const void* a_scale, const void* b_scale, const void* bias, bool bf16,
+                       const void* a_scale, const void* b_scale, const void* bias, bool bf16, int flags,
                        void* y, int32_t* acc_out, void* workspace, int64_t workspace_bytes,
                        hipStream_t s) {
     SkinnyParams p{};
@@ -295,7 +460,7 @@ int gemm_i8_skinny_run(const int8_t* a, const int8_t* b, int64_t M, int64_t N, i
     p.acc_out = acc_out;
     p.K = K;
     p.N = N;
-    p.exact = bf16 ? 2 : 0;
+    p.exact = (bf16 ? 2 : 0) | ((flags & 2) ? 4 : 0);
     const Plan pl = make_plan(M, K, N);
     const int64_t nblocks = (N + kNB - 1) / kNB;
     const int rows_max = (int)(M < pl.rows ? M : pl.rows);

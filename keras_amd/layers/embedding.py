@@ -1,0 +1,544 @@
+"""`Embedding` and `ReversibleEmbedding` with the int8 / int4 quantized forward on MI355X.
+
+Mirrors the quantization-related surface of `keras.layers.Embedding`
+(keras/src/layers/core/embedding.py) and `keras.layers.ReversibleEmbedding`
+(keras/src/layers/core/reversible_embedding.py): variable names, shapes and dtypes
+(`_embeddings` int8 `[vocab, dim]` or packed int4 `[vocab, ceil(dim/2)]`,
+`embeddings_scale`, `embeddings_zero`, `g_idx`, and the `reverse_*` twins of an untied
+layer), `quantize(mode, config)`, the dtype-policy names it leaves behind and the
+positional store order.  The lookup runs `k3q_embedding_lookup`; the int8 reverse
+projection (the LM head) runs the int8 GEMM / decode kernels with the tied table read in
+place as an `[N, K]` operand.
+
+Both layers set `autocast = False` in the reference (embedding.py:132): their float
+variables are read in their own dtype, and torch's type promotion decides the output dtype
+(a float32 scale under a bfloat16 compute dtype gives float32 outputs).
+"""
+
+import math
+
+import torch
+
+from keras_amd import dtype_policies, ops as kops, quantizers
+from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.quantization_config import (
+    Int4QuantizationConfig,
+    QuantizationConfig,
+    get_block_size_for_layer,
+)
+
+
+def uniform_initializer(shape, dtype, generator=None):
+    """keras "uniform": U(-0.05, 0.05) (keras/src/initializers/random_initializers.py:118-170)."""
+    return ((torch.rand(shape, generator=generator) * 2.0 - 1.0) * 0.05).to(dtype)
+
+
+def _promote(a, b):
+    return a if a == b else torch.float32
+
+
+class Embedding(Layer):
+    def __init__(self, input_dim, output_dim, embeddings_initializer=None, mask_zero=False,
+                 dtype=None, name=None, device=None, quantization_config=None):
+        if not isinstance(input_dim, int) or isinstance(input_dim, bool) or input_dim <= 0:
+            raise ValueError(
+                "`input_dim` must be a positive integer. "
+                f"Received: input_dim={input_dim} (of type {type(input_dim).__name__})."
+            )
+        if not isinstance(output_dim, int) or isinstance(output_dim, bool) or output_dim <= 0:
+            raise ValueError(
+                "`output_dim` must be a positive integer. "
+                f"Received: output_dim={output_dim} (of type {type(output_dim).__name__})."
+            )
+        super().__init__(dtype=dtype, name=name, device=device)
+        self.input_dim = input_dim
+        self.output_dim = output_dim
+        self.embeddings_initializer = embeddings_initializer or uniform_initializer
+        self.mask_zero = mask_zero
+        self.autocast = False
+        self.lora_enabled = False
+        self.quantization_config = quantization_config
+        # raise IndexError for ids outside the table as the reference does; costs one
+        # device -> host read per call, switch off in a serving loop
+        self.check_ids = True
+
+    # ---- build --------------------------------------------------------------
+    def build(self, input_shape=None):
+        if self.built:
+            return
+        embeddings_shape = (self.input_dim, self.output_dim)
+        if self.quantization_mode:
+            self.quantized_build(embeddings_shape, mode=self.quantization_mode,
+                                 config=self.quantization_config)
+        if self.quantization_mode not in ("int8", "int4"):
+            self._embeddings = self.add_weight(
+                name="embeddings", shape=embeddings_shape,
+                initializer=self.embeddings_initializer, trainable=True,
+            )
+        self.built = True
+
+    @property
+    def embeddings(self):
+        """The table as a consumer sees it: int4 comes back unpacked to int8
+        `[vocab, dim]` (embedding.py:169-191)."""
+        if not self.built:
+            raise AttributeError("You must build the layer before accessing `embeddings`.")
+        embeddings = as_tensor(self._embeddings)
+        if self.quantization_mode == "int4":
+            embeddings = quantizers.unpack_int4(embeddings, self._orig_output_dim, axis=-1)
+        return embeddings
+
+    def __call__(self, inputs, training=None, **kwargs):
+        # ids are not cast to the compute dtype (layer.py:883-901 only touches floats)
+        if not isinstance(inputs, torch.Tensor):
+            inputs = torch.as_tensor(inputs)
+        if not self.built:
+            self.build(tuple(inputs.shape))
+        if inputs.device != self.device:
+            inputs = inputs.to(self.device)
+        if self.quantization_mode is not None:
+            return self.quantized_call(inputs, **kwargs)
+        return self.call(inputs, **kwargs)
+
+    def call(self, inputs):
+        if inputs.dtype not in (torch.int32, torch.int64):
+            inputs = inputs.to(torch.int32)
+        idx = inputs.long()
+        idx = torch.where(idx < 0, idx + self.input_dim, idx)
+        out = torch.nn.functional.embedding(idx, as_tensor(self._embeddings))
+        return out.to(to_torch_dtype(self.compute_dtype))
+
+    def compute_mask(self, inputs, mask=None):
+        if not self.mask_zero:
+            return None
+        return torch.not_equal(inputs, 0)
+
+    def compute_output_shape(self, input_shape):
+        return (*input_shape, self.output_dim)
+
+    # ---- quantized variables --------------------------------------------------
+    @property
+    def variable_serialization_spec(self):
+        """embedding.py:409-428."""
+        return {
+            None: ["embeddings"],
+            "int8": ["embeddings", "embeddings_scale"],
+            "int4": ["embeddings", "embeddings_scale", "embeddings_zero", "g_idx"],
+        }
+
+    def quantized_build(self, embeddings_shape, mode, config=None):
+        if mode == "int8":
+            self._int8_build(embeddings_shape, config)
+        elif mode == "int4":
+            self._int4_build(embeddings_shape, config)
+        else:
+            raise self._quantization_mode_error(mode)
+        self._is_quantized = True
+
+    def _int8_build(self, embeddings_shape, config=None):
+        self._embeddings = self.add_weight(name="embeddings", shape=embeddings_shape, dtype="int8")
+        # one scale per vocabulary row: the reduction runs over output_dim (embedding.py:447-455)
+        self.embeddings_scale = self.add_weight(
+            name="embeddings_scale", shape=(self.input_dim,), initializer="ones"
+        )
+
+    def _int4_build(self, embeddings_shape, config=None):
+        input_dim, output_dim = embeddings_shape
+        packed_cols = (output_dim + 1) // 2
+        self._embeddings = self.add_weight(
+            name="embeddings", shape=(input_dim, packed_cols), dtype="int8"
+        )
+        block_size = get_block_size_for_layer(self, config)
+        self._int4_block_size = block_size
+        if block_size is None or block_size == -1:
+            scale_shape = (self.input_dim,)
+        else:
+            scale_shape = (self.input_dim, math.ceil(output_dim / block_size))
+        self.embeddings_scale = self.add_weight(
+            name="embeddings_scale", shape=scale_shape, initializer="ones"
+        )
+        if block_size is not None and block_size > 0:
+            self.embeddings_zero = self.add_weight(
+                name="embeddings_zero", shape=scale_shape, dtype="int8"
+            )
+            # float32 on purpose, as in the reference (embedding.py:500-516)
+            self.g_idx = self.add_weight(
+                name="g_idx", shape=(output_dim,), dtype="float32",
+                initializer=lambda shape, dtype: torch.floor_divide(
+                    torch.arange(output_dim, dtype=dtype), block_size),
+            )
+        self._orig_output_dim = output_dim
+
+    # ---- quantized forward -------------------------------------------------------
+    def _lookup_dtype(self):
+        return _promote(to_torch_dtype(self.compute_dtype), as_tensor(self.embeddings_scale).dtype)
+
+    def _int8_call(self, inputs, training=None):
+        """embedding.py:521-541: gather rows and scales, cast, divide -- one kernel."""
+        if self.lora_enabled:
+            raise NotImplementedError("LoRA on a quantized Embedding is outside this inference path.")
+        return kops.embedding_lookup(
+            inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
+            self.output_dim, bits=8, out_dtype=self._lookup_dtype(), check_ids=self.check_ids,
+        )
+
+    def _int4_call(self, inputs, training=None):
+        """embedding.py:542-582: the packed rows are gathered and de-quantised in one kernel;
+        the table is never unpacked in memory."""
+        if self.lora_enabled:
+            raise NotImplementedError("LoRA on a quantized Embedding is outside this inference path.")
+        block_size = getattr(self, "_int4_block_size", None)
+        grouped = block_size is not None and block_size > 0
+        return kops.embedding_lookup(
+            inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
+            self._orig_output_dim, bits=4,
+            zero=as_tensor(self.embeddings_zero) if grouped else None,
+            block_size=block_size if grouped else None,
+            out_dtype=self._lookup_dtype(), check_ids=self.check_ids,
+        )
+
+    # ---- quantize (one-time, host side) ---------------------------------------------
+    def _drop(self, attr):
+        var = getattr(self, attr)
+        self._variables = [v for v in self._variables if v is not var]
+        delattr(self, attr)
+
+    def _quantize_table(self, mode, config, block_size):
+        """Quantised forward table: (value int8 [V, D] or packed, scale, zero | None)."""
+        table = as_tensor(self._embeddings)
+        if mode == "int8":
+            wq = QuantizationConfig.weight_quantizer_or_default(
+                config, quantizers.AbsMaxQuantizer(axis=-1))
+            value, scale = wq(table, to_numpy=True)
+            return value, torch.squeeze(scale, dim=-1), None
+        use_grouped = block_size is not None and block_size != -1
+        zero = None
+        if not use_grouped:
+            wq = QuantizationConfig.weight_quantizer_or_default(
+                config, quantizers.AbsMaxQuantizer(axis=-1, value_range=(-8, 7), output_dtype="int8"))
+            value, scale = wq(table, to_numpy=True)
+            scale = torch.squeeze(scale, dim=-1)
+        else:
+            # grouped along output_dim: quantise the transpose, transpose back
+            value_t, scale_t, zero_t = quantizers.abs_max_quantize_grouped_with_zero_point(
+                torch.transpose(table, 0, 1), block_size=block_size, value_range=(-8, 7),
+                dtype="int8", to_numpy=True,
+            )
+            value = torch.transpose(value_t, 0, 1).contiguous()
+            scale = torch.transpose(scale_t, 0, 1).contiguous()
+            zero = torch.transpose(zero_t, 0, 1).contiguous()
+        packed, _, _ = quantizers.pack_int4(value.to(self.device), axis=-1)
+        return packed, scale, zero
+
+    def _set_quantized_policy(self, mode, config):
+        if self.dtype_policy.quantization_mode is None:
+            policy_name = mode
+            if mode == "int4":
+                block_size = get_block_size_for_layer(self, config)
+                policy_name = f"int4/{-1 if block_size is None else block_size}"
+            self._dtype_policy = dtype_policies.get(f"{policy_name}_from_{self.dtype_policy.name}")
+
+    def _quantize(self, mode, config, type_check=True):
+        """embedding.py:584-684."""
+        if type_check and type(self) is not Embedding:
+            raise self._not_implemented_error(self.quantize)
+        if mode not in ("int8", "int4"):
+            raise self._quantization_mode_error(mode)
+        self.quantization_config = config
+        embeddings_shape = (self.input_dim, self.output_dim)
+        block_size = get_block_size_for_layer(self, config) if mode == "int4" else None
+        value, scale, zero = self._quantize_table(mode, config, block_size)
+        self._drop("_embeddings")
+        self.quantized_build(embeddings_shape, mode, config)
+        self._embeddings.assign(value)
+        self.embeddings_scale.assign(scale)
+        if zero is not None:
+            self.embeddings_zero.assign(zero)
+        self._set_quantized_policy(mode, config)
+
+    def _quantization_mode_error(self, mode):
+        return NotImplementedError(
+            "Invalid quantization mode. Expected one of ('int8', 'int4'). "
+            f"Received: quantization_mode={mode}"
+        )
+
+    # ---- serialization ----------------------------------------------------------------
+    def _spec_entries(self):
+        """(name, variable) in store order, skipping entries this configuration lacks
+        (embedding.py:276-372)."""
+        mode = self.quantization_mode
+        if mode not in self.variable_serialization_spec:
+            raise self._quantization_mode_error(mode)
+        out = []
+        for name in self.variable_serialization_spec[mode]:
+            attr = "_embeddings" if name == "embeddings" else name
+            if not hasattr(self, attr):
+                continue
+            out.append((name, getattr(self, attr)))
+        return out
+
+    def save_own_variables(self, store):
+        if not self.built:
+            return
+        for idx, (_, var) in enumerate(self._spec_entries()):
+            store[str(idx)] = as_tensor(var)
+
+    def load_own_variables(self, store):
+        if not self.built:
+            return
+        for idx, (name, var) in enumerate(self._spec_entries()):
+            value = store[str(idx)]
+            if name == "g_idx" and isinstance(value, torch.Tensor):
+                value = value.to(as_tensor(var).dtype)
+            var.assign(value)
+
+    def get_config(self):
+        return {
+            "name": self.name,
+            "input_dim": self.input_dim,
+            "output_dim": self.output_dim,
+            "mask_zero": self.mask_zero,
+            "dtype": self.dtype_policy.name,
+            "quantization_config": (
+                None if self.quantization_config is None else {
+                    "class_name": type(self.quantization_config).__name__,
+                    "config": self.quantization_config.get_config(),
+                }
+            ),
+        }
+
+
+class ReversibleEmbedding(Embedding):
+    """`Embedding` that can also project back to the vocabulary (`reverse=True`), i.e. the
+    LM head (reversible_embedding.py:16-541)."""
+
+    def __init__(self, input_dim, output_dim, tie_weights=True, embeddings_initializer=None,
+                 mask_zero=False, reverse_dtype=None, logit_soft_cap=None, **kwargs):
+        super().__init__(input_dim, output_dim, embeddings_initializer=embeddings_initializer,
+                         mask_zero=mask_zero, **kwargs)
+        self.tie_weights = tie_weights
+        self.reverse_dtype = reverse_dtype
+        self.logit_soft_cap = logit_soft_cap
+        self.exact_epilogue = None
+        self._cache = {}
+
+    def build(self, input_shape=None):
+        if self.built:
+            return
+        super().build(input_shape)
+        if not self.tie_weights and self.quantization_mode not in ("int8", "int4"):
+            self.reverse_embeddings = self.add_weight(
+                name="reverse_embeddings", shape=(self.output_dim, self.input_dim),
+                initializer=self.embeddings_initializer, trainable=True,
+            )
+
+    def __call__(self, inputs, reverse=False, training=None):
+        if not reverse:
+            return super().__call__(inputs)
+        if not isinstance(inputs, torch.Tensor):
+            inputs = torch.as_tensor(inputs)
+        if not self.built:
+            self.build()
+        if inputs.device != self.device:
+            inputs = inputs.to(self.device)
+        cd = to_torch_dtype(self.compute_dtype)
+        if inputs.dtype.is_floating_point and inputs.dtype != cd:
+            inputs = inputs.to(cd)
+        if self.quantization_mode is not None:
+            return self.quantized_call(inputs, reverse=True)
+        return self.call(inputs, reverse=True)
+
+    def call(self, inputs, reverse=False):
+        if not reverse:
+            return super().call(inputs)
+        if self.tie_weights:
+            kernel = torch.transpose(as_tensor(self._embeddings), 0, 1)
+        else:
+            kernel = as_tensor(self.reverse_embeddings)
+        if self.reverse_dtype is not None:
+            rd = to_torch_dtype(self.reverse_dtype)
+            inputs, kernel = inputs.to(rd), kernel.to(rd)
+        rt = _promote(inputs.dtype, kernel.dtype)
+        logits = torch.matmul(inputs.to(rt), kernel.to(rt))
+        return self._soft_cap(logits)
+
+    def _soft_cap(self, logits):
+        if self.logit_soft_cap is None:
+            return logits
+        cap = self.logit_soft_cap
+        return torch.multiply(torch.tanh(torch.divide(logits, cap)), cap)
+
+    def compute_mask(self, inputs, mask=None):
+        return None
+
+    def compute_output_shape(self, input_shape, reverse=False):
+        output_shape = list(input_shape)
+        if reverse:
+            output_shape[-1] = self.input_dim
+        else:
+            output_shape += [self.output_dim]
+        return output_shape
+
+    # ---- quantized variables ------------------------------------------------------
+    @property
+    def variable_serialization_spec(self):
+        """reversible_embedding.py:176-189."""
+        spec = {k: list(v) for k, v in super().variable_serialization_spec.items()}
+        if not self.tie_weights:
+            for mode, names in spec.items():
+                names.append("reverse_embeddings")
+                if mode in ("int4", "int8"):
+                    names.append("reverse_embeddings_scale")
+                if mode == "int4":
+                    names.append("reverse_embeddings_zero")
+        return spec
+
+    def _int8_build(self, embeddings_shape, config=None):
+        super()._int8_build(embeddings_shape, config)
+        self.inputs_quantizer = QuantizationConfig.activation_quantizer_or_default(
+            config, quantizers.AbsMaxQuantizer(axis=-1))
+        if not self.tie_weights:
+            self.reverse_embeddings = self.add_weight(
+                name="reverse_embeddings", shape=(self.output_dim, self.input_dim), dtype="int8")
+            self.reverse_embeddings_scale = self.add_weight(
+                name="reverse_embeddings_scale", shape=(self.input_dim,), initializer="ones")
+
+    def _int4_build(self, embeddings_shape, config=None):
+        super()._int4_build(embeddings_shape, config)
+        self.inputs_quantizer = QuantizationConfig.activation_quantizer_or_default(
+            config, quantizers.AbsMaxQuantizer(axis=-1))
+        if not self.tie_weights:
+            packed_rows = (self.output_dim + 1) // 2
+            self.reverse_embeddings = self.add_weight(
+                name="reverse_embeddings", shape=(packed_rows, self.input_dim), dtype="int8")
+            block_size = get_block_size_for_layer(self, config)
+            if block_size is None or block_size == -1:
+                reverse_scale_shape = (self.input_dim,)
+            else:
+                reverse_scale_shape = (math.ceil(self.output_dim / block_size), self.input_dim)
+            self.reverse_embeddings_scale = self.add_weight(
+                name="reverse_embeddings_scale", shape=reverse_scale_shape, initializer="ones")
+            if block_size is not None and block_size != -1:
+                # variable dtype (not int8), as in the reference (reversible_embedding.py:262-269)
+                self.reverse_embeddings_zero = self.add_weight(
+                    name="reverse_embeddings_zero", shape=reverse_scale_shape)
+
+    # ---- quantized forward -----------------------------------------------------------
+    def _cached(self, key, var, make):
+        hit = self._cache.get(key)
+        if hit is not None and hit[0] == var.version and hit[1] is var:
+            return hit[2]
+        value = make(as_tensor(var))
+        self._cache[key] = (var.version, var, value)
+        return value
+
+    def _int8_call(self, inputs, reverse=False, training=None):
+        """reversible_embedding.py:272-296.  Tied weights: the `[vocab, dim]` int8 table IS
+        the `[N, K]` operand of the GEMM; nothing is transposed."""
+        if not reverse:
+            return super()._int8_call(inputs)
+        if not self.inputs_quantizer:
+            raise NotImplementedError(
+                "Weight-only int8 reverse projection (no activation quantizer) is not on the "
+                "fused path yet."
+            )
+        cd = to_torch_dtype(self.compute_dtype)
+        lead = inputs.shape[:-1]
+        x2 = inputs.reshape(-1, inputs.shape[-1])
+        q, in_scale = self.inputs_quantizer(x2, axis=-1)
+        scale_var = self.embeddings_scale if self.tie_weights else self.reverse_embeddings_scale
+        out_dtype = _promote(cd, as_tensor(scale_var).dtype)
+        M, N = x2.shape[0], self.input_dim
+        exact = self.exact_epilogue
+        if exact is None:
+            exact = M * N <= (1 << 22)
+        in_scale = in_scale.to(out_dtype)  # widening an existing value is exact
+        round_acc = cd == torch.bfloat16 and out_dtype == torch.float32
+        if self.tie_weights:
+            logits = kops.int8_matmul_nk(
+                q, as_tensor(self._embeddings), a_scale=in_scale,
+                kernel_scale=as_tensor(scale_var), out_dtype=out_dtype,
+                exact_epilogue=exact, round_acc_bf16=round_acc,
+            )
+        else:
+            if round_acc:
+                raise NotImplementedError(
+                    "Untied int8 reverse projection with bfloat16 compute and float32 scales "
+                    "is not on the fused path yet."
+                )
+            logits = kops.int8_matmul(
+                q, as_tensor(self.reverse_embeddings), a_scale=in_scale,
+                kernel_scale=as_tensor(scale_var), out_dtype=out_dtype,
+                prepacked=self._cached("prepacked", self.reverse_embeddings,
+                                       kops.prepack_int8_kernel),
+                exact_epilogue=exact,
+            )
+        return self._soft_cap(logits.reshape(*lead, N))
+
+    def _int4_call(self, inputs, reverse=False, training=None):
+        if not reverse:
+            return super()._int4_call(inputs)
+        raise NotImplementedError(
+            "The int4 reverse projection (activation-quantized int4 matmul, "
+            "reversible_embedding.py:298-381) is not on the fused path yet."
+        )
+
+    # ---- quantize -----------------------------------------------------------------------
+    def _quantize(self, mode, config, type_check=True):
+        """reversible_embedding.py:383-541."""
+        if type_check and type(self) is not ReversibleEmbedding:
+            raise self._not_implemented_error(self.quantize)
+        if mode not in ("int8", "int4"):
+            raise self._quantization_mode_error(mode)
+        self.quantization_config = config
+        embeddings_shape = (self.input_dim, self.output_dim)
+        # the reference reads the block size from the config object only here (:439-444)
+        block_size = None
+        if mode == "int4" and isinstance(config, Int4QuantizationConfig):
+            block_size = config.block_size
+        use_grouped = block_size is not None and block_size != -1
+        value, scale, zero = self._quantize_table(mode, config, block_size)
+        self._drop("_embeddings")
+        rev = None
+        if not self.tie_weights:
+            rtable = as_tensor(self.reverse_embeddings)
+            if mode == "int8":
+                wq = QuantizationConfig.weight_quantizer_or_default(
+                    config, quantizers.AbsMaxQuantizer(axis=0))
+                rvalue, rscale = wq(rtable, to_numpy=True)
+                rev = (rvalue, torch.squeeze(rscale, dim=0), None)
+            else:
+                if not use_grouped:
+                    wq = QuantizationConfig.weight_quantizer_or_default(
+                        config,
+                        quantizers.AbsMaxQuantizer(axis=0, value_range=(-8, 7), output_dtype="int8"))
+                    rvalue, rscale = wq(rtable, to_numpy=True)
+                    rscale, rzero = torch.squeeze(rscale, dim=0), None
+                else:
+                    rvalue, rscale, rzero = quantizers.abs_max_quantize_grouped_with_zero_point(
+                        rtable, block_size=block_size, value_range=(-8, 7), dtype="int8",
+                        to_numpy=True)
+                rpacked, _, _ = quantizers.pack_int4(rvalue.to(self.device), axis=0)
+                rev = (rpacked, rscale, rzero)
+            self._drop("reverse_embeddings")
+        self.quantized_build(embeddings_shape, mode, config)
+        self._embeddings.assign(value)
+        self.embeddings_scale.assign(scale)
+        if zero is not None:
+            self.embeddings_zero.assign(zero)
+        if rev is not None:
+            self.reverse_embeddings.assign(rev[0])
+            self.reverse_embeddings_scale.assign(rev[1])
+            if rev[2] is not None:
+                self.reverse_embeddings_zero.assign(rev[2])
+        self._set_quantized_policy(mode, config)
+        self._cache.clear()
+
+    def get_config(self):
+        config = super().get_config()
+        config.update({
+            "tie_weights": self.tie_weights,
+            "reverse_dtype": self.reverse_dtype,
+            "logit_soft_cap": self.logit_soft_cap,
+        })
+        return config

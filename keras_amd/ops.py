@@ -155,3 +155,97 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
     if want_acc and want_y:
         return y, acc
     return acc if want_acc else y
+
+
+GEMM_ROUND_ACC_BF16 = 2
+
+
+def int8_matmul_nk(a, kernel_nk, a_scale=None, kernel_scale=None, out_dtype=None,
+                   exact_epilogue=False, want_acc=False, round_acc_bf16=False):
+    """`a[M, K] int8 . kernel_nk[N, K]^T` with the de-scale fused: the kernel is given
+    with K contiguous, which is how a tied int8 embedding table `[vocab, dim]` serves as
+    the LM head (keras/src/layers/core/reversible_embedding.py:272-296).  Nothing is
+    transposed or copied; decode-sized M runs the bandwidth-bound kernel, larger M the
+    MFMA GEMM.  round_acc_bf16 (float32 output): the accumulator is cast to bfloat16
+    before the division, as a bfloat16-compute layer with float32 scales does.
+    """
+    _lib.require_device(a, kernel_nk, a_scale, kernel_scale)
+    if a.dtype != torch.int8 or kernel_nk.dtype != torch.int8:
+        raise TypeError("int8_matmul_nk takes int8 operands")
+    M, K = a.shape
+    if kernel_nk.dim() != 2 or kernel_nk.shape[1] != K:
+        raise ValueError(f"inner dimensions differ: {tuple(a.shape)} x {tuple(kernel_nk.shape)}^T")
+    N = kernel_nk.shape[0]
+    if out_dtype is None:
+        out_dtype = a_scale.dtype if a_scale is not None else torch.float32
+    code = _lib.dtype_code(out_dtype)
+    for t in (a_scale, kernel_scale):
+        if t is not None and t.dtype != out_dtype:
+            raise TypeError("scales must be read in the output dtype")
+    a = a if a.is_contiguous() else a.contiguous()
+    b = kernel_nk if kernel_nk.is_contiguous() else kernel_nk.contiguous()
+    sa = a_scale.reshape(-1).contiguous() if a_scale is not None else None
+    sb = kernel_scale.reshape(-1).contiguous() if kernel_scale is not None else None
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
+    lib = _lib.load()
+    ws, ws_bytes = None, 0
+    if M <= SKINNY_MAX_ROWS:
+        ws = _workspace(a.device, lib.k3q_gemm_i8_workspace_bytes(M, N, K))
+        ws_bytes = ws.numel()
+    rc = lib.k3q_gemm_i8(
+        _lib.ptr(a), _lib.ptr(b), 1, M, N, K, _lib.ptr(sa), _lib.ptr(sb), None, code,
+        (GEMM_EXACT_EPILOGUE if exact_epilogue else 0)
+        | (GEMM_ROUND_ACC_BF16 if round_acc_bf16 else 0),
+        _lib.ptr(y), _lib.ptr(acc), _lib.ptr(ws), ws_bytes, _lib.stream_ptr(a.device),
+    )
+    _lib.check(rc, "k3q_gemm_i8")
+    return (y, acc) if want_acc else y
+
+
+def embedding_lookup(ids, table, scale, dim, bits=8, zero=None, block_size=None,
+                     out_dtype=None, check_ids=True):
+    """Rows `ids` of a quantized embedding table, de-quantised.
+
+    table: int8 [vocab, dim] (bits=8) or packed int4 [vocab, ceil(dim/2)] (bits=4).
+    scale: [vocab], or [vocab, groups] with `zero` int8 of the same shape for grouped int4.
+    out_dtype: the dtype the reference's chain ends in, i.e. the promotion of the compute
+    dtype and the scale dtype; bfloat16 only with bfloat16 scales.
+    check_ids: raise IndexError for ids outside [-vocab, vocab) as the reference does
+    (reads a flag back from the device, i.e. synchronises); without it such ids give rows of
+    zeros.  Reference: keras/src/layers/core/embedding.py:521-582.
+    """
+    _lib.require_device(ids, table, scale, zero)
+    if ids.dtype not in (torch.int32, torch.int64):
+        ids = ids.to(torch.int32)
+    ids = ids if ids.is_contiguous() else ids.contiguous()
+    if table.dtype != torch.int8 or table.dim() != 2:
+        raise TypeError("the embedding table must be a 2-D int8 tensor")
+    vocab = table.shape[0]
+    want_cols = dim if bits == 8 else (dim + 1) // 2
+    if table.shape[1] != want_cols:
+        raise ValueError(f"table has {table.shape[1]} columns, expected {want_cols}")
+    grouped = block_size is not None and block_size > 0
+    if out_dtype is None:
+        out_dtype = scale.dtype
+    if out_dtype == torch.bfloat16 and scale.dtype != torch.bfloat16:
+        raise TypeError("float32 scales promote the result to float32")
+    table = table if table.is_contiguous() else table.contiguous()
+    scale = scale if scale.is_contiguous() else scale.contiguous()
+    if grouped:
+        if zero is None:
+            raise ValueError("grouped int4 needs the zero points")
+        zero = zero if zero.is_contiguous() else zero.contiguous()
+    count = ids.numel()
+    out = torch.empty((count, dim), dtype=out_dtype, device=table.device)
+    flag = torch.zeros(1, dtype=torch.int32, device=table.device) if check_ids else None
+    rc = _lib.load().k3q_embedding_lookup(
+        _lib.ptr(ids), _lib.K3Q_I64 if ids.dtype == torch.int64 else _lib.K3Q_I32, count,
+        _lib.ptr(table), vocab, int(dim), int(bits), _lib.ptr(scale), _lib.dtype_code(scale.dtype),
+        _lib.ptr(zero) if grouped else None, int(block_size) if grouped else -1,
+        _lib.dtype_code(out_dtype), _lib.ptr(out), _lib.ptr(flag), _lib.stream_ptr(table.device),
+    )
+    _lib.check(rc, "k3q_embedding_lookup")
+    if check_ids and int(flag.item()) != 0:
+        raise IndexError("index out of range in self")
+    return out.reshape(*ids.shape, dim)

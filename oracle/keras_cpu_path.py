@@ -558,6 +558,97 @@ def einsum_dense_int4_call(inputs, qk, equation, bias=None, compute_dtype=None,
 
 
 # --------------------------------------------------------------------------
+# next rows: Embedding / ReversibleEmbedding
+# --------------------------------------------------------------------------
+def take_rows(x, indices):
+    """`ops.take(x, indices, axis=0)` for a 2-D x on the torch backend
+    (keras/src/backend/torch/numpy.py:2005-2017): negative ids wrap once, then
+    `torch.nn.functional.embedding` (which raises IndexError when out of range);
+    1-D x goes through index_select (:2021-2028)."""
+    indices = indices.long()
+    indices = torch.where(indices < 0, indices + x.shape[0], indices)
+    if x.dim() == 2:
+        if x.dtype.is_floating_point:
+            return torch.nn.functional.embedding(indices, x)
+        return x[indices]  # F.embedding rejects integer tables on some builds; same gather
+    return torch.index_select(x, 0, indices.ravel()).reshape(indices.shape)
+
+
+def embedding_quantize_int8(embeddings):
+    """keras/src/layers/core/embedding.py:595-612 -> (int8 [V,D], scale [V])."""
+    q, s = AbsMaxQuantizer(axis=-1)(embeddings, to_numpy=True)
+    return q, torch.squeeze(s, dim=-1)
+
+
+def embedding_quantize_int4(embeddings, block_size=128):
+    """keras/src/layers/core/embedding.py:613-668.  Returns dict(embeddings=packed int8
+    [V, ceil(D/2)], embeddings_scale [V] | [V,G], embeddings_zero [V,G] | None, g_idx [D] |
+    None, unpacked int8 [V,D])."""
+    V, D = embeddings.shape
+    if block_size is None or block_size == -1:
+        q, s = AbsMaxQuantizer(axis=-1, value_range=(-8, 7))(embeddings, to_numpy=True)
+        s = torch.squeeze(s, dim=-1)
+        zero = None
+        g_idx = None
+    else:
+        q_t, s_t, z_t = abs_max_quantize_grouped_with_zero_point(
+            torch.transpose(embeddings, 0, 1), block_size=block_size
+        )
+        q = torch.transpose(q_t, 0, 1)
+        s = torch.transpose(s_t, 0, 1)
+        zero = torch.transpose(z_t, 0, 1)
+        # embedding.py:500-516: float32 floor(arange(D) / block_size)
+        g_idx = torch.floor_divide(torch.arange(D, dtype=torch.float32), block_size)
+    packed, _, _ = pack_int4(q, axis=-1)
+    return dict(embeddings=packed, embeddings_scale=s, embeddings_zero=zero, g_idx=g_idx,
+                unpacked=q)
+
+
+def embedding_int8_call(ids, embeddings, embeddings_scale, compute_dtype="float32"):
+    """keras/src/layers/core/embedding.py:521-541 (no LoRA).  The layer sets
+    `autocast = False` (:132), so the scale is read in its own dtype and torch's type
+    promotion decides the result dtype."""
+    cd = _tdtype(compute_dtype)
+    scale = take_rows(embeddings_scale, ids)
+    outputs = take_rows(embeddings, ids)
+    return torch.divide(outputs.to(cd), torch.unsqueeze(scale, -1))
+
+
+def embedding_int4_call(ids, embeddings, embeddings_scale, orig_output_dim,
+                        embeddings_zero=None, g_idx=None, block_size=None,
+                        compute_dtype="float32"):
+    """keras/src/layers/core/embedding.py:542-582 (no LoRA)."""
+    cd = _tdtype(compute_dtype)
+    unpacked = unpack_int4(embeddings, orig_output_dim, axis=-1)
+    outputs = take_rows(unpacked, ids)
+    if block_size is None or block_size == -1:
+        scale = take_rows(embeddings_scale, ids)
+        return torch.divide(outputs.to(cd), torch.unsqueeze(scale, -1))
+    scale = take_rows(embeddings_scale, ids)
+    zero = take_rows(embeddings_zero, ids)
+    return dequantize_with_sz_map(outputs.to(cd), scale, zero, g_idx, group_axis=-1)
+
+
+def reversible_embedding_int8_reverse(inputs, embeddings, embeddings_scale,
+                                      compute_dtype=None, logit_soft_cap=None,
+                                      return_intermediates=False):
+    """keras/src/layers/core/reversible_embedding.py:272-296 with tied weights:
+    kernel = transpose(embeddings [V,D]), scale = transpose(scale [V]) (a no-op on 1-D)."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    kernel = torch.transpose(embeddings, 0, 1)
+    q, s_in = AbsMaxQuantizer(axis=-1)(inputs)
+    acc = matmul(q, kernel)
+    logits = acc.to(cd)
+    logits = torch.divide(logits, torch.multiply(s_in, embeddings_scale))
+    if logit_soft_cap is not None:
+        logits = torch.multiply(torch.tanh(torch.divide(logits, logit_soft_cap)), logit_soft_cap)
+    if return_intermediates:
+        return logits, dict(q=q, inputs_scale=s_in, acc=acc)
+    return logits
+
+
+# --------------------------------------------------------------------------
 # helpers shared by tests / bench (input generators named in the configs)
 # --------------------------------------------------------------------------
 def glorot_uniform(fan_in, fan_out, shape=None, generator=None):

@@ -1,0 +1,250 @@
+"""GPU parity: quantized Embedding lookup, ReversibleEmbedding reverse projection and the
+[N, K]-layout int8 matmul, through the C ABI, against the CPU oracle."""
+
+import pytest
+import torch
+
+from keras_amd import ops as kops
+from keras_amd.layers import Embedding, ReversibleEmbedding
+from keras_amd.quantization_config import Int4QuantizationConfig
+from oracle import keras_cpu_path as ref
+from tests.helpers import RTOL, c_gemm_i8, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def bits(t):
+    return t.view(torch.int16) if t.dtype == torch.bfloat16 else t.view(torch.int32)
+
+
+def table(V, D, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.rand(V, D, generator=g) * 2.0 - 1.0) * 0.05
+
+
+def some_ids(V, shape, seed, dtype=torch.int64):
+    ids = torch.randint(-V, V, shape, generator=torch.Generator().manual_seed(seed))
+    flat = ids.view(-1)
+    flat[0], flat[-1] = V - 1, -V  # both ends of the valid range
+    return ids.to(dtype)
+
+
+# ---- k3q_embedding_lookup ----------------------------------------------------------------
+@pytest.mark.parametrize("scale_dtype,out_dtype", [(torch.float32, torch.float32),
+                                                   (torch.bfloat16, torch.bfloat16),
+                                                   (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("V,D", [(1000, 4096), (37, 64), (50, 48), (9, 33), (5, 1)])
+@pytest.mark.parametrize("ids_dtype", [torch.int32, torch.int64])
+def test_lookup_int8(dev, scale_dtype, out_dtype, V, D, ids_dtype):
+    q, s = ref.embedding_quantize_int8(table(V, D))
+    s = s.to(scale_dtype)
+    ids = some_ids(V, (3, 17), seed=1, dtype=ids_dtype)
+    cd = "bfloat16" if out_dtype == torch.bfloat16 or scale_dtype == torch.bfloat16 else "float32"
+    if scale_dtype == torch.bfloat16 and out_dtype == torch.float32:
+        cd = "float32"  # float32 compute with a bfloat16 scale variable
+    want = ref.embedding_int8_call(ids, q, s, compute_dtype=cd)
+    assert want.dtype == out_dtype
+    got = kops.embedding_lookup(ids.to(dev), q.to(dev), s.to(dev), D, bits=8, out_dtype=out_dtype)
+    assert got.dtype == out_dtype and tuple(got.shape) == (3, 17, D)
+    assert torch.equal(bits(got.cpu()), bits(want))
+
+
+@pytest.mark.parametrize("scale_dtype,out_dtype", [(torch.float32, torch.float32),
+                                                   (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("V,D,block", [(500, 4096, 128), (500, 4096, None), (40, 256, 64),
+                                       (40, 256, -1), (11, 96, 32), (11, 100, 20), (7, 33, 8),
+                                       (7, 33, None), (10, 16, 4)])
+def test_lookup_int4(dev, scale_dtype, out_dtype, V, D, block):
+    qd = ref.embedding_quantize_int4(table(V, D, seed=2), block_size=block)
+    s = qd["embeddings_scale"].to(scale_dtype)
+    ids = some_ids(V, (29,), seed=3)
+    cd = "bfloat16" if out_dtype == torch.bfloat16 else "float32"
+    want = ref.embedding_int4_call(ids, qd["embeddings"], s, D, embeddings_zero=qd["embeddings_zero"],
+                                   g_idx=qd["g_idx"], block_size=block, compute_dtype=cd)
+    grouped = block is not None and block > 0
+    got = kops.embedding_lookup(
+        ids.to(dev), qd["embeddings"].to(dev), s.to(dev), D, bits=4,
+        zero=qd["embeddings_zero"].to(dev) if grouped else None,
+        block_size=block if grouped else None, out_dtype=out_dtype)
+    assert torch.equal(bits(got.cpu()), bits(want))
+
+
+def test_lookup_out_of_range(dev):
+    q, s = ref.embedding_quantize_int8(table(10, 32))
+    qd, sd = q.to(dev), s.to(dev)
+    for bad in (10, -11, 1 << 40):
+        ids = torch.tensor([1, bad, 2], device=dev)
+        with pytest.raises(IndexError):
+            kops.embedding_lookup(ids, qd, sd, 32)
+        out = kops.embedding_lookup(ids, qd, sd, 32, check_ids=False)
+        want = ref.embedding_int8_call(torch.tensor([1, 2]), q, s)
+        assert torch.equal(out[[0, 2]].cpu(), want)
+        assert torch.count_nonzero(out[1]).item() == 0
+    assert kops.embedding_lookup(torch.zeros((0,), dtype=torch.int64, device=dev), qd, sd, 32).shape == (0, 32)
+    with pytest.raises(RuntimeError):
+        kops.embedding_lookup(torch.tensor([1]), q, s, 32)  # host tensors: no CPU path
+
+
+# ---- int8 matmul with an [N, K] kernel -----------------------------------------------------
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,K,N", [(1, 4096, 32000), (8, 4096, 32000), (16, 256, 1000),
+                                   (5, 4096, 64), (3, 64, 7), (17, 512, 333), (64, 1024, 2048),
+                                   (40, 128, 50), (300, 256, 1000), (65, 4096, 512)])
+def test_int8_matmul_nk(dev, out_dtype, M, K, N):
+    g = torch.Generator().manual_seed(M * 7 + N)
+    a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    sa = (torch.rand(M, generator=g) * 50 + 1).to(out_dtype)
+    sb = (torch.rand(N, generator=g) * 50 + 1).to(out_dtype)
+    y, acc = kops.int8_matmul_nk(a.to(dev), b.to(dev), a_scale=sa.to(dev), kernel_scale=sb.to(dev),
+                                 out_dtype=out_dtype, exact_epilogue=True, want_acc=True)
+    want_acc = c_gemm_i8(a, b.t().contiguous())
+    assert torch.equal(acc.cpu(), want_acc)
+    want = torch.divide(want_acc.to(out_dtype), torch.multiply(sa.unsqueeze(-1), sb))
+    assert torch.equal(bits(y.cpu()), bits(want))
+
+
+def test_int8_matmul_nk_round_acc(dev):
+    g = torch.Generator().manual_seed(5)
+    for M, K, N in [(4, 4096, 1000), (200, 256, 512)]:
+        a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+        b = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+        sa = (torch.rand(M, generator=g) * 50 + 1).to(torch.bfloat16).float()
+        sb = torch.rand(N, generator=g) * 50 + 1
+        y = kops.int8_matmul_nk(a.to(dev), b.to(dev), a_scale=sa.to(dev), kernel_scale=sb.to(dev),
+                                out_dtype=torch.float32, exact_epilogue=True, round_acc_bf16=True)
+        acc = c_gemm_i8(a, b.t().contiguous())
+        want = torch.divide(acc.to(torch.bfloat16), torch.multiply(sa.unsqueeze(-1), sb))
+        assert want.dtype == torch.float32
+        assert torch.equal(y.cpu(), want)
+
+
+# ---- layers -----------------------------------------------------------------------------------
+def build_embedding(cls, dev, V, D, policy, seed, **kw):
+    g = torch.Generator().manual_seed(seed)
+    layer = cls(V, D, dtype=policy, device=dev,
+                embeddings_initializer=lambda s, d: ((torch.rand(s, generator=g) * 2 - 1) * 0.05).to(d), **kw)
+    layer.build()
+    return layer
+
+
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16", "bfloat16"])
+@pytest.mark.parametrize("V,D", [(10, 16), (100, 256), (1000, 4096)])
+def test_embedding_int8_layer(dev, policy, V, D):
+    layer = build_embedding(Embedding, dev, V, D, policy, seed=0)
+    t = layer._embeddings.value.cpu()
+    ids = torch.randint(0, V - 1, (64, 3), generator=torch.Generator().manual_seed(1))
+    y_float = layer(ids)
+    layer.quantize("int8")
+    assert layer.dtype_policy.name == f"int8_from_{policy}"
+    assert layer._embeddings.dtype == "int8" and layer.embeddings_scale.dtype == layer.variable_dtype
+    q, s = ref.embedding_quantize_int8(t)
+    assert torch.equal(layer._embeddings.value.cpu(), q)
+    assert torch.equal(bits(layer.embeddings_scale.value.cpu()), bits(s))
+    y = layer(ids)
+    want = ref.embedding_int8_call(ids, q, s, compute_dtype=layer.compute_dtype)
+    assert y.dtype == want.dtype and torch.equal(bits(y.cpu()), bits(want))
+    # embedding_test.py:364-394
+    assert (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item() < 1e-3
+    with pytest.raises(ValueError):
+        layer.quantize("int8")
+    store = {}
+    layer.save_own_variables(store)
+    assert sorted(store) == ["0", "1"]
+    clone = Embedding(V, D, dtype=layer.dtype_policy.name, device=dev)
+    clone.build()
+    clone.load_own_variables(store)
+    assert torch.equal(bits(clone(ids).cpu()), bits(want))
+
+
+@pytest.mark.parametrize("policy", ["float32", "bfloat16"])
+@pytest.mark.parametrize("block_size", [128, 64, 8, None, -1])
+@pytest.mark.parametrize("V,D", [(10, 16), (100, 256), (300, 4096)])
+def test_embedding_int4_layer(dev, policy, block_size, V, D):
+    layer = build_embedding(Embedding, dev, V, D, policy, seed=2)
+    t = layer._embeddings.value.cpu()
+    ids = torch.randint(0, V, (4, 8), generator=torch.Generator().manual_seed(3))
+    y_float = layer(ids)
+    layer.quantize("int4", config=Int4QuantizationConfig(block_size=block_size))
+    assert layer._int4_block_size == block_size
+    bs_name = -1 if block_size is None else block_size
+    assert layer.dtype_policy.name == f"int4/{bs_name}_from_{policy}"
+    qd = ref.embedding_quantize_int4(t, block_size=block_size)
+    assert torch.equal(layer._embeddings.value.cpu(), qd["embeddings"])
+    assert torch.equal(bits(layer.embeddings_scale.value.cpu()), bits(qd["embeddings_scale"]))
+    grouped = block_size is not None and block_size > 0
+    if grouped:
+        assert torch.equal(layer.embeddings_zero.value.cpu(), qd["embeddings_zero"])
+        assert torch.equal(layer.g_idx.value.cpu(), qd["g_idx"]) and layer.g_idx.dtype == "float32"
+    else:
+        assert not hasattr(layer, "g_idx") and not hasattr(layer, "embeddings_zero")
+    assert torch.equal(layer.embeddings.cpu(), qd["unpacked"])
+    y = layer(ids)
+    want = ref.embedding_int4_call(ids, qd["embeddings"], qd["embeddings_scale"], D,
+                                   embeddings_zero=qd["embeddings_zero"], g_idx=qd["g_idx"],
+                                   block_size=block_size, compute_dtype=layer.compute_dtype)
+    assert y.dtype == want.dtype and torch.equal(bits(y.cpu()), bits(want))
+    assert (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item() < 1e-3
+    store = {}
+    layer.save_own_variables(store)
+    assert len(store) == (4 if grouped else 2)
+
+
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16", "bfloat16"])
+@pytest.mark.parametrize("M,V,D", [(1, 32000, 4096), (8, 32000, 4096), (16, 1000, 256),
+                                   (300, 1000, 256), (5, 77, 64)])
+def test_reversible_embedding_int8_tied(dev, policy, M, V, D):
+    layer = build_embedding(ReversibleEmbedding, dev, V, D, policy, seed=4)
+    t = layer._embeddings.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(5))
+    y_float = layer(x, reverse=True)
+    layer.quantize("int8")
+    q, s = ref.embedding_quantize_int8(t)
+    assert torch.equal(layer._embeddings.value.cpu(), q)
+    layer.exact_epilogue = True
+    y = layer(x, reverse=True)
+    want = ref.reversible_embedding_int8_reverse(x.to(cd), q, s.to(TORCH[layer.variable_dtype]),
+                                                 compute_dtype=cd)
+    assert y.dtype == want.dtype and tuple(y.shape) == (M, V)
+    assert torch.equal(bits(y.cpu()), bits(want))
+    layer.exact_epilogue = False
+    assert max_rel_err(layer(x, reverse=True), want) <= RTOL[cd]
+    err = (y_float.float().cpu() - y.float().cpu()).abs().max().item()
+    assert err <= 0.05 * y_float.float().abs().max().item() + 1e-3
+    # the forward lookup of the same layer still works
+    ids = torch.randint(0, V, (2, 5), generator=torch.Generator().manual_seed(6))
+    assert torch.equal(bits(layer(ids).cpu()),
+                       bits(ref.embedding_int8_call(ids, q, s, compute_dtype=layer.compute_dtype)))
+
+
+@pytest.mark.parametrize("M", [4, 100])
+def test_reversible_embedding_int8_untied_and_soft_cap(dev, M):
+    V, D = 512, 128
+    layer = build_embedding(ReversibleEmbedding, dev, V, D, "float32", seed=7, tie_weights=False,
+                            logit_soft_cap=0.3)
+    rt = layer.reverse_embeddings.value.cpu()
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(8))
+    layer.quantize("int8")
+    assert layer.reverse_embeddings.dtype == "int8" and layer.reverse_embeddings.shape == (D, V)
+    rq, rs = ref.dense_quantize_int8(rt)  # AbsMaxQuantizer(axis=0) on [D, V], as Dense does
+    assert torch.equal(layer.reverse_embeddings.value.cpu(), rq)
+    layer.exact_epilogue = True
+    y = layer(x, reverse=True)
+    logits = ref.dense_int8_call(x, rq, rs)
+    want = torch.multiply(torch.tanh(torch.divide(logits, 0.3)), 0.3)
+    assert torch.allclose(y.cpu(), want, rtol=1e-6, atol=1e-7)
+    store = {}
+    layer.save_own_variables(store)
+    assert len(store) == 4
+
+
+def test_reversible_embedding_int4_reverse_raises(dev):
+    layer = build_embedding(ReversibleEmbedding, dev, 64, 32, "float32", seed=9)
+    layer.quantize("int4")
+    ids = torch.tensor([1, 2, 3])
+    assert layer(ids).shape == (3, 32)
+    with pytest.raises(NotImplementedError):
+        layer(torch.randn(2, 32), reverse=True)

@@ -1,0 +1,146 @@
+"""CPU: pins for the Embedding / ReversibleEmbedding functions of the oracle.
+
+The functions compose primitives that tests/test_oracle.py already pins (abs-max quantizer,
+pack / unpack, the grouped quantizer, the int8 matmul); what is checked here is the
+composition: which axis is reduced, which scale meets which row, multiply versus divide,
+the nibble order along the output dim -- each against plain Python loops on small tables,
+plus the reference's own property tests (embedding_test.py:364-394, :793-824, :921-941).
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import keras_cpu_path as ref
+
+
+def table(V, D, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.rand(V, D, generator=g) * 2.0 - 1.0) * 0.05  # keras "uniform" initializer
+
+
+def test_int8_table_quantization_and_lookup_by_loops():
+    V, D = 7, 12
+    t = table(V, D)
+    q, s = ref.embedding_quantize_int8(t)
+    assert q.dtype == torch.int8 and tuple(s.shape) == (V,)
+    tn = t.numpy()
+    for v in range(V):
+        amax = np.abs(tn[v]).max()
+        sc = np.float32(127.0) / (np.float32(amax) + np.float32(1e-7))
+        assert s[v].item() == pytest.approx(float(sc), rel=1e-6)
+        for d in range(D):
+            want = int(np.clip(np.round(np.float32(tn[v, d]) * sc), -127, 127))
+            assert q[v, d].item() == want
+    ids = torch.tensor([[0, 6], [3, -1]])  # -1 wraps to the last row
+    out = ref.embedding_int8_call(ids, q, s)
+    assert tuple(out.shape) == (2, 2, D) and out.dtype == torch.float32
+    for (i, j), v in {(0, 0): 0, (0, 1): 6, (1, 0): 3, (1, 1): V - 1}.items():
+        for d in range(D):
+            assert out[i, j, d].item() == np.float32(q[v, d].item()) / np.float32(s[v].item())
+
+
+@pytest.mark.parametrize("block_size", [None, 4, 8])
+def test_int4_table_by_loops(block_size):
+    V, D = 6, 16
+    t = table(V, D, seed=1)
+    qd = ref.embedding_quantize_int4(t, block_size=block_size)
+    packed, unpacked = qd["embeddings"], qd["unpacked"]
+    assert tuple(packed.shape) == (V, D // 2)
+    # nibble order along the output dim: low nibble = even column
+    for v in range(V):
+        for j in range(D // 2):
+            byte = packed[v, j].item() & 0xFF
+            lo, hi = byte & 0xF, byte >> 4
+            assert ((lo ^ 8) - 8) == unpacked[v, 2 * j].item()
+            assert ((hi ^ 8) - 8) == unpacked[v, 2 * j + 1].item()
+    ids = torch.tensor([5, 0, 2])
+    out = ref.embedding_int4_call(ids, packed, qd["embeddings_scale"], D,
+                                  embeddings_zero=qd["embeddings_zero"], g_idx=qd["g_idx"],
+                                  block_size=block_size)
+    if block_size is None:
+        assert tuple(qd["embeddings_scale"].shape) == (V,)
+        for r, v in enumerate(ids.tolist()):
+            for d in range(D):
+                want = np.float32(unpacked[v, d].item()) / np.float32(qd["embeddings_scale"][v].item())
+                assert out[r, d].item() == want
+    else:
+        G = math.ceil(D / block_size)
+        assert tuple(qd["embeddings_scale"].shape) == (V, G)
+        assert tuple(qd["embeddings_zero"].shape) == (V, G) and qd["embeddings_zero"].dtype == torch.int8
+        # embedding_test.py:921-941
+        assert torch.equal(qd["g_idx"], torch.tensor(np.arange(D) // block_size, dtype=torch.float32))
+        for r, v in enumerate(ids.tolist()):
+            for d in range(D):
+                gi = d // block_size
+                want = (np.float32(unpacked[v, d].item()) - np.float32(qd["embeddings_zero"][v, gi].item())) \
+                    * np.float32(qd["embeddings_scale"][v, gi].item())
+                assert out[r, d].item() == want
+        # the grouped parameters are those of the group's own min / max (asymmetric)
+        tn = t.numpy()
+        for v in range(V):
+            for gi in range(G):
+                seg = tn[v, gi * block_size:(gi + 1) * block_size]
+                sc = (np.float32(seg.max()) - np.float32(seg.min()) + np.float32(1e-7)) / np.float32(15)
+                assert qd["embeddings_scale"][v, gi].item() == pytest.approx(float(sc), rel=1e-6)
+
+
+@pytest.mark.parametrize("mode,V,D,block", [("int8", 10, 16, None), ("int4", 10, 16, 128),
+                                            ("int4", 100, 256, 64), ("int4", 100, 256, None)])
+def test_reference_weak_mse_property(mode, V, D, block):
+    # embedding_test.py:364-394 and :793-824: mean squared error against the float layer < 1e-3
+    t = table(V, D, seed=2)
+    ids = torch.randint(0, V - 1, (64, 3), generator=torch.Generator().manual_seed(3))
+    y_float = t[ids]
+    if mode == "int8":
+        q, s = ref.embedding_quantize_int8(t)
+        y = ref.embedding_int8_call(ids, q, s)
+    else:
+        qd = ref.embedding_quantize_int4(t, block_size=block)
+        y = ref.embedding_int4_call(ids, qd["embeddings"], qd["embeddings_scale"], D,
+                                    embeddings_zero=qd["embeddings_zero"], g_idx=qd["g_idx"],
+                                    block_size=block)
+    assert (y_float - y).pow(2).mean().item() < 1e-3
+
+
+def test_lookup_dtype_promotion_without_autocast():
+    # bfloat16 compute, float32 scale variable (the layer does not autocast): float32 out
+    t = table(5, 8, seed=4)
+    q, s = ref.embedding_quantize_int8(t)
+    out = ref.embedding_int8_call(torch.tensor([1, 2]), q, s, compute_dtype="bfloat16")
+    assert out.dtype == torch.float32
+    assert torch.equal(out, q[[1, 2]].float() / s[[1, 2]].unsqueeze(-1))
+    out_bf = ref.embedding_int8_call(torch.tensor([1, 2]), q, s.to(torch.bfloat16), compute_dtype="bfloat16")
+    assert out_bf.dtype == torch.bfloat16
+
+
+def test_out_of_range_ids_raise():
+    t = table(5, 8)
+    q, s = ref.embedding_quantize_int8(t)
+    with pytest.raises(IndexError):
+        ref.embedding_int8_call(torch.tensor([5]), q, s)
+    with pytest.raises(IndexError):
+        ref.embedding_int8_call(torch.tensor([-6]), q, s)
+
+
+def test_reverse_projection_tied_int8_closed_form():
+    V, D, M = 9, 32, 3
+    t = table(V, D, seed=5)
+    q, s = ref.embedding_quantize_int8(t)
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(6))
+    logits, inter = ref.reversible_embedding_int8_reverse(x, q, s, return_intermediates=True)
+    assert tuple(logits.shape) == (M, V)
+    xq, xs = inter["q"], inter["inputs_scale"]
+    for m in range(M):
+        for v in range(V):
+            acc = sum(int(xq[m, d]) * int(q[v, d]) for d in range(D))
+            assert inter["acc"][m, v].item() == acc
+            want = np.float32(acc) / (np.float32(xs[m, 0].item()) * np.float32(s[v].item()))
+            assert logits[m, v].item() == want
+    # and it approximates the float projection
+    want_f = x @ t.T
+    assert (logits - want_f).abs().max().item() < 0.05 * want_f.abs().max().item() + 1e-3
+    capped = ref.reversible_embedding_int8_reverse(x, q, s, logit_soft_cap=0.5)
+    assert torch.allclose(capped, torch.tanh(logits / 0.5) * 0.5)
