@@ -27,6 +27,7 @@ struct EmbParams {
     void* out;
     int* oob_flag;
     int64_t count, vocab, dim, row_bytes, groups, block_size;
+    int64_t parts, part_pieces;  // waves per row and 16-byte output pieces per wave (vector kernel)
 };
 
 template <bool kBF16>
@@ -44,29 +45,6 @@ __device__ __forceinline__ float dequant(float q, float s, float z, bool grouped
     return kOutBF16 ? round_bf16(q / s) : q / s;
 }
 
-template <bool kOutBF16>
-__device__ __forceinline__ void store16(void* out, int64_t first, const float* v) {
-    // 16 consecutive outputs starting at element `first` (a multiple of 16)
-    if (kOutBF16) {
-        v4u o[2];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-                o[h][d] = f32_to_bf16_bits(v[8 * h + 2 * d]) | (f32_to_bf16_bits(v[8 * h + 2 * d + 1]) << 16);
-        v4u* dst = (v4u*)((uint16_t*)out + first);
-        __builtin_nontemporal_store(o[0], dst);
-        __builtin_nontemporal_store(o[1], dst + 1);
-    } else {
-        v4f* dst = (v4f*)((float*)out + first);
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-            v4f o = {v[4 * h], v[4 * h + 1], v[4 * h + 2], v[4 * h + 3]};
-            __builtin_nontemporal_store(o, dst + h);
-        }
-    }
-}
-
 template <typename IdT>
 __device__ __forceinline__ int64_t row_of(const EmbParams& p, int64_t t, bool* ok) {
     int64_t r = (int64_t)((const IdT*)p.ids)[t];
@@ -79,66 +57,76 @@ __device__ __forceinline__ int64_t row_of(const EmbParams& p, int64_t t, bool* o
     return r;
 }
 
-// One wave per token, 16-byte pieces of the table row per lane.  kBits == 8: dim % 16 == 0;
-// kBits == 4: dim % 32 == 0 (so that a piece is 32 whole columns) and, grouped,
-// block_size % 32 == 0 (a piece never straddles a group).
+// One wave per token.  A lane's piece is whatever de-quantises to one 16-byte store (4
+// float32 or 8 bfloat16 outputs, i.e. 2..8 bytes of the table row), so that consecutive
+// lanes read consecutive table bytes and every store instruction of the wave writes 1 KiB
+// of contiguous output.  Needs dim % piece == 0 and, grouped, block_size % piece == 0.
 template <int kBits, bool kScaleBF16, bool kOutBF16, bool kGrouped, typename IdT>
 __global__ __launch_bounds__(256) void embedding_rows(EmbParams p) {
+    constexpr int kOut = kOutBF16 ? 8 : 4;       // outputs per piece
+    constexpr int kIn = kOut * kBits / 8;        // table bytes per piece: 8, 4 or 2
+    constexpr int kUnroll = 4;
     const int lane = threadIdx.x & 63;
-    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    // a row is shared by p.parts waves (more than one only when there are few tokens)
+    const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t t = wid / p.parts;
     if (t >= p.count) return;
     bool ok;
     const int64_t row = row_of<IdT>(p, t, &ok);
-    const v4u* src = (const v4u*)(p.table + row * p.row_bytes);
-    const int64_t pieces = p.row_bytes / 16;
-    constexpr int kPerPiece = kBits == 8 ? 16 : 32;
+    const char* src = (const char*)p.table + row * p.row_bytes;
+    const int64_t first = (wid - t * p.parts) * p.part_pieces;
+    int64_t pieces = first + p.part_pieces;
+    if (pieces > p.dim / kOut) pieces = p.dim / kOut;
     float s_row = 1.0f;
     if (!kGrouped) s_row = scale_at<kScaleBF16>(p.scale, row);
-    for (int64_t c0 = 0; c0 < pieces; c0 += 256) {
-        // up to four pieces in flight per lane
-        v4u w[4];
+    for (int64_t c0 = first; c0 < pieces; c0 += 64 * kUnroll) {
+        uint64_t w[kUnroll];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kUnroll; ++u) {
             const int64_t c = c0 + 64 * u + lane;
-            if (c < pieces) w[u] = __builtin_nontemporal_load(src + c);
+            w[u] = 0;
+            if (c < pieces) {
+                if (kIn == 8)
+                    w[u] = __builtin_nontemporal_load((const uint64_t*)(src + c * 8));
+                else if (kIn == 4)
+                    w[u] = __builtin_nontemporal_load((const u32*)(src + c * 4));
+                else
+                    w[u] = __builtin_nontemporal_load((const uint16_t*)(src + c * 2));
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kUnroll; ++u) {
             const int64_t c = c0 + 64 * u + lane;
             if (c >= pieces) continue;
-            const int64_t col = c * kPerPiece;
+            const int64_t col = c * kOut;
             float s = s_row, z = 0.0f;
             if (kGrouped) {
                 const int64_t gi = row * p.groups + col / p.block_size;
                 s = scale_at<kScaleBF16>(p.scale, gi);
                 z = (float)p.zero[gi];
             }
-            float v[kPerPiece];
+            float v[kOut];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                const u32 word = ok ? w[u][d] : 0u;
+            for (int e = 0; e < kOut; ++e) {
+                float q;
                 if (kBits == 8) {
-#pragma unroll
-                    for (int b = 0; b < 4; ++b)
-                        v[4 * d + b] = (float)(int)(int8_t)(word >> (8 * b));
+                    q = (float)(int)(int8_t)(w[u] >> (8 * e));
                 } else {
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        const u32 byte = (word >> (8 * b)) & 0xffu;
-                        v[8 * d + 2 * b] = (float)((int)((byte & 0xfu) ^ 8u) - 8);
-                        v[8 * d + 2 * b + 1] = (float)((int)((byte >> 4) ^ 8u) - 8);
-                    }
+                    const u32 nib = (u32)(w[u] >> (4 * e)) & 0xfu;  // low nibble = even column
+                    q = (float)((int)(nib ^ 8u) - 8);
                 }
+                v[e] = ok ? dequant<kOutBF16>(q, s, z, kGrouped) : 0.0f;
             }
-            if (ok) {
+            if (kOutBF16) {
+                v4u o;
 #pragma unroll
-                for (int e = 0; e < kPerPiece; ++e) v[e] = dequant<kOutBF16>(v[e], s, z, kGrouped);
+                for (int d = 0; d < 4; ++d)
+                    o[d] = f32_to_bf16_bits(v[2 * d]) | (f32_to_bf16_bits(v[2 * d + 1]) << 16);
+                __builtin_nontemporal_store(o, (v4u*)((uint16_t*)p.out + t * p.dim + col));
             } else {
-#pragma unroll
-                for (int e = 0; e < kPerPiece; ++e) v[e] = 0.0f;
+                v4f o = {v[0], v[1], v[2], v[3]};
+                __builtin_nontemporal_store(o, (v4f*)((float*)p.out + t * p.dim + col));
             }
-            store16<kOutBF16>(p.out, t * p.dim + col, v);
-            if (kBits == 4) store16<kOutBF16>(p.out, t * p.dim + col + 16, v + 16);
         }
     }
 }
@@ -178,8 +166,15 @@ __global__ __launch_bounds__(256) void embedding_generic(EmbParams p) {
 template <int kBits, bool kScaleBF16, bool kOutBF16, bool kGrouped, typename IdT>
 void launch(const EmbParams& p, bool vec, hipStream_t s) {
     if (vec) {
+        // few tokens (decode): spread each row over several waves, down to 64 pieces a wave
+        EmbParams q = p;
+        const int64_t pieces = p.dim / (kOutBF16 ? 8 : 4);
+        int64_t parts = 1;
+        while (p.count * parts < 2048 && pieces / (parts * 2) >= 64) parts *= 2;
+        q.parts = parts;
+        q.part_pieces = ((pieces + parts - 1) / parts + 63) / 64 * 64;
         embedding_rows<kBits, kScaleBF16, kOutBF16, kGrouped, IdT>
-            <<<(unsigned)((p.count + 3) / 4), 256, 0, s>>>(p);
+            <<<(unsigned)((p.count * parts + 3) / 4), 256, 0, s>>>(q);
     } else {
         // grid.y is limited to 65535 tokens per launch
         for (int64_t t0 = 0; t0 < p.count; t0 += 65535) {
@@ -256,9 +251,10 @@ extern "C" int k3q_embedding_lookup(const void* ids, int ids_dtype, int64_t coun
     p.row_bytes = bits == 8 ? dim : (dim + 1) / 2;
     p.block_size = grouped ? block_size : 0;
     p.groups = grouped ? (dim + block_size - 1) / block_size : 0;
-    const int per_piece = bits == 8 ? 16 : 32;
-    const bool vec = (dim % per_piece) == 0 && aligned_to(table, 16) && aligned_to(out, 16) &&
-                     (!grouped || (block_size % 32) == 0);
+    // a piece is one 16-byte store: 4 float32 or 8 bfloat16 outputs
+    const int piece = out_dtype == K3Q_BF16 ? 8 : 4;
+    const bool vec = (dim % piece) == 0 && aligned_to(table, 8) && aligned_to(out, 16) &&
+                     (!grouped || (block_size % piece) == 0);
     hipStream_t s = (hipStream_t)stream;
     if (bits == 8)
         launch_types<8, false>(p, ids_dtype, scale_dtype, out_dtype, vec, s);

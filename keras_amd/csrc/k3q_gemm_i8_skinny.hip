@@ -268,27 +268,49 @@ __global__ __launch_bounds__(256) void gemm_i8_skinny_nk(SkinnyParams p) {
 #pragma unroll
     for (int t = 0; t < kTiles; ++t) acc[t] = v4i{0, 0, 0, 0};
 
-    for (int64_t k0 = k_begin; k0 < k_end; k0 += 64 * kNkUnroll) {
-        v4u wv[kNkUnroll][kTiles], xv[kNkUnroll];
+    // two register buffers of kNkUnroll steps each: the next batch is requested before the
+    // current one is consumed, so a wave always has loads in flight
+    v4u wv[2][kNkUnroll][kTiles], xv[2][kNkUnroll];
+    constexpr int64_t kBatch = 64 * kNkUnroll;
+    auto load_batch = [&](int b, int64_t k0) {
 #pragma unroll
         for (int u = 0; u < kNkUnroll; ++u) {
             // steps past the slice end re-read the last valid step and meet a zero x operand
             const int64_t k = k0 + 64 * u < k_end ? k0 + 64 * u : k_end - 64;
 #pragma unroll
             for (int t = 0; t < kTiles; ++t)
-                wv[u][t] = __builtin_nontemporal_load((const v4u*)(wrow[t] + k));
-            xv[u] = *(const v4u*)(xrow + k);
+                wv[b][u][t] = __builtin_nontemporal_load((const v4u*)(wrow[t] + k));
+            xv[b][u] = *(const v4u*)(xrow + k);
         }
+    };
+    auto compute_batch = [&](int b, int64_t k0) {
 #pragma unroll
         for (int u = 0; u < kNkUnroll; ++u) {
             const u32 m = k0 + 64 * u < k_end ? xmask : 0u;
-            const v4u xm = {xv[u][0] & m, xv[u][1] & m, xv[u][2] & m, xv[u][3] & m};
+            const v4u xm = {xv[b][u][0] & m, xv[b][u][1] & m, xv[b][u][2] & m, xv[b][u][3] & m};
 #pragma unroll
             for (int t = 0; t < kTiles; ++t)
-                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, wv[u][t]),
-                                                               __builtin_bit_cast(v4i, xm), acc[t],
-                                                               0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                    __builtin_bit_cast(v4i, wv[b][u][t]), __builtin_bit_cast(v4i, xm), acc[t], 0, 0, 0);
         }
+    };
+    // Rows are K bytes apart, typically a multiple of every channel interleave, so waves that
+    // walk K in step would all sit on the same memory channels at the same time.  Integer
+    // sums do not care about order: each wave starts at its own batch and wraps around.
+    const int nbatch = (int)((k_end - k_begin + kBatch - 1) / kBatch);
+    const int rot = (int)(((int64_t)blockIdx.x * 4 + wave) % nbatch);
+    auto batch_k = [&](int j) {
+        int r = j + rot;
+        if (r >= nbatch) r -= nbatch;
+        return k_begin + (int64_t)r * kBatch;
+    };
+    load_batch(0, batch_k(0));
+#pragma unroll 1
+    for (int j = 0; j < nbatch; j += 2) {
+        if (j + 1 < nbatch) load_batch(1, batch_k(j + 1));
+        compute_batch(0, batch_k(j));
+        if (j + 2 < nbatch) load_batch(0, batch_k(j + 2));
+        if (j + 1 < nbatch) compute_batch(1, batch_k(j + 1));
     }
 
     // lane holds rows n0 + 16t + 4c + r (r = 0..3) of x row i
@@ -326,7 +348,7 @@ struct NkPlan {
 
 NkPlan make_nk_plan(int64_t N, int64_t K) {
     NkPlan pl{};
-    pl.tiles = N >= 16384 ? 2 : 1;
+    pl.tiles = 1;
     const int64_t waves = (N + 16 * pl.tiles - 1) / (16 * pl.tiles);
     int64_t ks = 1;
     // aim at >= 2048 waves (8 per CU), keep at least 512 bytes of K per slice
