@@ -1,0 +1,226 @@
+"""Llama-style decoder assembled from the quantizable layer mirrors: the caller of the path.
+
+Every weight matrix of the network sits in a `Dense`, `EinsumDense` or
+`ReversibleEmbedding`, so after `model.quantize("int8" | "int4")` every matmul of a
+forward pass goes through the k3q kernels; what is left to torch is glue that the
+reference also leaves to backend ops (RMS norm, rotary embedding, softmax attention over
+the KV cache, SwiGLU gating, residual adds, argmax).
+
+Shape of the network (d_model, heads, ffn, vocab, layers) follows the usual Llama layout:
+pre-norm blocks, attention projections as einsum layers `btd,dnh->btnh` / `btnh,nhd->btd`,
+a gated feed-forward of three Dense layers, tied input / output embeddings.
+"""
+
+import math
+
+import torch
+
+from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding
+from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.models import Model
+
+
+class RMSNorm(Layer):
+    def __init__(self, dim, epsilon=1e-6, dtype=None, name=None, device=None):
+        super().__init__(dtype=dtype, name=name, device=device)
+        self.dim = dim
+        self.epsilon = epsilon
+        self.build((None, dim))
+
+    def build(self, input_shape):
+        self.scale = self.add_weight(name="scale", shape=(self.dim,), initializer="ones", trainable=True)
+        self.built = True
+
+    def call(self, x, training=None):
+        xf = x.float()
+        var = xf.pow(2).mean(dim=-1, keepdim=True)
+        y = xf * torch.rsqrt(var + self.epsilon)
+        return (y * self.read(self.scale).float()).to(x.dtype)
+
+
+def rope_tables(head_dim, max_len, device, base=10000.0):
+    inv = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    ang = torch.outer(torch.arange(max_len, dtype=torch.float32), inv)
+    return torch.cos(ang).to(device), torch.sin(ang).to(device)
+
+
+def apply_rope(x, cos, sin):
+    """x [B, T, H, hd]; cos / sin [T, hd/2] for the positions of these T tokens."""
+    xf = x.float()
+    x1, x2 = xf[..., 0::2], xf[..., 1::2]
+    c, s = cos[None, :, None, :], sin[None, :, None, :]
+    out = torch.stack((x1 * c - x2 * s, x1 * s + x2 * c), dim=-1).flatten(-2)
+    return out.to(x.dtype)
+
+
+class DecoderBlock(Layer):
+    def __init__(self, d_model, n_heads, ffn_dim, dtype=None, layer_dtype=None, name=None,
+                 device=None, init=None):
+        """dtype: policy of the block and its norms; layer_dtype: policy of the
+        weight-carrying layers (a quantized policy name builds them already quantized)."""
+        super().__init__(dtype=dtype, name=name, device=device)
+        hd = d_model // n_heads
+        kw = dict(dtype=layer_dtype or dtype, device=device, kernel_initializer=init)
+        self.n_heads, self.head_dim = n_heads, hd
+        self.attn_norm = RMSNorm(d_model, dtype=dtype, device=device, name=f"{name}_attn_norm")
+        self.query = EinsumDense("btd,dnh->btnh", (None, n_heads, hd), name=f"{name}_query", **kw)
+        self.key = EinsumDense("btd,dnh->btnh", (None, n_heads, hd), name=f"{name}_key", **kw)
+        self.value = EinsumDense("btd,dnh->btnh", (None, n_heads, hd), name=f"{name}_value", **kw)
+        self.attn_out = EinsumDense("btnh,nhd->btd", (None, d_model), name=f"{name}_attn_out", **kw)
+        self.ffn_norm = RMSNorm(d_model, dtype=dtype, device=device, name=f"{name}_ffn_norm")
+        self.gate = Dense(ffn_dim, use_bias=False, name=f"{name}_ffn_gate", **kw)
+        self.up = Dense(ffn_dim, use_bias=False, name=f"{name}_ffn_up", **kw)
+        self.down = Dense(d_model, use_bias=False, name=f"{name}_ffn_down", **kw)
+        for layer in (self.query, self.key, self.value):
+            layer.build((None, None, d_model))
+        self.attn_out.build((None, None, n_heads, hd))
+        self.gate.build((None, d_model))
+        self.up.build((None, d_model))
+        self.down.build((None, ffn_dim))
+        self.built = True
+
+    def forward(self, x, cos, sin, cache, pos, mask):
+        """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
+        (an int64 device tensor [T]); mask [T, maxT] True where a key may be attended to."""
+        h = self.attn_norm(x)
+        q = apply_rope(self.query(h), cos, sin)
+        k = apply_rope(self.key(h), cos, sin)
+        v = self.value(h)
+        kc, vc = cache
+        kc.index_copy_(2, pos, k.transpose(1, 2))
+        vc.index_copy_(2, pos, v.transpose(1, 2))
+        a = torch.nn.functional.scaled_dot_product_attention(
+            q.transpose(1, 2), kc, vc, attn_mask=mask[None, None])
+        x = x + self.attn_out(a.transpose(1, 2))
+        h = self.ffn_norm(x)
+        return x + self.down(torch.nn.functional.silu(self.gate(h)) * self.up(h))
+
+
+class LlamaStyleDecoder(Model):
+    def __init__(self, vocab=32000, d_model=4096, n_heads=32, ffn_dim=14336, n_layers=32,
+                 max_len=256, dtype="bfloat16", device=None, seed=0, layer_policy=None):
+        """layer_policy: dtype-policy name for the weight-carrying layers, e.g.
+        "int4/128_from_bfloat16": the layers are then built already quantized (zero
+        weights, to be filled by `load_own_variables` or `randomize_quantized_weights`)
+        instead of being built in float and converted."""
+        super().__init__(dtype=dtype, name="llama_style_decoder", device=device)
+        self.vocab, self.d_model, self.n_heads = vocab, d_model, n_heads
+        self.head_dim = d_model // n_heads
+        self.max_len = max_len
+        gen = torch.Generator().manual_seed(seed)
+        wdtype = layer_policy or dtype
+
+        def init(shape, dt):
+            # N(0, 1/fan_in); the output projection [heads, head_dim, d_model] contracts its
+            # two leading axes, every other kernel its first
+            fan_in = shape[0] * shape[1] if len(shape) == 3 and shape[0] == n_heads else shape[0]
+            return (torch.randn(shape, generator=gen) * (1.0 / math.sqrt(fan_in))).to(dt)
+
+        self.token_embedding = ReversibleEmbedding(
+            vocab, d_model, dtype=wdtype, device=self.device, name="token_embedding",
+            embeddings_initializer=lambda s, dt: (torch.randn(s, generator=gen) * 0.02).to(dt))
+        self.token_embedding.build()
+        self.token_embedding.check_ids = False
+        self.blocks = [
+            DecoderBlock(d_model, n_heads, ffn_dim, dtype=dtype, layer_dtype=wdtype,
+                         device=self.device, name=f"block{i}", init=init)
+            for i in range(n_layers)
+        ]
+        self.final_norm = RMSNorm(d_model, dtype=dtype, device=self.device, name="final_norm")
+        self.cos, self.sin = rope_tables(self.head_dim, max_len, self.device)
+        self._graphs = {}
+
+    # ---- synthetic quantized weights ---------------------------------------------------
+    def randomize_quantized_weights(self, seed=0):
+        """Fill already-quantized layers with random int8 / packed-int4 values and plausible
+        scales, on the device (throughput runs at sizes where converting float weights on
+        the host would take minutes).  Values are not a quantisation of anything."""
+        g = torch.Generator(device=self.device).manual_seed(seed)
+        for layer in self._flatten_layers():
+            for var in getattr(layer, "_variables", []):
+                t = as_tensor(var)
+                short = var.name.rsplit("/", 1)[-1]
+                if short == "g_idx":
+                    continue
+                if t.dtype == torch.int8 and short.endswith("zero"):
+                    var.assign(torch.randint(-2, 3, t.shape, generator=g, device=self.device, dtype=torch.int8))
+                elif t.dtype == torch.int8:
+                    var.assign(torch.randint(-128, 128, t.shape, generator=g, device=self.device, dtype=torch.int8))
+                elif short.endswith("_scale"):
+                    # keep de-quantised magnitudes near 1/sqrt(fan_in) so activations stay finite
+                    grouped = (getattr(layer, "_int4_block_size", None) or -1) > 0
+                    u = torch.rand(t.shape, generator=g, device=self.device)
+                    if layer.quantization_mode == "int4" and grouped:
+                        v = u * 0.002 + 0.002       # value = (q - zero) * scale
+                    elif layer.quantization_mode == "int4":
+                        v = u * 200.0 + 300.0       # value = q / scale, |q| <= 8
+                    else:
+                        v = u * 2000.0 + 4000.0     # value = q / scale, |q| <= 127
+                    var.assign(v.to(t.dtype))
+
+    # ---- forward ---------------------------------------------------------------------------
+    def new_cache(self, batch):
+        cd = to_torch_dtype(self.compute_dtype)
+        shape = (batch, self.n_heads, self.max_len, self.head_dim)
+        return [(torch.zeros(shape, dtype=cd, device=self.device),
+                 torch.zeros(shape, dtype=cd, device=self.device)) for _ in self.blocks]
+
+    def forward(self, ids, pos, cache, last_only=True):
+        """ids [B, T] token ids at positions pos [T] (int64 device tensor) -> logits."""
+        x = self.token_embedding(ids)
+        cd = to_torch_dtype(self.compute_dtype)
+        if x.dtype != cd:
+            x = x.to(cd)
+        cos = self.cos.index_select(0, pos)
+        sin = self.sin.index_select(0, pos)
+        keys = torch.arange(self.max_len, device=self.device)
+        mask = keys[None, :] <= pos[:, None]
+        for block, kv in zip(self.blocks, cache):
+            x = block.forward(x, cos, sin, kv, pos, mask)
+        if last_only:
+            x = x[:, -1:, :]
+        return self.token_embedding(self.final_norm(x), reverse=True)
+
+    def generate(self, prompt, steps, use_graph=True):
+        """Greedy decode: prompt [B, P] -> generated ids [B, steps].  The prompt is one
+        forward over P positions; each later step is one forward over one position, replayed
+        from a HIP graph when use_graph is set (shapes and buffers are static)."""
+        prompt = prompt.to(self.device)
+        B, P = prompt.shape
+        if P + steps > self.max_len:
+            raise ValueError(f"prompt {P} + steps {steps} exceeds max_len {self.max_len}")
+        cache = self.new_cache(B)
+        logits = self.forward(prompt, torch.arange(P, device=self.device), cache)
+        token = logits[:, -1, :].argmax(dim=-1)
+        out = [token]
+        if steps == 1:
+            return torch.stack(out, dim=1)
+        tok_buf = token.clone().reshape(B, 1)
+        pos_buf = torch.full((1,), P, dtype=torch.int64, device=self.device)
+        next_buf = torch.empty((B,), dtype=torch.int64, device=self.device)
+
+        def step():
+            lg = self.forward(tok_buf, pos_buf, cache)
+            next_buf.copy_(lg[:, -1, :].argmax(dim=-1))
+
+        graph = None
+        if use_graph:
+            side = torch.cuda.Stream(self.device)
+            side.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(side):
+                # warm-up outside capture (first-call set-up, scratch allocation); it writes
+                # cache position P only, with the values the first replay writes again
+                step()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    step()
+            torch.cuda.current_stream(self.device).wait_stream(side)
+        for i in range(1, steps):
+            if graph is not None:
+                graph.replay()
+            else:
+                step()
+            out.append(next_buf.clone())
+            tok_buf.copy_(next_buf.reshape(B, 1))
+            pos_buf.add_(1)
+        return torch.stack(out, dim=1)
