@@ -156,6 +156,23 @@ int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N
                      int64_t workspace_bytes, const int* plan, void* stream);
 
 /*
+ * Weight-only int4 matmul for decode-sized M with the kernel stored K-contiguous:
+ *     y[m,n] = sum_k x[m,k] * W[n,k],  w_packed int8 [N, ceil(K/2)], low nibble = even k
+ *   block_size <= 0: scale [N];                         y = T(T(acc) / scale[n])
+ *   block_size  > 0: scale, zero [N, ceil(K/block)];     y = T(x . ((W - zero) * scale))
+ * This is a tied int4 embedding table [vocab, ceil(dim/2)] used as the LM head: the reverse
+ * branch of ReversibleEmbedding._int4_call without an activation quantizer
+ * (keras/src/layers/core/reversible_embedding.py:298-381: transpose, unpack_int4 along
+ * axis 0, dequantize_with_sz_map | divide, matmul).  x: [M, K] float32 or bfloat16;
+ * y: [M, N], bfloat16 when x and scale are both bfloat16, float32 otherwise (the
+ * reference's promotion).  Any M (tuned for M <= 8); the fast kernel needs K % 128 == 0
+ * and, grouped, block_size % 128 == 0; other shapes run a plain kernel.
+ */
+int k3q_gemv_w4_nk(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                   const int8_t* w_packed, const void* scale, int scale_dtype,
+                   const int8_t* zero, int64_t block_size, void* y, void* stream);
+
+/*
  * Quantized embedding lookup: out[t, :] = dequantise(table[ids[t], :]), t < count.
  * Replaces the take + cast + divide chain of Embedding._int8_call
  * (keras/src/layers/core/embedding.py:521-541) and the unpack_int4 + take +

@@ -181,46 +181,58 @@ class LlamaStyleDecoder(Model):
             x = x[:, -1:, :]
         return self.token_embedding(self.final_norm(x), reverse=True)
 
-    def generate(self, prompt, steps, use_graph=True):
+    def generate(self, prompt, steps, use_graph=True, stats=None):
         """Greedy decode: prompt [B, P] -> generated ids [B, steps].  The prompt is one
-        forward over P positions; each later step is one forward over one position, replayed
-        from a HIP graph when use_graph is set (shapes and buffers are static)."""
+        forward over P positions; each later step is one forward over one position that also
+        feeds its token back, replayed from a HIP graph when use_graph is set (shapes and
+        buffers are static, the position lives on the device).  `stats` (a dict) receives
+        prefill_ms, decode_ms, decode_steps as measured with device events."""
         prompt = prompt.to(self.device)
         B, P = prompt.shape
         if P + steps > self.max_len:
             raise ValueError(f"prompt {P} + steps {steps} exceeds max_len {self.max_len}")
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         cache = self.new_cache(B)
+        ev[0].record()
         logits = self.forward(prompt, torch.arange(P, device=self.device), cache)
         token = logits[:, -1, :].argmax(dim=-1)
-        out = [token]
-        if steps == 1:
-            return torch.stack(out, dim=1)
+        ev[1].record()
+        out_buf = torch.zeros((B, steps), dtype=torch.int64, device=self.device)
+        out_buf[:, 0] = token
         tok_buf = token.clone().reshape(B, 1)
         pos_buf = torch.full((1,), P, dtype=torch.int64, device=self.device)
-        next_buf = torch.empty((B,), dtype=torch.int64, device=self.device)
+        idx_buf = torch.ones((1,), dtype=torch.int64, device=self.device)
 
         def step():
             lg = self.forward(tok_buf, pos_buf, cache)
-            next_buf.copy_(lg[:, -1, :].argmax(dim=-1))
+            nxt = lg[:, -1, :].argmax(dim=-1, keepdim=True)
+            out_buf.index_copy_(1, idx_buf, nxt)
+            tok_buf.copy_(nxt)
+            pos_buf.add_(1)
+            idx_buf.add_(1)
 
+        done = 1
         graph = None
-        if use_graph:
+        if use_graph and steps > 2:
             side = torch.cuda.Stream(self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))
             with torch.cuda.stream(side):
-                # warm-up outside capture (first-call set-up, scratch allocation); it writes
-                # cache position P only, with the values the first replay writes again
-                step()
+                step()  # a real step, run eagerly: first-call set-up and scratch allocation
+                done += 1
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph, stream=side):
                     step()
             torch.cuda.current_stream(self.device).wait_stream(side)
-        for i in range(1, steps):
+        ev[2].record()
+        timed = steps - done
+        for _ in range(timed):
             if graph is not None:
                 graph.replay()
             else:
                 step()
-            out.append(next_buf.clone())
-            tok_buf.copy_(next_buf.reshape(B, 1))
-            pos_buf.add_(1)
-        return torch.stack(out, dim=1)
+        ev[3].record()
+        if stats is not None:
+            torch.cuda.synchronize(self.device)
+            stats.update(prefill_ms=ev[0].elapsed_time(ev[1]), decode_ms=ev[2].elapsed_time(ev[3]),
+                         decode_steps=timed, batch=B)
+        return out_buf

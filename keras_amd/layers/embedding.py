@@ -476,12 +476,29 @@ class ReversibleEmbedding(Embedding):
         return self._soft_cap(logits.reshape(*lead, N))
 
     def _int4_call(self, inputs, reverse=False, training=None):
+        """reversible_embedding.py:298-381.  Tied weights without an activation quantizer
+        (the default int4 config): the packed `[vocab, ceil(dim/2)]` table is the K-contiguous
+        int4 kernel of the projection and is read in place."""
         if not reverse:
             return super()._int4_call(inputs)
-        raise NotImplementedError(
-            "The int4 reverse projection (activation-quantized int4 matmul, "
-            "reversible_embedding.py:298-381) is not on the fused path yet."
+        if self.inputs_quantizer:
+            raise NotImplementedError(
+                "The int4 reverse projection with an activation quantizer is not on the fused "
+                "path yet."
+            )
+        if not self.tie_weights:
+            raise NotImplementedError(
+                "The untied int4 reverse projection (kernel packed along its first axis) is not "
+                "on the fused path yet."
+            )
+        block_size = getattr(self, "_int4_block_size", None)
+        grouped = block_size is not None and block_size > 0
+        logits = kops.int4_matmul_nk(
+            inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
+            zero=as_tensor(self.embeddings_zero) if grouped else None,
+            block_size=block_size if grouped else None,
         )
+        return self._soft_cap(logits)
 
     # ---- quantize -----------------------------------------------------------------------
     def _quantize(self, mode, config, type_check=True):

@@ -249,3 +249,38 @@ def embedding_lookup(ids, table, scale, dim, bits=8, zero=None, block_size=None,
     if check_ids and int(flag.item()) != 0:
         raise IndexError("index out of range in self")
     return out.reshape(*ids.shape, dim)
+
+
+def int4_matmul_nk(x, table_packed, scale, zero=None, block_size=None):
+    """`x[..., K] . W4[N, K]^T` for an int4 kernel stored K-contiguous: int8
+    [N, ceil(K/2)], low nibble = even k -- a tied int4 embedding table used as the LM head
+    (keras/src/layers/core/reversible_embedding.py:298-381, no activation quantizer).
+    scale: [N] (per row) or [N, G] with `zero` int8 [N, G] (grouped along K).
+    Returns [..., N] in bfloat16 when x and scale are bfloat16, float32 otherwise.
+    """
+    _lib.require_device(x, table_packed, scale, zero)
+    xcode = _lib.dtype_code(x.dtype)
+    scode = _lib.dtype_code(scale.dtype)
+    K = x.shape[-1]
+    if table_packed.dtype != torch.int8 or table_packed.dim() != 2 or table_packed.shape[1] != (K + 1) // 2:
+        raise ValueError("table must be int8 of shape [N, ceil(K / 2)]")
+    N = table_packed.shape[0]
+    grouped = block_size is not None and block_size > 0
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    tp = table_packed if table_packed.is_contiguous() else table_packed.contiguous()
+    sc = scale if scale.is_contiguous() else scale.contiguous()
+    zp = None
+    if grouped:
+        if zero is None:
+            raise ValueError("grouped int4 needs the zero points")
+        zp = zero if zero.is_contiguous() else zero.contiguous()
+    out_dtype = torch.bfloat16 if (x.dtype == torch.bfloat16 and scale.dtype == torch.bfloat16) else torch.float32
+    y = torch.empty((x2.shape[0], N), dtype=out_dtype, device=x.device)
+    rc = _lib.load().k3q_gemv_w4_nk(
+        _lib.ptr(x2), xcode, x2.shape[0], K, N, _lib.ptr(tp), _lib.ptr(sc), scode, _lib.ptr(zp),
+        int(block_size) if grouped else -1, _lib.ptr(y), _lib.stream_ptr(x.device),
+    )
+    _lib.check(rc, "k3q_gemv_w4_nk")
+    return y.reshape(*lead, N)

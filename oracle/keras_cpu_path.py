@@ -648,6 +648,33 @@ def reversible_embedding_int8_reverse(inputs, embeddings, embeddings_scale,
     return logits
 
 
+def reversible_embedding_int4_reverse(inputs, embeddings, embeddings_scale, output_dim,
+                                      embeddings_zero=None, g_idx=None, block_size=None,
+                                      compute_dtype=None, logit_soft_cap=None):
+    """keras/src/layers/core/reversible_embedding.py:298-381 with tied weights and no
+    activation quantizer (the default Int4QuantizationConfig): `inputs_scale` is
+    `ones((1,), compute_dtype)`; the packed table [V, ceil(D/2)] is transposed and unpacked
+    along axis 0 to int8 [D, V]."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    unpacked = unpack_int4(torch.transpose(embeddings, 0, 1), output_dim, axis=0)
+    inputs_scale = torch.ones((1,), dtype=cd)
+    if block_size is None or block_size == -1:
+        scale = embeddings_scale  # transpose of a 1-D tensor
+        logits = matmul(inputs, unpacked)
+        logits = logits.to(cd)
+        logits = torch.divide(logits, torch.multiply(inputs_scale, scale))
+    else:
+        scale_t = torch.transpose(embeddings_scale, 0, 1)
+        zero_t = torch.transpose(embeddings_zero, 0, 1)
+        float_embeddings = dequantize_with_sz_map(unpacked.to(cd), scale_t, zero_t, g_idx, group_axis=0)
+        logits = matmul(inputs, float_embeddings)
+        logits = torch.divide(logits, inputs_scale)
+    if logit_soft_cap is not None:
+        logits = torch.multiply(torch.tanh(torch.divide(logits, logit_soft_cap)), logit_soft_cap)
+    return logits
+
+
 # --------------------------------------------------------------------------
 # helpers shared by tests / bench (input generators named in the configs)
 # --------------------------------------------------------------------------

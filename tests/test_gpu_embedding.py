@@ -241,10 +241,66 @@ def test_reversible_embedding_int8_untied_and_soft_cap(dev, M):
     assert len(store) == 4
 
 
-def test_reversible_embedding_int4_reverse_raises(dev):
-    layer = build_embedding(ReversibleEmbedding, dev, 64, 32, "float32", seed=9)
-    layer.quantize("int4")
+@pytest.mark.parametrize("x_dtype,scale_dtype", [(torch.float32, torch.float32),
+                                                 (torch.bfloat16, torch.bfloat16),
+                                                 (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,V,D,block", [(1, 4000, 4096, 128), (8, 4000, 4096, None), (3, 500, 256, 128),
+                                         (11, 77, 384, 128), (2, 64, 512, 256), (4, 33, 256, -1),
+                                         (5, 40, 96, 32), (2, 21, 100, 20), (3, 17, 33, None)])
+def test_int4_matmul_nk(dev, x_dtype, scale_dtype, M, V, D, block):
+    qd = ref.embedding_quantize_int4(table(V, D, seed=11), block_size=block)
+    s = qd["embeddings_scale"].to(scale_dtype)
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(12)).to(x_dtype)
+    want = ref.reversible_embedding_int4_reverse(
+        x, qd["embeddings"], s, D, embeddings_zero=qd["embeddings_zero"], g_idx=qd["g_idx"],
+        block_size=block, compute_dtype=x_dtype)
+    grouped = block is not None and block > 0
+    got = kops.int4_matmul_nk(x.to(dev), qd["embeddings"].to(dev), s.to(dev),
+                              zero=qd["embeddings_zero"].to(dev) if grouped else None,
+                              block_size=block if grouped else None)
+    assert got.dtype == want.dtype and tuple(got.shape) == (M, V)
+    # float64 value of the same product: both must sit within the dtype's tolerance of it
+    w = qd["unpacked"].double()
+    if grouped:
+        gi = qd["g_idx"].long()
+        w = (w - qd["embeddings_zero"].double()[:, gi]) * s.double()[:, gi]
+        exact = x.double() @ w.T
+    else:
+        exact = (x.double() @ w.T) / s.double()
+    tol = RTOL[torch.bfloat16 if x_dtype == torch.bfloat16 else torch.float32]
+    assert max_rel_err(got, exact) <= tol
+    assert max_rel_err(got, want) <= tol
+
+
+@pytest.mark.parametrize("policy", ["float32", "bfloat16", "mixed_bfloat16"])
+@pytest.mark.parametrize("block_size", [128, None])
+def test_reversible_embedding_int4_tied(dev, policy, block_size):
+    V, D, M = 1000, 512, 6
+    layer = build_embedding(ReversibleEmbedding, dev, V, D, policy, seed=13)
+    t = layer._embeddings.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(14))
+    y_float = layer(x, reverse=True)
+    layer.quantize("int4", config=Int4QuantizationConfig(block_size=block_size))
+    qd = ref.embedding_quantize_int4(t.float(), block_size=block_size)
+    assert torch.equal(layer._embeddings.value.cpu(), qd["embeddings"])
+    y = layer(x, reverse=True)
+    vd = TORCH[layer.variable_dtype]
+    want = ref.reversible_embedding_int4_reverse(
+        x.to(cd), qd["embeddings"], qd["embeddings_scale"].to(vd), D,
+        embeddings_zero=qd["embeddings_zero"], g_idx=qd["g_idx"], block_size=block_size,
+        compute_dtype=cd)
+    assert y.dtype == want.dtype and tuple(y.shape) == (M, V)
+    assert max_rel_err(y, want) <= RTOL[cd]
+    err = (y_float.float().cpu() - y.float().cpu()).abs().max().item()
+    assert err <= 0.2 * y_float.float().abs().max().item() + 1e-3
     ids = torch.tensor([1, 2, 3])
-    assert layer(ids).shape == (3, 32)
+    assert layer(ids).shape == (3, D)
+
+
+def test_reversible_embedding_int4_untied_reverse_raises(dev):
+    layer = build_embedding(ReversibleEmbedding, dev, 64, 32, "float32", seed=9, tie_weights=False)
+    layer.quantize("int4")
+    assert layer(torch.tensor([1, 2, 3])).shape == (3, 32)
     with pytest.raises(NotImplementedError):
         layer(torch.randn(2, 32), reverse=True)

@@ -144,3 +144,29 @@ def test_reverse_projection_tied_int8_closed_form():
     assert (logits - want_f).abs().max().item() < 0.05 * want_f.abs().max().item() + 1e-3
     capped = ref.reversible_embedding_int8_reverse(x, q, s, logit_soft_cap=0.5)
     assert torch.allclose(capped, torch.tanh(logits / 0.5) * 0.5)
+
+
+@pytest.mark.parametrize("block_size", [None, 8])
+def test_reverse_projection_tied_int4_by_loops(block_size):
+    V, D, M = 5, 16, 2
+    t = table(V, D, seed=7)
+    qd = ref.embedding_quantize_int4(t, block_size=block_size)
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(8))
+    logits = ref.reversible_embedding_int4_reverse(
+        x, qd["embeddings"], qd["embeddings_scale"], D, embeddings_zero=qd["embeddings_zero"],
+        g_idx=qd["g_idx"], block_size=block_size)
+    assert tuple(logits.shape) == (M, V) and logits.dtype == torch.float32
+    w = qd["unpacked"]
+    for m in range(M):
+        for v in range(V):
+            if block_size is None:
+                acc = sum(float(x[m, d]) * float(w[v, d]) for d in range(D))
+                want = acc / float(qd["embeddings_scale"][v])
+            else:
+                want = sum(
+                    float(x[m, d]) * (float(w[v, d]) - float(qd["embeddings_zero"][v, d // block_size]))
+                    * float(qd["embeddings_scale"][v, d // block_size]) for d in range(D))
+            assert logits[m, v].item() == pytest.approx(want, rel=2e-5, abs=1e-6)
+    # and it approximates the float projection (int4: coarse)
+    want_f = x @ t.T
+    assert (logits - want_f).abs().max().item() < 0.25 * want_f.abs().max().item() + 1e-3
