@@ -15,9 +15,11 @@ import math
 
 import torch
 
+from keras_amd import dtype_policies
 from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
 from keras_amd.models import Model
+from keras_amd.quantization_config import Int4QuantizationConfig
 
 
 class RMSNorm(Layer):
@@ -116,8 +118,16 @@ class LlamaStyleDecoder(Model):
             fan_in = shape[0] * shape[1] if len(shape) == 3 and shape[0] == n_heads else shape[0]
             return (torch.randn(shape, generator=gen) * (1.0 / math.sqrt(fan_in))).to(dt)
 
+        # A layer built straight from an int4 policy has no config and would fall back to the
+        # default activation quantizer (reversible_embedding.py:229-233); pass the config that
+        # `quantize("int4")` resolves to, so that both construction paths give the same layer.
+        emb_config = None
+        policy = dtype_policies.get(wdtype)
+        if policy.quantization_mode == "int4":
+            emb_config = Int4QuantizationConfig(block_size=policy.block_size)
         self.token_embedding = ReversibleEmbedding(
             vocab, d_model, dtype=wdtype, device=self.device, name="token_embedding",
+            quantization_config=emb_config,
             embeddings_initializer=lambda s, dt: (torch.randn(s, generator=gen) * 0.02).to(dt))
         self.token_embedding.build()
         self.token_embedding.check_ids = False

@@ -56,7 +56,13 @@ def oracle_forward(model, ids):
     elif emb.quantization_mode is None:
         x = cpu(emb._embeddings)[ids]
     else:
-        raise AssertionError("unexpected embedding mode")
+        bs = emb._int4_block_size
+        grouped = bs is not None and bs > 0
+        x = ref.embedding_int4_call(
+            ids, cpu(emb._embeddings), cpu(emb.embeddings_scale), emb.output_dim,
+            embeddings_zero=cpu(emb.embeddings_zero) if grouped else None,
+            g_idx=cpu(emb.g_idx) if grouped else None, block_size=bs,
+            compute_dtype=emb.compute_dtype)
     cos, sin = rope_tables(model.head_dim, model.max_len, torch.device("cpu"))
     cos, sin = cos[:T], sin[:T]
     causal = torch.ones(T, T, dtype=torch.bool).tril()
@@ -82,15 +88,20 @@ def oracle_forward(model, ids):
         return ref.reversible_embedding_int8_reverse(
             x.reshape(B * T, -1), cpu(emb._embeddings), cpu(emb.embeddings_scale),
             compute_dtype=emb.compute_dtype).reshape(B, T, -1)
+    if emb.quantization_mode == "int4":
+        bs = emb._int4_block_size
+        grouped = bs is not None and bs > 0
+        return ref.reversible_embedding_int4_reverse(
+            x.reshape(B * T, -1), cpu(emb._embeddings), cpu(emb.embeddings_scale), emb.output_dim,
+            embeddings_zero=cpu(emb.embeddings_zero) if grouped else None,
+            g_idx=cpu(emb.g_idx) if grouped else None, block_size=bs,
+            compute_dtype=emb.compute_dtype).reshape(B, T, -1)
     return x @ cpu(emb._embeddings).T
 
 
 def quantize(model, mode):
     with warnings.catch_warnings():
         warnings.simplefilter("ignore")
-        if mode == "int4":
-            # the int4 reverse projection is not on the fused path: keep the embedding in float
-            return model.quantize("int4", filters=lambda l: l.name != "token_embedding")
         return model.quantize(mode)
 
 
@@ -99,14 +110,19 @@ def test_model_quantize_report(dev, mode):
     model = LlamaStyleDecoder(dtype="float32", device=dev, **CFG)
     report = quantize(model, mode)
     per_block = 7
-    n_q = per_block * CFG["n_layers"] + (1 if mode == "int8" else 0)
+    n_q = per_block * CFG["n_layers"] + 1
     assert report.mode == mode and report.num_quantized == n_q
     # norms (2 per block + final) and the blocks themselves have no quantized form
     unsupported = report.skipped_by_reason(QuantizationReport.SKIP_NO_SUPPORT)
     assert len(unsupported) == 3 * CFG["n_layers"] + 1
     if mode == "int4":
-        assert report.skipped_by_reason(QuantizationReport.SKIP_FILTERED) == ["token_embedding"]
         assert all(s == "int4/128_from_float32" for _, _, s in report.quantized)
+    model2 = LlamaStyleDecoder(dtype="float32", device=dev, **CFG)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        filtered = model2.quantize(mode, filters=lambda l: l.name != "token_embedding")
+    assert filtered.skipped_by_reason(QuantizationReport.SKIP_FILTERED) == ["token_embedding"]
+    assert filtered.num_quantized == n_q - 1
     again = quantize(model, mode)
     assert again.num_quantized == 0
     assert len(again.skipped_by_reason(QuantizationReport.SKIP_ALREADY_QUANTIZED)) == n_q
@@ -150,17 +166,17 @@ def test_generate_graph_equals_eager(dev, mode, dtype):
     assert torch.equal(graphed.cpu(), again.cpu())
 
 
-def test_prebuilt_quantized_decoder_runs(dev):
-    model = LlamaStyleDecoder(dtype="bfloat16", device=dev, layer_policy="int4/128_from_bfloat16",
+@pytest.mark.parametrize("policy", ["int4/128_from_bfloat16", "int4/-1_from_bfloat16", "int8_from_bfloat16"])
+def test_prebuilt_quantized_decoder_runs(dev, policy):
+    model = LlamaStyleDecoder(dtype="bfloat16", device=dev, layer_policy=policy,
                               **{**CFG, "d_model": 256, "ffn_dim": 512})
-    assert model.blocks[0].gate.quantization_mode == "int4"
+    mode = policy[:4]
+    assert model.blocks[0].gate.quantization_mode == mode
     assert model.blocks[0].gate._kernel.dtype == "int8"
+    assert model.token_embedding.quantization_mode == mode
     model.randomize_quantized_weights()
-    model.token_embedding  # int4 table: lookup works, reverse is not on the fused path
     prompt = torch.randint(0, CFG["vocab"], (2, 8), generator=torch.Generator().manual_seed(4))
-    with pytest.raises(NotImplementedError):
-        model.generate(prompt, 4)
-    model8 = LlamaStyleDecoder(dtype="bfloat16", device=dev, layer_policy="int8_from_bfloat16", **CFG)
-    model8.randomize_quantized_weights()
-    out = model8.generate(prompt, 6)
+    stats = {}
+    out = model.generate(prompt, 6, stats=stats)
     assert tuple(out.shape) == (2, 6) and int(out.min()) >= 0 and int(out.max()) < CFG["vocab"]
+    assert stats["decode_steps"] == 4 and stats["decode_ms"] > 0
