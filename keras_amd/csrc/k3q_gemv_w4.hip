@@ -529,6 +529,24 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     int64_t klen = K * nblocks / ((int64_t)target * waves);
     klen = klen / chunk * chunk;
     if (klen < chunk) klen = chunk;
+    // at least two chunks per wave (so that loads and MFMAs overlap) while that still leaves
+    // one workgroup per CU
+    if (!grouped && klen < 2 * chunk && K * nblocks / (2 * chunk * (int64_t)waves) >= kTargetWorkgroups)
+        klen = 2 * chunk;
+    if (grouped) {
+        // a slice that straddles group boundaries pays an extra flush per wave: snap to a
+        // multiple of the group size, or to a fraction of it (14 us instead of 21 us at
+        // K = 4096, N = 14336, where the formula above gives 96 rows for groups of 128)
+        if (4 * klen >= 3 * block_size) {
+            klen = (klen + block_size / 2) / block_size * block_size;
+        } else {
+            int64_t frac = block_size;
+            while (frac / 2 >= chunk && (frac / 2) % chunk == 0 && 3 * (frac / 2) >= 2 * klen &&
+                   frac > klen)
+                frac /= 2;
+            klen = frac;
+        }
+    }
     if (plan_override && plan_override[3] > 0) klen = (plan_override[3] + chunk - 1) / chunk * chunk;
     if (klen > K) klen = (K + chunk - 1) / chunk * chunk;
     pl.klen = (int)klen;

@@ -34,25 +34,23 @@ class RMSNorm(Layer):
         self.built = True
 
     def call(self, x, training=None):
-        xf = x.float()
-        var = xf.pow(2).mean(dim=-1, keepdim=True)
-        y = xf * torch.rsqrt(var + self.epsilon)
-        return (y * self.read(self.scale).float()).to(x.dtype)
+        return torch.nn.functional.rms_norm(x, (self.dim,), self.read(self.scale), self.epsilon)
 
 
-def rope_tables(head_dim, max_len, device, base=10000.0):
+def rope_tables(head_dim, max_len, device, base=10000.0, dtype=torch.float32):
+    """cos / sin [max_len, head_dim] for the rotate-half form: the half-width table repeated."""
     inv = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
     ang = torch.outer(torch.arange(max_len, dtype=torch.float32), inv)
-    return torch.cos(ang).to(device), torch.sin(ang).to(device)
+    ang = torch.cat((ang, ang), dim=-1)
+    return torch.cos(ang).to(device=device, dtype=dtype), torch.sin(ang).to(device=device, dtype=dtype)
 
 
 def apply_rope(x, cos, sin):
-    """x [B, T, H, hd]; cos / sin [T, hd/2] for the positions of these T tokens."""
-    xf = x.float()
-    x1, x2 = xf[..., 0::2], xf[..., 1::2]
-    c, s = cos[None, :, None, :], sin[None, :, None, :]
-    out = torch.stack((x1 * c - x2 * s, x1 * s + x2 * c), dim=-1).flatten(-2)
-    return out.to(x.dtype)
+    """x [B, T, H, hd]; cos / sin [T, hd] for the positions of these T tokens
+    (rotate-half: pairs are (i, i + hd/2))."""
+    half = x.shape[-1] // 2
+    rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return x * cos[None, :, None, :] + rot * sin[None, :, None, :]
 
 
 class DecoderBlock(Layer):
@@ -137,7 +135,8 @@ class LlamaStyleDecoder(Model):
             for i in range(n_layers)
         ]
         self.final_norm = RMSNorm(d_model, dtype=dtype, device=self.device, name="final_norm")
-        self.cos, self.sin = rope_tables(self.head_dim, max_len, self.device)
+        self.cos, self.sin = rope_tables(self.head_dim, max_len, self.device,
+                                         dtype=to_torch_dtype(self.compute_dtype))
         self._graphs = {}
 
     # ---- synthetic quantized weights ---------------------------------------------------

@@ -63,14 +63,12 @@ def oracle_forward(model, ids):
             embeddings_zero=cpu(emb.embeddings_zero) if grouped else None,
             g_idx=cpu(emb.g_idx) if grouped else None, block_size=bs,
             compute_dtype=emb.compute_dtype)
-    cos, sin = rope_tables(model.head_dim, model.max_len, torch.device("cpu"))
+    cos, sin = rope_tables(model.head_dim, model.max_len, torch.device("cpu"), dtype=x.dtype)
     cos, sin = cos[:T], sin[:T]
     causal = torch.ones(T, T, dtype=torch.bool).tril()
 
     def norm(layer, v):
-        vf = v.float()
-        y = vf * torch.rsqrt(vf.pow(2).mean(-1, keepdim=True) + layer.epsilon)
-        return (y * cpu(layer.scale).float()).to(v.dtype)
+        return torch.nn.functional.rms_norm(v, (layer.dim,), cpu(layer.scale).to(v.dtype), layer.epsilon)
 
     for blk in model.blocks:
         h = norm(blk.attn_norm, x)
