@@ -53,6 +53,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
+    ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the quantized Dense path has no multi-GPU leg "
@@ -179,6 +180,37 @@ def main():
             del graph
         del xg
 
+    # ------------------------------------------------------------------ end-to-end decode
+    # Llama-style 32-layer decoder (d_model 4096, 32 heads, SwiGLU 14336, vocab 32000), every
+    # weight matrix int4 (grouped, block 128) with synthetic values written on the device;
+    # prompt of 128 random ids, greedy decode of 128 steps, decode steps replayed from a HIP
+    # graph.  Matmuls, embedding lookup and LM head run the k3q kernels; norms, RoPE,
+    # attention and the gating are torch ops.
+    decode = None
+    if not args.no_decode:
+        from keras_amd.decoder_harness import LlamaStyleDecoder
+
+        w4_host = packs[0].cpu()
+        del packs
+        torch.cuda.empty_cache()
+        model = LlamaStyleDecoder(max_len=256, dtype="bfloat16", device=dev,
+                                  layer_policy="int4/128_from_bfloat16")
+        model.randomize_quantized_weights()
+        decode = []
+        for batch in (1, 8):
+            prompt = torch.randint(0, model.vocab, (batch, 128), generator=g)
+            model.generate(prompt, 8)  # first-call set-up
+            st = {}
+            model.generate(prompt, 128, stats=st)
+            decode.append({
+                "batch": batch, "prompt": 128, "steps": 128,
+                "prefill_ms": round(st["prefill_ms"], 2),
+                "decode_ms_per_step": round(st["decode_ms"] / st["decode_steps"], 3),
+                "tokens_per_s": round(batch * st["decode_steps"] / st["decode_ms"] * 1e3, 1),
+            })
+        del model
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None
     if not args.no_cpu_baseline:
@@ -198,7 +230,7 @@ def main():
                       f"{Mc} of {M} rows, K=N={K}, one pass, {cpu_s:.1f} s; host has {os.cpu_count()} cpus",
         }
         # int4 decode GEMV on the host: unpack + float matmul per call, as the reference does
-        w4 = packs[0].cpu()
+        w4 = w4_host if decode is not None else packs[0].cpu()
         x1 = torch.randn(1, Kg, generator=g).to(torch.bfloat16)
         ref.dense_int4_call(x1, w4, pc_scale.cpu().float(), Ng, compute_dtype=torch.bfloat16)
         t0 = time.perf_counter()
@@ -234,6 +266,7 @@ def main():
                                    "frac": round(quant_bytes / (quant_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                                    "traffic": QUANT_HBM_TRAFFIC_BYTES}},
         "int4_gemv": gemv,
+        "llama_decode_int4": decode,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
