@@ -1,0 +1,19 @@
+// bfloat16 x bfloat16 -> float32 GEMM on the tile machinery of the int8 GEMM
+// (k3q_gemm_i8.hip): y[M,N] = T(T(a[M,K] . bt[N,K]^T) / scale[n]) (+ bias), bfloat16 in and out.
+// Used for prefill-sized int4 matmuls, where bt is the int4 kernel de-quantised into scratch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace k3q {
+
+// K % 64 == 0, N % 4 == 0, 16-byte aligned operands
+bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* bt,
+                            const void* y);
+
+// b_scale (bfloat16 [N]) and bias (bfloat16 [N]) may be null
+int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
+                     const void* b_scale, const void* bias, void* y, hipStream_t s);
+
+}  // namespace k3q

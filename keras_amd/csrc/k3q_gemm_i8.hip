@@ -18,6 +18,7 @@
 // the activation tile the second (column) operand, so a lane ends up with ONE
 // output row m and groups of four consecutive n: stores are 8 or 16 bytes wide.
 #include "k3q_common.h"
+#include "k3q_gemm_bf16.h"
 #include "k3q_gemm_i8_skinny.h"
 
 namespace k3q {
@@ -59,6 +60,7 @@ struct GemmParams {
     void* y;                // T [M, N] or null
     int32_t* acc_out;       // [M, N] or null
     int64_t M, N, K;
+    int64_t row_bytes;      // bytes per row of a and bt: K (int8) or 2K (bfloat16 operands)
     int tiles_m, tiles_n;
     int flags;
 };
@@ -89,8 +91,31 @@ __device__ __forceinline__ float load_t(const void* p, int64_t i) {
     return ((const float*)p)[i];
 }
 
-template <bool kBF16, bool kExact>
-__global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
+// Operand kinds.  The byte geometry is the same for both: a lane's MFMA fragment is 16
+// bytes of one row, a stage is 128 bytes of K per row -- 128 int8 or 64 bfloat16 values.
+constexpr int kKindI8 = 0;    // int8 x int8 -> int32, v_mfma_i32_32x32x32_i8
+constexpr int kKindBF16 = 1;  // bfloat16 x bfloat16 -> float32, v_mfma_f32_32x32x16_bf16
+
+template <int kKind>
+struct Mma;
+template <>
+struct Mma<kKindI8> {
+    typedef v16i Acc;
+    static __device__ __forceinline__ Acc run(const v4i& b, const v4i& a, const Acc& c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<kKindBF16> {
+    typedef v16f Acc;
+    static __device__ __forceinline__ Acc run(const v4i& b, const v4i& a, const Acc& c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, b),
+                                                       __builtin_bit_cast(v8bf, a), c, 0, 0, 0);
+    }
+};
+
+template <int kKind, bool kBF16, bool kExact>
+__global__ __launch_bounds__(kThreads) void gemm_mfma(GemmParams p) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 #ifdef K3Q_GEMM_PROBE_CLOCK
     const uint64_t clk0 = __builtin_readcyclecounter();
@@ -132,7 +157,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
         int64_t grow = (is_b ? n0 : m0) + row;
         const int64_t lim = (is_b ? p.N : p.M) - 1;
         grow = grow < lim ? grow : lim;
-        src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.K + chunk * 16;
+        src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16;
     }
     auto issue_stage = [&](int kt) {
         char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
@@ -173,7 +198,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
             af[fb][mb] = *(const v4i*)(st + a_row[mb] + (((2 * ks + fg) ^ a_swz[mb]) << 4));
     };
 
-    v16i acc[kNBlk][kMBlk];
+    typename Mma<kKind>::Acc acc[kNBlk][kMBlk];
 #pragma unroll
     for (int nb = 0; nb < kNBlk; ++nb)
 #pragma unroll
@@ -187,7 +212,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
     // matrix core has work queued while waves meet.  At that barrier every wave holds its
     // last fragments of stage kt in registers, so stage kt+2 may be DMA-ed over stage kt, and
     // stage kt+1 (whose DMA every wave has waited for) may be read.
-    const int KT = (int)(p.K / kBK);
+    const int KT = (int)(p.row_bytes / kBK);
     issue_stage(0);
     if (KT > 1) {
         issue_stage(1);
@@ -209,8 +234,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
             for (int nb = 0; nb < kNBlk / 2; ++nb)
 #pragma unroll
                 for (int mb = 0; mb < kMBlk; ++mb)
-                    acc[nb][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][nb], af[ks & 1][mb],
-                                                                        acc[nb][mb], 0, 0, 0);
+                    acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
 #endif
             __builtin_amdgcn_sched_barrier(0);
             if (ks + 1 < kKSteps) {
@@ -229,12 +253,11 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
             for (int nb = kNBlk / 2; nb < kNBlk; ++nb)
 #pragma unroll
                 for (int mb = 0; mb < kMBlk; ++mb)
-                    acc[nb][mb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[ks & 1][nb], af[ks & 1][mb],
-                                                                        acc[nb][mb], 0, 0, 0);
+                    acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
 #else
             // probe build: consume the fragments so that the reads stay
 #pragma unroll
-            for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] ^= af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1];
+            for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] += (af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1]);
 #endif
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -259,7 +282,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
 #pragma unroll
             for (int mb = 0; mb < kMBlk; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sink ^= acc[nb][mb][r];
+                for (int r = 0; r < 16; ++r) sink ^= (int)acc[nb][mb][r];
         if (sink == 0x7fffffff && p.y) ((char*)p.y)[0] = 1;
         return;
     }
@@ -279,6 +302,39 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
         ep[2 * kBN + t] = kExact ? sav : 1.0f / sav;
     }
     __syncthreads();
+    if constexpr (kKind == kKindBF16) {
+        // float operands (a de-quantised int4 kernel): y = T(T(acc) / scale[n]) (+ bias), or
+        // with a null scale y = T(acc) (+ bias); bfloat16 output.
+        const bool has_b = p.bias != nullptr, has_s = p.b_scale != nullptr;
+#pragma unroll
+        for (int mb = 0; mb < kMBlk; ++mb) {
+            const int ml = wm * kWM + mb * 32 + fi;
+            const int64_t m = m0 + ml;
+            if (m >= p.M) continue;
+#pragma unroll
+            for (int nb = 0; nb < kNBlk; ++nb) {
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+                    const int64_t n = n0 + nl;
+                    if (n >= p.N) continue;
+                    const v4f sb = *(const v4f*)(ep + nl);
+                    const v4f bv = *(const v4f*)(ep + kBN + nl);
+                    u32 h[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float r = round_bf16((float)acc[nb][mb][4 * rg + e]);
+                        if (has_s) r = round_bf16(r / sb[e]);
+                        if (has_b) r = round_bf16(r + bv[e]);
+                        h[e] = f32_to_bf16_bits(r);
+                    }
+                    v2u o = {h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+                    *(v2u*)((uint16_t*)p.y + m * p.N + n) = o;
+                }
+            }
+        }
+        return;
+    }
     const bool has_bias = p.bias != nullptr;
     const bool round_acc = (p.flags & kFlagRoundAccBF16) != 0;
     // Row-major store order: the eight 8-byte (16-byte for float32) pieces that make up one
@@ -297,8 +353,8 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_mfma(GemmParams p) {
                 const int64_t n = n0 + nl;
                 if (n >= p.N) continue;  // N % 4 == 0 on this path: all four columns in or out
                 if (p.acc_out) {
-                    v4i o = {acc[nb][mb][4 * rg], acc[nb][mb][4 * rg + 1], acc[nb][mb][4 * rg + 2],
-                             acc[nb][mb][4 * rg + 3]};
+                    v4i o = {(int)acc[nb][mb][4 * rg], (int)acc[nb][mb][4 * rg + 1],
+                             (int)acc[nb][mb][4 * rg + 2], (int)acc[nb][mb][4 * rg + 3]};
                     *(v4i*)(p.acc_out + m * p.N + n) = o;
                 }
                 if (!p.y) continue;
@@ -386,25 +442,49 @@ __global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ i
     }
 }
 
-bool g_lds_attr_set[4] = {false, false, false, false};
+bool g_lds_attr_set[8] = {};
 
-template <bool kBF16, bool kExact>
+template <int kKind, bool kBF16, bool kExact>
 int launch_mfma(const GemmParams& p, hipStream_t s) {
     // 128 KiB of dynamic LDS needs the attribute raised once per kernel (idempotent).
-    constexpr int slot = (kBF16 ? 1 : 0) + (kExact ? 2 : 0);
+    constexpr int slot = (kBF16 ? 1 : 0) + (kExact ? 2 : 0) + 4 * kKind;
     if (!g_lds_attr_set[slot]) {
-        if (hipFuncSetAttribute((const void*)gemm_i8_mfma<kBF16, kExact>,
+        if (hipFuncSetAttribute((const void*)gemm_mfma<kKind, kBF16, kExact>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
             return K3Q_ERR_LAUNCH;
         g_lds_attr_set[slot] = true;
     }
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    gemm_i8_mfma<kBF16, kExact><<<grid, kThreads, kLdsBytes, s>>>(p);
+    gemm_mfma<kKind, kBF16, kExact><<<grid, kThreads, kLdsBytes, s>>>(p);
     return launch_status();
 }
 
 }  // namespace
+
+bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* bt,
+                            const void* y) {
+    return M > 0 && (2 * K) % kBK == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(bt, 16) &&
+           aligned_to(y, 8) && ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) < (1 << 28);
+}
+
+int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
+                     const void* b_scale, const void* bias, void* y, hipStream_t s) {
+    GemmParams p{};
+    p.a = (const int8_t*)a;
+    p.bt = (const int8_t*)bt;
+    p.b_scale = b_scale;
+    p.bias = bias;
+    p.y = y;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.row_bytes = 2 * K;
+    p.tiles_m = (int)((M + kBM - 1) / kBM);
+    p.tiles_n = (int)((N + kBN - 1) / kBN);
+    return launch_mfma<kKindBF16, true, true>(p, s);
+}
+
 }  // namespace k3q
 
 using namespace k3q;
@@ -453,6 +533,7 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     p.M = M;
     p.N = N;
     p.K = K;
+    p.row_bytes = K;
     p.flags = flags;
     p.tiles_m = (int)((M + kBM - 1) / kBM);
     p.tiles_n = (int)((N + kBN - 1) / kBN);
@@ -483,8 +564,8 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     }
     if (fast) {
         const bool exact = (flags & kFlagExactEpilogue) != 0;
-        if (bf16) return exact ? launch_mfma<true, true>(p, s) : launch_mfma<true, false>(p, s);
-        return exact ? launch_mfma<false, true>(p, s) : launch_mfma<false, false>(p, s);
+        if (bf16) return exact ? launch_mfma<kKindI8, true, true>(p, s) : launch_mfma<kKindI8, true, false>(p, s);
+        return exact ? launch_mfma<kKindI8, false, true>(p, s) : launch_mfma<kKindI8, false, false>(p, s);
     }
 
     if (M > 65535) return K3Q_ERR_SHAPE;

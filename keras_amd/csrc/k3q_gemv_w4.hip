@@ -36,6 +36,7 @@
 // workgroup, which on this multi-XCD part means an L2 write-back and
 // invalidate each: measured 2-5x slower than the second launch.)
 #include "k3q_common.h"
+#include "k3q_gemm_bf16.h"
 
 namespace k3q {
 namespace {
@@ -475,6 +476,82 @@ __global__ __launch_bounds__(256) void gemv_w4_generic(GemvParams p) {
     finish<kBF16, kGrouped>(p, m, n, total);
 }
 
+// Prefill-sized M: the packed kernel is de-quantised once per call into a bfloat16 [N, K]
+// scratch matrix (K contiguous, what the MFMA GEMM consumes) and the product runs on the
+// matrix cores at full tile size.  Per-channel: the scratch holds the plain nibble values
+// (exact) and the GEMM epilogue divides by the scale, as the reference's matmul + divide does;
+// grouped: it holds T((w - zero) * scale), rounded to bfloat16 per weight exactly as the
+// reference's de-quantised kernel is.
+constexpr int kDqK = 128;  // tile: 128 rows of K x 64 columns
+constexpr int kDqN = 64;
+
+template <bool kGrouped>
+__global__ __launch_bounds__(256) void dequant_w4_to_bf16_nk(const uint8_t* __restrict__ w,
+                                                            const uint16_t* __restrict__ scale,
+                                                            const int8_t* __restrict__ zero,
+                                                            uint16_t* __restrict__ out, int64_t K,
+                                                            int64_t N, int block_size) {
+    __shared__ uint16_t tile[kDqK][kDqN + 2];
+    const int64_t k0 = (int64_t)blockIdx.y * kDqK;
+    const int64_t n0 = (int64_t)blockIdx.x * kDqN;
+    {
+        // thread -> (row k, 32 columns): one 16-byte load of packed nibbles
+        const int r = threadIdx.x >> 1, h = threadIdx.x & 1;
+        const int64_t k = k0 + r, n = n0 + 32 * h;
+        const v4u pk = *(const v4u*)(w + k * (N / 2) + n / 2);
+        float sc[32], zp[32];
+        if (kGrouped) {
+            const int64_t g = k / block_size;
+            const v4u* sp = (const v4u*)(scale + g * N + n);
+            const v4u* zq = (const v4u*)(zero + g * N + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const v4u sv = sp[q];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    sc[8 * q + 2 * d] = __uint_as_float(sv[d] << 16);
+                    sc[8 * q + 2 * d + 1] = __uint_as_float(sv[d] & 0xffff0000u);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const v4u zv = zq[q];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) zp[16 * q + e] = (float)(int)(int8_t)(zv[e >> 2] >> (8 * (e & 3)));
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            const u32 nib = (pk[e >> 3] >> (4 * (e & 7))) & 0xfu;  // low nibble = even column
+            float v = (float)((int)(nib ^ 8u) - 8);
+            if (kGrouped) v = (v - zp[e]) * sc[e];  // the difference is exact, one rounding
+            tile[r][32 * h + e] = (uint16_t)f32_to_bf16_bits(v);
+        }
+    }
+    __syncthreads();
+    {
+        // thread -> (column n, 32 rows of k): 64 contiguous bytes of output row n
+        const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
+        v4u o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int kk = 32 * part + 8 * q + 2 * d;
+                o[q][d] = (u32)tile[kk][c] | ((u32)tile[kk + 1][c] << 16);
+            }
+        v4u* dst = (v4u*)(out + (n0 + c) * K + k0 + 32 * part);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dst[q] = o[q];
+    }
+}
+
+constexpr int64_t kGemmMinRows = 64;  // from here on the GEMM route beats 16-row decode passes
+
+inline bool gemm_route_ok(int x_dtype, int64_t M, int64_t K, int64_t N) {
+    return x_dtype == K3Q_BF16 && M >= kGemmMinRows && (K % kDqK) == 0 && (N % kDqN) == 0;
+}
+
 struct Plan {
     bool fast;
     int vec;     // dwords per lane per k row
@@ -627,6 +704,20 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
     p.row_bytes = (N + 1) / 2;
     p.block_size = grouped ? (int)block_size : 0;
 
+    if (!plan_override && gemm_route_ok(x_dtype, M, K, N) && workspace &&
+        workspace_bytes >= N * K * 2 && aligned_to(workspace, 16) && aligned_to(w_packed, 16) &&
+        aligned_to(scale, 16) && (!zero || aligned_to(zero, 16)) &&
+        gemm_bf16_nk_supported(M, N, K, x, workspace, y)) {
+        dim3 grid((unsigned)(N / kDqN), (unsigned)(K / kDqK));
+        if (grouped)
+            dequant_w4_to_bf16_nk<true><<<grid, 256, 0, s>>>(
+                (const uint8_t*)w_packed, (const uint16_t*)scale, (const int8_t*)zero,
+                (uint16_t*)workspace, K, N, (int)block_size);
+        else
+            dequant_w4_to_bf16_nk<false><<<grid, 256, 0, s>>>(
+                (const uint8_t*)w_packed, nullptr, nullptr, (uint16_t*)workspace, K, N, 0);
+        return gemm_bf16_nk_run(x, workspace, M, N, K, grouped ? nullptr : scale, bias, y, s);
+    }
     Plan pl = make_plan(x_dtype, M, K, N, block_size, plan_override);
     // vector loads of x rows, packed rows, scales and zero points
     if (pl.fast && (!aligned_to(x, 16) || !aligned_to(w_packed, 16) || !aligned_to(scale, 16) ||
@@ -709,6 +800,8 @@ extern "C" int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N) 
             const int64_t b = (int64_t)pl.ks * rows * N * 4;
             if (b > part) part = b;
         }
+    // prefill sizes: room for the bfloat16 [N, K] copy of the de-quantised kernel
+    if (gemm_route_ok(K3Q_BF16, M, K, N) && N * K * 2 > part) part = N * K * 2;
     return part;
 }
 
