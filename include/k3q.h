@@ -121,21 +121,26 @@ int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64
                 void* stream);
 
 /*
- * Weight-only int4 matmul for decode-sized inputs (any M; tuned for M <= 16):
+ * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; 16-row
+ * passes up to M = 255; from M = 256 on, for bfloat16 x with K % 128 == 0 and
+ * N % 64 == 0, the kernel is de-quantised once into `workspace` as bfloat16 [N, K]
+ * and the product runs on the MFMA tile kernel):
  *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)
  *     grouped     (block_size  > 0):  y = T(x . ((unpack(w) - zero[g]) * scale[g]))  (+ bias),  g = k / block_size
  * x: [M, K] of x_dtype, contiguous.  w_packed: the layer's int4 kernel as stored,
  * int8 [K, ceil(N/2)], low nibble = even column.  scale: x_dtype, [N] or
  * [ceil(K/block_size), N].  zero: int8 [ceil(K/block_size), N] (grouped only).
- * bias: x_dtype [N] or null.  y: x_dtype [M, N].  The packed kernel is read
- * once from HBM and is neither unpacked nor de-quantised in memory.
+ * bias: x_dtype [N] or null.  y: x_dtype [M, N].  At decode sizes the packed kernel
+ * is read once from HBM and is neither unpacked nor de-quantised in memory.
  * Replaces, per call, unpack_int4 + (dequantize_with_sz_map | cast) + matmul +
  * divide of Dense._int4_call (keras/src/layers/core/dense.py:988-1095) and the
  * int4 branch of EinsumDense (keras/src/layers/core/einsum_dense.py:1120-1261).
  *
  * workspace: k3q_gemv_w4_workspace_bytes(M, K, N) bytes, 16-byte aligned, contents
  * irrelevant.  It holds the fp32 partial sums of the K split between the two
- * kernels of a call, so two calls that overlap in time must not share one.
+ * kernels of a call (decode sizes) or the de-quantised kernel (prefill sizes), so
+ * two calls that overlap in time must not share one.  Without it (null / too small)
+ * prefill sizes fall back to the 16-row passes.
  */
 int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
