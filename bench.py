@@ -8,8 +8,10 @@ de-scale epilogue, at BASELINE's target shape M=4096, K=N=8192, bfloat16
 activations (inputs and weights already resident in HBM).  `value` is
 2*M*N*K / step time in TOP/s.  The int4 decode GEMV (K=N=8192, M in {1,4,16}),
 the second half of BASELINE's metric, is reported under `int4_gemv` with its own
-HBM roofline.  The CPU oracle (a restatement of the reference's torch-CPU op
-sequence) is timed on the host cores on a bounded sample as `cpu_baseline`.
+HBM roofline; `llama_decode_int4` is the end-to-end greedy decode of a 32-layer
+Llama-style decoder whose weight matrices are all int4 (tokens/s at batch 1 and 8).
+The CPU oracle (a restatement of the reference's torch-CPU op sequence) is timed
+on the host cores on a bounded sample as `cpu_baseline`.
 
 Prints ONE JSON line.
 """
@@ -31,14 +33,14 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
 # `--pmc WRITE_SIZE` (KiB per dispatch), each scaled by what the same counter reads for a plain
 # device copy of known size (FETCH_SIZE reads 0.50x, WRITE_SIZE 1.00x):
 # profiles/bench_dense_int8_M4096_K8192_N8192_and_int4_decode.md
-GEMM_HBM_TRAFFIC_BYTES = int((196835.4 * 2.0 + 83429.4) * 1024)
-QUANT_HBM_TRAFFIC_BYTES = int((32812.2 * 2.0 + 32832.0) * 1024)
+GEMM_HBM_TRAFFIC_BYTES = int((196814.6 * 2.0 + 90450.7) * 1024)
+QUANT_HBM_TRAFFIC_BYTES = int((32830.5 * 2.0 + 32832.0) * 1024)
 # int4 decode main kernel, keyed by (M > 8, grouped)
 GEMV_HBM_TRAFFIC_BYTES = {
-    (False, False): int((16600.1 * 2.0 + 640.0) * 1024),
-    (False, True): int((17411.1 * 2.0 + 640.0) * 1024),
-    (True, False): int((17472.0 * 2.0 + 4096.0) * 1024),
-    (True, True): int((34648.5 * 2.0 + 2048.0) * 1024),
+    (False, False): int((16601.6 * 2.0 + 1280.0) * 1024),
+    (False, True): int((17419.6 * 2.0 + 640.0) * 1024),
+    (True, False): int((17477.0 * 2.0 + 4096.0) * 1024),
+    (True, True): int((18469.1 * 2.0 + 2048.0) * 1024),
 }
 
 
@@ -257,7 +259,7 @@ def main():
                                "glorot-uniform kernel quantized per channel, kernel prepacked once"},
         "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": INT8_PEAK_TOPS,
                      "unit": "TFLOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 4),
-                     "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "gemm_i8_mfma",
+                     "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "gemm_mfma<int8>",
                      "avg_launch_us": round(gemm_ms * 1e3, 1), "ops_per_launch": ops_per_step,
                      "note": "int8 multiply-accumulate counted as 2 ops; peak is the published dense int8 figure"},
         "quantizer": {"kernel": "quantize_rows_vec", "avg_launch_us": round(quant_ms * 1e3, 1),
