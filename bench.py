@@ -4,10 +4,10 @@
 
 One "step" is one forward pass of an int8-quantized Dense layer over one batch:
 the fused abs-max activation quantizer followed by the int8 MFMA GEMM with the
-de-scale epilogue, at BASELINE's target shape M=4096, K=N=8192, bfloat16
+de-scale epilogue, at the target shape M=4096, K=N=8192, bfloat16
 activations (inputs and weights already resident in HBM).  `value` is
 2*M*N*K / step time in TOP/s.  The int4 decode GEMV (K=N=8192, M in {1,4,16}),
-the second half of BASELINE's metric, is reported under `int4_gemv` with its own
+the second half of the headline metric, is reported under `int4_gemv` with its own
 HBM roofline; `llama_decode_int4` is the end-to-end greedy decode of a 32-layer
 Llama-style decoder whose weight matrices are all int4 (tokens/s at batch 1 and 8).
 The CPU oracle (a restatement of the reference's torch-CPU op sequence) is timed

@@ -63,7 +63,7 @@ def test_int4_matmul_small(dev, M, K, N, block_size, dtype):
 @pytest.mark.parametrize("M", [1, 4, 16])
 @pytest.mark.parametrize("block_size", [None, 128])
 def test_int4_decode_config(dev, M, block_size):
-    # BASELINE config 2: K = N = 8192, bf16 inputs, M in {1, 4, 16}
+    # target configuration 2: K = N = 8192, bf16 inputs, M in {1, 4, 16}
     run_case(dev, M, 8192, 8192, block_size, torch.bfloat16, with_bias=False)
 
 

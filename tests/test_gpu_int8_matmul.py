@@ -65,7 +65,7 @@ def test_dense_int8_fast_epilogue(dev, M, K, N, dtype):
 
 
 def test_config1_dense_4096(dev):
-    # BASELINE config 1: Dense(4096) on [16, 4096] float32 inputs, bias, seed 0
+    # target configuration 1: Dense(4096) on [16, 4096] float32 inputs, bias, seed 0
     run_dense_int8(dev, 16, 4096, 4096, torch.float32, prepack=True, exact=True, seed=0)
 
 
@@ -84,7 +84,7 @@ def test_gemm_extreme_values(dev):
 
 @pytest.mark.parametrize("M,K,N", [(4096, 8192, 8192), (2048, 4096, 4096), (512, 8192, 28672)])
 def test_gemm_full_size_accumulators(dev, M, K, N):
-    # full BASELINE sizes: sampled rows against the CPU oracle (bit-exact) plus two
+    # full target sizes: sampled rows against the CPU oracle (bit-exact) plus two
     # size-independent integer identities over the whole output
     g = torch.Generator().manual_seed(7)
     a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)

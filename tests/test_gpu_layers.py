@@ -114,7 +114,7 @@ def test_variables_reload_round_trip(dev):
 
 
 EQUATIONS = [
-    # equation, output_shape, input_shape  (einsum_dense_test.py:556-691 and BASELINE config 4 shapes, scaled)
+    # equation, output_shape, input_shape  (einsum_dense_test.py:556-691 and the target attention-projection shapes, scaled)
     ("btnh,nhd->btd", (None, 8), (1, 2, 2, 4)),
     ("btd,ndh->btnh", (None, 2, 8), (1, 2, 4)),
     ("btd,df->btf", (None, 4), (1, 2, 4)),
@@ -174,7 +174,7 @@ def test_einsum_dense_int4(dev, equation, output_shape, input_shape, block_size)
 
 @pytest.mark.parametrize("t", [1, 512])
 def test_config4_attention_projections(dev, t):
-    # BASELINE config 4: d_model 4096, 32 heads x 128, batch 8, bf16
+    # target configuration 4: d_model 4096, 32 heads x 128, batch 8, bf16
     g = torch.Generator().manual_seed(4)
     for equation, out_shape, in_shape in [
         ("btd,dnh->btnh", (None, 32, 128), (8, t, 4096)),
