@@ -122,7 +122,7 @@ int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64
 
 /*
  * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; 16-row
- * passes up to M = 255; from M = 256 on, for bfloat16 x with K % 128 == 0 and
+ * passes up to M = 127; from M = 128 on, for bfloat16 x with K % 128 == 0 and
  * N % 64 == 0, the kernel is de-quantised once into `workspace` as bfloat16 [N, K]
  * and the product runs on the MFMA tile kernel):
  *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)

@@ -24,32 +24,44 @@
 namespace k3q {
 namespace {
 
-constexpr int kBM = 256;  // tile rows of a / y
-constexpr int kBN = 256;  // tile rows of the prepacked weight = columns of y
 constexpr int kBK = 128;  // bytes of K per stage: one full 128-byte line per row
 constexpr int kStages = 2;
 constexpr int kKSteps = kBK / 32;  // MFMA K steps per stage
+constexpr int kRowChunks = kBK / 16;  // 16-byte chunks per LDS row
 #ifndef K3Q_GEMM_WAVES_N
 #define K3Q_GEMM_WAVES_N 4
 #define K3Q_GEMM_WAVES_M 2
 #endif
-constexpr int kWavesN = K3Q_GEMM_WAVES_N;  // waves along N
-constexpr int kWavesM = K3Q_GEMM_WAVES_M;  // waves along M
-constexpr int kThreads = 64 * kWavesN * kWavesM;
-constexpr int kWN = kBN / kWavesN;  // 64 columns per wave
-constexpr int kWM = kBM / kWavesM;  // 128 rows per wave
-constexpr int kNBlk = kWN / 32;     // 2 MFMA blocks along N per wave
-constexpr int kMBlk = kWM / 32;     // 4 MFMA blocks along M per wave
-constexpr int kTileBytes = kBM * kBK;             // 16 KiB per operand tile
-constexpr int kStageBytes = 2 * kTileBytes;       // 32 KiB
-constexpr int kLdsBytes = kStages * kStageBytes;  // 128 KiB
-constexpr int kDmaPerTile = kTileBytes / 1024;                        // 32 DMA instructions per operand tile
-constexpr int kDmaPerWave = (2 * kDmaPerTile) / (kThreads / 64);      // 8 per wave per stage
-constexpr int kRowChunks = kBK / 16;                                  // 16-byte chunks per LDS row
+
+// Tile shape of a workgroup: BM rows of a / y, BN rows of the prepacked weight (= columns of
+// y), waves laid out WN (along N) x WM (along M).
+template <int BM, int BN, int WN_, int WM_>
+struct Tile {
+    static constexpr int kBM = BM, kBN = BN, kWavesN = WN_, kWavesM = WM_;
+    static constexpr int kThreads = 64 * WN_ * WM_;
+    static constexpr int kWN = BN / WN_;      // columns per wave
+    static constexpr int kWM = BM / WM_;      // rows per wave
+    static constexpr int kNBlk = kWN / 32;    // MFMA blocks along N per wave
+    static constexpr int kMBlk = kWM / 32;    // MFMA blocks along M per wave
+    static constexpr int kATileBytes = BM * kBK;
+    static constexpr int kBTileBytes = BN * kBK;
+    static constexpr int kStageBytes = kATileBytes + kBTileBytes;
+    static constexpr int kLdsBytes = kStages * kStageBytes;
+    static constexpr int kDmaA = kATileBytes / 1024;  // DMA instructions (1 KiB each) per A tile
+    static constexpr int kDmaB = kBTileBytes / 1024;
+    static constexpr int kDmaPerWave = (kDmaA + kDmaB) / (kThreads / 64);
+};
+// 256 x 256, 8 waves, 128 KiB of LDS: one workgroup per CU; the shape for large problems.
+typedef Tile<256, 256, K3Q_GEMM_WAVES_N, K3Q_GEMM_WAVES_M> TileLarge;
+// 128 x 128, 4 waves, 64 KiB of LDS: two workgroups per CU; used while the large tile would
+// leave CUs without work.
+typedef Tile<128, 128, 2, 2> TileSmall;
 
 constexpr int kFlagExactEpilogue = 1;
 constexpr int kFlagRoundAccBF16 = 2;   // float32 output of a bfloat16 layer: acc is cast to bfloat16 first
 constexpr int kFlagSkipEpilogue = 1024;  // undocumented timing aid
+constexpr int kFlagForceSmallTile = 2048;  // undocumented tuning aids
+constexpr int kFlagForceLargeTile = 4096;
 
 struct GemmParams {
     const int8_t* a;        // [M, K]
@@ -74,6 +86,7 @@ __device__ __forceinline__ int swz(int row) {
 
 // gfx9 s_waitcnt encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]
 __device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+template <int kDmaPerWave>
 __device__ __forceinline__ void wait_vmcnt_one_stage() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kDmaPerWave & 0xF) | ((kDmaPerWave >> 4) << 14));
 }
@@ -114,8 +127,12 @@ struct Mma<kKindBF16> {
     }
 };
 
-template <int kKind, bool kBF16, bool kExact>
-__global__ __launch_bounds__(kThreads) void gemm_mfma(GemmParams p) {
+template <class T, int kKind, bool kBF16, bool kExact>
+__global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
+    constexpr int kBM = T::kBM, kBN = T::kBN, kWavesN = T::kWavesN, kThreads = T::kThreads;
+    constexpr int kWN = T::kWN, kWM = T::kWM, kNBlk = T::kNBlk, kMBlk = T::kMBlk;
+    constexpr int kATileBytes = T::kATileBytes, kStageBytes = T::kStageBytes;
+    constexpr int kDmaA = T::kDmaA, kDmaPerWave = T::kDmaPerWave;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 #ifdef K3Q_GEMM_PROBE_CLOCK
     const uint64_t clk0 = __builtin_readcyclecounter();
@@ -146,13 +163,14 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma(GemmParams p) {
 
     // ---- DMA source addresses ----
     // DMA instruction d of this wave fills LDS bytes [(wave * kDmaPerWave + d) * 1024, +1024) of
-    // the stage: 8 rows x 128 B.  Instructions 0..31 of a stage are the A tile, 32..63 the B tile.
+    // the stage: 8 rows x 128 B.  The first kDmaA instructions of a stage are the A tile, the
+    // rest the B tile.
     const char* src[kDmaPerWave];
 #pragma unroll
     for (int d = 0; d < kDmaPerWave; ++d) {
         const int inst = wave * kDmaPerWave + d;
-        const bool is_b = inst >= kDmaPerTile;
-        const int row = (inst % kDmaPerTile) * 8 + lane / kRowChunks;
+        const bool is_b = inst >= kDmaA;
+        const int row = (is_b ? inst - kDmaA : inst) * 8 + lane / kRowChunks;
         const int chunk = (lane & (kRowChunks - 1)) ^ swz(row);
         int64_t grow = (is_b ? n0 : m0) + row;
         const int64_t lim = (is_b ? p.N : p.M) - 1;
@@ -184,7 +202,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma(GemmParams p) {
 #pragma unroll
     for (int nb = 0; nb < kNBlk; ++nb) {
         const int row = wn * kWN + nb * 32 + fi;
-        b_row[nb] = kTileBytes + row * kBK;
+        b_row[nb] = kATileBytes + row * kBK;
         b_swz[nb] = swz(row);
     }
     v4i af[2][kMBlk], bf[2][kNBlk];
@@ -216,7 +234,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma(GemmParams p) {
     issue_stage(0);
     if (KT > 1) {
         issue_stage(1);
-        wait_vmcnt_one_stage();
+        wait_vmcnt_one_stage<kDmaPerWave>();
     } else {
         wait_vmcnt0();
     }
@@ -442,22 +460,32 @@ __global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ i
     }
 }
 
-bool g_lds_attr_set[8] = {};
+template <class T, int kKind, bool kBF16, bool kExact>
+int launch_tile(GemmParams p, hipStream_t s) {
+    // more than 64 KiB of dynamic LDS needs the attribute raised once per kernel
+    static const bool raised =
+        hipFuncSetAttribute((const void*)gemm_mfma<T, kKind, kBF16, kExact>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes) == hipSuccess;
+    if (!raised) return K3Q_ERR_LAUNCH;
+    p.tiles_m = (int)((p.M + T::kBM - 1) / T::kBM);
+    p.tiles_n = (int)((p.N + T::kBN - 1) / T::kBN);
+    const int total = p.tiles_m * p.tiles_n;
+    const int grid = ((total + 7) / 8) * 8;
+    gemm_mfma<T, kKind, kBF16, kExact><<<grid, T::kThreads, T::kLdsBytes, s>>>(p);
+    return launch_status();
+}
+
+// The large tile needs about one tile per CU to pay off; below that the small tile (four
+// times as many workgroups, two per CU) keeps the chip busy.
+constexpr int64_t kLargeTileMinTiles = 224;
 
 template <int kKind, bool kBF16, bool kExact>
 int launch_mfma(const GemmParams& p, hipStream_t s) {
-    // 128 KiB of dynamic LDS needs the attribute raised once per kernel (idempotent).
-    constexpr int slot = (kBF16 ? 1 : 0) + (kExact ? 2 : 0) + 4 * kKind;
-    if (!g_lds_attr_set[slot]) {
-        if (hipFuncSetAttribute((const void*)gemm_mfma<kKind, kBF16, kExact>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
-            return K3Q_ERR_LAUNCH;
-        g_lds_attr_set[slot] = true;
-    }
-    const int total = p.tiles_m * p.tiles_n;
-    const int grid = ((total + 7) / 8) * 8;
-    gemm_mfma<kKind, kBF16, kExact><<<grid, kThreads, kLdsBytes, s>>>(p);
-    return launch_status();
+    const int64_t large_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
+    const bool large = (p.flags & kFlagForceLargeTile) ||
+                       (large_tiles >= kLargeTileMinTiles && !(p.flags & kFlagForceSmallTile));
+    if (large) return launch_tile<TileLarge, kKind, kBF16, kExact>(p, s);
+    return launch_tile<TileSmall, kKind, kBF16, kExact>(p, s);
 }
 
 }  // namespace
@@ -465,7 +493,7 @@ int launch_mfma(const GemmParams& p, hipStream_t s) {
 bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* bt,
                             const void* y) {
     return M > 0 && (2 * K) % kBK == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(bt, 16) &&
-           aligned_to(y, 8) && ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) < (1 << 28);
+           aligned_to(y, 8) && ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);
 }
 
 int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
@@ -480,8 +508,6 @@ int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_
     p.N = N;
     p.K = K;
     p.row_bytes = 2 * K;
-    p.tiles_m = (int)((M + kBM - 1) / kBM);
-    p.tiles_n = (int)((N + kBN - 1) / kBN);
     return launch_mfma<kKindBF16, true, true>(p, s);
 }
 
@@ -535,8 +561,6 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     p.K = K;
     p.row_bytes = K;
     p.flags = flags;
-    p.tiles_m = (int)((M + kBM - 1) / kBM);
-    p.tiles_n = (int)((N + kBN - 1) / kBN);
 
     const size_t el = bf16 ? 2 : 4;
     // decode-sized M: bandwidth-bound kernel that reads the [K,N] kernel in place
@@ -549,7 +573,7 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     bool fast = (K % kBK) == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
                 (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
                 (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&
-                (int64_t)p.tiles_m * p.tiles_n < (1 << 28);
+                ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);
     if (fast && b_layout == 0) {
         // needs the [N,K] copy: made here per call when the caller supplies scratch for it
         if (workspace && workspace_bytes >= N * K && aligned_to(workspace, 16)) {

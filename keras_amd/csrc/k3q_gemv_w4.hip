@@ -546,9 +546,9 @@ __global__ __launch_bounds__(256) void dequant_w4_to_bf16_nk(const uint8_t* __re
     }
 }
 
-// Below this the GEMM has too few 256-row tiles to fill the chip and the 16-row decode passes
-// are faster (M = 128, K = N = 4096: 72 us in passes, 119 us on the GEMM route).
-constexpr int64_t kGemmMinRows = 256;
+// Below this the 16-row decode passes are faster (K = N = 4096: 51 us at 64 rows; at 128 rows
+// the passes take 96 us, de-quantise + GEMM 67 us).
+constexpr int64_t kGemmMinRows = 128;
 
 inline bool gemm_route_ok(int x_dtype, int64_t M, int64_t K, int64_t N) {
     return x_dtype == K3Q_BF16 && M >= kGemmMinRows && (K % kDqK) == 0 && (N % kDqN) == 0;

@@ -96,10 +96,10 @@ def test_int4_repeatable(dev):
         assert torch.equal(first, again)
 
 
-# prefill sizes: bfloat16 inputs with M >= 256, K % 128 == 0, N % 64 == 0 take the
+# prefill sizes: bfloat16 inputs with M >= 128, K % 128 == 0, N % 64 == 0 take the
 # de-quantise + MFMA GEMM route; everything else stays on the 16-row passes
 @pytest.mark.parametrize("M,K,N,block_size", [
-    (256, 128, 64, None), (256, 256, 128, 128), (300, 512, 320, 64), (257, 1024, 512, 32),
+    (128, 128, 64, None), (129, 256, 128, 128), (300, 512, 320, 64), (257, 1024, 512, 32),
     (1024, 4096, 4096, 128), (512, 4096, 14336, 128), (300, 2048, 1024, -1), (260, 384, 192, 128),
     (1000, 256, 64, 256),
 ])
@@ -111,7 +111,7 @@ def test_int4_prefill_route(dev, M, K, N, block_size):
     (300, 256, 128, 128, torch.float32),   # float32: not on the GEMM route
     (300, 192, 128, 64, torch.bfloat16),   # K % 128 != 0
     (280, 256, 96, None, torch.bfloat16),  # N % 64 != 0
-    (200, 256, 128, 128, torch.bfloat16),  # M below the GEMM threshold
+    (100, 256, 128, 128, torch.bfloat16),  # M below the GEMM threshold
 ])
 def test_int4_large_m_off_route(dev, M, K, N, block_size, dtype):
     run_case(dev, M, K, N, block_size, dtype, with_bias=True)
