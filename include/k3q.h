@@ -98,10 +98,12 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  * flags bit 1 (K3Q_GEMM_ROUND_ACC_BF16, float32 output only): acc is cast to bfloat16
  * before the division, which is what a bfloat16-compute layer with float32 scales
  * computes (ReversibleEmbedding reads its scale without autocast).
- * Decode sizes (M <= 64) run bandwidth-bound kernels that read b once, in either
- * layout (b_layout 0: N % 16 == 0, K % 8 == 0; b_layout 1, e.g. a tied int8
- * embedding table used as the LM head: K % 64 == 0), always with the exact
- * epilogue; they may split K and then need `workspace` for int32 partials.
+ * Decode sizes run bandwidth-bound kernels that stream b in place, always with the
+ * exact epilogue: b_layout 0 up to 64 rows (N % 16 == 0, K % 8 == 0; passes of 16
+ * rows), b_layout 1 -- e.g. a tied int8 embedding table used as the LM head -- up to
+ * 16 rows (K % 64 == 0; up to 64 rows when the MFMA kernel's conditions do not hold).
+ * They may split K and then need `workspace` for int32 partials.  The MFMA kernel
+ * itself picks 128 x 128 tiles while 256 x 256 tiles would leave CUs idle.
  * The reverse projection of ReversibleEmbedding._int8_call
  * (keras/src/layers/core/reversible_embedding.py:272-296) is this call with
  * b = the [vocab, dim] table as stored, b_layout 1 and no bias.

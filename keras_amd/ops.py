@@ -89,8 +89,9 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
 
 
 GEMM_EXACT_EPILOGUE = 1
-# up to this many rows the int8 matmul is bandwidth-bound and reads the [K, N] kernel in place
-SKINNY_MAX_ROWS = 64
+# up to this many rows the int8 matmul streams the [K, N] kernel in place (passes of 16 rows);
+# above, the prepacked copy on 128-row MFMA tiles is faster
+SKINNY_MAX_ROWS = 32
 
 
 def prepack_int8_kernel(kernel):
@@ -190,7 +191,7 @@ def int8_matmul_nk(a, kernel_nk, a_scale=None, kernel_scale=None, out_dtype=None
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
     lib = _lib.load()
     ws, ws_bytes = None, 0
-    if M <= SKINNY_MAX_ROWS:
+    if M <= 64:  # the decode kernels may split K and then need room for int32 partials
         ws = _workspace(a.device, lib.k3q_gemm_i8_workspace_bytes(M, N, K))
         ws_bytes = ws.numel()
     rc = lib.k3q_gemm_i8(
