@@ -83,8 +83,9 @@ class DecoderBlock(Layer):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
         (an int64 device tensor [T]); mask [T, maxT] True where a key may be attended to."""
         h = self.attn_norm(x)
-        q = apply_rope(self.query(h), cos, sin)
-        k = apply_rope(self.key(h), cos, sin)
+        # one rotation over the query and key heads together (half the elementwise launches)
+        qk = apply_rope(torch.cat((self.query(h), self.key(h)), dim=2), cos, sin)
+        q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
         v = self.value(h)
         kc, vc = cache
         kc.index_copy_(2, pos, k.transpose(1, 2))
