@@ -123,6 +123,24 @@ int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64
                 void* stream);
 
 /*
+ * Weight-only int8 matmul: float activations, int8 kernel (a Dense int8 layer whose
+ * config has no activation quantizer):
+ *     y = T(T(x . b) / b_scale[n]) (+ bias)
+ * x: [M, K] float32 or bfloat16; b as in k3q_gemm_i8 ([K,N] with b_layout 0, the
+ * prepacked [N,K] with b_layout 1); b_scale, bias, y of x_dtype.  bfloat16 x with
+ * K % 64 == 0, N % 4 == 0 and `workspace` (k3q_gemm_w8_workspace_bytes, 16-byte
+ * aligned) widens the kernel to bfloat16 in scratch (exact) and runs the MFMA tile
+ * kernel; everything else runs a plain kernel with fp32 accumulation.
+ * Replaces matmul (float x int8: both cast to the float type,
+ * keras/src/backend/torch/numpy.py:139-157), cast, divide, add of Dense._int8_call
+ * without inputs_quantizer (keras/src/layers/core/dense.py:961-983).
+ */
+int64_t k3q_gemm_w8_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64_t M, int64_t N,
+                int64_t K, const void* b_scale, const void* bias, void* y, void* workspace,
+                int64_t workspace_bytes, void* stream);
+
+/*
  * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; 16-row
  * passes up to M = 127; from M = 128 on, for bfloat16 x with K % 128 == 0 and
  * N % 64 == 0, the kernel is de-quantised once into `workspace` as bfloat16 [N, K]
@@ -152,7 +170,7 @@ int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
 
 /*
  * Same as k3q_gemv_w4 with the launch plan overridden, for tuning sweeps:
- * plan = {dwords per lane per k row (1|2|4), 16-row steps per chunk (1|2),
+ * plan = {dwords per lane per k row (1|2), 16-row steps per chunk (1|2),
  * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null
  * `plan` keep the built-in choice.  The workspace must then hold
  * ceil(K / (waves * rows per wave)) * min(M, 16) * N floats.  No counterpart in the reference.

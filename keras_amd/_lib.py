@@ -49,6 +49,11 @@ SIGNATURES = {
         [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _int, _int, _ptr, _ptr, _ptr,
          _i64, _ptr],
     ),
+    "k3q_gemm_w8_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "k3q_gemm_w8": (
+        _int,
+        [_ptr, _int, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr],
+    ),
     "k3q_gemv_w4_nk": (
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _int, _ptr, _i64, _ptr, _ptr],

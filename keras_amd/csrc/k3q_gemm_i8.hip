@@ -460,6 +460,71 @@ __global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ i
     }
 }
 
+// ---- weight-only int8: the int8 kernel widened to bfloat16 [N, K] in scratch (exact) ----
+// [N, K] int8 -> [N, K] bfloat16, 16 values per thread
+__global__ __launch_bounds__(256) void widen_i8_to_bf16(const int8_t* __restrict__ in,
+                                                        uint16_t* __restrict__ out, int64_t count16) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count16) return;
+    const v4u v = *(const v4u*)(in + i * 16);
+    v4u o[2];
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        const u32 lo = f32_to_bf16_bits((float)(int)(int8_t)(v[e >> 2] >> (8 * (e & 3))));
+        const u32 hi = f32_to_bf16_bits((float)(int)(int8_t)(v[(e + 1) >> 2] >> (8 * ((e + 1) & 3))));
+        o[e >> 3][(e & 7) >> 1] = lo | (hi << 16);
+    }
+    v4u* dst = (v4u*)(out + i * 16);
+    dst[0] = o[0];
+    dst[1] = o[1];
+}
+
+// [K, N] int8 -> [N, K] bfloat16 through a padded LDS tile
+__global__ __launch_bounds__(256) void transpose_widen_i8_to_bf16(const int8_t* __restrict__ in,
+                                                                  uint16_t* __restrict__ out,
+                                                                  int64_t K, int64_t N) {
+    __shared__ int8_t tile[64][64 + 4];
+    const int64_t k0 = (int64_t)blockIdx.y * 64;
+    const int64_t n0 = (int64_t)blockIdx.x * 64;
+    for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+        const int r = e / 64, c = e % 64;
+        int8_t v = 0;
+        if (k0 + r < K && n0 + c < N) v = in[(k0 + r) * N + n0 + c];
+        tile[r][c] = v;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+        const int r = e / 64, c = e % 64;  // r: n within tile, c: k within tile
+        if (n0 + r < N && k0 + c < K)
+            out[(n0 + r) * K + k0 + c] = (uint16_t)f32_to_bf16_bits((float)tile[c][r]);
+    }
+}
+
+// Any shape and dtype: one thread per output, fp32 accumulation.
+template <bool kBF16>
+__global__ __launch_bounds__(256) void gemm_w8_simple(const void* x, const int8_t* b,
+                                                      int64_t b_stride_k, int64_t b_stride_n,
+                                                      const void* scale, const void* bias, void* y,
+                                                      int64_t N, int64_t K) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t m = blockIdx.y;
+    if (n >= N) return;
+    float acc = 0.f;
+    for (int64_t k = 0; k < K; ++k)
+        acc = fmaf(load_t<kBF16>(x, m * K + k), (float)b[k * b_stride_k + n * b_stride_n], acc);
+    if (kBF16) {
+        float r = round_bf16(acc);
+        if (scale) r = round_bf16(r / load_t<true>(scale, n));
+        if (bias) r = round_bf16(r + load_t<true>(bias, n));
+        ((uint16_t*)y)[m * N + n] = (uint16_t)f32_to_bf16_bits(r);
+    } else {
+        float r = acc;
+        if (scale) r = r / load_t<false>(scale, n);
+        if (bias) r = r + load_t<false>(bias, n);
+        ((float*)y)[m * N + n] = r;
+    }
+}
+
 template <class T, int kKind, bool kBF16, bool kExact>
 int launch_tile(GemmParams p, hipStream_t s) {
     // more than 64 KiB of dynamic LDS needs the attribute raised once per kernel
@@ -605,5 +670,45 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
         gemm_i8_simple<true><<<grid, 256, 0, s>>>(a, b, sk, sn, p);
     else
         gemm_i8_simple<false><<<grid, 256, 0, s>>>(a, b, sk, sn, p);
+    return launch_status();
+}
+
+extern "C" int64_t k3q_gemm_w8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return N * K * 2;  // the kernel widened to bfloat16
+}
+
+extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64_t M,
+                           int64_t N, int64_t K, const void* b_scale, const void* bias, void* y,
+                           void* workspace, int64_t workspace_bytes, void* stream) {
+    if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || N <= 0 || K <= 0) return K3Q_ERR_SHAPE;
+    if (b_layout != 0 && b_layout != 1) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (!x || !b || !y) return K3Q_ERR_NULL;
+    hipStream_t s = (hipStream_t)stream;
+    const bool bf16 = x_dtype == K3Q_BF16;
+    const bool fast = bf16 && workspace && workspace_bytes >= N * K * 2 && aligned_to(workspace, 16) &&
+                      aligned_to(b, 16) && (!b_scale || aligned_to(b_scale, 2)) &&
+                      gemm_bf16_nk_supported(M, N, K, x, workspace, y) && (K % 16) == 0;
+    if (fast) {
+        if (b_layout == 1) {
+            const int64_t count16 = N * K / 16;
+            widen_i8_to_bf16<<<(unsigned)((count16 + 255) / 256), 256, 0, s>>>(b, (uint16_t*)workspace,
+                                                                              count16);
+        } else {
+            dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
+            transpose_widen_i8_to_bf16<<<grid, 256, 0, s>>>(b, (uint16_t*)workspace, K, N);
+        }
+        return gemm_bf16_nk_run(x, workspace, M, N, K, b_scale, bias, y, s);
+    }
+    if (M > 65535) return K3Q_ERR_SHAPE;
+    dim3 grid((unsigned)((N + 255) / 256), (unsigned)M);
+    const int64_t sk = b_layout == 0 ? N : 1;
+    const int64_t sn = b_layout == 0 ? 1 : K;
+    if (bf16)
+        gemm_w8_simple<true><<<grid, 256, 0, s>>>(x, b, sk, sn, b_scale, bias, y, N, K);
+    else
+        gemm_w8_simple<false><<<grid, 256, 0, s>>>(x, b, sk, sn, b_scale, bias, y, N, K);
     return launch_status();
 }

@@ -96,11 +96,7 @@ struct Packed {
 template <int kVec>
 __device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
     Packed<kVec> r;
-    if (kVec == 4) {
-        v4u v = __builtin_nontemporal_load((const v4u*)p);
-#pragma unroll
-        for (int q = 0; q < kVec; ++q) r.d[q] = v[q];
-    } else if (kVec == 2) {
+    if (kVec == 2) {
         v2u v = __builtin_nontemporal_load((const v2u*)p);
 #pragma unroll
         for (int q = 0; q < kVec; ++q) r.d[q] = v[q];
@@ -585,7 +581,7 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     int vec = (grouped && pl.sets == 2) ? 1 : 2;
     if (plan_override && plan_override[0] > 0) vec = plan_override[0];
     while (vec > 1 && (N % (8 * vec)) != 0) vec >>= 1;
-    if (vec != 1 && vec != 2 && vec != 4) vec = 1;
+    if (vec != 1 && vec != 2) vec = vec > 2 ? 2 : 1;  // 16-byte loads per lane lost every sweep
     pl.vec = vec;
 
     int steps = 2;
@@ -670,8 +666,6 @@ void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, bool g
                  int threads, size_t lds, hipStream_t s) {
     const int key = pl.vec * 10 + pl.steps;
     switch (key) {
-        case 42: launch2<4, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
-        case 41: launch2<4, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
         case 22: launch2<2, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
         case 21: launch2<2, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
         case 12: launch2<1, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;

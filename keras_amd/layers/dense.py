@@ -216,9 +216,16 @@ class Dense(Layer):
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized Dense is outside this inference path.")
         if not self.inputs_quantizer:
-            raise NotImplementedError(
-                "Weight-only int8 (no activation quantizer) is not on the fused path yet."
+            # weight-only: float activations against the int8 kernel, then the de-scale
+            y = kops.int8_weight_only_matmul(
+                inputs, as_tensor(self._kernel),
+                self._read_cached("kernel_scale", self.kernel_scale),
+                bias=self._read_cached("bias", self.bias),
+                prepacked=self._cached("prepacked", self._kernel, kops.prepack_int8_kernel),
             )
+            if self.activation is not None:
+                y = self.activation(y)
+            return y
         lead = inputs.shape[:-1]
         x2 = inputs.reshape(-1, inputs.shape[-1])
         q, scale = self.inputs_quantizer(x2, axis=-1)
@@ -244,12 +251,30 @@ class Dense(Layer):
         consumed in place (no unpack, no de-quantised copy)."""
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized Dense is outside this inference path.")
-        if self.inputs_quantizer:
-            raise NotImplementedError(
-                "int4 with an activation quantizer is not on the fused path yet."
-            )
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
+        if self.inputs_quantizer:
+            if grouped:
+                raise NotImplementedError(
+                    "Grouped int4 with an activation quantizer has no counterpart in the "
+                    "reference (dense.py:1040-1084 ignores the quantizer there)."
+                )
+            # activation-quantized, per-channel (dense.py:1023-1031): int8 rows against the
+            # nibbles unpacked to int8 in scratch, exact int32 accumulation, one de-scale
+            lead = inputs.shape[:-1]
+            x2 = inputs.reshape(-1, inputs.shape[-1])
+            q, scale = self.inputs_quantizer(x2, axis=-1)
+            unpacked = quantizers.unpack_int4(as_tensor(self._kernel), self._orig_output_dim, axis=-1)
+            y = kops.int8_matmul(
+                q, unpacked, a_scale=scale,
+                kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
+                bias=self._read_cached("bias", self.bias),
+                out_dtype=to_torch_dtype(self.compute_dtype), exact_epilogue=True,
+            )
+            y = y.reshape(*lead, self._orig_output_dim)
+            if self.activation is not None:
+                y = self.activation(y)
+            return y
         y = kops.int4_matmul(
             inputs, as_tensor(self._kernel),
             self._read_cached("kernel_scale", self.kernel_scale), self._orig_output_dim,

@@ -285,3 +285,32 @@ def int4_matmul_nk(x, table_packed, scale, zero=None, block_size=None):
     )
     _lib.check(rc, "k3q_gemv_w4_nk")
     return y.reshape(*lead, N)
+
+
+def int8_weight_only_matmul(x, kernel, kernel_scale, bias=None, prepacked=None):
+    """`x[..., K] (float) . kernel[K, N] (int8)` with the per-channel de-scale:
+    `y = T(T(x . W) / kernel_scale) + bias` -- a Dense int8 layer without an activation
+    quantizer (keras/src/layers/core/dense.py:961-983).  Scale and bias in x.dtype."""
+    _lib.require_device(x, kernel, kernel_scale, bias, prepacked)
+    code = _lib.dtype_code(x.dtype)
+    K, N = kernel.shape
+    if x.shape[-1] != K:
+        raise ValueError(f"last axis of the input ({x.shape[-1]}) does not match the kernel ({K})")
+    if kernel_scale.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise TypeError("kernel_scale and bias must be read in the input's dtype")
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    if prepacked is not None:
+        b, layout = prepacked, 1
+    else:
+        b, layout = (kernel if kernel.is_contiguous() else kernel.contiguous()), 0
+    lib = _lib.load()
+    ws = _workspace(x.device, lib.k3q_gemm_w8_workspace_bytes(M, N, K))
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    rc = lib.k3q_gemm_w8(_lib.ptr(x2), code, _lib.ptr(b), layout, M, N, K,
+                         _lib.ptr(kernel_scale.reshape(-1).contiguous()), _lib.ptr(bias), _lib.ptr(y),
+                         _lib.ptr(ws), ws.numel(), _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemm_w8")
+    return y.reshape(*lead, N)

@@ -209,3 +209,49 @@ def test_unsupported_paths_raise(dev):
     cpu_layer.quantize("int8")
     with pytest.raises(RuntimeError):
         cpu_layer(torch.randn(2, 32))  # no CPU fallback
+
+
+# ---- non-default configs: weight-only int8, activation-quantized int4 --------------------
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16", "bfloat16"])
+@pytest.mark.parametrize("M,K,N", [(16, 4096, 4096), (5, 128, 48), (300, 256, 512), (2, 100, 30),
+                                   (700, 1024, 2048)])
+def test_dense_int8_weight_only(dev, policy, M, K, N):
+    layer = build_dense(dev, K, N, policy, seed=5)
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(6))
+    layer.quantize("int8", config=ka.Int8QuantizationConfig(activation_quantizer=None))
+    assert layer.inputs_quantizer is None
+    qk, ks = ref.dense_quantize_int8(kernel_f)
+    assert torch.equal(layer._kernel.value.cpu(), qk)
+    y = layer(x)
+    want = ref.dense_int8_call(x.to(cd), qk, ks, bias_f, compute_dtype=cd, quantize_inputs=False)
+    assert y.dtype == cd and tuple(y.shape) == (M, N)
+    assert max_rel_err(y, want) <= RTOL[cd]
+    # and against the exact value: float64 matmul of the same operands
+    exact = (x.to(cd).double() @ qk.double()) / ks.to(cd).double() + bias_f.to(cd).double()
+    assert max_rel_err(y, exact) <= RTOL[cd]
+
+
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 512), (16, 512, 384), (7, 300, 64), (40, 256, 96),
+                                   (300, 512, 256)])
+def test_dense_int4_activation_quantized(dev, policy, M, K, N):
+    layer = build_dense(dev, K, N, policy, seed=7)
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(8))
+    config = ka.Int4QuantizationConfig(block_size=None, activation_quantizer=ka.quantizers.AbsMaxQuantizer())
+    layer.quantize("int4", config=config)
+    assert layer.inputs_quantizer is not None
+    qk = ref.dense_quantize_int4(kernel_f, None)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    y = layer(x)
+    want, inter = ref.dense_int4_call(
+        x.to(cd), qk["kernel"], qk["kernel_scale"], N, block_size=None, bias=bias_f,
+        compute_dtype=cd, quantize_inputs=True, return_intermediates=True)
+    assert inter["acc"].dtype == torch.int32
+    # integer accumulation and the exact epilogue: bit-identical to the reference chain
+    assert y.dtype == cd and torch.equal(bits(y.cpu()), bits(want))
