@@ -141,8 +141,8 @@ int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64
                 int64_t workspace_bytes, void* stream);
 
 /*
- * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; 16-row
- * passes up to M = 127; from M = 128 on, for bfloat16 x with K % 128 == 0 and
+ * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; passes of
+ * 32 rows (bfloat16) or 8 rows (float32) up to M = 127; from M = 128 on, for bfloat16 x with K % 128 == 0 and
  * N % 64 == 0, the kernel is de-quantised once into `workspace` as bfloat16 [N, K]
  * and the product runs on the MFMA tile kernel):
  *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)
@@ -160,7 +160,7 @@ int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64
  * irrelevant.  It holds the fp32 partial sums of the K split between the two
  * kernels of a call (decode sizes) or the de-quantised kernel (prefill sizes), so
  * two calls that overlap in time must not share one.  Without it (null / too small)
- * prefill sizes fall back to the 16-row passes.
+ * prefill sizes fall back to the passes.
  */
 int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,

@@ -110,7 +110,7 @@ __device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
 }
 
 // kVec: dwords (8 columns each) a lane loads per k row; the block is 128*kVec columns.
-// kSteps: 16-row K steps per chunk.  kSets: 1 -> up to 8 rows of bf16 x; 2 -> up to 16
+// kSteps: 16-row K steps per chunk.  kSets: n -> up to 8n rows of bf16 x (n = 1, 2, 4); 2 -> also
 // rows of bf16 x, or up to 8 rows of f32 x split into two bf16 parts.
 template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
 __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
@@ -581,22 +581,26 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     pl.fast = (N % 8) == 0 && (K % 16) == 0 && (!grouped || block_size % 16 == 0);
     if (!pl.fast) return pl;
     const bool f32 = x_dtype == K3Q_F32;
-    pl.rows = f32 ? 8 : (M > 8 ? 16 : 8);
-    pl.sets = f32 ? 2 : (M > 8 ? 2 : 1);
+    // rows of x per pass: 8 per row set; bfloat16 takes up to four sets (32 rows), so that
+    // 17..127 rows need a half to a quarter of the passes over the kernel
+    pl.rows = f32 ? 8 : (M > 16 ? 32 : M > 8 ? 16 : 8);
+    pl.sets = f32 ? 2 : pl.rows / 8;
     const int rows_used = (int)(M < pl.rows ? M : pl.rows);
 
     // Measured on MI355X at K = N = 8192: 8 waves per workgroup, 8-byte loads per lane and
     // one or two workgroups per CU beat wider loads and finer K splits.
-    int vec = (grouped && pl.sets == 2) ? 1 : 2;
+    int vec = ((grouped && pl.sets == 2) || pl.sets == 4) ? 1 : 2;
     if (plan_override && plan_override[0] > 0) vec = plan_override[0];
     while (vec > 1 && (N % (8 * vec)) != 0) vec >>= 1;
     if (vec != 1 && vec != 2) vec = vec > 2 ? 2 : 1;  // 16-byte loads per lane lost every sweep
+    if (pl.sets == 4) vec = 1;                       // the only width built for four row sets
     pl.vec = vec;
 
     int steps = 2;
     if (plan_override && plan_override[1] > 0) steps = plan_override[1];
     if (steps != 1 && steps != 2) steps = 2;
     if ((K % 32) != 0 || (grouped && (block_size % 32) != 0)) steps = 1;
+    if (grouped && pl.sets == 4) steps = 1;  // two steps would spill registers
     pl.steps = steps;
     const int chunk = steps * 16;
 
@@ -663,12 +667,16 @@ void launch4(const GemvParams& p, bool grouped, dim3 grid, int threads, size_t l
 template <int kVec, int kSteps>
 void launch2(int sets, bool f32, const GemvParams& p, bool grouped, dim3 grid, int threads,
              size_t lds, hipStream_t s) {
-    if (f32)
+    if (f32) {
         launch4<kVec, kSteps, 2, true>(p, grouped, grid, threads, lds, s);
-    else if (sets == 2)
+    } else if (sets == 4) {
+        // four row sets only with 4-byte loads per lane (register budget)
+        if constexpr (kVec == 1) launch4<1, kSteps, 4, false>(p, grouped, grid, threads, lds, s);
+    } else if (sets == 2) {
         launch4<kVec, kSteps, 2, false>(p, grouped, grid, threads, lds, s);
-    else
+    } else {
         launch4<kVec, kSteps, 1, false>(p, grouped, grid, threads, lds, s);
+    }
 }
 
 void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, bool grouped, dim3 grid,
@@ -769,7 +777,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         p.per_xcd = (int)(grid.x / 8);
         p.ks = pl.ks;
         const size_t lds = (size_t)pl.waves * rows * (nb_cols + kRedPad) * sizeof(float);
-        const int sets = (!f32 && rows > 8) ? 2 : (f32 ? 2 : 1);
+        const int sets = f32 ? 2 : (rows > 16 ? 4 : rows > 8 ? 2 : 1);
         launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
         if (pl.ks > 1) {
             dim3 rgrid((unsigned)((N / 4 + 255) / 256), rows);

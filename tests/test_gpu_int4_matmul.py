@@ -39,7 +39,12 @@ def run_case(dev, M, K, N, block_size, dtype, with_bias, seed=0, plan=None):
     e_exact = max_rel_err(got, exact)
     e_ref_exact = max_rel_err(want, exact)
     tol = RTOL[dtype]
-    assert e_ref <= tol, f"vs oracle: {e_ref:.3e} > {tol:.0e}"
+    # One bfloat16 ulp of an output in [4, 8) is 0.7 % of max|y| here, so two correctly
+    # rounded chains (the reference rounds every de-quantised weight to bfloat16, the kernel
+    # keeps fp32 until the end) can sit 1.5 ulp apart while each is within 0.7 % of the
+    # float64 value.  Such a case passes only if the kernel is the one closer to that value.
+    assert e_ref <= tol or (e_ref <= 1.5 * tol and e_exact <= e_ref_exact), \
+        f"vs oracle: {e_ref:.3e} > {tol:.0e} (vs float64: kernel {e_exact:.3e}, oracle {e_ref_exact:.3e})"
     # the kernel must be at least about as close to the true value as the reference path is
     assert e_exact <= max(2.0 * e_ref_exact, tol / 4), (e_exact, e_ref_exact)
     return e_ref, e_exact
@@ -115,3 +120,13 @@ def test_int4_prefill_route(dev, M, K, N, block_size):
 ])
 def test_int4_large_m_off_route(dev, M, K, N, block_size, dtype):
     run_case(dev, M, K, N, block_size, dtype, with_bias=True)
+
+
+# 17..127 rows: passes of 32 rows (four row sets), last pass narrower
+@pytest.mark.parametrize("M,K,N,block_size", [
+    (17, 256, 512, 128), (32, 512, 1024, None), (33, 1024, 256, 64), (64, 4096, 4096, 128),
+    (100, 512, 384, 32), (127, 2048, 1024, None), (40, 100, 30, 50), (31, 4096, 14336, 128),
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_int4_mid_rows(dev, M, K, N, block_size, dtype):
+    run_case(dev, M, K, N, block_size, dtype, with_bias=(M % 2 == 0))
