@@ -476,29 +476,69 @@ class ReversibleEmbedding(Embedding):
         return self._soft_cap(logits.reshape(*lead, N))
 
     def _int4_call(self, inputs, reverse=False, training=None):
-        """reversible_embedding.py:298-381.  Tied weights without an activation quantizer
-        (the default int4 config): the packed `[vocab, ceil(dim/2)]` table is the K-contiguous
-        int4 kernel of the projection and is read in place."""
+        """reversible_embedding.py:298-381.
+
+        Tied weights: the packed `[vocab, ceil(dim/2)]` table is the K-contiguous int4 kernel
+        of the projection and is read in place.  Untied weights: `reverse_embeddings` is
+        packed along its first axis (two k per byte); it is re-packed once, on the device,
+        into the Dense layout (two columns per byte, same size) and cached, after which the
+        call is a Dense int4 call.  With an activation quantizer (a layer built from a policy
+        without a config): per-row scales go through the exact int8 GEMM on the table unpacked
+        once to int8; grouped scales multiply the quantised rows, as float values, with the
+        de-quantised kernel and divide by the input scale afterwards, as the reference does."""
         if not reverse:
             return super()._int4_call(inputs)
-        if self.inputs_quantizer:
-            raise NotImplementedError(
-                "The int4 reverse projection with an activation quantizer is not on the fused "
-                "path yet."
-            )
-        if not self.tie_weights:
-            raise NotImplementedError(
-                "The untied int4 reverse projection (kernel packed along its first axis) is not "
-                "on the fused path yet."
-            )
+        cd = to_torch_dtype(self.compute_dtype)
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
-        logits = kops.int4_matmul_nk(
-            inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
-            zero=as_tensor(self.embeddings_zero) if grouped else None,
-            block_size=block_size if grouped else None,
-        )
-        return self._soft_cap(logits)
+        lead = inputs.shape[:-1]
+        x2 = inputs.reshape(-1, inputs.shape[-1])
+        in_scale = None
+        if self.inputs_quantizer:
+            x2, in_scale = self.inputs_quantizer(x2, axis=-1)
+        if self.tie_weights:
+            scale = as_tensor(self.embeddings_scale)
+            if in_scale is not None and not grouped:
+                # int8 rows x int4 table: exact int32 accumulation, one de-scale
+                out_dtype = _promote(cd, scale.dtype)
+                table8 = self._cached(
+                    "unpacked", self._embeddings,
+                    lambda t: quantizers.unpack_int4(t, self._orig_output_dim, axis=-1))
+                logits = kops.int8_matmul_nk(
+                    x2, table8, a_scale=in_scale.to(out_dtype), kernel_scale=scale,
+                    out_dtype=out_dtype, exact_epilogue=True,
+                    round_acc_bf16=(cd == torch.bfloat16 and out_dtype == torch.float32))
+            else:
+                logits = kops.int4_matmul_nk(
+                    x2 if in_scale is None else x2.to(cd), as_tensor(self._embeddings), scale,
+                    zero=as_tensor(self.embeddings_zero) if grouped else None,
+                    block_size=block_size if grouped else None)
+                if in_scale is not None:
+                    logits = torch.divide(logits, in_scale)
+        else:
+            scale = as_tensor(self.reverse_embeddings_scale)
+            if in_scale is not None:
+                raise NotImplementedError(
+                    "The untied int4 reverse projection with an activation quantizer is not on "
+                    "the fused path yet."
+                )
+            if scale.dtype != cd:
+                raise NotImplementedError(
+                    "The untied int4 reverse projection needs its scales in the compute dtype "
+                    f"(got {scale.dtype} scales under {cd} compute)."
+                )
+            relaid = self._cached(
+                "relaid", self.reverse_embeddings,
+                lambda t: quantizers.pack_int4(
+                    quantizers.unpack_int4(t, self.output_dim, axis=0), axis=-1)[0])
+            zero = None
+            if grouped:
+                zero = self._cached("zero_i8", self.reverse_embeddings_zero,
+                                    lambda t: t.to(torch.int8).contiguous())
+            logits = kops.int4_matmul(
+                x2, relaid, scale, self.input_dim, kernel_zero=zero,
+                block_size=block_size if grouped else None)
+        return self._soft_cap(logits.reshape(*lead, self.input_dim))
 
     # ---- quantize -----------------------------------------------------------------------
     def _quantize(self, mode, config, type_check=True):

@@ -650,29 +650,59 @@ def reversible_embedding_int8_reverse(inputs, embeddings, embeddings_scale,
 
 def reversible_embedding_int4_reverse(inputs, embeddings, embeddings_scale, output_dim,
                                       embeddings_zero=None, g_idx=None, block_size=None,
-                                      compute_dtype=None, logit_soft_cap=None):
-    """keras/src/layers/core/reversible_embedding.py:298-381 with tied weights and no
-    activation quantizer (the default Int4QuantizationConfig): `inputs_scale` is
-    `ones((1,), compute_dtype)`; the packed table [V, ceil(D/2)] is transposed and unpacked
-    along axis 0 to int8 [D, V]."""
+                                      compute_dtype=None, logit_soft_cap=None,
+                                      tie_weights=True, quantize_inputs=False):
+    """keras/src/layers/core/reversible_embedding.py:298-381 (torch backend).
+
+    tie_weights: `embeddings` is the packed table [V, ceil(D/2)], scale [V] or [V, G], zero
+    [V, G]; it is transposed and unpacked along axis 0 to int8 [D, V].  Untied: `embeddings`
+    is `reverse_embeddings` [ceil(D/2), V], scale [V] or [G, V], zero [G, V].
+    quantize_inputs: the layer has an activation quantizer (AbsMaxQuantizer(axis=-1));
+    otherwise `inputs_scale` is `ones((1,), compute_dtype)`."""
     cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
     inputs = inputs.to(cd)
-    unpacked = unpack_int4(torch.transpose(embeddings, 0, 1), output_dim, axis=0)
-    inputs_scale = torch.ones((1,), dtype=cd)
-    if block_size is None or block_size == -1:
-        scale = embeddings_scale  # transpose of a 1-D tensor
+    grouped = not (block_size is None or block_size == -1)
+    if tie_weights:
+        kernel = torch.transpose(embeddings, 0, 1)
+        scale = embeddings_scale
+    else:
+        kernel = embeddings
+        scale = embeddings_scale
+    unpacked = unpack_int4(kernel, output_dim, axis=0)
+    if quantize_inputs:
+        inputs, inputs_scale = AbsMaxQuantizer(axis=-1)(inputs)
+    else:
+        inputs_scale = torch.ones((1,), dtype=cd)
+    if not grouped:
         logits = matmul(inputs, unpacked)
         logits = logits.to(cd)
         logits = torch.divide(logits, torch.multiply(inputs_scale, scale))
     else:
-        scale_t = torch.transpose(embeddings_scale, 0, 1)
-        zero_t = torch.transpose(embeddings_zero, 0, 1)
-        float_embeddings = dequantize_with_sz_map(unpacked.to(cd), scale_t, zero_t, g_idx, group_axis=0)
+        if tie_weights:
+            scale_g = torch.transpose(scale, 0, 1)
+            zero_g = torch.transpose(embeddings_zero, 0, 1)
+        else:
+            scale_g, zero_g = scale, embeddings_zero
+        float_embeddings = dequantize_with_sz_map(unpacked.to(cd), scale_g, zero_g, g_idx, group_axis=0)
         logits = matmul(inputs, float_embeddings)
         logits = torch.divide(logits, inputs_scale)
     if logit_soft_cap is not None:
         logits = torch.multiply(torch.tanh(torch.divide(logits, logit_soft_cap)), logit_soft_cap)
     return logits
+
+
+def reversible_embedding_quantize_reverse_int4(reverse_embeddings, block_size=128):
+    """Untied `reverse_embeddings` [D, V] -> dict(reverse_embeddings=packed int8
+    [ceil(D/2), V], scale [V] | [G, V], zero (float, as stored) [G, V] | None)
+    (reversible_embedding.py:478-515)."""
+    if block_size is None or block_size == -1:
+        q, s = AbsMaxQuantizer(axis=0, value_range=(-8, 7))(reverse_embeddings, to_numpy=True)
+        s = torch.squeeze(s, dim=0)
+        zero = None
+    else:
+        q, s, zero = abs_max_quantize_grouped_with_zero_point(reverse_embeddings, block_size=block_size)
+    packed, _, _ = pack_int4(q, axis=0)
+    return dict(reverse_embeddings=packed, scale=s, zero=zero, unpacked=q)
 
 
 # --------------------------------------------------------------------------

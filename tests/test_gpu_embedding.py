@@ -298,9 +298,84 @@ def test_reversible_embedding_int4_tied(dev, policy, block_size):
     assert layer(ids).shape == (3, D)
 
 
-def test_reversible_embedding_int4_untied_reverse_raises(dev):
-    layer = build_embedding(ReversibleEmbedding, dev, 64, 32, "float32", seed=9, tie_weights=False)
-    layer.quantize("int4")
-    assert layer(torch.tensor([1, 2, 3])).shape == (3, 32)
-    with pytest.raises(NotImplementedError):
-        layer(torch.randn(2, 32), reverse=True)
+@pytest.mark.parametrize("policy", ["float32", "bfloat16"])
+@pytest.mark.parametrize("block_size", [128, 32, None])
+@pytest.mark.parametrize("M,V,D", [(4, 512, 256), (40, 1000, 384)])
+def test_reversible_embedding_int4_untied(dev, policy, block_size, M, V, D):
+    layer = build_embedding(ReversibleEmbedding, dev, V, D, policy, seed=15, tie_weights=False)
+    rt = layer.reverse_embeddings.value.cpu()
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(16))
+    y_float = layer(x, reverse=True)
+    layer.quantize("int4", config=Int4QuantizationConfig(block_size=block_size))
+    assert layer.reverse_embeddings.dtype == "int8" and layer.reverse_embeddings.shape == (D // 2, V)
+    assert layer.reverse_embeddings_scale.dtype == layer.variable_dtype
+    qd = ref.reversible_embedding_quantize_reverse_int4(rt.float(), block_size=block_size)
+    assert torch.equal(layer.reverse_embeddings.value.cpu(), qd["reverse_embeddings"])
+    grouped = block_size is not None
+    vd = TORCH[layer.variable_dtype]
+    if grouped:
+        assert layer.reverse_embeddings_zero.dtype == layer.variable_dtype
+        assert torch.equal(layer.reverse_embeddings_zero.value.float().cpu(), qd["zero"].float())
+    y = layer(x, reverse=True)
+    want = ref.reversible_embedding_int4_reverse(
+        x.to(cd), qd["reverse_embeddings"], qd["scale"].to(vd), D,
+        embeddings_zero=qd["zero"].to(vd) if grouped else None,
+        g_idx=layer.g_idx.value.cpu() if grouped else None, block_size=block_size,
+        compute_dtype=cd, tie_weights=False)
+    assert y.dtype == want.dtype and tuple(y.shape) == (M, V)
+    assert max_rel_err(y, want) <= RTOL[cd]
+    err = (y_float.float().cpu() - y.float().cpu()).abs().max().item()
+    assert err <= 0.25 * y_float.float().abs().max().item() + 1e-3
+    store = {}
+    layer.save_own_variables(store)
+    assert len(store) == (7 if grouped else 4)
+
+
+@pytest.mark.parametrize("policy,block", [("int4/128_from_float32", 128), ("int4/-1_from_float32", None),
+                                          ("int4/-1_from_bfloat16", None), ("int4/-1_from_mixed_bfloat16", None),
+                                          ("int4/128_from_bfloat16", 128)])
+def test_reversible_embedding_int4_policy_built_quantizes_inputs(dev, policy, block):
+    # a layer built from a policy has no config: the reference gives it the default
+    # activation quantizer (reversible_embedding.py:229-233)
+    V, D, M = 600, 256, 5
+    src = build_embedding(ReversibleEmbedding, dev, V, D, policy.split("_from_")[1], seed=17)
+    src.quantize("int4", config=Int4QuantizationConfig(block_size=block))
+    store = {}
+    src.save_own_variables(store)
+    layer = ReversibleEmbedding(V, D, dtype=policy, device=dev)
+    layer.build()
+    layer.load_own_variables(store)
+    assert layer.inputs_quantizer is not None and src.inputs_quantizer is None
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(18))
+    y = layer(x, reverse=True)
+    grouped = block is not None
+    want = ref.reversible_embedding_int4_reverse(
+        x.to(cd), store["0"].cpu(), store["1"].cpu(), D,
+        embeddings_zero=store["2"].cpu() if grouped else None,
+        g_idx=store["3"].cpu() if grouped else None, block_size=block, compute_dtype=cd,
+        quantize_inputs=True)
+    assert y.dtype == want.dtype
+    if grouped:
+        assert max_rel_err(y, want) <= RTOL[cd]
+    else:
+        assert torch.equal(bits(y.cpu()), bits(want))  # integer accumulation, exact epilogue
+
+
+@pytest.mark.parametrize("mode", ["int4", "int8"])
+@pytest.mark.parametrize("tie_weights", [True, False])
+def test_reversible_embedding_reference_property(dev, mode, tie_weights):
+    # reversible_embedding_test.py:156-185: (10, 16) layer, uniform inputs, weak MSE bounds
+    g = torch.Generator().manual_seed(19)
+    layer = build_embedding(ReversibleEmbedding, dev, 10, 16, "float32", seed=20, tie_weights=tie_weights)
+    x = torch.randint(0, 9, (64, 3), generator=g)
+    x_reverse = torch.rand(64, 16, generator=g)
+    y_float, y_reverse_float = layer(x), layer(x_reverse, reverse=True)
+    layer.quantize(mode)
+    if not tie_weights:
+        assert layer.reverse_embeddings.dtype == "int8"
+        assert layer.reverse_embeddings_scale.dtype == layer.variable_dtype
+    mse = (y_float - layer(x)).pow(2).mean().item()
+    mse_reverse = (y_reverse_float - layer(x_reverse, reverse=True)).pow(2).mean().item()
+    assert mse < 1e-3 and mse_reverse < 1e-2

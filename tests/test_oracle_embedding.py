@@ -170,3 +170,58 @@ def test_reverse_projection_tied_int4_by_loops(block_size):
     # and it approximates the float projection (int4: coarse)
     want_f = x @ t.T
     assert (logits - want_f).abs().max().item() < 0.25 * want_f.abs().max().item() + 1e-3
+
+
+@pytest.mark.parametrize("block_size", [None, 8])
+@pytest.mark.parametrize("quantize_inputs", [False, True])
+def test_reverse_projection_untied_int4_by_loops(block_size, quantize_inputs):
+    V, D, M = 5, 16, 2
+    rt = table(D, V, seed=9)  # reverse_embeddings [D, V]
+    qd = ref.reversible_embedding_quantize_reverse_int4(rt, block_size=block_size)
+    assert tuple(qd["reverse_embeddings"].shape) == (D // 2, V)
+    w = qd["unpacked"]  # [D, V]
+    # packed along axis 0: low nibble = even row
+    for j in range(D // 2):
+        for v in range(V):
+            byte = qd["reverse_embeddings"][j, v].item() & 0xFF
+            assert ((byte & 0xF) ^ 8) - 8 == w[2 * j, v].item()
+            assert ((byte >> 4) ^ 8) - 8 == w[2 * j + 1, v].item()
+    g_idx = None if block_size is None else torch.floor_divide(torch.arange(D, dtype=torch.float32), block_size)
+    zero = None if qd["zero"] is None else qd["zero"].float()
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(10))
+    logits = ref.reversible_embedding_int4_reverse(
+        x, qd["reverse_embeddings"], qd["scale"], D, embeddings_zero=zero, g_idx=g_idx,
+        block_size=block_size, tie_weights=False, quantize_inputs=quantize_inputs)
+    if quantize_inputs:
+        xq, xs = ref.abs_max_quantize(x, axis=-1)
+        xv, xdiv = xq.float(), xs
+    else:
+        xv, xdiv = x, torch.ones(M, 1)
+    for m in range(M):
+        for v in range(V):
+            if block_size is None:
+                acc = sum(float(xv[m, d]) * float(w[d, v]) for d in range(D))
+                want = acc / (float(xdiv[m, 0]) * float(qd["scale"][v]))
+            else:
+                acc = sum(float(xv[m, d]) * (float(w[d, v]) - float(zero[d // block_size, v]))
+                          * float(qd["scale"][d // block_size, v]) for d in range(D))
+                want = acc / float(xdiv[m, 0])
+            assert logits[m, v].item() == pytest.approx(want, rel=3e-5, abs=1e-6)
+    want_f = x @ rt
+    assert (logits - want_f).abs().max().item() < 0.3 * want_f.abs().max().item() + 1e-3
+
+
+def test_reverse_projection_tied_int4_with_input_quantizer():
+    V, D, M = 6, 16, 3
+    t = table(V, D, seed=11)
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(12))
+    qd = ref.embedding_quantize_int4(t, block_size=None)
+    logits = ref.reversible_embedding_int4_reverse(x, qd["embeddings"], qd["embeddings_scale"], D,
+                                                   block_size=None, quantize_inputs=True)
+    xq, xs = ref.abs_max_quantize(x, axis=-1)
+    for m in range(M):
+        for v in range(V):
+            acc = sum(int(xq[m, d]) * int(qd["unpacked"][v, d]) for d in range(D))
+            import numpy as np
+            want = np.float32(acc) / (np.float32(xs[m, 0].item()) * np.float32(qd["embeddings_scale"][v].item()))
+            assert logits[m, v].item() == want
