@@ -426,13 +426,8 @@ class EinsumDense(Layer):
         """keras/src/layers/core/einsum_dense.py:1030-1118 as quantise-rows + int8 GEMM."""
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
-        if not self.inputs_quantizer:
-            raise NotImplementedError(
-                "Weight-only int8 (no activation quantizer) is not on the fused path yet."
-            )
         gv = self._gemm_view()
         x2, free_shape = self._input_rows(inputs, gv)
-        q, scale = self.inputs_quantizer(x2, axis=-1)
         cd = to_torch_dtype(self.compute_dtype)
 
         def kernel_matrix(t):
@@ -443,6 +438,18 @@ class EinsumDense(Layer):
         n = k2.shape[1]
         pre = self._cached("prepacked", self._kernel, lambda t: kops.prepack_int8_kernel(kernel_matrix(t)))
         bias, fused = self._fusable_bias(gv, n)
+        if not self.inputs_quantizer:
+            # Weight-only (einsum_dense.py:1085-1101).  The torch backend divides every weight
+            # by its scale first and contracts in float; here the contraction runs on the
+            # exact int8 values and the scale divides the result -- the same quantity without
+            # the per-weight rounding.
+            y2 = kops.int8_weight_only_matmul(
+                x2, k2,
+                self._cached("kernel_scale", self.kernel_scale,
+                             lambda t: t.to(cd).reshape(-1).contiguous()),
+                bias=bias, prepacked=pre)
+            return self._finish(y2, free_shape, gv, fused)
+        q, scale = self.inputs_quantizer(x2, axis=-1)
         exact = self.exact_epilogue
         if exact is None:
             exact = x2.shape[0] * n <= _EXACT_EPILOGUE_MAX_OUTPUTS
@@ -458,8 +465,6 @@ class EinsumDense(Layer):
         """keras/src/layers/core/einsum_dense.py:1120-1261, weight-only."""
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
-        if self.inputs_quantizer:
-            raise NotImplementedError("int4 with an activation quantizer is not on the fused path yet.")
         gv = self._gemm_view()
         if not gv.k_plain:
             raise NotImplementedError(
@@ -471,6 +476,26 @@ class EinsumDense(Layer):
         block_size = self._int4_block_size
         grouped = block_size is not None and block_size > 0
         bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
+        if self.inputs_quantizer:
+            if grouped:
+                raise NotImplementedError(
+                    "Grouped int4 with an activation quantizer has no counterpart in the "
+                    "reference (einsum_dense.py:1188-1261 ignores the quantizer there)."
+                )
+            # Activation-quantized, per-channel (einsum_dense.py:1163-1187).  The torch
+            # backend contracts the quantised rows, cast back to float, with the kernel
+            # divided by its scale weight by weight; here the contraction is the exact int32
+            # one and both scales divide the result -- the same quantity without the
+            # per-weight rounding.
+            q, scale = self.inputs_quantizer(x2, axis=-1)
+            unpacked = quantizers.unpack_int4(
+                as_tensor(self._kernel), self._int4_unpacked_column_size, axis=-1)
+            y2 = kops.int8_matmul(
+                q, unpacked, a_scale=scale,
+                kernel_scale=self._cached("kernel_scale", self.kernel_scale,
+                                          lambda t: t.to(cd).reshape(-1).contiguous()),
+                bias=bias, out_dtype=cd, exact_epilogue=True)
+            return self._finish(y2, free_shape, gv, fused)
         y2 = kops.int4_matmul(
             x2, as_tensor(self._kernel),
             self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).contiguous()),

@@ -488,6 +488,55 @@ def _adjust_scale(scale, part):
     return scale
 
 
+def _adjust_scale_for_dequant(scale, part):
+    """einsum_dense.py:1625-1648: the inverse of `_adjust_scale` (kernel scale back to a
+    shape that broadcasts against the kernel)."""
+    for a in sorted(part["squeeze"]):
+        scale = torch.unsqueeze(scale, a)
+    for a in sorted(part["expand"], reverse=True):
+        scale = torch.squeeze(scale, a)
+    if part["transpose"]:
+        perm = part["transpose"]
+        reverse = sorted(range(len(perm)), key=perm.__getitem__)
+        scale = scale.permute(reverse)
+    return scale
+
+
+def einsum_dense_int8_weight_only_call(inputs, kernel, kernel_scale, equation, bias=None,
+                                       compute_dtype=None):
+    """keras/src/layers/core/einsum_dense.py:1085-1101, torch branch: every weight is divided
+    by its scale in the compute dtype, then a float einsum."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    info = einsum_quantization_info(equation, inputs.dim())
+    ks = _adjust_scale_for_dequant(_read_var(kernel_scale, cd), info["kernel"])
+    float_kernel = torch.divide(kernel.to(cd), ks)
+    x = torch.einsum(equation, inputs, float_kernel)
+    if bias is not None:
+        x = torch.add(x, _read_var(bias, cd))
+    return x
+
+
+def einsum_dense_int4_activation_quantized_call(inputs, qk, equation, bias=None,
+                                                compute_dtype=None):
+    """keras/src/layers/core/einsum_dense.py:1163-1187, per-channel, torch branch: kernel
+    de-quantised weight by weight, quantised inputs cast back to float, float einsum,
+    division by the input scale."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    inputs = inputs.to(cd)
+    info = qk["info"]
+    ks = _read_var(qk["kernel_scale"], cd)
+    unpacked = unpack_int4(qk["kernel"], qk["cols"], axis=-1)
+    float_kernel = torch.reshape(torch.divide(unpacked.to(cd), ks), qk["original_kernel_shape"])
+    q, s_in = AbsMaxQuantizer()(inputs, axis=tuple(info["input"]["reduced"]))
+    s_adj = _adjust_scale(s_in, info["input"])
+    x = torch.einsum(equation, q.to(cd), float_kernel)
+    x = torch.divide(x, s_adj)
+    if bias is not None:
+        x = torch.add(x, _read_var(bias, cd))
+    return x
+
+
 def einsum_dense_quantize_int8(kernel, equation, input_rank):
     """keras/src/layers/core/einsum_dense.py:1364-1381."""
     info = einsum_quantization_info(equation, input_rank)

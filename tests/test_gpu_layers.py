@@ -255,3 +255,45 @@ def test_dense_int4_activation_quantized(dev, policy, M, K, N):
     assert inter["acc"].dtype == torch.int32
     # integer accumulation and the exact epilogue: bit-identical to the reference chain
     assert y.dtype == cd and torch.equal(bits(y.cpu()), bits(want))
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape", EQUATIONS)
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_einsum_dense_int8_weight_only(dev, equation, output_shape, input_shape, policy):
+    g = torch.Generator().manual_seed(2024)
+    layer = EinsumDense(equation, output_shape, dtype=policy, device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    x = torch.rand(input_shape, generator=g)
+    layer.quantize("int8", config=ka.Int8QuantizationConfig(activation_quantizer=None))
+    assert layer.inputs_quantizer is None
+    qk, ks, _ = ref.einsum_dense_quantize_int8(kernel_f, equation, len(input_shape))
+    y = layer(x)
+    want = ref.einsum_dense_int8_weight_only_call(x.to(cd), qk, ks, equation, compute_dtype=cd)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    # the reference rounds every de-quantised weight to the compute dtype, the kernel divides
+    # once at the end: same quantity, float tolerance
+    assert max_rel_err(y, want) <= RTOL[cd]
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape", [EQUATIONS[0], EQUATIONS[2], EQUATIONS[4], EQUATIONS[5]])
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_einsum_dense_int4_activation_quantized(dev, equation, output_shape, input_shape, policy):
+    g = torch.Generator().manual_seed(2025)
+    layer = EinsumDense(equation, output_shape, dtype=policy, device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    x = torch.rand(input_shape, generator=g)
+    config = ka.Int4QuantizationConfig(block_size=None, activation_quantizer=ka.quantizers.AbsMaxQuantizer())
+    layer.quantize("int4", config=config)
+    assert layer.inputs_quantizer is not None
+    qk = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), None)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    y = layer(x)
+    want = ref.einsum_dense_int4_activation_quantized_call(x.to(cd), qk, equation, compute_dtype=cd)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    assert max_rel_err(y, want) <= RTOL[cd]

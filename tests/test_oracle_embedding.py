@@ -225,3 +225,27 @@ def test_reverse_projection_tied_int4_with_input_quantizer():
             import numpy as np
             want = np.float32(acc) / (np.float32(xs[m, 0].item()) * np.float32(qd["embeddings_scale"][v].item()))
             assert logits[m, v].item() == want
+
+
+def test_einsum_non_default_configs_against_float64():
+    # weight-only int8 and activation-quantized int4 EinsumDense (torch branch): the value is
+    # einsum(x, q / scale) resp. einsum(xq, q4 / scale) / x_scale, checked in float64
+    g = torch.Generator().manual_seed(21)
+    for equation, kshape, xshape in [("btd,dnh->btnh", (16, 2, 4), (2, 3, 16)),
+                                     ("btnh,nhd->btd", (2, 4, 8), (2, 3, 2, 4)),
+                                     ("ab,bc->ac", (8, 6), (5, 8))]:
+        kernel = torch.rand(kshape, generator=g) - 0.5
+        x = torch.rand(xshape, generator=g)
+        q8, s8, info = ref.einsum_dense_quantize_int8(kernel, equation, len(xshape))
+        got = ref.einsum_dense_int8_weight_only_call(x, q8, s8, equation)
+        s_full = ref._adjust_scale_for_dequant(s8, info["kernel"])
+        want = torch.einsum(equation, x.double(), q8.double() / s_full.double())
+        assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-6)
+        assert (got - torch.einsum(equation, x, kernel)).abs().max() < 0.05
+        qk = ref.einsum_dense_quantize_int4(kernel, equation, len(xshape), None)
+        got4 = ref.einsum_dense_int4_activation_quantized_call(x, qk, equation)
+        xq, xs = ref.abs_max_quantize(x, axis=tuple(qk["info"]["input"]["reduced"]))
+        w = (qk["unpacked"].double() / qk["kernel_scale"].double()).reshape(kshape)
+        want4 = torch.einsum(equation, xq.double(), w) / ref._adjust_scale(xs, qk["info"]["input"]).double()
+        assert torch.allclose(got4.double(), want4, rtol=1e-5, atol=1e-6)
+        assert (got4 - torch.einsum(equation, x, kernel)).abs().max() < 0.35
