@@ -437,14 +437,27 @@ class ReversibleEmbedding(Embedding):
         the `[N, K]` operand of the GEMM; nothing is transposed."""
         if not reverse:
             return super()._int8_call(inputs)
-        if not self.inputs_quantizer:
-            raise NotImplementedError(
-                "Weight-only int8 reverse projection (no activation quantizer) is not on the "
-                "fused path yet."
-            )
         cd = to_torch_dtype(self.compute_dtype)
         lead = inputs.shape[:-1]
         x2 = inputs.reshape(-1, inputs.shape[-1])
+        if not self.inputs_quantizer:
+            # weight-only: float rows against the int8 kernel, then the de-scale
+            scale_var = self.embeddings_scale if self.tie_weights else self.reverse_embeddings_scale
+            scale = as_tensor(scale_var)
+            if scale.dtype != cd:
+                raise NotImplementedError(
+                    "The weight-only int8 reverse projection needs its scales in the compute "
+                    f"dtype (got {scale.dtype} scales under {cd} compute)."
+                )
+            if self.tie_weights:
+                logits = kops.int8_weight_only_matmul(x2, None, scale,
+                                                      prepacked=as_tensor(self._embeddings))
+            else:
+                logits = kops.int8_weight_only_matmul(
+                    x2, as_tensor(self.reverse_embeddings), scale,
+                    prepacked=self._cached("prepacked", self.reverse_embeddings,
+                                           kops.prepack_int8_kernel))
+            return self._soft_cap(logits.reshape(*lead, self.input_dim))
         q, in_scale = self.inputs_quantizer(x2, axis=-1)
         scale_var = self.embeddings_scale if self.tie_weights else self.reverse_embeddings_scale
         out_dtype = _promote(cd, as_tensor(scale_var).dtype)

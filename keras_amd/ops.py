@@ -293,7 +293,10 @@ def int8_weight_only_matmul(x, kernel, kernel_scale, bias=None, prepacked=None):
     quantizer (keras/src/layers/core/dense.py:961-983).  Scale and bias in x.dtype."""
     _lib.require_device(x, kernel, kernel_scale, bias, prepacked)
     code = _lib.dtype_code(x.dtype)
-    K, N = kernel.shape
+    if kernel is None:  # only the [N, K] form is at hand (a tied embedding table)
+        N, K = prepacked.shape
+    else:
+        K, N = kernel.shape
     if x.shape[-1] != K:
         raise ValueError(f"last axis of the input ({x.shape[-1]}) does not match the kernel ({K})")
     if kernel_scale.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):

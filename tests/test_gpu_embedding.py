@@ -379,3 +379,26 @@ def test_reversible_embedding_reference_property(dev, mode, tie_weights):
     mse = (y_float - layer(x)).pow(2).mean().item()
     mse_reverse = (y_reverse_float - layer(x_reverse, reverse=True)).pow(2).mean().item()
     assert mse < 1e-3 and mse_reverse < 1e-2
+
+
+@pytest.mark.parametrize("policy", ["float32", "bfloat16"])
+@pytest.mark.parametrize("tie_weights", [True, False])
+def test_reversible_embedding_int8_weight_only(dev, policy, tie_weights):
+    from keras_amd.quantization_config import Int8QuantizationConfig
+
+    V, D, M = 640, 256, 9
+    layer = build_embedding(ReversibleEmbedding, dev, V, D, policy, seed=21, tie_weights=tie_weights)
+    cd = TORCH[layer.compute_dtype]
+    table_f = (layer._embeddings if tie_weights else layer.reverse_embeddings).value.cpu().float()
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(22))
+    layer.quantize("int8", config=Int8QuantizationConfig(activation_quantizer=None))
+    assert layer.inputs_quantizer is None
+    y = layer(x, reverse=True)
+    if tie_weights:
+        q, s = ref.embedding_quantize_int8(table_f)
+        kernel = q.t()
+    else:
+        kernel, s = ref.dense_quantize_int8(table_f)
+    # reversible_embedding.py:272-296 with inputs_scale = ones: float matmul, cast, divide
+    want = torch.divide(ref.matmul(x.to(cd), kernel).to(cd), torch.multiply(torch.ones(1, dtype=cd), s.to(cd)))
+    assert y.dtype == cd and max_rel_err(y, want) <= RTOL[cd]
