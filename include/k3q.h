@@ -142,9 +142,11 @@ int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64
 
 /*
  * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; passes of
- * 32 rows (bfloat16) or 8 rows (float32) up to M = 127; from M = 128 on, for bfloat16 x with K % 128 == 0 and
- * N % 64 == 0, the kernel is de-quantised once into `workspace` as bfloat16 [N, K]
- * and the product runs on the MFMA tile kernel):
+ * 32 rows (bfloat16) or 8 rows (float32) below prefill sizes; from M = 128 .. 320 rows on
+ * (the longer K, the later), for K % 128 == 0 and N % 64 == 0, the kernel is de-quantised
+ * once per call into `workspace` as bfloat16 [N, K] and the product runs on the MFMA tile
+ * kernel; float32 x and the float32 de-quantised kernel go there as high + low bfloat16
+ * parts concatenated along K, which keeps float32 accuracy to about 2^-17):
  *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)
  *     grouped     (block_size  > 0):  y = T(x . ((unpack(w) - zero[g]) * scale[g]))  (+ bias),  g = k / block_size
  * x: [M, K] of x_dtype, contiguous.  w_packed: the layer's int4 kernel as stored,

@@ -23,17 +23,33 @@ constexpr int kWave = 64;
 
 __device__ __forceinline__ float bf16_bits_to_f32(u32 h) { return __uint_as_float(h << 16); }
 
-// float -> bfloat16 bits, round to nearest even (finite inputs; NaN stays NaN).
+// float -> bfloat16 bits, round to nearest even (NaN stays NaN): one v_cvt_pk_bf16_f32.
 __device__ __forceinline__ u32 f32_to_bf16_bits(float f) {
-    u32 u = __float_as_uint(f);
-    u32 r = u + 0x7fffu + ((u >> 16) & 1u);
-    r = ((u & 0x7fffffffu) > 0x7f800000u) ? (u | 0x00400000u) : r;
-    return r >> 16;
+    return (u32)__builtin_bit_cast(unsigned short, (__bf16)f);
+}
+
+// two floats -> packed bfloat16 pair (lo in bits 0..15), one conversion instruction
+__device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(u32, __builtin_convertvector(v, bf2));
 }
 
 // value of f after a round trip through bfloat16
-__device__ __forceinline__ float round_bf16(float f) {
-    return __uint_as_float(f32_to_bf16_bits(f) << 16);
+__device__ __forceinline__ float round_bf16(float f) { return (float)(__bf16)f; }
+
+// bfloat16(a / b) for a and b that are themselves bfloat16 values, bit-identical to rounding
+// the IEEE float32 quotient.  Such a quotient is never closer than 2^-17 (relative) to the
+// midpoint of two bfloat16 values: with 8-bit significands A, B the distance is
+// |512 A - (2j+1) B| / (512 B), a non-zero integer over less than 2^17.  a * rcp(b) is within
+// 2^-22, so it rounds the same way.  Operands outside [2^-60, 2^60] (where rcp or the product
+// could leave the normal range) take the IEEE division.
+__device__ __forceinline__ float div_round_bf16(float a, float b) {
+    const u32 ea = (__float_as_uint(a) >> 23) & 0xffu, eb = (__float_as_uint(b) >> 23) & 0xffu;
+    const bool a_ok = (ea - 67u) <= 120u || (__float_as_uint(a) << 1) == 0u;
+    if (__builtin_expect(a_ok && (eb - 67u) <= 120u, 1)) return round_bf16(a * __builtin_amdgcn_rcpf(b));
+    return round_bf16(a / b);
 }
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -1,5 +1,5 @@
 // bfloat16 x bfloat16 -> float32 GEMM on the tile machinery of the int8 GEMM
-// (k3q_gemm_i8.hip): y[M,N] = T(T(a[M,K] . bt[N,K]^T) / scale[n]) (+ bias), bfloat16 in and out.
+// (k3q_gemm_i8.hip): y[M,N] = T(T(a[M,K] . bt[N,K]^T) / scale[n]) (+ bias), bfloat16 operands.
 // Used for prefill-sized int4 matmuls, where bt is the int4 kernel de-quantised into scratch.
 #pragma once
 
@@ -12,8 +12,9 @@ namespace k3q {
 bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* bt,
                             const void* y);
 
-// b_scale (bfloat16 [N]) and bias (bfloat16 [N]) may be null
+// b_scale [N] and bias [N] may be null; they and y are bfloat16, or float32 with out_f32 (the
+// operands then being high / low bfloat16 parts of float32 values, concatenated along K)
 int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
-                     const void* b_scale, const void* bias, void* y, hipStream_t s);
+                     const void* b_scale, const void* bias, void* y, bool out_f32, hipStream_t s);
 
 }  // namespace k3q

@@ -17,6 +17,8 @@
 // MFMA: v_mfma_i32_32x32x32_i8.  The weight tile is the first (row) operand and
 // the activation tile the second (column) operand, so a lane ends up with ONE
 // output row m and groups of four consecutive n: stores are 8 or 16 bytes wide.
+#include <type_traits>
+
 #include "k3q_common.h"
 #include "k3q_gemm_bf16.h"
 #include "k3q_gemm_i8_skinny.h"
@@ -150,265 +152,323 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
     // XCD runs at a time share A rows and B rows in its L2.
     const int total = p.tiles_m * p.tiles_n;
     const int per_xcd = (total + 7) / 8;
-    const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (t >= total) return;
-    constexpr int kBand = 4;
-    const int band = t / (kBand * p.tiles_n);
-    const int band_rows = min(kBand, p.tiles_m - band * kBand);
-    const int within = t - band * kBand * p.tiles_n;
-    const int tile_m = band * kBand + within % band_rows;
-    const int tile_n = within / band_rows;
-    const int64_t m0 = (int64_t)tile_m * kBM;
-    const int64_t n0 = (int64_t)tile_n * kBN;
+    // A workgroup stays on its CU and walks every (gridDim / 8)-th tile of its XCD's range:
+    // the output stores of one tile drain while the next tile's loads are already running.
+    const int tl_first = blockIdx.x / 8, tl_step = gridDim.x / 8;
+    for (int tl = tl_first; tl < per_xcd; tl += tl_step) {
+        const int t = (blockIdx.x % 8) * per_xcd + tl;
+        if (t >= total) break;
+        if (tl != tl_first) __syncthreads();  // the previous tile's epilogue is done with the LDS
+        constexpr int kBand = 4;
+        const int band = t / (kBand * p.tiles_n);
+        const int band_rows = min(kBand, p.tiles_m - band * kBand);
+        const int within = t - band * kBand * p.tiles_n;
+        const int tile_m = band * kBand + within % band_rows;
+        const int tile_n = within / band_rows;
+        const int64_t m0 = (int64_t)tile_m * kBM;
+        const int64_t n0 = (int64_t)tile_n * kBN;
 
-    // ---- DMA source addresses ----
-    // DMA instruction d of this wave fills LDS bytes [(wave * kDmaPerWave + d) * 1024, +1024) of
-    // the stage: 8 rows x 128 B.  The first kDmaA instructions of a stage are the A tile, the
-    // rest the B tile.
-    const char* src[kDmaPerWave];
-#pragma unroll
-    for (int d = 0; d < kDmaPerWave; ++d) {
-        const int inst = wave * kDmaPerWave + d;
-        const bool is_b = inst >= kDmaA;
-        const int row = (is_b ? inst - kDmaA : inst) * 8 + lane / kRowChunks;
-        const int chunk = (lane & (kRowChunks - 1)) ^ swz(row);
-        int64_t grow = (is_b ? n0 : m0) + row;
-        const int64_t lim = (is_b ? p.N : p.M) - 1;
-        grow = grow < lim ? grow : lim;
-        src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16;
-    }
-    auto issue_stage = [&](int kt) {
-        char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
+        // ---- DMA source addresses ----
+        // DMA instruction d of this wave fills LDS bytes [(wave * kDmaPerWave + d) * 1024, +1024) of
+        // the stage: 8 rows x 128 B.  The first kDmaA instructions of a stage are the A tile, the
+        // rest the B tile.
+        const char* src[kDmaPerWave];
 #pragma unroll
         for (int d = 0; d < kDmaPerWave; ++d) {
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
-                (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
+            const int inst = wave * kDmaPerWave + d;
+            const bool is_b = inst >= kDmaA;
+            const int row = (is_b ? inst - kDmaA : inst) * 8 + lane / kRowChunks;
+            const int chunk = (lane & (kRowChunks - 1)) ^ swz(row);
+            int64_t grow = (is_b ? n0 : m0) + row;
+            const int64_t lim = (is_b ? p.N : p.M) - 1;
+            grow = grow < lim ? grow : lim;
+            src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16;
         }
-    };
-
-    // ---- fragment reads ----
-    // MFMA operand lane (i = lane % 32, g = lane / 32) holds row i, bytes [16g, 16g+16) of the
-    // 32-byte K step, i.e. logical chunk 2*ks + g of the row.
-    const int fi = lane & 31;
-    const int fg = lane >> 5;
-    int a_row[kMBlk], a_swz[kMBlk], b_row[kNBlk], b_swz[kNBlk];
+        auto issue_stage = [&](int kt) {
+            char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
 #pragma unroll
-    for (int mb = 0; mb < kMBlk; ++mb) {
-        const int row = wm * kWM + mb * 32 + fi;
-        a_row[mb] = row * kBK;
-        a_swz[mb] = swz(row);
-    }
-#pragma unroll
-    for (int nb = 0; nb < kNBlk; ++nb) {
-        const int row = wn * kWN + nb * 32 + fi;
-        b_row[nb] = kATileBytes + row * kBK;
-        b_swz[nb] = swz(row);
-    }
-    v4i af[2][kMBlk], bf[2][kNBlk];
-    auto read_frags = [&](int fb, int stage, int ks) {
-        const char* st = lds + stage * kStageBytes;
-#pragma unroll
-        for (int nb = 0; nb < kNBlk; ++nb)
-            bf[fb][nb] = *(const v4i*)(st + b_row[nb] + (((2 * ks + fg) ^ b_swz[nb]) << 4));
-#pragma unroll
-        for (int mb = 0; mb < kMBlk; ++mb)
-            af[fb][mb] = *(const v4i*)(st + a_row[mb] + (((2 * ks + fg) ^ a_swz[mb]) << 4));
-    };
-
-    typename Mma<kKind>::Acc acc[kNBlk][kMBlk];
-#pragma unroll
-    for (int nb = 0; nb < kNBlk; ++nb)
-#pragma unroll
-        for (int mb = 0; mb < kMBlk; ++mb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0;
-
-    // ---- main loop ----
-    // Two LDS stages.  The fragments of K step ks+1 are read in the middle of the MFMAs of
-    // step ks; the one barrier per stage sits in the middle of the LAST step's MFMAs, so the
-    // matrix core has work queued while waves meet.  At that barrier every wave holds its
-    // last fragments of stage kt in registers, so stage kt+2 may be DMA-ed over stage kt, and
-    // stage kt+1 (whose DMA every wave has waited for) may be read.
-    const int KT = (int)(p.row_bytes / kBK);
-    issue_stage(0);
-    if (KT > 1) {
-        issue_stage(1);
-        wait_vmcnt_one_stage<kDmaPerWave>();
-    } else {
-        wait_vmcnt0();
-    }
-    bare_barrier();
-    read_frags(0, 0, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-#pragma unroll
-        for (int ks = 0; ks < kKSteps; ++ks) {
-            // first half of this step's MFMAs, then the reads for the next step, then the
-            // second half: the reads get half a step of matrix-core time to come back
-            __builtin_amdgcn_sched_barrier(0);
-#ifndef K3Q_GEMM_PROBE_NO_MMA
-#pragma unroll
-            for (int nb = 0; nb < kNBlk / 2; ++nb)
-#pragma unroll
-                for (int mb = 0; mb < kMBlk; ++mb)
-                    acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
-#endif
-            __builtin_amdgcn_sched_barrier(0);
-            if (ks + 1 < kKSteps) {
-                read_frags((ks + 1) & 1, cur, ks + 1);
-            } else if (kt + 1 < KT) {
-                wait_vmcnt0();  // own DMA of stage kt+1 has landed (own reads of stage kt are done)
-                bare_barrier();
-#ifndef K3Q_GEMM_PROBE_NO_DMA
-                if (kt + 2 < KT) issue_stage(kt + 2);
-#endif
-                read_frags(0, cur ^ 1, 0);
+            for (int d = 0; d < kDmaPerWave; ++d) {
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
+                    (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-#ifndef K3Q_GEMM_PROBE_NO_MMA
-#pragma unroll
-            for (int nb = kNBlk / 2; nb < kNBlk; ++nb)
-#pragma unroll
-                for (int mb = 0; mb < kMBlk; ++mb)
-                    acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
-#else
-            // probe build: consume the fragments so that the reads stay
-#pragma unroll
-            for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] += (af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1]);
-#endif
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
+        };
 
-#ifdef K3Q_GEMM_PROBE_CLOCK
-    if (p.acc_out && tid == 0 && blockIdx.x < 64) {
-        uint64_t* d = (uint64_t*)p.acc_out + 2 * blockIdx.x;
-        d[0] = __builtin_readcyclecounter() - clk0;
-        d[1] = __builtin_amdgcn_s_memrealtime() - rt0;
-    }
-    if (p.acc_out) return;
-#endif
-    // ---- epilogue ----
-    // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
-    // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: a lane owns one row of y per mb
-    // and groups of four consecutive columns.
-    if (p.flags & kFlagSkipEpilogue) {  // timing aid: main loop only
-        int sink = 0;
+        // ---- fragment reads ----
+        // MFMA operand lane (i = lane % 32, g = lane / 32) holds row i, bytes [16g, 16g+16) of the
+        // 32-byte K step, i.e. logical chunk 2*ks + g of the row.
+        const int fi = lane & 31;
+        const int fg = lane >> 5;
+        int a_row[kMBlk], a_swz[kMBlk], b_row[kNBlk], b_swz[kNBlk];
+#pragma unroll
+        for (int mb = 0; mb < kMBlk; ++mb) {
+            const int row = wm * kWM + mb * 32 + fi;
+            a_row[mb] = row * kBK;
+            a_swz[mb] = swz(row);
+        }
+#pragma unroll
+        for (int nb = 0; nb < kNBlk; ++nb) {
+            const int row = wn * kWN + nb * 32 + fi;
+            b_row[nb] = kATileBytes + row * kBK;
+            b_swz[nb] = swz(row);
+        }
+        v4i af[2][kMBlk], bf[2][kNBlk];
+        auto read_frags = [&](int fb, int stage, int ks) {
+            const char* st = lds + stage * kStageBytes;
+#pragma unroll
+            for (int nb = 0; nb < kNBlk; ++nb)
+                bf[fb][nb] = *(const v4i*)(st + b_row[nb] + (((2 * ks + fg) ^ b_swz[nb]) << 4));
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb)
+                af[fb][mb] = *(const v4i*)(st + a_row[mb] + (((2 * ks + fg) ^ a_swz[mb]) << 4));
+        };
+
+        typename Mma<kKind>::Acc acc[kNBlk][kMBlk];
 #pragma unroll
         for (int nb = 0; nb < kNBlk; ++nb)
 #pragma unroll
             for (int mb = 0; mb < kMBlk; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sink ^= (int)acc[nb][mb][r];
-        if (sink == 0x7fffffff && p.y) ((char*)p.y)[0] = 1;
-        return;
-    }
-    // Stage the tile's scales and bias in LDS as floats (the main loop is done with it): the
-    // per-lane reads below are then cheap and need no large register arrays.
-    float* ep = (float*)lds;  // [0,256) b_scale or its reciprocal, [256,512) bias, [512,768) a_scale or reciprocal
-    __syncthreads();
-    for (int t = tid; t < kBN; t += kThreads) {
-        const int64_t n = n0 + t < p.N ? n0 + t : p.N - 1;
-        const float sbv = p.b_scale ? load_t<kBF16>(p.b_scale, n) : 1.0f;
-        ep[t] = kExact ? sbv : 1.0f / sbv;
-        ep[kBN + t] = p.bias ? load_t<kBF16>(p.bias, n) : 0.0f;
-    }
-    for (int t = tid; t < kBM; t += kThreads) {
-        const int64_t m = m0 + t < p.M ? m0 + t : p.M - 1;
-        const float sav = p.a_scale ? load_t<kBF16>(p.a_scale, m) : 1.0f;
-        ep[2 * kBN + t] = kExact ? sav : 1.0f / sav;
-    }
-    __syncthreads();
-    if constexpr (kKind == kKindBF16) {
-        // float operands (a de-quantised int4 kernel): y = T(T(acc) / scale[n]) (+ bias), or
-        // with a null scale y = T(acc) (+ bias); bfloat16 output.
-        const bool has_b = p.bias != nullptr, has_s = p.b_scale != nullptr;
+                for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0;
+
+        // ---- main loop ----
+        // Two LDS stages.  The fragments of K step ks+1 are read in the middle of the MFMAs of
+        // step ks; the one barrier per stage sits in the middle of the LAST step's MFMAs, so the
+        // matrix core has work queued while waves meet.  At that barrier every wave holds its
+        // last fragments of stage kt in registers, so stage kt+2 may be DMA-ed over stage kt, and
+        // stage kt+1 (whose DMA every wave has waited for) may be read.
+        const int KT = (int)(p.row_bytes / kBK);
+        issue_stage(0);
+        if (KT > 1) {
+            issue_stage(1);
+            wait_vmcnt_one_stage<kDmaPerWave>();
+        } else {
+            wait_vmcnt0();
+        }
+        bare_barrier();
+        read_frags(0, 0, 0);
+        for (int kt = 0; kt < KT; ++kt) {
+            const int cur = kt & 1;
 #pragma unroll
-        for (int mb = 0; mb < kMBlk; ++mb) {
-            const int ml = wm * kWM + mb * 32 + fi;
-            const int64_t m = m0 + ml;
-            if (m >= p.M) continue;
+            for (int ks = 0; ks < kKSteps; ++ks) {
+                // first half of this step's MFMAs, then the reads for the next step, then the
+                // second half: the reads get half a step of matrix-core time to come back
+                __builtin_amdgcn_sched_barrier(0);
+#ifndef K3Q_GEMM_PROBE_NO_MMA
 #pragma unroll
-            for (int nb = 0; nb < kNBlk; ++nb) {
+                for (int nb = 0; nb < kNBlk / 2; ++nb)
 #pragma unroll
-                for (int rg = 0; rg < 4; ++rg) {
-                    const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
-                    const int64_t n = n0 + nl;
-                    if (n >= p.N) continue;
-                    const v4f sb = *(const v4f*)(ep + nl);
-                    const v4f bv = *(const v4f*)(ep + kBN + nl);
-                    u32 h[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        float r = round_bf16((float)acc[nb][mb][4 * rg + e]);
-                        if (has_s) r = round_bf16(r / sb[e]);
-                        if (has_b) r = round_bf16(r + bv[e]);
-                        h[e] = f32_to_bf16_bits(r);
-                    }
-                    v2u o = {h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
-                    *(v2u*)((uint16_t*)p.y + m * p.N + n) = o;
+                    for (int mb = 0; mb < kMBlk; ++mb)
+                        acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
+#endif
+                __builtin_amdgcn_sched_barrier(0);
+                if (ks + 1 < kKSteps) {
+                    read_frags((ks + 1) & 1, cur, ks + 1);
+                } else if (kt + 1 < KT) {
+                    wait_vmcnt0();  // own DMA of stage kt+1 has landed (own reads of stage kt are done)
+                    bare_barrier();
+#ifndef K3Q_GEMM_PROBE_NO_DMA
+                    if (kt + 2 < KT) issue_stage(kt + 2);
+#endif
+                    read_frags(0, cur ^ 1, 0);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+#ifndef K3Q_GEMM_PROBE_NO_MMA
+#pragma unroll
+                for (int nb = kNBlk / 2; nb < kNBlk; ++nb)
+#pragma unroll
+                    for (int mb = 0; mb < kMBlk; ++mb)
+                        acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
+#else
+                // probe build: consume the fragments so that the reads stay
+#pragma unroll
+                for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] += (af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1]);
+#endif
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        return;
-    }
-    const bool has_bias = p.bias != nullptr;
-    const bool round_acc = (p.flags & kFlagRoundAccBF16) != 0;
-    // Row-major store order: the eight 8-byte (16-byte for float32) pieces that make up one
-    // 128-byte line of a row of y leave back to back, so that the L2 can merge them.
+
+#ifdef K3Q_GEMM_PROBE_CLOCK
+        if (p.acc_out && tid == 0 && blockIdx.x < 64) {
+            uint64_t* d = (uint64_t*)p.acc_out + 2 * blockIdx.x;
+            d[0] = __builtin_readcyclecounter() - clk0;
+            d[1] = __builtin_amdgcn_s_memrealtime() - rt0;
+        }
+        if (p.acc_out) return;
+#endif
+        // ---- epilogue ----
+        // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
+        // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: a lane owns one row of y per mb
+        // and groups of four consecutive columns.
+        if (p.flags & kFlagSkipEpilogue) {  // timing aid: main loop only
+            int sink = 0;
 #pragma unroll
-    for (int mb = 0; mb < kMBlk; ++mb) {
-        const int ml = wm * kWM + mb * 32 + fi;
-        const int64_t m = m0 + ml;
-        if (m >= p.M) continue;
-        const float sa = ep[2 * kBN + ml];
+            for (int nb = 0; nb < kNBlk; ++nb)
 #pragma unroll
-        for (int nb = 0; nb < kNBlk; ++nb) {
+                for (int mb = 0; mb < kMBlk; ++mb)
 #pragma unroll
-            for (int rg = 0; rg < 4; ++rg) {
-                const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
-                const int64_t n = n0 + nl;
-                if (n >= p.N) continue;  // N % 4 == 0 on this path: all four columns in or out
-                if (p.acc_out) {
-                    v4i o = {(int)acc[nb][mb][4 * rg], (int)acc[nb][mb][4 * rg + 1],
-                             (int)acc[nb][mb][4 * rg + 2], (int)acc[nb][mb][4 * rg + 3]};
-                    *(v4i*)(p.acc_out + m * p.N + n) = o;
-                }
-                if (!p.y) continue;
-                const v4f sb = *(const v4f*)(ep + nl);
-                const v4f bv = *(const v4f*)(ep + kBN + nl);
-                float v[4];
+                    for (int r = 0; r < 16; ++r) sink ^= (int)acc[nb][mb][r];
+            if (sink == 0x7fffffff && p.y) ((char*)p.y)[0] = 1;
+            continue;
+        }
+        // Stage the tile's scales and bias in LDS as floats (the main loop is done with it): the
+        // per-lane reads below are then cheap and need no large register arrays.
+        float* ep = (float*)lds;  // [0,256) b_scale or its reciprocal, [256,512) bias, [512,768) a_scale or reciprocal
+        __syncthreads();
+        // scales outside [2^-30, 2^30] send the tile to the IEEE division (see div_round_bf16:
+        // with both in range, the product of two and an int32 over it stay normal numbers)
+        int wide_scale = 0;
+        auto out_of_range = [](float v) { return (((__float_as_uint(v) >> 23) & 0xffu) - 97u) > 60u; };
+        for (int t = tid; t < kBN; t += kThreads) {
+            const int64_t n = n0 + t < p.N ? n0 + t : p.N - 1;
+            const float sbv = p.b_scale ? load_t<kBF16>(p.b_scale, n) : 1.0f;
+            wide_scale |= out_of_range(sbv);
+            ep[t] = kExact ? sbv : 1.0f / sbv;
+            ep[kBN + t] = p.bias ? load_t<kBF16>(p.bias, n) : 0.0f;
+        }
+        for (int t = tid; t < kBM; t += kThreads) {
+            const int64_t m = m0 + t < p.M ? m0 + t : p.M - 1;
+            const float sav = p.a_scale ? load_t<kBF16>(p.a_scale, m) : 1.0f;
+            wide_scale |= out_of_range(sav);
+            ep[2 * kBN + t] = kExact ? sav : 1.0f / sav;
+        }
+        const bool ieee_div = __syncthreads_or(wide_scale) != 0;
+        // Output staging.  A lane's accumulators are four consecutive columns of 32 different
+        // rows: stored as they are, a wave instruction would touch 32 lines with 8 or 16 bytes
+        // each.  Instead every wave passes its 32-row blocks through a private LDS area
+        // ([32][kWN] outputs, rows padded by 16 bytes against bank conflicts) and stores them
+        // row-contiguous, 16 bytes per lane: whole 128-byte lines per instruction.
+        constexpr int kE = kBF16 ? 2 : 4;            // bytes per output
+        constexpr int kPitch = kWN * kE + 16;
+        constexpr int kChunks = kWN * kE / 16;       // 16-byte chunks per staged row
+        constexpr int kRowsPerPass = 64 / kChunks;
+        static_assert((2 * kBN + kBM) * 4 <= 4096, "scales and bias fit below the staging areas");
+        static_assert(4096 + (kThreads / 64) * 32 * kPitch <= T::kLdsBytes, "staging fits in LDS");
+        char* wst = lds + 4096 + wave * (32 * kPitch);
+        const bool wide = (((int64_t)p.N * kE) % 16 == 0) && (((uintptr_t)p.y) % 16 == 0);
+        auto stage4 = [&](int nb, int rg, const float (&v)[4]) {
+            char* d = wst + fi * kPitch + (nb * 32 + 8 * rg + 4 * fg) * kE;
+            if (kBF16) {
+                v2u o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+                *(v2u*)d = o;
+            } else {
+                v4f o = {v[0], v[1], v[2], v[3]};
+                *(v4f*)d = o;
+            }
+        };
+        auto flush_rows = [&](int mb) {
+            // LDS operations of one wave complete in order: waiting for the writes is enough
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float accf = (float)acc[nb][mb][4 * rg + e];
-                    if (!kBF16 && round_acc) accf = round_bf16(accf);
-                    float r;
-                    if (kExact) {
-                        // the reference's op sequence, every step rounded to T
-                        if (kBF16) {
-                            const float os = round_bf16(sb[e] * sa);
-                            r = round_bf16(round_bf16(accf) / os);
-                            if (has_bias) r = round_bf16(r + bv[e]);
-                        } else {
-                            r = accf / (sb[e] * sa);
-                            if (has_bias) r = r + bv[e];
-                        }
-                    } else {
-                        r = (accf * sa) * sb[e] + bv[e];  // sa, sb hold reciprocals here
-                    }
-                    v[e] = r;
-                }
-                if (kBF16) {
-                    v2u o;
-                    o[0] = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-                    o[1] = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
-                    *(v2u*)((uint16_t*)p.y + m * p.N + n) = o;
+            for (int ps = 0; ps < 32 / kRowsPerPass; ++ps) {
+                const int row = ps * kRowsPerPass + lane / kChunks;
+                const int chunk = lane % kChunks;
+                const v4u d = *(const v4u*)(wst + row * kPitch + chunk * 16);
+                const int64_t m = m0 + wm * kWM + mb * 32 + row;
+                const int64_t n = n0 + wn * kWN + chunk * (16 / kE);
+                if (m >= p.M || n >= p.N) continue;
+                char* dst = (char*)p.y + (m * p.N + n) * kE;
+                const bool full = n + 16 / kE <= p.N;  // else the first 8 bytes (N % 4 == 0)
+                if (wide && full) {
+                    __builtin_nontemporal_store(d, (v4u*)dst);
                 } else {
-                    v4f o = {v[0], v[1], v[2], v[3]};
-                    *(v4f*)((float*)p.y + m * p.N + n) = o;
+                    v2u lo = {d[0], d[1]}, hi = {d[2], d[3]};
+                    __builtin_nontemporal_store(lo, (v2u*)dst);
+                    if (full) __builtin_nontemporal_store(hi, (v2u*)(dst + 8));
                 }
             }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next block's writes
+        };
+        if constexpr (kKind == kKindBF16) {
+            // float operands (a de-quantised int4 / widened int8 kernel): y = T(T(acc) / scale[n])
+            // (+ bias), or with a null scale y = T(acc) (+ bias).  T = bfloat16, or float32 when the
+            // operands are the high / low bfloat16 parts of float32 values.
+            const bool has_b = p.bias != nullptr, has_s = p.b_scale != nullptr;
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb) {
+#pragma unroll
+                for (int nb = 0; nb < kNBlk; ++nb) {
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+                        const v4f sb = *(const v4f*)(ep + nl);
+                        const v4f bv = *(const v4f*)(ep + kBN + nl);
+                        float r[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            r[e] = (float)acc[nb][mb][4 * rg + e];
+                            if (kBF16) {
+                                r[e] = round_bf16(r[e]);
+                                if (has_s) r[e] = div_round_bf16(r[e], sb[e]);
+                                if (has_b) r[e] = round_bf16(r[e] + bv[e]);
+                            } else {
+                                if (has_s) r[e] = r[e] / sb[e];
+                                if (has_b) r[e] = r[e] + bv[e];
+                            }
+                        }
+                        stage4(nb, rg, r);
+                    }
+                }
+                flush_rows(mb);
+            }
+            continue;
+        }
+        const bool has_bias = p.bias != nullptr;
+        const bool round_acc = (p.flags & kFlagRoundAccBF16) != 0;
+        auto descale = [&](auto rcp_div) {
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb) {
+                const int ml = wm * kWM + mb * 32 + fi;
+                const int64_t m = m0 + ml;
+                const float sa = ep[2 * kBN + ml];
+#pragma unroll
+                for (int nb = 0; nb < kNBlk; ++nb) {
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+                        const int64_t n = n0 + nl;
+                        if (p.acc_out && m < p.M && n < p.N) {  // N % 4 == 0 on this path
+                            v4i o = {(int)acc[nb][mb][4 * rg], (int)acc[nb][mb][4 * rg + 1],
+                                     (int)acc[nb][mb][4 * rg + 2], (int)acc[nb][mb][4 * rg + 3]};
+                            *(v4i*)(p.acc_out + m * p.N + n) = o;
+                        }
+                        if (!p.y) continue;
+                        const v4f sb = *(const v4f*)(ep + nl);
+                        const v4f bv = *(const v4f*)(ep + kBN + nl);
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float accf = (float)acc[nb][mb][4 * rg + e];
+                            if (!kBF16 && round_acc) accf = round_bf16(accf);
+                            float r;
+                            if (kExact) {
+                                // the reference's op sequence, every step rounded to T
+                                if (kBF16) {
+                                    const float os = round_bf16(sb[e] * sa);
+                                    const float ab = round_bf16(accf);
+                                    r = round_bf16(decltype(rcp_div)::value ? ab * __builtin_amdgcn_rcpf(os)
+                                                                            : ab / os);
+                                    if (has_bias) r = round_bf16(r + bv[e]);
+                                } else {
+                                    r = accf / (sb[e] * sa);
+                                    if (has_bias) r = r + bv[e];
+                                }
+                            } else {
+                                r = (accf * sa) * sb[e] + bv[e];  // sa, sb hold reciprocals here
+                            }
+                            v[e] = r;
+                        }
+                        stage4(nb, rg, v);
+                    }
+                }
+                if (p.y) flush_rows(mb);
+            }
+        };
+        if constexpr (kExact && kBF16) {
+            if (ieee_div) descale(std::false_type{});
+            else descale(std::true_type{});
+        } else {
+            descale(std::false_type{});
         }
     }
 }
@@ -525,6 +585,19 @@ __global__ __launch_bounds__(256) void gemm_w8_simple(const void* x, const int8_
     }
 }
 
+// compute units of the current device
+inline int cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+        cached[dev] = n > 0 ? n : -1;
+    }
+    return cached[dev] > 0 ? cached[dev] : 0;
+}
+
 template <class T, int kKind, bool kBF16, bool kExact>
 int launch_tile(GemmParams p, hipStream_t s) {
     // more than 64 KiB of dynamic LDS needs the attribute raised once per kernel
@@ -535,7 +608,11 @@ int launch_tile(GemmParams p, hipStream_t s) {
     p.tiles_m = (int)((p.M + T::kBM - 1) / T::kBM);
     p.tiles_n = (int)((p.N + T::kBN - 1) / T::kBN);
     const int total = p.tiles_m * p.tiles_n;
-    const int grid = ((total + 7) / 8) * 8;
+    // one resident set of workgroups (as many as fit on the chip at once, a multiple of the
+    // 8 XCDs); each walks its share of the tiles
+    const int resident = cu_count() * (T::kLdsBytes <= 64 * 1024 ? 2 : 1) / 8 * 8;
+    int grid = ((total + 7) / 8) * 8;
+    if (resident >= 8 && grid > resident) grid = resident;
     gemm_mfma<T, kKind, kBF16, kExact><<<grid, T::kThreads, T::kLdsBytes, s>>>(p);
     return launch_status();
 }
@@ -562,7 +639,7 @@ bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, cons
 }
 
 int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
-                     const void* b_scale, const void* bias, void* y, hipStream_t s) {
+                     const void* b_scale, const void* bias, void* y, bool out_f32, hipStream_t s) {
     GemmParams p{};
     p.a = (const int8_t*)a;
     p.bt = (const int8_t*)bt;
@@ -573,6 +650,7 @@ int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_
     p.N = N;
     p.K = K;
     p.row_bytes = 2 * K;
+    if (out_f32) return launch_mfma<kKindBF16, false, true>(p, s);
     return launch_mfma<kKindBF16, true, true>(p, s);
 }
 
@@ -700,7 +778,7 @@ extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_la
             dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
             transpose_widen_i8_to_bf16<<<grid, 256, 0, s>>>(b, (uint16_t*)workspace, K, N);
         }
-        return gemm_bf16_nk_run(x, workspace, M, N, K, b_scale, bias, y, s);
+        return gemm_bf16_nk_run(x, workspace, M, N, K, b_scale, bias, y, false, s);
     }
     if (M > 65535) return K3Q_ERR_SHAPE;
     dim3 grid((unsigned)((N + 255) / 256), (unsigned)M);

@@ -553,10 +553,104 @@ __global__ __launch_bounds__(256) void dequant_w4_to_bf16_nk(const uint8_t* __re
 
 // Below this the 16-row decode passes are faster (K = N = 4096: 51 us at 64 rows; at 128 rows
 // the passes take 96 us, de-quantise + GEMM 67 us).
+// ---- float32 inputs on the same route -------------------------------------------------
+// A float32 value is the sum of two bfloat16 values to 2^-17: hi = its top 16 bits, lo = the
+// rounded remainder.  With x = xh + xl and w = wh + wl,  x.w = xh.wh + xl.wh + xh.wl (+ 2^-18),
+// which is ONE bfloat16 GEMM over a K axis of three segments: a = [xh | xl | xh],
+// b = [wh | wh | wl].  Per-channel kernels are small integers (wl = 0): two segments.
+__global__ __launch_bounds__(256) void split_f32_rows(const float* __restrict__ x,
+                                                      uint16_t* __restrict__ out, int64_t M,
+                                                      int64_t K, int parts) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // 4 elements per thread
+    if (i >= M * K) return;
+    const int64_t m = i / K, k = i - m * K;
+    const v4u f = *(const v4u*)(x + i);
+    u32 hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const u32 top = f[e] & 0xffff0000u;
+        hi[e] = top >> 16;
+        lo[e] = f32_to_bf16_bits(__uint_as_float(f[e]) - __uint_as_float(top));
+    }
+    const v2u h2 = {hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16)};
+    const v2u l2 = {lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16)};
+    uint16_t* row = out + m * parts * K + k;
+    *(v2u*)row = h2;
+    *(v2u*)(row + K) = l2;
+    if (parts == 3) *(v2u*)(row + 2 * K) = h2;
+}
+
+// As dequant_w4_to_bf16_nk, for float32 scales: output rows of `parts` segments of K values,
+// [w | w] (per-channel, exact) or [wh | wh | wl] of w = (nibble - zero) * scale.
+template <bool kGrouped>
+__global__ __launch_bounds__(256) void dequant_w4_to_bf16_parts_nk(const uint8_t* __restrict__ w,
+                                                                  const float* __restrict__ scale,
+                                                                  const int8_t* __restrict__ zero,
+                                                                  uint16_t* __restrict__ out,
+                                                                  int64_t K, int64_t N, int block_size) {
+    constexpr int kParts = kGrouped ? 3 : 2;
+    __shared__ uint16_t thi[kDqK][kDqN + 2];
+    __shared__ uint16_t tlo[kGrouped ? kDqK : 1][kDqN + 2];
+    const int64_t k0 = (int64_t)blockIdx.y * kDqK;
+    const int64_t n0 = (int64_t)blockIdx.x * kDqN;
+    {
+        const int r = threadIdx.x >> 1, h = threadIdx.x & 1;
+        const int64_t k = k0 + r, n = n0 + 32 * h;
+        const v4u pk = *(const v4u*)(w + k * (N / 2) + n / 2);
+        const int64_t g = kGrouped ? k / block_size : 0;
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            const u32 nib = (pk[e >> 3] >> (4 * (e & 7))) & 0xfu;
+            float v = (float)((int)(nib ^ 8u) - 8);
+            if (kGrouped) {
+                v = (v - (float)zero[g * N + n + e]) * scale[g * N + n + e];
+                const u32 top = __float_as_uint(v) & 0xffff0000u;
+                thi[r][32 * h + e] = (uint16_t)(top >> 16);
+                tlo[r][32 * h + e] = (uint16_t)f32_to_bf16_bits(v - __uint_as_float(top));
+            } else {
+                thi[r][32 * h + e] = (uint16_t)f32_to_bf16_bits(v);
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
+        v4u oh[4], ol[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int kk = 32 * part + 8 * q + 2 * d;
+                oh[q][d] = (u32)thi[kk][c] | ((u32)thi[kk + 1][c] << 16);
+                if (kGrouped) ol[q][d] = (u32)tlo[kk][c] | ((u32)tlo[kk + 1][c] << 16);
+            }
+        v4u* dst = (v4u*)(out + (n0 + c) * kParts * K + k0 + 32 * part);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            dst[q] = oh[q];
+            dst[q + K / 8] = oh[q];
+            if (kGrouped) dst[q + 2 * (K / 8)] = ol[q];
+        }
+    }
+}
+
 constexpr int64_t kGemmMinRows = 128;
 
-inline bool gemm_route_ok(int x_dtype, int64_t M, int64_t K, int64_t N) {
-    return x_dtype == K3Q_BF16 && M >= kGemmMinRows && (K % kDqK) == 0 && (N % kDqN) == 0;
+// The route's cost is nearly flat in M (the de-quantisation of the whole kernel, and a GEMM
+// whose few tiles each walk all of K), the row passes cost per 32 rows: the longer K, the more
+// rows the route needs to win (measured crossovers).
+inline bool gemm_route_ok(bool f32, int64_t M, int64_t K, int64_t N) {
+    int64_t min_rows = kGemmMinRows;
+    if (K > 2048) min_rows = 192;
+    if (f32 && K > 4096) min_rows = K > 8192 ? 320 : 256;
+    return M >= min_rows && (K % kDqK) == 0 && (N % kDqN) == 0;
+}
+
+// scratch of the GEMM route: the de-quantised kernel and, for float32 inputs, the split rows
+inline int64_t gemm_route_bytes(bool f32, bool grouped, int64_t M, int64_t K, int64_t N) {
+    if (!f32) return N * K * 2;
+    const int64_t parts = grouped ? 3 : 2;
+    return (N + M) * parts * K * 2;
 }
 
 struct Plan {
@@ -717,19 +811,37 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
     p.row_bytes = (N + 1) / 2;
     p.block_size = grouped ? (int)block_size : 0;
 
-    if (!plan_override && gemm_route_ok(x_dtype, M, K, N) && workspace &&
-        workspace_bytes >= N * K * 2 && aligned_to(workspace, 16) && aligned_to(w_packed, 16) &&
-        aligned_to(scale, 16) && (!zero || aligned_to(zero, 16)) &&
-        gemm_bf16_nk_supported(M, N, K, x, workspace, y)) {
+    if (!plan_override && gemm_route_ok(f32, M, K, N) && workspace &&
+        workspace_bytes >= gemm_route_bytes(f32, grouped, M, K, N) && aligned_to(workspace, 16) &&
+        aligned_to(w_packed, 16) && aligned_to(scale, 16) && (!zero || aligned_to(zero, 16)) &&
+        aligned_to(x, 16) && aligned_to(y, 16)) {
         dim3 grid((unsigned)(N / kDqN), (unsigned)(K / kDqK));
+        if (!f32) {
+            if (grouped)
+                dequant_w4_to_bf16_nk<true><<<grid, 256, 0, s>>>(
+                    (const uint8_t*)w_packed, (const uint16_t*)scale, (const int8_t*)zero,
+                    (uint16_t*)workspace, K, N, (int)block_size);
+            else
+                dequant_w4_to_bf16_nk<false><<<grid, 256, 0, s>>>(
+                    (const uint8_t*)w_packed, nullptr, nullptr, (uint16_t*)workspace, K, N, 0);
+            if (!gemm_bf16_nk_supported(M, N, K, x, workspace, y)) return K3Q_ERR_SHAPE;
+            return gemm_bf16_nk_run(x, workspace, M, N, K, grouped ? nullptr : scale, bias, y, false, s);
+        }
+        const int parts = grouped ? 3 : 2;
+        uint16_t* wt = (uint16_t*)workspace;            // [N, parts * K]
+        uint16_t* xs = wt + (int64_t)N * parts * K;      // [M, parts * K]
         if (grouped)
-            dequant_w4_to_bf16_nk<true><<<grid, 256, 0, s>>>(
-                (const uint8_t*)w_packed, (const uint16_t*)scale, (const int8_t*)zero,
-                (uint16_t*)workspace, K, N, (int)block_size);
+            dequant_w4_to_bf16_parts_nk<true><<<grid, 256, 0, s>>>(
+                (const uint8_t*)w_packed, (const float*)scale, (const int8_t*)zero, wt, K, N,
+                (int)block_size);
         else
-            dequant_w4_to_bf16_nk<false><<<grid, 256, 0, s>>>(
-                (const uint8_t*)w_packed, nullptr, nullptr, (uint16_t*)workspace, K, N, 0);
-        return gemm_bf16_nk_run(x, workspace, M, N, K, grouped ? nullptr : scale, bias, y, s);
+            dequant_w4_to_bf16_parts_nk<false><<<grid, 256, 0, s>>>(
+                (const uint8_t*)w_packed, nullptr, nullptr, wt, K, N, 0);
+        split_f32_rows<<<(unsigned)((M * K / 4 + 255) / 256), 256, 0, s>>>((const float*)x, xs, M, K,
+                                                                          parts);
+        if (!gemm_bf16_nk_supported(M, N, (int64_t)parts * K, xs, wt, y)) return K3Q_ERR_SHAPE;
+        return gemm_bf16_nk_run(xs, wt, M, N, (int64_t)parts * K, grouped ? nullptr : scale, bias, y,
+                                true, s);
     }
     Plan pl = make_plan(x_dtype, M, K, N, block_size, plan_override);
     // vector loads of x rows, packed rows, scales and zero points
@@ -817,7 +929,11 @@ extern "C" int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N) 
             if (b > part) part = b;
         }
     // prefill sizes: room for the bfloat16 [N, K] copy of the de-quantised kernel
-    if (gemm_route_ok(K3Q_BF16, M, K, N) && N * K * 2 > part) part = N * K * 2;
+    for (int f32 = 0; f32 < 2; ++f32)
+        if (gemm_route_ok(f32, M, K, N)) {
+            const int64_t need = gemm_route_bytes(f32, true, M, K, N);
+            if (need > part) part = need;
+        }
     return part;
 }
 

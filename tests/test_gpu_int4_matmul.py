@@ -101,8 +101,8 @@ def test_int4_repeatable(dev):
         assert torch.equal(first, again)
 
 
-# prefill sizes: bfloat16 inputs with M >= 128, K % 128 == 0, N % 64 == 0 take the
-# de-quantise + MFMA GEMM route; everything else stays on the 16-row passes
+# prefill sizes: M >= 128, K % 128 == 0, N % 64 == 0 take the de-quantise + MFMA GEMM route;
+# everything else stays on the row passes
 @pytest.mark.parametrize("M,K,N,block_size", [
     (128, 128, 64, None), (129, 256, 128, 128), (300, 512, 320, 64), (257, 1024, 512, 32),
     (1024, 4096, 4096, 128), (512, 4096, 14336, 128), (300, 2048, 1024, -1), (260, 384, 192, 128),
@@ -112,8 +112,20 @@ def test_int4_prefill_route(dev, M, K, N, block_size):
     run_case(dev, M, K, N, block_size, torch.bfloat16, with_bias=(N % 128 == 0))
 
 
+# float32 inputs on that route: the GEMM runs over the high / low bfloat16 parts of x and of the
+# de-quantised kernel, which must leave the result at float32 accuracy (far inside 1e-3)
+@pytest.mark.parametrize("M,K,N,block_size", [
+    (128, 128, 64, None), (129, 256, 128, 128), (300, 512, 320, 64), (257, 1024, 512, 32),
+    (1024, 4096, 4096, 128), (256, 4096, 14336, 128), (300, 2048, 1024, -1), (260, 384, 192, 128),
+    (1000, 256, 64, 256), (512, 4096, 4096, None),
+])
+def test_int4_prefill_route_f32(dev, M, K, N, block_size):
+    _, e_exact = run_case(dev, M, K, N, block_size, torch.float32, with_bias=(N % 128 == 0))
+    assert e_exact < 5e-5, e_exact
+
+
 @pytest.mark.parametrize("M,K,N,block_size,dtype", [
-    (300, 256, 128, 128, torch.float32),   # float32: not on the GEMM route
+    (300, 192, 128, 64, torch.float32),    # K % 128 != 0, float32
     (300, 192, 128, 64, torch.bfloat16),   # K % 128 != 0
     (280, 256, 96, None, torch.bfloat16),  # N % 64 != 0
     (100, 256, 128, 128, torch.bfloat16),  # M below the GEMM threshold

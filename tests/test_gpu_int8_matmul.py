@@ -20,8 +20,10 @@ def make_case(M, K, N, dtype, seed, with_bias=True):
     return x, qkernel, kscale, bias
 
 
-def run_dense_int8(dev, M, K, N, dtype, prepack, exact, seed=0, with_bias=True):
+def run_dense_int8(dev, M, K, N, dtype, prepack, exact, seed=0, with_bias=True, row_gain=None):
     x, qk, ks, bias = make_case(M, K, N, dtype, seed, with_bias)
+    if row_gain is not None:
+        x = (x.float() * row_gain[:, None]).to(dtype)
     want, inter = ref.dense_int8_call(x, qk, ks, bias, compute_dtype=dtype, return_intermediates=True)
     q, s = kq.abs_max_quantize(x.to(dev), axis=-1)
     assert torch.equal(q.cpu(), inter["q"])
@@ -62,6 +64,21 @@ def test_dense_int8_exact_epilogue(dev, M, K, N, dtype, prepack):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_dense_int8_fast_epilogue(dev, M, K, N, dtype):
     run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=False)
+
+
+@pytest.mark.parametrize("M,K,N", [(300, 640, 772), (16, 512, 256), (513, 256, 1028)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_int8_wide_range_scales(dev, M, K, N, dtype):
+    # rows of x spread over 60 decades: input scales from 1e-28 to 1e32, so the de-scale
+    # divides by very small and very large numbers (the bfloat16 epilogue switches from the
+    # reciprocal to the IEEE division per tile) and some outputs are tiny
+    gains = torch.tensor([1e-30, 1e-12, 1e-3, 1.0, 1e5, 1e12, 1e30])
+    row_gain = gains[torch.arange(M) % len(gains)]
+    run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True, row_gain=row_gain)
+    # one well-scaled block of rows next to the rest: tiles of both kinds in one call
+    row_gain = torch.ones(M)
+    row_gain[M // 2:] = gains[torch.arange(M - M // 2) % len(gains)]
+    run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True, row_gain=row_gain, seed=3)
 
 
 def test_config1_dense_4096(dev):
