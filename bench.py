@@ -49,6 +49,20 @@ def gemv_algorithmic_bytes(M, K, N, grouped, block=128):
     return K * (N // 2) + scales + 2 * M * K + 2 * M * N
 
 
+# The GPU's clocks take tens of milliseconds of load to come up from idle (measured: the same
+# GEMM runs 300 -> 240 us over its first 40 ms), and drop again while the host prepares the next
+# section.  Every timed region below is therefore preceded by this much untimed work of the
+# same kind, in addition to the --warmup steps.
+CLOCK_SPIN_UP_S = 0.2
+
+
+def spin_up(torch, fn, seconds=CLOCK_SPIN_UP_S):
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end:
+        fn()
+        torch.cuda.synchronize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -103,6 +117,7 @@ def main():
             for _ in range(args.steps):
                 step()
     torch.cuda.synchronize()
+    spin_up(torch, graph.replay)
     t0 = time.perf_counter()
     graph.replay()
     torch.cuda.synchronize()
@@ -115,6 +130,13 @@ def main():
     # dominant kernel alone, HIP events on the stream it is launched on
     q, s = kq.abs_max_quantize(x, axis=-1)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * args.steps)]
+
+    def gemm_burst():
+        for _ in range(20):
+            kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
+                             prepacked=prepacked)
+
+    spin_up(torch, gemm_burst)
     for i in range(args.steps):
         ev[2 * i].record()
         kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
@@ -160,8 +182,7 @@ def main():
                     for i in range(reps):
                         call(i)
             torch.cuda.synchronize()
-            graph.replay()
-            torch.cuda.synchronize()
+            spin_up(torch, graph.replay, 0.05)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(3):
@@ -249,6 +270,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "clock_spin_up_s": CLOCK_SPIN_UP_S,  # untimed work before each timed region, besides warmup
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
