@@ -188,6 +188,9 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
             char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
 #pragma unroll
             for (int d = 0; d < kDmaPerWave; ++d) {
+#ifdef K3Q_GEMM_PROBE_NO_BDMA
+                if (wave * kDmaPerWave + d >= kDmaA) continue;
+#endif
                 __builtin_amdgcn_global_load_lds(
                     (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
                     (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
@@ -215,9 +218,11 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         v4i af[2][kMBlk], bf[2][kNBlk];
         auto read_frags = [&](int fb, int stage, int ks) {
             const char* st = lds + stage * kStageBytes;
+#ifndef K3Q_GEMM_PROBE_NO_BREAD
 #pragma unroll
             for (int nb = 0; nb < kNBlk; ++nb)
                 bf[fb][nb] = *(const v4i*)(st + b_row[nb] + (((2 * ks + fg) ^ b_swz[nb]) << 4));
+#endif
 #pragma unroll
             for (int mb = 0; mb < kMBlk; ++mb)
                 af[fb][mb] = *(const v4i*)(st + a_row[mb] + (((2 * ks + fg) ^ a_swz[mb]) << 4));
@@ -247,6 +252,47 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         }
         bare_barrier();
         read_frags(0, 0, 0);
+        // The DMA of a stage is not issued as one burst: the texture unit takes an instruction
+        // per ~16 clocks and the workgroup's 64 would hold every wave (an in-order issuer) away
+        // from its MFMAs for up to a thousand clocks.  Instead one DMA instruction follows every
+        // kDmaStride-th MFMA, starting at the hand-over (second half of the last K step, into the
+        // buffer just released) and ending in the second K step of the next stage, which
+        // leaves the last one half a stage to land.
+        constexpr int kHalfMmas = kNBlk / 2 * kMBlk;
+        constexpr int kDmaStride = 5 * kHalfMmas / kDmaPerWave >= 2 ? 2 : 1;
+        static_assert(kKSteps == 4 && 5 * kHalfMmas / kDmaStride >= kDmaPerWave, "DMA slots");
+        auto issue_one = [&](int kt, int d) {
+#ifdef K3Q_GEMM_PROBE_NO_BDMA
+            if (wave * kDmaPerWave + d >= kDmaA) return;
+#endif
+            char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
+                (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
+        };
+        auto mma_half = [&](int ks, int half, int kt) {
+            // halves since the hand-over: 0 = second half of the last step (feeds stage kt+2),
+            // 1..4 = the two halves of steps 0 and 1 (feed stage kt+1, begun one stage earlier)
+            const int hh = (ks == kKSteps - 1 && half == 1) ? 0 : (ks <= 1 ? 1 + 2 * ks + half : -1);
+#pragma unroll
+            for (int j = 0; j < kHalfMmas; ++j) {
+                const int nb = half * (kNBlk / 2) + j / kMBlk, mb = j % kMBlk;
+#ifndef K3Q_GEMM_PROBE_NO_MMA
+                acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
+#endif
+#ifndef K3Q_GEMM_PROBE_NO_DMA
+                const int pos = hh * kHalfMmas + j;
+                if (hh >= 0 && pos % kDmaStride == kDmaStride - 1 && pos / kDmaStride < kDmaPerWave) {
+                    const int target = hh == 0 ? kt + 2 : kt + 1;
+                    if ((hh == 0 || kt >= 1) && target < KT) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        issue_one(target, pos / kDmaStride);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+#endif
+            }
+        };
         for (int kt = 0; kt < KT; ++kt) {
             const int cur = kt & 1;
 #pragma unroll
@@ -254,32 +300,18 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                 // first half of this step's MFMAs, then the reads for the next step, then the
                 // second half: the reads get half a step of matrix-core time to come back
                 __builtin_amdgcn_sched_barrier(0);
-#ifndef K3Q_GEMM_PROBE_NO_MMA
-#pragma unroll
-                for (int nb = 0; nb < kNBlk / 2; ++nb)
-#pragma unroll
-                    for (int mb = 0; mb < kMBlk; ++mb)
-                        acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
-#endif
+                mma_half(ks, 0, kt);
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks + 1 < kKSteps) {
                     read_frags((ks + 1) & 1, cur, ks + 1);
                 } else if (kt + 1 < KT) {
                     wait_vmcnt0();  // own DMA of stage kt+1 has landed (own reads of stage kt are done)
                     bare_barrier();
-#ifndef K3Q_GEMM_PROBE_NO_DMA
-                    if (kt + 2 < KT) issue_stage(kt + 2);
-#endif
                     read_frags(0, cur ^ 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-#ifndef K3Q_GEMM_PROBE_NO_MMA
-#pragma unroll
-                for (int nb = kNBlk / 2; nb < kNBlk; ++nb)
-#pragma unroll
-                    for (int mb = 0; mb < kMBlk; ++mb)
-                        acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
-#else
+                mma_half(ks, 1, kt);
+#ifdef K3Q_GEMM_PROBE_NO_MMA
                 // probe build: consume the fragments so that the reads stay
 #pragma unroll
                 for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] += (af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1]);
