@@ -18,7 +18,7 @@ import string
 import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
-from keras_amd.layers.dense import _ACTIVATIONS, _EXACT_EPILOGUE_MAX_OUTPUTS, glorot_uniform
+from keras_amd.layers.dense import _ACTIVATIONS, glorot_uniform
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
 from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
 
@@ -452,7 +452,7 @@ class EinsumDense(Layer):
         q, scale = self.inputs_quantizer(x2, axis=-1)
         exact = self.exact_epilogue
         if exact is None:
-            exact = x2.shape[0] * n <= _EXACT_EPILOGUE_MAX_OUTPUTS
+            exact = True
         y2 = kops.int8_matmul(
             q, k2, a_scale=scale,
             kernel_scale=self._cached("kernel_scale", self.kernel_scale,

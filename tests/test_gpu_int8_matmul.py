@@ -119,6 +119,28 @@ def test_gemm_full_size_accumulators(dev, M, K, N):
     assert torch.equal(acc.to(torch.int64).sum(1).cpu(), a.to(torch.int64) @ rowsum_b)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_dense_int8_full_size_rows_bit_exact(dev, dtype):
+    # the benchmark configuration end to end (quantize + GEMM + de-scale + bias); every row of
+    # the layer is independent of the others, so sampled rows are checked against the oracle
+    # run on those rows alone, bit for bit
+    M, K, N = 4096, 8192, 8192
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    kernel = ref.glorot_uniform(K, N, generator=g)
+    bias = torch.randn(N, generator=g) * 0.02
+    qk, ks = ref.dense_quantize_int8(kernel)
+    q, s = kq.abs_max_quantize(x.to(dev), axis=-1)
+    qk_d = qk.to(dev)
+    y = kops.int8_matmul(q, qk_d, a_scale=s, kernel_scale=ks.to(dtype).to(dev),
+                         bias=bias.to(dtype).to(dev), out_dtype=dtype,
+                         prepacked=kops.prepack_int8_kernel(qk_d), exact_epilogue=True)
+    rows = torch.cat([torch.tensor([0, 255, 256, M - 1]), torch.randint(0, M, (28,), generator=g)])
+    want = ref.dense_int8_call(x[rows], qk, ks, bias, compute_dtype=dtype)
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    assert torch.equal(y[rows.to(dev)].cpu().view(bits), want.view(bits))
+
+
 def test_prepack_is_transpose(dev):
     g = torch.Generator().manual_seed(1)
     for K, N in [(128, 64), (100, 37), (4096, 4096), (65, 129)]:
