@@ -33,8 +33,8 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
 # `--pmc WRITE_SIZE` (KiB per dispatch), each scaled by what the same counter reads for a plain
 # device copy of known size (FETCH_SIZE reads 0.50x, WRITE_SIZE 1.00x):
 # profiles/bench_dense_int8_M4096_K8192_N8192_and_int4_decode.md
-GEMM_HBM_TRAFFIC_BYTES = int((196814.6 * 2.0 + 90450.7) * 1024)
-QUANT_HBM_TRAFFIC_BYTES = int((32830.5 * 2.0 + 32832.0) * 1024)
+GEMM_HBM_TRAFFIC_BYTES = int((198717.9 * 2.0 + 67607.1) * 1024)
+QUANT_HBM_TRAFFIC_BYTES = int((32840.4 * 2.0 + 32832.0) * 1024)
 # int4 decode main kernel, keyed by (M > 8, grouped)
 GEMV_HBM_TRAFFIC_BYTES = {
     (False, False): int((16601.6 * 2.0 + 1280.0) * 1024),
