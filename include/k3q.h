@@ -103,7 +103,13 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  * rows), b_layout 1 -- e.g. a tied int8 embedding table used as the LM head -- up to
  * 16 rows (K % 64 == 0; up to 64 rows when the MFMA kernel's conditions do not hold).
  * They may split K and then need `workspace` for int32 partials.  The MFMA kernel
- * itself picks 128 x 128 tiles while 256 x 256 tiles would leave CUs idle.
+ * itself picks 128 x 128 tiles while 256 x 256 tiles would leave CUs idle, and where
+ * even those are few and K is long (e.g. M = 128, K = N = 8192) it splits K over
+ * workgroups: int32 partials in `workspace` after the [N,K] copy's place
+ * (ceil16(N * K) bytes in; with b_layout 1 only that second part is of use and a
+ * workspace of k3q_gemm_i8_workspace_bytes - ceil16(N * K) bytes may be passed), summed
+ * by a second kernel that applies the epilogue; results are the same bits either way.
+ * Without that room K is not split.
  * The reverse projection of ReversibleEmbedding._int8_call
  * (keras/src/layers/core/reversible_embedding.py:272-296) is this call with
  * b = the [vocab, dim] table as stored, b_layout 1 and no bias.
@@ -142,11 +148,12 @@ int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64
 
 /*
  * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; passes of
- * 32 rows (bfloat16) or 8 rows (float32) below prefill sizes; from M = 128 .. 320 rows on
- * (the longer K, the later), for K % 128 == 0 and N % 64 == 0, the kernel is de-quantised
- * once per call into `workspace` as bfloat16 [N, K] and the product runs on the MFMA tile
- * kernel; float32 x and the float32 de-quantised kernel go there as high + low bfloat16
- * parts concatenated along K, which keeps float32 accuracy to about 2^-17):
+ * 32 rows (bfloat16) or 8 rows (float32) below prefill sizes; from M = 128 rows on, for
+ * K % 128 == 0 and N % 64 == 0, the kernel is de-quantised once per call into `workspace`
+ * as bfloat16 [N, K] and the product runs on the MFMA tile kernel (which splits K over
+ * workgroups while its tiles are few); float32 x and the float32 de-quantised kernel go
+ * there as high + low bfloat16 parts concatenated along K, which keeps float32 accuracy to
+ * about 2^-17):
  *     per-channel (block_size <= 0):  y = T(T(x . unpack(w)) / scale[n])   (+ bias)
  *     grouped     (block_size  > 0):  y = T(x . ((unpack(w) - zero[g]) * scale[g]))  (+ bias),  g = k / block_size
  * x: [M, K] of x_dtype, contiguous.  w_packed: the layer's int4 kernel as stored,

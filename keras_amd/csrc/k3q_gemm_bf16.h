@@ -12,9 +12,14 @@ namespace k3q {
 bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* bt,
                             const void* y);
 
+// scratch for the partial sums of a K split (problems with few tiles and a long K); 0 if none
+int64_t gemm_bf16_nk_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
 // b_scale [N] and bias [N] may be null; they and y are bfloat16, or float32 with out_f32 (the
-// operands then being high / low bfloat16 parts of float32 values, concatenated along K)
+// operands then being high / low bfloat16 parts of float32 values, concatenated along K).
+// workspace (may be null: then K is not split) is 16-byte aligned scratch.
 int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
-                     const void* b_scale, const void* bias, void* y, bool out_f32, hipStream_t s);
+                     const void* b_scale, const void* bias, void* y, bool out_f32, void* workspace,
+                     int64_t workspace_bytes, hipStream_t s);
 
 }  // namespace k3q

@@ -77,6 +77,13 @@ struct GemmParams {
     int64_t row_bytes;      // bytes per row of a and bt: K (int8) or 2K (bfloat16 operands)
     int tiles_m, tiles_n;
     int flags;
+    // split of K over workgroups (problems with few tiles and a long K): split sp takes the
+    // stages [sp * kt_split, min((sp + 1) * kt_split, stages)) and stores its raw
+    // accumulators to part[sp][M][N] (int32 or float32); gemm_split_reduce sums them in
+    // split order and applies the epilogue
+    int splits, kt_split;
+    void* part;
+    int64_t part_bytes;
 };
 
 // 16-byte chunk swizzle of a 128-byte LDS row (8 chunks): chunk c of row r lives at chunk
@@ -111,6 +118,11 @@ __device__ __forceinline__ float load_t(const void* p, int64_t i) {
 constexpr int kKindI8 = 0;    // int8 x int8 -> int32, v_mfma_i32_32x32x32_i8
 constexpr int kKindBF16 = 1;  // bfloat16 x bfloat16 -> float32, v_mfma_f32_32x32x16_bf16
 
+__device__ __forceinline__ u32 raw_bits(int v) { return (u32)v; }
+__device__ __forceinline__ u32 raw_bits(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ void from_bits(u32 b, int& v) { v = (int)b; }
+__device__ __forceinline__ void from_bits(u32 b, float& v) { v = __uint_as_float(b); }
+
 template <int kKind>
 struct Mma;
 template <>
@@ -128,6 +140,47 @@ struct Mma<kKindBF16> {
                                                        __builtin_bit_cast(v8bf, a), c, 0, 0, 0);
     }
 };
+
+// De-scale of one int32 accumulator.  kExact: the reference's op sequence, every step rounded
+// to T (sa, sb are the scales); otherwise one final rounding (sa, sb are their reciprocals, bv
+// is 0 without a bias).  kDiv selects the bfloat16 division: 0 IEEE, 1 reciprocal (the caller
+// has checked the scales' range), 2 reciprocal with a range check per element; all three
+// give the same bits.
+template <bool kBF16, bool kExact, int kDiv>
+__device__ __forceinline__ float descale_i8(int acc, float sa, float sb, float bv, bool has_bias,
+                                            bool round_acc) {
+    float accf = (float)acc;
+    if (!kBF16 && round_acc) accf = round_bf16(accf);
+    if (!kExact) return (accf * sa) * sb + bv;
+    if (kBF16) {
+        const float os = round_bf16(sb * sa);
+        const float ab = round_bf16(accf);
+        float r = kDiv == 0   ? round_bf16(ab / os)
+                  : kDiv == 1 ? round_bf16(ab * __builtin_amdgcn_rcpf(os))
+                              : div_round_bf16(ab, os);
+        if (has_bias) r = round_bf16(r + bv);
+        return r;
+    }
+    float r = accf / (sb * sa);
+    if (has_bias) r = r + bv;
+    return r;
+}
+
+// De-scale of one float accumulator of the bfloat16-operand kind: y = T(T(acc) / scale[n])
+// (+ bias); T = bfloat16 or float32.
+template <bool kBF16>
+__device__ __forceinline__ float descale_f(float acc, float sb, float bv, bool has_s, bool has_b) {
+    float r = acc;
+    if (kBF16) {
+        r = round_bf16(r);
+        if (has_s) r = div_round_bf16(r, sb);
+        if (has_b) r = round_bf16(r + bv);
+    } else {
+        if (has_s) r = r / sb;
+        if (has_b) r = r + bv;
+    }
+    return r;
+}
 
 template <class T, int kKind, bool kBF16, bool kExact>
 __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
@@ -150,15 +203,16 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
     // Workgroups are dealt round-robin to the 8 XCDs; each XCD walks a contiguous range of
     // the tile list, and the list is ordered in bands of 4 tile rows so that the 32 tiles an
     // XCD runs at a time share A rows and B rows in its L2.
-    const int total = p.tiles_m * p.tiles_n;
+    const int total = p.tiles_m * p.tiles_n * p.splits;  // work items: (tile, split of K)
     const int per_xcd = (total + 7) / 8;
     // A workgroup stays on its CU and walks every (gridDim / 8)-th tile of its XCD's range:
     // the output stores of one tile drain while the next tile's loads are already running.
     const int tl_first = blockIdx.x / 8, tl_step = gridDim.x / 8;
     for (int tl = tl_first; tl < per_xcd; tl += tl_step) {
-        const int t = (blockIdx.x % 8) * per_xcd + tl;
-        if (t >= total) break;
+        const int item = (blockIdx.x % 8) * per_xcd + tl;
+        if (item >= total) break;
         if (tl != tl_first) __syncthreads();  // the previous tile's epilogue is done with the LDS
+        const int t = item / p.splits, sp = item - t * p.splits;
         constexpr int kBand = 4;
         const int band = t / (kBand * p.tiles_n);
         const int band_rows = min(kBand, p.tiles_m - band * kBand);
@@ -182,7 +236,8 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
             int64_t grow = (is_b ? n0 : m0) + row;
             const int64_t lim = (is_b ? p.N : p.M) - 1;
             grow = grow < lim ? grow : lim;
-            src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16;
+            src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16 +
+                     (int64_t)sp * p.kt_split * kBK;
         }
         auto issue_stage = [&](int kt) {
             char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
@@ -242,7 +297,8 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         // matrix core has work queued while waves meet.  At that barrier every wave holds its
         // last fragments of stage kt in registers, so stage kt+2 may be DMA-ed over stage kt, and
         // stage kt+1 (whose DMA every wave has waited for) may be read.
-        const int KT = (int)(p.row_bytes / kBK);
+        const int kt_first = sp * p.kt_split;  // this split's stages (all of K without a split)
+        const int KT = min(p.kt_split, (int)(p.row_bytes / kBK) - kt_first);
         issue_stage(0);
         if (KT > 1) {
             issue_stage(1);
@@ -328,6 +384,25 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         }
         if (p.acc_out) return;
 #endif
+        if (p.splits > 1) {
+            // raw accumulators of this split, as they lie (16 bytes per lane and column group)
+#pragma unroll
+            for (int mb = 0; mb < kMBlk; ++mb) {
+                const int64_t m = m0 + wm * kWM + mb * 32 + fi;
+#pragma unroll
+                for (int nb = 0; nb < kNBlk; ++nb)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int64_t n = n0 + wn * kWN + nb * 32 + 8 * rg + 4 * fg;
+                        if (m >= p.M || n >= p.N) continue;
+                        v4u o;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = raw_bits(acc[nb][mb][4 * rg + e]);
+                        *(v4u*)((u32*)p.part + ((int64_t)sp * p.M + m) * p.N + n) = o;
+                    }
+            }
+            continue;
+        }
         // ---- epilogue ----
         // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
         // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: a lane owns one row of y per mb
@@ -402,11 +477,11 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                 char* dst = (char*)p.y + (m * p.N + n) * kE;
                 const bool full = n + 16 / kE <= p.N;  // else the first 8 bytes (N % 4 == 0)
                 if (wide && full) {
-                    __builtin_nontemporal_store(d, (v4u*)dst);
+                    *(v4u*)dst = d;
                 } else {
                     v2u lo = {d[0], d[1]}, hi = {d[2], d[3]};
-                    __builtin_nontemporal_store(lo, (v2u*)dst);
-                    if (full) __builtin_nontemporal_store(hi, (v2u*)(dst + 8));
+                    *(v2u*)dst = lo;
+                    if (full) *(v2u*)(dst + 8) = hi;
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next block's writes
@@ -427,17 +502,8 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                         const v4f bv = *(const v4f*)(ep + kBN + nl);
                         float r[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            r[e] = (float)acc[nb][mb][4 * rg + e];
-                            if (kBF16) {
-                                r[e] = round_bf16(r[e]);
-                                if (has_s) r[e] = div_round_bf16(r[e], sb[e]);
-                                if (has_b) r[e] = round_bf16(r[e] + bv[e]);
-                            } else {
-                                if (has_s) r[e] = r[e] / sb[e];
-                                if (has_b) r[e] = r[e] + bv[e];
-                            }
-                        }
+                        for (int e = 0; e < 4; ++e)
+                            r[e] = descale_f<kBF16>((float)acc[nb][mb][4 * rg + e], sb[e], bv[e], has_s, has_b);
                         stage4(nb, rg, r);
                     }
                 }
@@ -469,27 +535,9 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                         const v4f bv = *(const v4f*)(ep + kBN + nl);
                         float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            float accf = (float)acc[nb][mb][4 * rg + e];
-                            if (!kBF16 && round_acc) accf = round_bf16(accf);
-                            float r;
-                            if (kExact) {
-                                // the reference's op sequence, every step rounded to T
-                                if (kBF16) {
-                                    const float os = round_bf16(sb[e] * sa);
-                                    const float ab = round_bf16(accf);
-                                    r = round_bf16(decltype(rcp_div)::value ? ab * __builtin_amdgcn_rcpf(os)
-                                                                            : ab / os);
-                                    if (has_bias) r = round_bf16(r + bv[e]);
-                                } else {
-                                    r = accf / (sb[e] * sa);
-                                    if (has_bias) r = r + bv[e];
-                                }
-                            } else {
-                                r = (accf * sa) * sb[e] + bv[e];  // sa, sb hold reciprocals here
-                            }
-                            v[e] = r;
-                        }
+                        for (int e = 0; e < 4; ++e)
+                            v[e] = descale_i8<kBF16, kExact, decltype(rcp_div)::value ? 1 : 0>(
+                                (int)acc[nb][mb][4 * rg + e], sa, sb[e], bv[e], has_bias, round_acc);
                         stage4(nb, rg, v);
                     }
                 }
@@ -630,6 +678,95 @@ inline int cu_count() {
     return cached[dev] > 0 ? cached[dev] : 0;
 }
 
+// Second kernel of a K split: sums part[0..splits)[m][n] in split order (int32: exact;
+// float32: one fixed order) and applies the epilogue of gemm_mfma.  One thread per four
+// consecutive columns of a row.
+template <int kKind, bool kBF16, bool kExact>
+__global__ __launch_bounds__(256) void gemm_split_reduce(GemmParams p) {
+    const int64_t quads = p.N / 4;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.M * quads) return;
+    const int64_t m = i / quads, n = (i - m * quads) * 4;
+    typedef typename std::conditional<kKind == kKindI8, int, float>::type Elem;
+    Elem sum[4] = {0, 0, 0, 0};
+    for (int sp = 0; sp < p.splits; ++sp) {
+        const v4u v = *(const v4u*)((const u32*)p.part + ((int64_t)sp * p.M + m) * p.N + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            Elem t;
+            from_bits(v[e], t);
+            sum[e] += t;
+        }
+    }
+    if constexpr (kKind == kKindI8) {
+        if (p.acc_out) {
+            v4i o = {(int)sum[0], (int)sum[1], (int)sum[2], (int)sum[3]};
+            *(v4i*)(p.acc_out + m * p.N + n) = o;
+        }
+    }
+    if (!p.y) return;
+    float r[4];
+    const bool has_bias = p.bias != nullptr;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float bv = has_bias ? load_t<kBF16>(p.bias, n + e) : 0.0f;
+        if constexpr (kKind == kKindBF16) {
+            const bool has_s = p.b_scale != nullptr;
+            r[e] = descale_f<kBF16>((float)sum[e], has_s ? load_t<kBF16>(p.b_scale, n + e) : 1.0f, bv,
+                                    has_s, has_bias);
+        } else {
+            float sa = p.a_scale ? load_t<kBF16>(p.a_scale, m) : 1.0f;
+            float sb = p.b_scale ? load_t<kBF16>(p.b_scale, n + e) : 1.0f;
+            if (!kExact) {
+                sa = 1.0f / sa;
+                sb = 1.0f / sb;
+            }
+            r[e] = descale_i8<kBF16, kExact, 2>((int)sum[e], sa, sb, bv, has_bias,
+                                                (p.flags & kFlagRoundAccBF16) != 0);
+        }
+    }
+    if (kBF16) {
+        v2u o = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+        *(v2u*)((uint16_t*)p.y + m * p.N + n) = o;
+    } else {
+        v4f o = {r[0], r[1], r[2], r[3]};
+        *(v4f*)((float*)p.y + m * p.N + n) = o;
+    }
+}
+
+// How many ways to split K.  A split pays where the tiles alone leave most of the chip idle
+// and K is long.  Cost model fitted to a sweep (128 x 128 tiles, M = 128 .. 1024, K = 2048 ..
+// 14336): an unsplit tile walks its stages at 0.65 us each, a split into sp saves
+// (1 - 1/sp) of that, costs 4 us for the second kernel and 0.052 us per tile and split for
+// writing and reading its 64 KiB of partials, and is taken while tiles * sp still fit on the
+// chip at once.  E.g. 32 tiles x 32 stages: 4; 64 x 64: 4; 32 x 112: 8; 128 x 64: 3;
+// 128 x 16 or 96 x 32: none.
+inline int choose_splits(int64_t tiles, int64_t stages, int resident, int forced) {
+    if (forced > 0) return (int)(forced < stages ? forced : stages);
+    int best = 1;
+    int64_t best_gain_ns = 0;
+    for (int sp = 2; sp <= 8; ++sp) {
+        if (tiles * sp > resident || stages / sp < 4) break;
+        const int64_t gain_ns = stages * 650 * (sp - 1) / sp - tiles * sp * 52 - 4000;
+        if (gain_ns > best_gain_ns) {
+            best_gain_ns = gain_ns;
+            best = sp;
+        }
+    }
+    return best;
+}
+
+constexpr int kFlagSplitShift = 16;  // undocumented tuning aid: bits 16..20 force the split count
+
+// Room for the partials of the largest split the launch may choose (sized for a chip of up
+// to 256 CUs; a launch that finds less room splits less).
+inline int64_t split_workspace_bytes(int64_t M, int64_t N, int64_t row_bytes) {
+    if (M <= 0 || (row_bytes % kBK) != 0 || (N % 4) != 0) return 0;
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    const int splits = choose_splits(tiles, row_bytes / kBK, 512, 0);
+    return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
+}
+
 template <class T, int kKind, bool kBF16, bool kExact>
 int launch_tile(GemmParams p, hipStream_t s) {
     // more than 64 KiB of dynamic LDS needs the attribute raised once per kernel
@@ -639,13 +776,27 @@ int launch_tile(GemmParams p, hipStream_t s) {
     if (!raised) return K3Q_ERR_LAUNCH;
     p.tiles_m = (int)((p.M + T::kBM - 1) / T::kBM);
     p.tiles_n = (int)((p.N + T::kBN - 1) / T::kBN);
-    const int total = p.tiles_m * p.tiles_n;
     // one resident set of workgroups (as many as fit on the chip at once, a multiple of the
     // 8 XCDs); each walks its share of the tiles
     const int resident = cu_count() * (T::kLdsBytes <= 64 * 1024 ? 2 : 1) / 8 * 8;
-    int grid = ((total + 7) / 8) * 8;
+    const int stages = (int)(p.row_bytes / kBK);
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    int splits = choose_splits(tiles, stages, resident, (p.flags >> kFlagSplitShift) & 31);
+    // partials need room, 16-byte rows (N % 4 == 0 holds on this path) and an output to make
+    if (splits > 1 && (!p.part || p.part_bytes < (int64_t)splits * p.M * p.N * 4)) {
+        const int64_t fit = p.part ? p.part_bytes / (p.M * p.N * 4) : 0;
+        splits = fit >= 2 ? (int)fit : 1;
+    }
+    p.kt_split = (stages + splits - 1) / splits;
+    p.splits = (stages + p.kt_split - 1) / p.kt_split;  // no empty split
+    const int64_t total = tiles * p.splits;
+    int64_t grid = ((total + 7) / 8) * 8;
     if (resident >= 8 && grid > resident) grid = resident;
-    gemm_mfma<T, kKind, kBF16, kExact><<<grid, T::kThreads, T::kLdsBytes, s>>>(p);
+    gemm_mfma<T, kKind, kBF16, kExact><<<(unsigned)grid, T::kThreads, T::kLdsBytes, s>>>(p);
+    if (p.splits > 1) {
+        const int64_t threads = p.M * (p.N / 4);
+        gemm_split_reduce<kKind, kBF16, kExact><<<(unsigned)((threads + 255) / 256), 256, 0, s>>>(p);
+    }
     return launch_status();
 }
 
@@ -670,9 +821,18 @@ bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, cons
            aligned_to(y, 8) && ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);
 }
 
+int64_t gemm_bf16_nk_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    return split_workspace_bytes(M, N, 2 * K);
+}
+
 int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_t K,
-                     const void* b_scale, const void* bias, void* y, bool out_f32, hipStream_t s) {
+                     const void* b_scale, const void* bias, void* y, bool out_f32, void* workspace,
+                     int64_t workspace_bytes, hipStream_t s) {
     GemmParams p{};
+    if (workspace && aligned_to(workspace, 16)) {
+        p.part = workspace;
+        p.part_bytes = workspace_bytes;
+    }
     p.a = (const int8_t*)a;
     p.bt = (const int8_t*)bt;
     p.b_scale = b_scale;
@@ -700,7 +860,8 @@ extern "C" int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K) 
         const int64_t nk = gemm_i8_skinny_nk_workspace_bytes(M, N, K);
         return kn > nk ? kn : nk;
     }
-    return N * K;
+    // the [N,K] copy (16-byte multiple), then the partials of a K split
+    return (N * K + 15) / 16 * 16 + split_workspace_bytes(M, N, K);
 }
 
 extern "C" int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N, int8_t* prepacked,
@@ -754,18 +915,25 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
         (M <= 16 || !fast))
         return gemm_i8_skinny_nk_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
                                      workspace, workspace_bytes, s);
+    char* scratch = (workspace && aligned_to(workspace, 16)) ? (char*)workspace : nullptr;
+    int64_t scratch_bytes = scratch ? workspace_bytes : 0;
     if (fast && b_layout == 0) {
         // needs the [N,K] copy: made here per call when the caller supplies scratch for it
-        if (workspace && workspace_bytes >= N * K && aligned_to(workspace, 16)) {
-            int rc = k3q_prepack_kernel_i8(b, K, N, (int8_t*)workspace, stream);
+        const int64_t copy_bytes = (N * K + 15) / 16 * 16;
+        if (scratch && scratch_bytes >= N * K) {
+            int rc = k3q_prepack_kernel_i8(b, K, N, (int8_t*)scratch, stream);
             if (rc != K3Q_OK) return rc;
-            p.bt = (const int8_t*)workspace;
+            p.bt = (const int8_t*)scratch;
+            scratch_bytes = scratch_bytes > copy_bytes ? scratch_bytes - copy_bytes : 0;
+            scratch += copy_bytes;
         } else {
             fast = false;
         }
     } else {
         p.bt = b;
     }
+    p.part = scratch_bytes > 0 ? scratch : nullptr;  // partials of a K split
+    p.part_bytes = scratch_bytes;
     if (fast) {
         const bool exact = (flags & kFlagExactEpilogue) != 0;
         if (bf16) return exact ? launch_mfma<kKindI8, true, true>(p, s) : launch_mfma<kKindI8, true, false>(p, s);
@@ -785,7 +953,8 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
 
 extern "C" int64_t k3q_gemm_w8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return N * K * 2;  // the kernel widened to bfloat16
+    // the kernel widened to bfloat16, then the partials of a K split
+    return N * K * 2 + split_workspace_bytes(M, N, 2 * K);
 }
 
 extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64_t M,
@@ -810,7 +979,9 @@ extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_la
             dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
             transpose_widen_i8_to_bf16<<<grid, 256, 0, s>>>(b, (uint16_t*)workspace, K, N);
         }
-        return gemm_bf16_nk_run(x, workspace, M, N, K, b_scale, bias, y, false, s);
+        char* rest = (char*)workspace + N * K * 2;
+        return gemm_bf16_nk_run(x, workspace, M, N, K, b_scale, bias, y, false, rest,
+                                workspace_bytes - N * K * 2, s);
     }
     if (M > 65535) return K3Q_ERR_SHAPE;
     dim3 grid((unsigned)((N + 255) / 256), (unsigned)M);

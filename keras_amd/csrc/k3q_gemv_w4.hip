@@ -636,14 +636,12 @@ __global__ __launch_bounds__(256) void dequant_w4_to_bf16_parts_nk(const uint8_t
 
 constexpr int64_t kGemmMinRows = 128;
 
-// The route's cost is nearly flat in M (the de-quantisation of the whole kernel, and a GEMM
-// whose few tiles each walk all of K), the row passes cost per 32 rows: the longer K, the more
-// rows the route needs to win (measured crossovers).
+// From 128 rows on the route wins: the row passes cost per 32 rows, the route's cost is
+// nearly flat in M up to a few hundred rows (the de-quantisation of the whole kernel, and a
+// GEMM that splits K while its tiles are few).
 inline bool gemm_route_ok(bool f32, int64_t M, int64_t K, int64_t N) {
-    int64_t min_rows = kGemmMinRows;
-    if (K > 2048) min_rows = 192;
-    if (f32 && K > 4096) min_rows = K > 8192 ? 320 : 256;
-    return M >= min_rows && (K % kDqK) == 0 && (N % kDqN) == 0;
+    (void)f32;
+    return M >= kGemmMinRows && (K % kDqK) == 0 && (N % kDqN) == 0;
 }
 
 // scratch of the GEMM route: the de-quantised kernel and, for float32 inputs, the split rows
@@ -651,6 +649,12 @@ inline int64_t gemm_route_bytes(bool f32, bool grouped, int64_t M, int64_t K, in
     if (!f32) return N * K * 2;
     const int64_t parts = grouped ? 3 : 2;
     return (N + M) * parts * K * 2;
+}
+
+// what the GEMM itself may use beyond that (partials of a K split)
+inline int64_t gemm_route_extra_bytes(bool f32, bool grouped, int64_t M, int64_t K, int64_t N) {
+    const int64_t parts = f32 ? (grouped ? 3 : 2) : 1;
+    return gemm_bf16_nk_workspace_bytes(M, N, parts * K);
 }
 
 struct Plan {
@@ -825,7 +829,9 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
                 dequant_w4_to_bf16_nk<false><<<grid, 256, 0, s>>>(
                     (const uint8_t*)w_packed, nullptr, nullptr, (uint16_t*)workspace, K, N, 0);
             if (!gemm_bf16_nk_supported(M, N, K, x, workspace, y)) return K3Q_ERR_SHAPE;
-            return gemm_bf16_nk_run(x, workspace, M, N, K, grouped ? nullptr : scale, bias, y, false, s);
+            const int64_t used = gemm_route_bytes(false, grouped, M, K, N);
+            return gemm_bf16_nk_run(x, workspace, M, N, K, grouped ? nullptr : scale, bias, y, false,
+                                    (char*)workspace + used, workspace_bytes - used, s);
         }
         const int parts = grouped ? 3 : 2;
         uint16_t* wt = (uint16_t*)workspace;            // [N, parts * K]
@@ -840,8 +846,9 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         split_f32_rows<<<(unsigned)((M * K / 4 + 255) / 256), 256, 0, s>>>((const float*)x, xs, M, K,
                                                                           parts);
         if (!gemm_bf16_nk_supported(M, N, (int64_t)parts * K, xs, wt, y)) return K3Q_ERR_SHAPE;
+        const int64_t used = gemm_route_bytes(true, grouped, M, K, N);
         return gemm_bf16_nk_run(xs, wt, M, N, (int64_t)parts * K, grouped ? nullptr : scale, bias, y,
-                                true, s);
+                                true, (char*)workspace + used, workspace_bytes - used, s);
     }
     Plan pl = make_plan(x_dtype, M, K, N, block_size, plan_override);
     // vector loads of x rows, packed rows, scales and zero points
@@ -931,7 +938,8 @@ extern "C" int64_t k3q_gemv_w4_workspace_bytes(int64_t M, int64_t K, int64_t N) 
     // prefill sizes: room for the bfloat16 [N, K] copy of the de-quantised kernel
     for (int f32 = 0; f32 < 2; ++f32)
         if (gemm_route_ok(f32, M, K, N)) {
-            const int64_t need = gemm_route_bytes(f32, true, M, K, N);
+            const int64_t need = gemm_route_bytes(f32, true, M, K, N) +
+                                 gemm_route_extra_bytes(f32, true, M, K, N);
             if (need > part) part = need;
         }
     return part;

@@ -140,13 +140,17 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
     lib = _lib.load()
     skinny = M <= SKINNY_MAX_ROWS and N % 16 == 0 and K % 8 == 0
+    nbytes = lib.k3q_gemm_i8_workspace_bytes(M, N, K)
     if prepacked is not None and not skinny:
-        b, layout, ws, ws_bytes = prepacked, 1, None, 0
+        # no per-call [N,K] copy: only the part of the scratch beyond it (partial sums of a
+        # K split, taken for few-tile problems) is of use
+        b, layout = prepacked, 1
+        nbytes = max(0, nbytes - (N * K + 15) // 16 * 16)
     else:
         b = kernel if kernel.is_contiguous() else kernel.contiguous()
         layout = 0
-        ws = _workspace(a.device, lib.k3q_gemm_i8_workspace_bytes(M, N, K))
-        ws_bytes = ws.numel()
+    ws = _workspace(a.device, nbytes) if nbytes > 0 else None
+    ws_bytes = nbytes if ws is not None else 0
     rc = lib.k3q_gemm_i8(
         _lib.ptr(a), _lib.ptr(b), layout, M, N, K, _lib.ptr(sa), _lib.ptr(sb), _lib.ptr(bias),
         code, GEMM_EXACT_EPILOGUE if exact_epilogue else 0, _lib.ptr(y), _lib.ptr(acc),

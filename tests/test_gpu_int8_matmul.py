@@ -40,8 +40,10 @@ def run_dense_int8(dev, M, K, N, dtype, prepack, exact, seed=0, with_bias=True, 
         assert torch.equal(y.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
                            want.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
     else:
+        # the opt-in fast epilogue rounds once where the reference's chain rounds four times:
+        # in bfloat16 the two can sit two ulps (2^-7 each) apart on the largest outputs
         e = max_rel_err(y, want)
-        assert e <= RTOL[dtype], e
+        assert e <= RTOL[dtype] * (2 if dtype == torch.bfloat16 else 1), e
     return y
 
 
@@ -79,6 +81,17 @@ def test_dense_int8_wide_range_scales(dev, M, K, N, dtype):
     row_gain = torch.ones(M)
     row_gain[M // 2:] = gains[torch.arange(M - M // 2) % len(gains)]
     run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True, row_gain=row_gain, seed=3)
+
+
+# few tiles and a long K: the tile kernel splits K over workgroups and a second kernel sums
+# the int32 partials and applies the epilogue; the result must not change by a bit
+@pytest.mark.parametrize("M,K,N", [(128, 4096, 4096), (130, 8192, 1028), (256, 14336, 512),
+                                   (384, 8192, 2048), (200, 4096, 260)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_int8_split_k(dev, M, K, N, dtype):
+    run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True)
+    run_dense_int8(dev, M, K, N, dtype, prepack=False, exact=True, seed=5, with_bias=False)
+    run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=False, seed=6)
 
 
 def test_config1_dense_4096(dev):
