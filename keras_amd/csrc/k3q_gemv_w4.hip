@@ -487,67 +487,96 @@ __global__ __launch_bounds__(256) void gemv_w4_generic(GemvParams p) {
 // (exact) and the GEMM epilogue divides by the scale, as the reference's matmul + divide does;
 // grouped: it holds T((w - zero) * scale), rounded to bfloat16 per weight exactly as the
 // reference's de-quantised kernel is.
-constexpr int kDqK = 128;  // tile: 128 rows of K x 64 columns
-constexpr int kDqN = 64;
+constexpr int kDqK = 64;    // tile of a workgroup: 64 rows of K x 256 columns, so that both the
+constexpr int kDqN = 256;   // packed rows read and the [n][k] rows written are whole 128-byte lines
+constexpr int kDqRouteK = 128, kDqRouteN = 64;  // shapes the route takes: K % 128 == 0, N % 64 == 0
 
-template <bool kGrouped>
-__global__ __launch_bounds__(256) void dequant_w4_to_bf16_nk(const uint8_t* __restrict__ w,
-                                                            const uint16_t* __restrict__ scale,
-                                                            const int8_t* __restrict__ zero,
-                                                            uint16_t* __restrict__ out, int64_t K,
-                                                            int64_t N, int block_size) {
-    __shared__ uint16_t tile[kDqK][kDqN + 2];
+// kF32 = false: bfloat16 scales, out[N][K] = T(w) or T((w - zero) * scale), rounded per weight
+// exactly as the reference's de-quantised kernel is.
+// kF32 = true: float32 scales, output rows of `parts` segments of K values for the float32
+// route below: [w | w] (per-channel, exact) or [wh | wh | wl] of w = (nibble - zero) * scale.
+//
+// Phase 1, thread = (row pair rp, 32-column chunk c): two 16-byte loads (rows 2rp, 2rp + 1),
+// each column's pair of values packed into one dword and written to the LDS tile [n][k]
+// (128 bytes of k per column, 16-byte chunks XOR-swizzled by the column so that phase 2's
+// reads spread over the banks).  Phase 2, thread = (column, 16-byte chunk of k): eight lanes
+// store one 128-byte piece of an output row.
+template <bool kGrouped, bool kF32>
+__global__ __launch_bounds__(256) void dequant_w4_nk(const uint8_t* __restrict__ w,
+                                                     const void* __restrict__ scale,
+                                                     const int8_t* __restrict__ zero,
+                                                     uint16_t* __restrict__ out, int64_t K, int64_t N,
+                                                     int block_size) {
+    constexpr bool kLow = kGrouped && kF32;  // a low part exists
+    constexpr int kParts = kF32 ? (kGrouped ? 3 : 2) : 1;
+    __shared__ __attribute__((aligned(16))) u32 thi[kDqN * 32];
+    __shared__ __attribute__((aligned(16))) u32 tlo[kLow ? kDqN * 32 : 4];
     const int64_t k0 = (int64_t)blockIdx.y * kDqK;
     const int64_t n0 = (int64_t)blockIdx.x * kDqN;
     {
-        // thread -> (row k, 32 columns): one 16-byte load of packed nibbles
-        const int r = threadIdx.x >> 1, h = threadIdx.x & 1;
-        const int64_t k = k0 + r, n = n0 + 32 * h;
-        const v4u pk = *(const v4u*)(w + k * (N / 2) + n / 2);
-        float sc[32], zp[32];
-        if (kGrouped) {
-            const int64_t g = k / block_size;
-            const v4u* sp = (const v4u*)(scale + g * N + n);
-            const v4u* zq = (const v4u*)(zero + g * N + n);
+        const int rp = threadIdx.x & 31, c = threadIdx.x >> 5;
+        const int64_t k = k0 + 2 * rp, n = n0 + 32 * c;
+        if (n < N) {  // N % 32 == 0: a chunk is inside or outside as a whole
+            const v4u p0 = *(const v4u*)(w + k * (N / 2) + n / 2);
+            const v4u p1 = *(const v4u*)(w + (k + 1) * (N / 2) + n / 2);
+            const int64_t g = kGrouped ? k / block_size : 0;  // block_size is even: one group for both rows
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const v4u sv = sp[q];
+                float sc[8], zp[8];
+                if (kGrouped) {
+                    const v2u zv = *(const v2u*)(zero + g * N + n + 8 * q);
 #pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    sc[8 * q + 2 * d] = __uint_as_float(sv[d] << 16);
-                    sc[8 * q + 2 * d + 1] = __uint_as_float(sv[d] & 0xffff0000u);
+                    for (int e = 0; e < 8; ++e) zp[e] = (float)(int)(int8_t)(zv[e >> 2] >> (8 * (e & 3)));
+                    if (kF32) {
+                        const v4f s0 = *(const v4f*)((const float*)scale + g * N + n + 8 * q);
+                        const v4f s1 = *(const v4f*)((const float*)scale + g * N + n + 8 * q + 4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            sc[e] = s0[e];
+                            sc[4 + e] = s1[e];
+                        }
+                    } else {
+                        const v4u sv = *(const v4u*)((const uint16_t*)scale + g * N + n + 8 * q);
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            sc[2 * d] = __uint_as_float(sv[d] << 16);
+                            sc[2 * d + 1] = __uint_as_float(sv[d] & 0xffff0000u);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    // low nibble = even column; sign-extended 4-bit field
+                    float v0 = (float)(int)__builtin_amdgcn_sbfe((int)p0[q], 4 * e, 4);  // the builtin's type is unsigned
+                    float v1 = (float)(int)__builtin_amdgcn_sbfe((int)p1[q], 4 * e, 4);
+                    if (kGrouped) {  // the difference is exact, the product rounds once
+                        v0 = (v0 - zp[e]) * sc[e];
+                        v1 = (v1 - zp[e]) * sc[e];
+                    }
+                    const int nl = 32 * c + 8 * q + e;
+                    const int at = nl * 32 + (rp ^ (((nl >> 1) & 7) << 2));
+                    if (kLow) {
+                        const u32 t0 = __float_as_uint(v0) & 0xffff0000u, t1 = __float_as_uint(v1) & 0xffff0000u;
+                        thi[at] = (t0 >> 16) | t1;
+                        tlo[at] = pack_bf16x2(v0 - __uint_as_float(t0), v1 - __uint_as_float(t1));
+                    } else {
+                        thi[at] = pack_bf16x2(v0, v1);
+                    }
                 }
             }
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const v4u zv = zq[q];
-#pragma unroll
-                for (int e = 0; e < 16; ++e) zp[16 * q + e] = (float)(int)(int8_t)(zv[e >> 2] >> (8 * (e & 3)));
-            }
-        }
-#pragma unroll
-        for (int e = 0; e < 32; ++e) {
-            const u32 nib = (pk[e >> 3] >> (4 * (e & 7))) & 0xfu;  // low nibble = even column
-            float v = (float)((int)(nib ^ 8u) - 8);
-            if (kGrouped) v = (v - zp[e]) * sc[e];  // the difference is exact, one rounding
-            tile[r][32 * h + e] = (uint16_t)f32_to_bf16_bits(v);
         }
     }
     __syncthreads();
-    {
-        // thread -> (column n, 32 rows of k): 64 contiguous bytes of output row n
-        const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
-        v4u o[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                const int kk = 32 * part + 8 * q + 2 * d;
-                o[q][d] = (u32)tile[kk][c] | ((u32)tile[kk + 1][c] << 16);
-            }
-        v4u* dst = (v4u*)(out + (n0 + c) * K + k0 + 32 * part);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) dst[q] = o[q];
+    for (int i = 0; i < 8; ++i) {
+        const int nl = (threadIdx.x >> 3) + 32 * i, j = threadIdx.x & 7;
+        if (n0 + nl >= N) continue;
+        const int at = nl * 32 + ((j ^ ((nl >> 1) & 7)) << 2);
+        const v4u hi = *(const v4u*)(thi + at);
+        uint16_t* dst = out + (n0 + nl) * kParts * K + k0 + 8 * j;
+        *(v4u*)dst = hi;
+        if (kF32) *(v4u*)(dst + K) = hi;
+        if (kLow) *(v4u*)(dst + 2 * K) = *(const v4u*)(tlo + at);
     }
 }
 
@@ -580,60 +609,6 @@ __global__ __launch_bounds__(256) void split_f32_rows(const float* __restrict__ 
     if (parts == 3) *(v2u*)(row + 2 * K) = h2;
 }
 
-// As dequant_w4_to_bf16_nk, for float32 scales: output rows of `parts` segments of K values,
-// [w | w] (per-channel, exact) or [wh | wh | wl] of w = (nibble - zero) * scale.
-template <bool kGrouped>
-__global__ __launch_bounds__(256) void dequant_w4_to_bf16_parts_nk(const uint8_t* __restrict__ w,
-                                                                  const float* __restrict__ scale,
-                                                                  const int8_t* __restrict__ zero,
-                                                                  uint16_t* __restrict__ out,
-                                                                  int64_t K, int64_t N, int block_size) {
-    constexpr int kParts = kGrouped ? 3 : 2;
-    __shared__ uint16_t thi[kDqK][kDqN + 2];
-    __shared__ uint16_t tlo[kGrouped ? kDqK : 1][kDqN + 2];
-    const int64_t k0 = (int64_t)blockIdx.y * kDqK;
-    const int64_t n0 = (int64_t)blockIdx.x * kDqN;
-    {
-        const int r = threadIdx.x >> 1, h = threadIdx.x & 1;
-        const int64_t k = k0 + r, n = n0 + 32 * h;
-        const v4u pk = *(const v4u*)(w + k * (N / 2) + n / 2);
-        const int64_t g = kGrouped ? k / block_size : 0;
-#pragma unroll
-        for (int e = 0; e < 32; ++e) {
-            const u32 nib = (pk[e >> 3] >> (4 * (e & 7))) & 0xfu;
-            float v = (float)((int)(nib ^ 8u) - 8);
-            if (kGrouped) {
-                v = (v - (float)zero[g * N + n + e]) * scale[g * N + n + e];
-                const u32 top = __float_as_uint(v) & 0xffff0000u;
-                thi[r][32 * h + e] = (uint16_t)(top >> 16);
-                tlo[r][32 * h + e] = (uint16_t)f32_to_bf16_bits(v - __uint_as_float(top));
-            } else {
-                thi[r][32 * h + e] = (uint16_t)f32_to_bf16_bits(v);
-            }
-        }
-    }
-    __syncthreads();
-    {
-        const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
-        v4u oh[4], ol[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                const int kk = 32 * part + 8 * q + 2 * d;
-                oh[q][d] = (u32)thi[kk][c] | ((u32)thi[kk + 1][c] << 16);
-                if (kGrouped) ol[q][d] = (u32)tlo[kk][c] | ((u32)tlo[kk + 1][c] << 16);
-            }
-        v4u* dst = (v4u*)(out + (n0 + c) * kParts * K + k0 + 32 * part);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            dst[q] = oh[q];
-            dst[q + K / 8] = oh[q];
-            if (kGrouped) dst[q + 2 * (K / 8)] = ol[q];
-        }
-    }
-}
-
 constexpr int64_t kGemmMinRows = 128;
 
 // From 128 rows on the route wins: the row passes cost per 32 rows, the route's cost is
@@ -641,7 +616,7 @@ constexpr int64_t kGemmMinRows = 128;
 // GEMM that splits K while its tiles are few).
 inline bool gemm_route_ok(bool f32, int64_t M, int64_t K, int64_t N) {
     (void)f32;
-    return M >= kGemmMinRows && (K % kDqK) == 0 && (N % kDqN) == 0;
+    return M >= kGemmMinRows && (K % kDqRouteK) == 0 && (N % kDqRouteN) == 0;
 }
 
 // scratch of the GEMM route: the de-quantised kernel and, for float32 inputs, the split rows
@@ -819,14 +794,14 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         workspace_bytes >= gemm_route_bytes(f32, grouped, M, K, N) && aligned_to(workspace, 16) &&
         aligned_to(w_packed, 16) && aligned_to(scale, 16) && (!zero || aligned_to(zero, 16)) &&
         aligned_to(x, 16) && aligned_to(y, 16)) {
-        dim3 grid((unsigned)(N / kDqN), (unsigned)(K / kDqK));
+        dim3 grid((unsigned)((N + kDqN - 1) / kDqN), (unsigned)(K / kDqK));
         if (!f32) {
             if (grouped)
-                dequant_w4_to_bf16_nk<true><<<grid, 256, 0, s>>>(
-                    (const uint8_t*)w_packed, (const uint16_t*)scale, (const int8_t*)zero,
-                    (uint16_t*)workspace, K, N, (int)block_size);
+                dequant_w4_nk<true, false><<<grid, 256, 0, s>>>(
+                    (const uint8_t*)w_packed, scale, (const int8_t*)zero, (uint16_t*)workspace, K, N,
+                    (int)block_size);
             else
-                dequant_w4_to_bf16_nk<false><<<grid, 256, 0, s>>>(
+                dequant_w4_nk<false, false><<<grid, 256, 0, s>>>(
                     (const uint8_t*)w_packed, nullptr, nullptr, (uint16_t*)workspace, K, N, 0);
             if (!gemm_bf16_nk_supported(M, N, K, x, workspace, y)) return K3Q_ERR_SHAPE;
             const int64_t used = gemm_route_bytes(false, grouped, M, K, N);
@@ -837,11 +812,10 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         uint16_t* wt = (uint16_t*)workspace;            // [N, parts * K]
         uint16_t* xs = wt + (int64_t)N * parts * K;      // [M, parts * K]
         if (grouped)
-            dequant_w4_to_bf16_parts_nk<true><<<grid, 256, 0, s>>>(
-                (const uint8_t*)w_packed, (const float*)scale, (const int8_t*)zero, wt, K, N,
-                (int)block_size);
+            dequant_w4_nk<true, true><<<grid, 256, 0, s>>>(
+                (const uint8_t*)w_packed, scale, (const int8_t*)zero, wt, K, N, (int)block_size);
         else
-            dequant_w4_to_bf16_parts_nk<false><<<grid, 256, 0, s>>>(
+            dequant_w4_nk<false, true><<<grid, 256, 0, s>>>(
                 (const uint8_t*)w_packed, nullptr, nullptr, wt, K, N, 0);
         split_f32_rows<<<(unsigned)((M * K / 4 + 255) / 256), 256, 0, s>>>((const float*)x, xs, M, K,
                                                                           parts);
