@@ -148,7 +148,7 @@ int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64
 
 /*
  * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; passes of
- * 32 rows (bfloat16) or 8 rows (float32) below prefill sizes; from M = 128 rows on, for
+ * 32 rows (bfloat16) or 8 rows (float32) below prefill sizes; from 65 (float32: 48 to 80) rows on, for
  * K % 128 == 0 and N % 64 == 0, the kernel is de-quantised once per call into `workspace`
  * as bfloat16 [N, K] and the product runs on the MFMA tile kernel (which splits K over
  * workgroups while its tiles are few); float32 x and the float32 de-quantised kernel go

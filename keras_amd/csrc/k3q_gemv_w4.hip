@@ -609,14 +609,18 @@ __global__ __launch_bounds__(256) void split_f32_rows(const float* __restrict__ 
     if (parts == 3) *(v2u*)(row + 2 * K) = h2;
 }
 
-constexpr int64_t kGemmMinRows = 128;
+// From here on the route wins: the row passes cost per 32 rows (bfloat16; K = N = 4096: 17 us
+// each) or per 8 rows (float32: 10 us each), the route's cost is nearly flat in M up to a few
+// hundred rows (the de-quantisation of the whole kernel, and a GEMM that splits K while its
+// tiles are few): 31 us at 128 bfloat16 rows, 56 us at 128 float32 rows.
+// The float32 route writes six bytes per weight before its GEMM starts, so on large kernels
+// it needs more rows to win (4096 x 14336: 167 us flat against 2.1 us per row in passes).
+constexpr int64_t kGemmMinRowsBF16 = 65, kGemmMinRowsF32 = 48, kGemmMinRowsF32Large = 80;
 
-// From 128 rows on the route wins: the row passes cost per 32 rows, the route's cost is
-// nearly flat in M up to a few hundred rows (the de-quantisation of the whole kernel, and a
-// GEMM that splits K while its tiles are few).
 inline bool gemm_route_ok(bool f32, int64_t M, int64_t K, int64_t N) {
-    (void)f32;
-    return M >= kGemmMinRows && (K % kDqRouteK) == 0 && (N % kDqRouteN) == 0;
+    const int64_t min_rows = !f32 ? kGemmMinRowsBF16
+                                  : (K * N > (int64_t(1) << 25) ? kGemmMinRowsF32Large : kGemmMinRowsF32);
+    return M >= min_rows && (K % kDqRouteK) == 0 && (N % kDqRouteN) == 0;
 }
 
 // scratch of the GEMM route: the de-quantised kernel and, for float32 inputs, the split rows

@@ -101,7 +101,7 @@ def test_int4_repeatable(dev):
         assert torch.equal(first, again)
 
 
-# prefill sizes: M >= 128, K % 128 == 0, N % 64 == 0 take the de-quantise + MFMA GEMM route;
+# prefill sizes: M > 64 (float32: >= 48), K % 128 == 0, N % 64 == 0 take the de-quantise + MFMA GEMM route;
 # everything else stays on the row passes
 @pytest.mark.parametrize("M,K,N,block_size", [
     (128, 128, 64, None), (129, 256, 128, 128), (300, 512, 320, 64), (257, 1024, 512, 32),
@@ -128,13 +128,14 @@ def test_int4_prefill_route_f32(dev, M, K, N, block_size):
     (300, 192, 128, 64, torch.float32),    # K % 128 != 0, float32
     (300, 192, 128, 64, torch.bfloat16),   # K % 128 != 0
     (280, 256, 96, None, torch.bfloat16),  # N % 64 != 0
-    (100, 256, 128, 128, torch.bfloat16),  # M below the GEMM threshold
+    (60, 256, 128, 128, torch.bfloat16),   # M below the GEMM threshold
 ])
 def test_int4_large_m_off_route(dev, M, K, N, block_size, dtype):
     run_case(dev, M, K, N, block_size, dtype, with_bias=True)
 
 
-# 17..127 rows: passes of 32 rows (four row sets), last pass narrower
+# 17..127 rows: passes of 32 rows (four row sets, last pass narrower) up to 64 rows, the GEMM
+# route beyond where the shape allows it
 @pytest.mark.parametrize("M,K,N,block_size", [
     (17, 256, 512, 128), (32, 512, 1024, None), (33, 1024, 256, 64), (64, 4096, 4096, 128),
     (100, 512, 384, 32), (127, 2048, 1024, None), (40, 100, 30, 50), (31, 4096, 14336, 128),
