@@ -101,7 +101,7 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  * Decode sizes run bandwidth-bound kernels that stream b in place, always with the
  * exact epilogue: b_layout 0 up to 64 rows (N % 16 == 0, K % 8 == 0; passes of 16
  * rows), b_layout 1 -- e.g. a tied int8 embedding table used as the LM head -- up to
- * 16 rows (K % 64 == 0; up to 64 rows when the MFMA kernel's conditions do not hold).
+ * 8 rows (K % 64 == 0; up to 64 rows when the MFMA kernel's conditions do not hold).
  * They may split K and then need `workspace` for int32 partials.  The MFMA kernel
  * itself picks 128 x 128 tiles while 256 x 256 tiles would leave CUs idle, and where
  * even those are few and K is long (e.g. M = 128, K = N = 8192) it splits K over

@@ -908,11 +908,11 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
                 (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
                 (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&
                 ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);
-    // [N,K] kernel at decode sizes: the streaming kernel up to 16 rows (one pass); beyond
-    // that the 128-row tiles read the kernel once where the passes would read it M/16 times
-    // (vocabulary 32000 x 4096: 16 rows 45 us, 64 rows 176 us in passes, 41 us tiled)
+    // [N,K] kernel at decode sizes: the streaming kernel up to 8 rows; beyond that the 128-row
+    // tiles (which split K while they are few) are as fast or faster (K = N = 8192, 16 rows:
+    // 24 us streamed, 19 us tiled; vocabulary 32000 x 4096, 64 rows: 176 us in passes, 41 us tiled)
     if (b_layout == 1 && !forced_tile && gemm_i8_skinny_nk_supported(M, N, K, a, b) &&
-        (M <= 16 || !fast))
+        (M <= 8 || !fast))
         return gemm_i8_skinny_nk_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
                                      workspace, workspace_bytes, s);
     char* scratch = (workspace && aligned_to(workspace, 16)) ? (char*)workspace : nullptr;

@@ -89,9 +89,10 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
 
 
 GEMM_EXACT_EPILOGUE = 1
-# up to this many rows the int8 matmul streams the [K, N] kernel in place (passes of 16 rows);
-# above, the prepacked copy on 128-row MFMA tiles is faster
-SKINNY_MAX_ROWS = 32
+# up to this many rows the int8 matmul streams the [K, N] kernel in place; above, the prepacked
+# copy on 128-row MFMA tiles (K split over workgroups while the tiles are few) is faster
+# (K = N = 4096, 17..64 rows: 11-13 us against 26-63 us in 16-row passes)
+SKINNY_MAX_ROWS = 8
 
 
 def prepack_int8_kernel(kernel):
