@@ -33,6 +33,19 @@ _ACTIVATIONS = {
 # bit (the default: it costs under 2 % of a prefill-sized matmul); False rounds once at the end.
 
 
+def activation_name(fn):
+    for name, f in _ACTIVATIONS.items():
+        if f is fn:
+            return name
+    raise ValueError(f"activation {fn} has no serializable name")
+
+
+def serialize_quantization_config(config):
+    if config is None:
+        return None
+    return {"class_name": type(config).__name__, "config": config.get_config()}
+
+
 def glorot_uniform(shape, dtype, generator=None):
     """U(-L, L), L = sqrt(6 / (fan_in + fan_out))
     (keras/src/initializers/random_initializers.py:292-318)."""
@@ -48,8 +61,10 @@ def glorot_uniform(shape, dtype, generator=None):
 
 class Dense(Layer):
     def __init__(self, units, activation=None, use_bias=True, kernel_initializer=None,
-                 bias_initializer="zeros", dtype=None, name=None, device=None):
+                 bias_initializer="zeros", dtype=None, name=None, device=None,
+                 quantization_config=None):
         super().__init__(dtype=dtype, name=name, device=device)
+        self.quantization_config = quantization_config  # dense.py:98-130
         if not isinstance(units, int) or units <= 0:
             raise ValueError(
                 f"Received an invalid value for `units`, expected a positive integer. Received: units={units}"
@@ -65,9 +80,11 @@ class Dense(Layer):
 
     # ---- build --------------------------------------------------------------
     def build(self, input_shape):
+        self._build_input_shape = tuple(input_shape)
         kernel_shape = (input_shape[-1], self.units)
         if self.quantization_mode:
-            self.quantized_build(kernel_shape, mode=self.quantization_mode)
+            self.quantized_build(kernel_shape, mode=self.quantization_mode,
+                                 config=self.quantization_config)
         if self.quantization_mode not in ("int8", "int4"):
             self._kernel = self.add_weight(
                 name="kernel", shape=kernel_shape, initializer=self.kernel_initializer, trainable=True
@@ -339,12 +356,8 @@ class Dense(Layer):
         return {
             "name": self.name,
             "units": self.units,
+            "activation": activation_name(self.activation),
             "use_bias": self.use_bias,
             "dtype": self.dtype_policy.name,
-            "quantization_config": (
-                None if self.quantization_config is None else {
-                    "class_name": type(self.quantization_config).__name__,
-                    "config": self.quantization_config.get_config(),
-                }
-            ),
+            "quantization_config": serialize_quantization_config(self.quantization_config),
         }

@@ -18,7 +18,8 @@ import string
 import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
-from keras_amd.layers.dense import _ACTIVATIONS, glorot_uniform
+from keras_amd.layers.dense import (_ACTIVATIONS, activation_name, glorot_uniform,
+                                    serialize_quantization_config)
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
 from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
 
@@ -196,8 +197,9 @@ class _GemmView:
 class EinsumDense(Layer):
     def __init__(self, equation, output_shape, activation=None, bias_axes=None,
                  kernel_initializer=None, bias_initializer="zeros", dtype=None, name=None,
-                 device=None):
+                 device=None, quantization_config=None):
         super().__init__(dtype=dtype, name=name, device=device)
+        self.quantization_config = quantization_config  # einsum_dense.py __init__ / build
         self.equation = equation
         self.partial_output_shape = (output_shape,) if isinstance(output_shape, int) else tuple(output_shape)
         self.bias_axes = bias_axes
@@ -210,6 +212,7 @@ class EinsumDense(Layer):
 
     # ---- build ---------------------------------------------------------------
     def build(self, input_shape):
+        self._build_input_shape = tuple(input_shape)
         kernel_shape, bias_shape, full_output_shape = analyze_einsum_shapes(
             self.equation, self.bias_axes, tuple(input_shape), self.partial_output_shape
         )
@@ -217,7 +220,8 @@ class EinsumDense(Layer):
         self.input_rank = len(input_shape)
         self.original_kernel_shape = kernel_shape
         if self.quantization_mode is not None:
-            self.quantized_build(kernel_shape, mode=self.quantization_mode)
+            self.quantized_build(kernel_shape, mode=self.quantization_mode,
+                                 config=self.quantization_config)
         if self.quantization_mode not in ("int8", "int4"):
             self._kernel = self.add_weight(
                 name="kernel", shape=kernel_shape, initializer=self.kernel_initializer, trainable=True
@@ -507,6 +511,17 @@ class EinsumDense(Layer):
         return self._finish(y2, free_shape, gv, fused)
 
     # ---- serialization -------------------------------------------------------------------------
+    def get_config(self):
+        return {
+            "name": self.name,
+            "output_shape": list(self.partial_output_shape),
+            "equation": self.equation,
+            "activation": activation_name(self.activation),
+            "bias_axes": self.bias_axes,
+            "dtype": self.dtype_policy.name,
+            "quantization_config": serialize_quantization_config(self.quantization_config),
+        }
+
     @property
     def variable_serialization_spec(self):
         """einsum_dense.py:560-610, the modes built here."""

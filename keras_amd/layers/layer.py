@@ -7,6 +7,8 @@ the dispatch to `_int8_call` / `_int4_call`
 (keras/src/layers/layer.py:243-261, :797-849, :874-1003, :1366-1458).
 """
 
+import re
+
 import numpy as np
 import torch
 
@@ -21,6 +23,12 @@ _TORCH_DTYPES = {
     "uint8": torch.uint8,
     "int32": torch.int32,
 }
+
+
+def _snake_case(name):
+    name = re.sub(r"\W+", "", name)
+    name = re.sub("(.)([A-Z][a-z]+)", r"\1_\2", name)
+    return re.sub("([a-z])([A-Z])", r"\1_\2", name).lower()
 
 
 def to_torch_dtype(name):
@@ -86,7 +94,9 @@ def as_tensor(x):
 
 class Layer:
     def __init__(self, dtype=None, name=None, device=None):
-        self.name = name or type(self).__name__.lower()
+        # default name: the snake-cased class name (keras/src/utils/naming.py; the reference
+        # also appends a per-process counter to later instances)
+        self.name = name or _snake_case(type(self).__name__)
         self._dtype_policy = dtype_policies.get(dtype)
         self.device = torch.device(device) if device is not None else default_device()
         self.built = False
@@ -149,6 +159,43 @@ class Layer:
         if t.dtype.is_floating_point and t.dtype != cd:
             return t.to(cd)
         return t
+
+    # ---- config ---------------------------------------------------------------
+    @classmethod
+    def from_config(cls, config):
+        """Layer from `get_config()` output (keras/src/layers/layer.py `from_config`; the
+        quantization config travels as {"class_name", "config"})."""
+        from keras_amd import quantization_config as qc
+
+        config = dict(config)
+        config.pop("trainable", None)
+        spec = config.pop("quantization_config", None)
+        if isinstance(config.get("dtype"), dict):  # a serialized policy object
+            config["dtype"] = dtype_policies.get(config["dtype"]["config"].get("name")
+                                                 or config["dtype"]["config"])
+        if spec is not None:
+            classes = {c.__name__: c for c in (qc.Int8QuantizationConfig, qc.Int4QuantizationConfig)}
+            if spec["class_name"] not in classes:
+                raise ValueError(f"Unknown quantization config class: {spec['class_name']}")
+            config["quantization_config"] = classes[spec["class_name"]].from_config(spec["config"])
+        return cls(**config)
+
+    # ---- stores ---------------------------------------------------------------
+    def save_own_variables(self, store):
+        """Every variable under "0", "1", ... in creation order
+        (keras/src/layers/layer.py:1478-1489); quantized layers override the order."""
+        for i, v in enumerate(self._variables):
+            store[str(i)] = v.value
+
+    def load_own_variables(self, store):
+        if len(store.keys()) != len(self._variables):
+            raise ValueError(
+                f"Layer '{self.name}' expected {len(self._variables)} variables, but received "
+                f"{len(store.keys())} variables during loading. "
+                f"Expected: {[v.name for v in self._variables]}"
+            )
+        for i, v in enumerate(self._variables):
+            v.assign(store[str(i)])
 
     # ---- call ---------------------------------------------------------------
     def __call__(self, inputs, training=None):

@@ -146,7 +146,46 @@ class Model(Layer):
 
     @property
     def layers(self):
-        return self._flatten_layers()
+        """The layers held directly by this model, containers flattened, sublayers of layers
+        not descended into (keras/src/models/model.py:174-176:
+        `_flatten_layers(include_self=False, recursive=False)`)."""
+        out, seen = [], {id(self)}
+
+        def visit(value):
+            if isinstance(value, Layer):
+                if id(value) not in seen:
+                    seen.add(id(value))
+                    out.append(value)
+            elif isinstance(value, (list, tuple)):
+                for v in value:
+                    visit(v)
+            elif isinstance(value, dict):
+                for v in value.values():
+                    visit(v)
+
+        for key, value in vars(self).items():
+            if not key.startswith("__"):
+                visit(value)
+        return out
+
+    # ---- saving (keras/src/models/model.py:save / save_weights / load_weights) ----------
+    def save(self, filepath, overwrite=True):
+        from keras_amd import saving
+
+        saving.save_model(self, filepath, overwrite=overwrite)
+
+    def save_weights(self, filepath, overwrite=True):
+        from keras_amd import saving
+
+        saving.save_weights(self, filepath, overwrite=overwrite)
+
+    def load_weights(self, filepath):
+        from keras_amd import saving
+
+        saving.load_weights(self, filepath)
+
+    def get_config(self):
+        return {"name": self.name, "dtype": self.dtype_policy.name}
 
     def quantize(self, mode=None, config=None, filters=None, verbose=False, **kwargs):
         type_check = kwargs.pop("type_check", True)
