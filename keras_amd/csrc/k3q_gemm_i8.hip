@@ -22,6 +22,7 @@
 #include "k3q_common.h"
 #include "k3q_gemm_bf16.h"
 #include "k3q_gemm_i8_skinny.h"
+#include "k3q_gemv_w8.h"
 
 namespace k3q {
 namespace {
@@ -967,6 +968,10 @@ extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_la
     if (!x || !b || !y) return K3Q_ERR_NULL;
     hipStream_t s = (hipStream_t)stream;
     const bool bf16 = x_dtype == K3Q_BF16;
+    // decode sizes on a K-contiguous kernel: streamed in place, nothing widened
+    if (b_layout == 1 && gemv_w8_nk_supported(M, N, K, x_dtype, x, b, y) &&
+        (!b_scale || aligned_to(b_scale, 4)) && (!bias || aligned_to(bias, 4)))
+        return gemv_w8_nk_run(x, x_dtype, b, M, N, K, b_scale, bias, y, s);
     const bool fast = bf16 && workspace && workspace_bytes >= N * K * 2 && aligned_to(workspace, 16) &&
                       aligned_to(b, 16) && (!b_scale || aligned_to(b_scale, 2)) &&
                       gemm_bf16_nk_supported(M, N, K, x, workspace, y) && (K % 16) == 0;

@@ -214,7 +214,10 @@ def test_unsupported_paths_raise(dev):
 # ---- non-default configs: weight-only int8, activation-quantized int4 --------------------
 @pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16", "bfloat16"])
 @pytest.mark.parametrize("M,K,N", [(16, 4096, 4096), (5, 128, 48), (300, 256, 512), (2, 100, 30),
-                                   (700, 1024, 2048)])
+                                   (700, 1024, 2048),
+                                   # decode sizes: the streaming kernel (1..8 rows, K % 16 == 0)
+                                   (1, 4096, 4096), (3, 8192, 1000), (4, 4096, 14336), (8, 1024, 7),
+                                   (7, 16, 33), (1, 16384, 64), (9, 4096, 512)])
 def test_dense_int8_weight_only(dev, policy, M, K, N):
     layer = build_dense(dev, K, N, policy, seed=5)
     kernel_f = layer._kernel.value.cpu()
