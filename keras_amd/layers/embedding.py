@@ -529,28 +529,41 @@ class ReversibleEmbedding(Embedding):
                 if in_scale is not None:
                     logits = torch.divide(logits, in_scale)
         else:
+            # the variable is read without autocast (float32 under a mixed policy): torch then
+            # promotes the whole de-scale / de-quantisation to that dtype
             scale = as_tensor(self.reverse_embeddings_scale)
-            if in_scale is not None:
-                raise NotImplementedError(
-                    "The untied int4 reverse projection with an activation quantizer is not on "
-                    "the fused path yet."
-                )
-            if scale.dtype != cd:
-                raise NotImplementedError(
-                    "The untied int4 reverse projection needs its scales in the compute dtype "
-                    f"(got {scale.dtype} scales under {cd} compute)."
-                )
-            relaid = self._cached(
-                "relaid", self.reverse_embeddings,
-                lambda t: quantizers.pack_int4(
-                    quantizers.unpack_int4(t, self.output_dim, axis=0), axis=-1)[0])
-            zero = None
-            if grouped:
-                zero = self._cached("zero_i8", self.reverse_embeddings_zero,
-                                    lambda t: t.to(torch.int8).contiguous())
-            logits = kops.int4_matmul(
-                x2, relaid, scale, self.input_dim, kernel_zero=zero,
-                block_size=block_size if grouped else None)
+            out_dtype = _promote(cd, scale.dtype)
+            if in_scale is not None and not grouped:
+                # int8 rows x int4 kernel: exact int32 accumulation, one de-scale
+                table8 = self._cached(
+                    "reverse_unpacked_nk", self.reverse_embeddings,
+                    lambda t: quantizers.unpack_int4(t, self.output_dim, axis=0).t().contiguous())
+                logits = kops.int8_matmul_nk(
+                    x2, table8, a_scale=in_scale.to(out_dtype), kernel_scale=scale,
+                    out_dtype=out_dtype, exact_epilogue=True,
+                    round_acc_bf16=(cd == torch.bfloat16 and out_dtype == torch.float32))
+            else:
+                relaid = self._cached(
+                    "relaid", self.reverse_embeddings,
+                    lambda t: quantizers.pack_int4(
+                        quantizers.unpack_int4(t, self.output_dim, axis=0), axis=-1)[0])
+                if grouped:
+                    # x . ((w - zero) * scale) in the promoted dtype (the quantised rows are
+                    # small integers: their cast is exact), then the input scale
+                    zero = self._cached("zero_i8", self.reverse_embeddings_zero,
+                                        lambda t: t.to(torch.int8).contiguous())
+                    logits = kops.int4_matmul(x2.to(out_dtype), relaid, scale, self.input_dim,
+                                              kernel_zero=zero, block_size=block_size)
+                    if in_scale is not None:
+                        logits = torch.divide(logits, in_scale)
+                elif out_dtype == cd:
+                    logits = kops.int4_matmul(x2, relaid, scale, self.input_dim)
+                else:
+                    # T(x . w) in the compute dtype, divided by the float32 scale afterwards
+                    ones = self._cached("ones_cd", self.reverse_embeddings_scale,
+                                        lambda t: torch.ones_like(t, dtype=cd))
+                    logits = kops.int4_matmul(x2, relaid, ones, self.input_dim)
+                    logits = torch.divide(logits.to(out_dtype), scale)
         return self._soft_cap(logits.reshape(*lead, self.input_dim))
 
     # ---- quantize -----------------------------------------------------------------------

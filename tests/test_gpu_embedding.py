@@ -298,7 +298,7 @@ def test_reversible_embedding_int4_tied(dev, policy, block_size):
     assert layer(ids).shape == (3, D)
 
 
-@pytest.mark.parametrize("policy", ["float32", "bfloat16"])
+@pytest.mark.parametrize("policy", ["float32", "bfloat16", "mixed_bfloat16"])
 @pytest.mark.parametrize("block_size", [128, 32, None])
 @pytest.mark.parametrize("M,V,D", [(4, 512, 256), (40, 1000, 384)])
 def test_reversible_embedding_int4_untied(dev, policy, block_size, M, V, D):
@@ -357,6 +357,40 @@ def test_reversible_embedding_int4_policy_built_quantizes_inputs(dev, policy, bl
         g_idx=store["3"].cpu() if grouped else None, block_size=block, compute_dtype=cd,
         quantize_inputs=True)
     assert y.dtype == want.dtype
+    if grouped:
+        assert max_rel_err(y, want) <= RTOL[cd]
+    else:
+        assert torch.equal(bits(y.cpu()), bits(want))  # integer accumulation, exact epilogue
+
+
+@pytest.mark.parametrize("policy,block", [("int4/128_from_float32", 128), ("int4/-1_from_float32", None),
+                                          ("int4/-1_from_bfloat16", None), ("int4/-1_from_mixed_bfloat16", None),
+                                          ("int4/128_from_bfloat16", 128), ("int4/32_from_mixed_bfloat16", 32)])
+def test_reversible_embedding_int4_untied_policy_built_quantizes_inputs(dev, policy, block):
+    # untied weights and the default activation quantizer of a policy-built layer: int8 rows
+    # against `reverse_embeddings`; float32 scales under bfloat16 compute promote the de-scale
+    V, D, M = 520, 256, 6
+    src = build_embedding(ReversibleEmbedding, dev, V, D, policy.split("_from_")[1], seed=27,
+                          tie_weights=False)
+    src.quantize("int4", config=Int4QuantizationConfig(block_size=block))
+    store = {}
+    src.save_own_variables(store)
+    layer = ReversibleEmbedding(V, D, tie_weights=False, dtype=policy, device=dev)
+    layer.build()
+    layer.load_own_variables(store)
+    assert layer.inputs_quantizer is not None
+    cd = TORCH[layer.compute_dtype]
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(28))
+    y = layer(x, reverse=True)
+    grouped = block is not None
+    names = [n for n, _ in layer._spec_entries()]
+    get = lambda n: store[str(names.index(n))].cpu()  # noqa: E731
+    want = ref.reversible_embedding_int4_reverse(
+        x.to(cd), get("reverse_embeddings"), get("reverse_embeddings_scale"), D,
+        embeddings_zero=get("reverse_embeddings_zero") if grouped else None,
+        g_idx=get("g_idx") if grouped else None, block_size=block, compute_dtype=cd,
+        tie_weights=False, quantize_inputs=True)
+    assert y.dtype == want.dtype and tuple(y.shape) == (M, V)
     if grouped:
         assert max_rel_err(y, want) <= RTOL[cd]
     else:
