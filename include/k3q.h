@@ -135,10 +135,12 @@ int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64
  * x: [M, K] float32 or bfloat16; b as in k3q_gemm_i8 ([K,N] with b_layout 0, the
  * prepacked [N,K] with b_layout 1); b_scale, bias, y of x_dtype.  Decode sizes (M <= 8,
  * b_layout 1, K % 16 == 0, 16-byte aligned x and b) stream the kernel in place, once per
- * four rows of x, with fp32 accumulation (K = N = 8192, M = 1: 13 us).  Otherwise bfloat16 x
- * with K % 64 == 0, N % 4 == 0 and `workspace` (k3q_gemm_w8_workspace_bytes, 16-byte
- * aligned) widens the kernel to bfloat16 in scratch (exact) and runs the MFMA tile
- * kernel; everything else runs a plain kernel with fp32 accumulation.
+ * four rows of x, with fp32 accumulation (K = N = 8192, M = 1: 13 us).  Otherwise, with
+ * K % 64 == 0, N % 4 == 0 and `workspace` (k3q_gemm_w8_workspace_bytes, 16-byte aligned),
+ * the kernel is widened to bfloat16 in scratch (exact) and the MFMA tile kernel runs on it;
+ * float32 x goes there as its high and low bfloat16 parts ([xh | xl] against [w | w], float32
+ * accumulation and epilogue, x to 2^-17 relative).  Everything else runs a plain kernel
+ * with fp32 accumulation.
  * Replaces matmul (float x int8: both cast to the float type,
  * keras/src/backend/torch/numpy.py:139-157), cast, divide, add of Dense._int8_call
  * without inputs_quantizer (keras/src/layers/core/dense.py:961-983).

@@ -22,4 +22,9 @@ int gemm_bf16_nk_run(const void* a, const void* bt, int64_t M, int64_t N, int64_
                      const void* b_scale, const void* bias, void* y, bool out_f32, void* workspace,
                      int64_t workspace_bytes, hipStream_t s);
 
+// out[M, parts * K] (bfloat16) = [xh | xl (| xh)] of float32 x[M, K]: xh = the top 16 bits of
+// a value, xl = the rounded remainder; K % 4 == 0 (k3q_gemv_w4.hip)
+void split_f32_rows_launch(const float* x, uint16_t* out, int64_t M, int64_t K, int parts,
+                           hipStream_t s);
+
 }  // namespace k3q

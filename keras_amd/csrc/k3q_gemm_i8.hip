@@ -602,28 +602,38 @@ __global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ i
 }
 
 // ---- weight-only int8: the int8 kernel widened to bfloat16 [N, K] in scratch (exact) ----
-// [N, K] int8 -> [N, K] bfloat16, 16 values per thread
+// [N, K] int8 -> bfloat16 rows of `out_stride` values, 16 values per thread; with `twice` the
+// K values of a row are written at +0 and at +K (the [w | w] rows of the float32 route)
 __global__ __launch_bounds__(256) void widen_i8_to_bf16(const int8_t* __restrict__ in,
-                                                        uint16_t* __restrict__ out, int64_t count16) {
+                                                        uint16_t* __restrict__ out, int64_t count16,
+                                                        int64_t K, int64_t out_stride, bool twice) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= count16) return;
     const v4u v = *(const v4u*)(in + i * 16);
     v4u o[2];
 #pragma unroll
     for (int e = 0; e < 16; e += 2) {
-        const u32 lo = f32_to_bf16_bits((float)(int)(int8_t)(v[e >> 2] >> (8 * (e & 3))));
-        const u32 hi = f32_to_bf16_bits((float)(int)(int8_t)(v[(e + 1) >> 2] >> (8 * ((e + 1) & 3))));
-        o[e >> 3][(e & 7) >> 1] = lo | (hi << 16);
+        const float lo = (float)(int)(int8_t)(v[e >> 2] >> (8 * (e & 3)));
+        const float hi = (float)(int)(int8_t)(v[(e + 1) >> 2] >> (8 * ((e + 1) & 3)));
+        o[e >> 3][(e & 7) >> 1] = pack_bf16x2(lo, hi);
     }
-    v4u* dst = (v4u*)(out + i * 16);
+    const int64_t n = (i * 16) / K, k = i * 16 - n * K;  // K % 16 == 0: a piece stays in its row
+    v4u* dst = (v4u*)(out + n * out_stride + k);
     dst[0] = o[0];
     dst[1] = o[1];
+    if (twice) {
+        dst = (v4u*)(out + n * out_stride + K + k);
+        dst[0] = o[0];
+        dst[1] = o[1];
+    }
 }
 
-// [K, N] int8 -> [N, K] bfloat16 through a padded LDS tile
+// [K, N] int8 -> [N, K] bfloat16 (rows of `out_stride` values, optionally twice) through a
+// padded LDS tile
 __global__ __launch_bounds__(256) void transpose_widen_i8_to_bf16(const int8_t* __restrict__ in,
                                                                   uint16_t* __restrict__ out,
-                                                                  int64_t K, int64_t N) {
+                                                                  int64_t K, int64_t N,
+                                                                  int64_t out_stride, bool twice) {
     __shared__ int8_t tile[64][64 + 4];
     const int64_t k0 = (int64_t)blockIdx.y * 64;
     const int64_t n0 = (int64_t)blockIdx.x * 64;
@@ -636,8 +646,11 @@ __global__ __launch_bounds__(256) void transpose_widen_i8_to_bf16(const int8_t* 
     __syncthreads();
     for (int e = threadIdx.x; e < 64 * 64; e += 256) {
         const int r = e / 64, c = e % 64;  // r: n within tile, c: k within tile
-        if (n0 + r < N && k0 + c < K)
-            out[(n0 + r) * K + k0 + c] = (uint16_t)f32_to_bf16_bits((float)tile[c][r]);
+        if (n0 + r < N && k0 + c < K) {
+            const uint16_t h = (uint16_t)f32_to_bf16_bits((float)tile[c][r]);
+            out[(n0 + r) * out_stride + k0 + c] = h;
+            if (twice) out[(n0 + r) * out_stride + K + k0 + c] = h;
+        }
     }
 }
 
@@ -954,8 +967,9 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
 
 extern "C" int64_t k3q_gemm_w8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    // the kernel widened to bfloat16, then the partials of a K split
-    return N * K * 2 + split_workspace_bytes(M, N, 2 * K);
+    // the kernel widened to bfloat16 (twice, plus the split rows of x, for float32 inputs:
+    // sized for that), then the partials of a K split
+    return (N + M) * 2 * K * 2 + split_workspace_bytes(M, N, 4 * K);
 }
 
 extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64_t M,
@@ -972,21 +986,31 @@ extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_la
     if (b_layout == 1 && gemv_w8_nk_supported(M, N, K, x_dtype, x, b, y) &&
         (!b_scale || aligned_to(b_scale, 4)) && (!bias || aligned_to(bias, 4)))
         return gemv_w8_nk_run(x, x_dtype, b, M, N, K, b_scale, bias, y, s);
-    const bool fast = bf16 && workspace && workspace_bytes >= N * K * 2 && aligned_to(workspace, 16) &&
-                      aligned_to(b, 16) && (!b_scale || aligned_to(b_scale, 2)) &&
-                      gemm_bf16_nk_supported(M, N, K, x, workspace, y) && (K % 16) == 0;
+    // MFMA route: the kernel widened to bfloat16 in scratch (exact).  float32 x goes there as
+    // its high and low bfloat16 parts side by side, [xh | xl] against [w | w]: one bfloat16
+    // GEMM over 2K with float32 accumulation and a float32 epilogue (x to 2^-17 relative).
+    const int64_t parts = bf16 ? 1 : 2;
+    const int64_t wt_bytes = N * parts * K * 2, xs_bytes = bf16 ? 0 : M * parts * K * 2;
+    const void* a_op = bf16 ? x : (const void*)((char*)workspace + wt_bytes);
+    const bool fast = workspace && workspace_bytes >= wt_bytes + xs_bytes && aligned_to(workspace, 16) &&
+                      aligned_to(b, 16) && aligned_to(x, 16) && (K % 64) == 0 &&
+                      (!b_scale || aligned_to(b_scale, 4)) &&
+                      gemm_bf16_nk_supported(M, N, parts * K, a_op, workspace, y) &&
+                      aligned_to(y, bf16 ? 8 : 16);
     if (fast) {
         if (b_layout == 1) {
             const int64_t count16 = N * K / 16;
-            widen_i8_to_bf16<<<(unsigned)((count16 + 255) / 256), 256, 0, s>>>(b, (uint16_t*)workspace,
-                                                                              count16);
+            widen_i8_to_bf16<<<(unsigned)((count16 + 255) / 256), 256, 0, s>>>(
+                b, (uint16_t*)workspace, count16, K, parts * K, !bf16);
         } else {
             dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
-            transpose_widen_i8_to_bf16<<<grid, 256, 0, s>>>(b, (uint16_t*)workspace, K, N);
+            transpose_widen_i8_to_bf16<<<grid, 256, 0, s>>>(b, (uint16_t*)workspace, K, N, parts * K,
+                                                            !bf16);
         }
-        char* rest = (char*)workspace + N * K * 2;
-        return gemm_bf16_nk_run(x, workspace, M, N, K, b_scale, bias, y, false, rest,
-                                workspace_bytes - N * K * 2, s);
+        if (!bf16) split_f32_rows_launch((const float*)x, (uint16_t*)a_op, M, K, 2, s);
+        char* rest = (char*)workspace + wt_bytes + xs_bytes;
+        return gemm_bf16_nk_run(a_op, workspace, M, N, parts * K, b_scale, bias, y, !bf16, rest,
+                                workspace_bytes - wt_bytes - xs_bytes, s);
     }
     if (M > 65535) return K3Q_ERR_SHAPE;
     dim3 grid((unsigned)((N + 255) / 256), (unsigned)M);

@@ -821,8 +821,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         else
             dequant_w4_nk<false, true><<<grid, 256, 0, s>>>(
                 (const uint8_t*)w_packed, nullptr, nullptr, wt, K, N, 0);
-        split_f32_rows<<<(unsigned)((M * K / 4 + 255) / 256), 256, 0, s>>>((const float*)x, xs, M, K,
-                                                                          parts);
+        split_f32_rows_launch((const float*)x, xs, M, K, parts, s);
         if (!gemm_bf16_nk_supported(M, N, (int64_t)parts * K, xs, wt, y)) return K3Q_ERR_SHAPE;
         const int64_t used = gemm_route_bytes(true, grouped, M, K, N);
         return gemm_bf16_nk_run(xs, wt, M, N, (int64_t)parts * K, grouped ? nullptr : scale, bias, y,
@@ -895,6 +894,12 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
 }
 
 }  // namespace
+
+void split_f32_rows_launch(const float* x, uint16_t* out, int64_t M, int64_t K, int parts,
+                           hipStream_t s) {
+    split_f32_rows<<<(unsigned)((M * K / 4 + 255) / 256), 256, 0, s>>>(x, out, M, K, parts);
+}
+
 }  // namespace k3q
 
 using namespace k3q;
