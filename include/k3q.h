@@ -91,7 +91,8 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  * reference's op chain does; otherwise y = T(acc * (1/a_scale) * (1/b_scale) + bias)
  * with one final rounding (differs from the chain by at most the chain's own
  * intermediate roundings).
- * The MFMA kernel needs K % 128 == 0, N % 4 == 0 and 16-byte aligned operands;
+ * The MFMA kernel needs K % 128 == 0 and 16-byte aligned operands (any N; with
+ * N % 4 != 0 the rows of y are stored element by element and K is never split);
  * other shapes run a plain kernel.  With b_layout 0 the MFMA kernel also needs
  * `workspace` (k3q_gemm_i8_workspace_bytes, 16-byte aligned) to hold the [N,K]
  * copy it makes on every call; callers that reuse a kernel should prepack once.

@@ -454,6 +454,7 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         static_assert(4096 + (kThreads / 64) * 32 * kPitch <= T::kLdsBytes, "staging fits in LDS");
         char* wst = lds + 4096 + wave * (32 * kPitch);
         const bool wide = (((int64_t)p.N * kE) % 16 == 0) && (((uintptr_t)p.y) % 16 == 0);
+        const bool quads = (p.N % 4) == 0;  // every row of y (and of acc_out) is 8-byte aligned
         auto stage4 = [&](int nb, int rg, const float (&v)[4]) {
             char* d = wst + fi * kPitch + (nb * 32 + 8 * rg + 4 * fg) * kE;
             if (kBF16) {
@@ -476,13 +477,23 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                 const int64_t n = n0 + wn * kWN + chunk * (16 / kE);
                 if (m >= p.M || n >= p.N) continue;
                 char* dst = (char*)p.y + (m * p.N + n) * kE;
-                const bool full = n + 16 / kE <= p.N;  // else the first 8 bytes (N % 4 == 0)
-                if (wide && full) {
+                const int valid = (int)min((int64_t)(16 / kE), p.N - n);  // columns of this piece in y
+                if (wide && valid == 16 / kE) {
                     *(v4u*)dst = d;
-                } else {
+                } else if (quads) {  // rows of y start on 8-byte boundaries
                     v2u lo = {d[0], d[1]}, hi = {d[2], d[3]};
                     *(v2u*)dst = lo;
-                    if (full) *(v2u*)(dst + 8) = hi;
+                    if (valid > 8 / kE) *(v2u*)(dst + 8) = hi;
+                } else {  // N % 4 != 0: rows of y start anywhere, element by element
+#pragma unroll
+                    for (int e = 0; e < 16 / kE; ++e) {
+                        if (e >= valid) break;
+                        const u32 word = d[e * kE / 4];
+                        if (kE == 2)
+                            ((uint16_t*)dst)[e] = (uint16_t)(word >> (16 * (e & 1)));
+                        else
+                            ((u32*)dst)[e] = word;
+                    }
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next block's writes
@@ -526,10 +537,16 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                     for (int rg = 0; rg < 4; ++rg) {
                         const int nl = wn * kWN + nb * 32 + 8 * rg + 4 * fg;
                         const int64_t n = n0 + nl;
-                        if (p.acc_out && m < p.M && n < p.N) {  // N % 4 == 0 on this path
-                            v4i o = {(int)acc[nb][mb][4 * rg], (int)acc[nb][mb][4 * rg + 1],
-                                     (int)acc[nb][mb][4 * rg + 2], (int)acc[nb][mb][4 * rg + 3]};
-                            *(v4i*)(p.acc_out + m * p.N + n) = o;
+                        if (p.acc_out && m < p.M && n < p.N) {
+                            if (quads) {
+                                v4i o = {(int)acc[nb][mb][4 * rg], (int)acc[nb][mb][4 * rg + 1],
+                                         (int)acc[nb][mb][4 * rg + 2], (int)acc[nb][mb][4 * rg + 3]};
+                                *(v4i*)(p.acc_out + m * p.N + n) = o;
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    if (n + e < p.N) p.acc_out[m * p.N + n + e] = (int)acc[nb][mb][4 * rg + e];
+                            }
                         }
                         if (!p.y) continue;
                         const v4f sb = *(const v4f*)(ep + nl);
@@ -795,8 +812,8 @@ int launch_tile(GemmParams p, hipStream_t s) {
     const int resident = cu_count() * (T::kLdsBytes <= 64 * 1024 ? 2 : 1) / 8 * 8;
     const int stages = (int)(p.row_bytes / kBK);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
-    int splits = choose_splits(tiles, stages, resident, (p.flags >> kFlagSplitShift) & 31);
-    // partials need room, 16-byte rows (N % 4 == 0 holds on this path) and an output to make
+    int splits = (p.N % 4) ? 1 : choose_splits(tiles, stages, resident, (p.flags >> kFlagSplitShift) & 31);
+    // partials need room and 16-byte rows (no split for N % 4 != 0, above)
     if (splits > 1 && (!p.part || p.part_bytes < (int64_t)splits * p.M * p.N * 4)) {
         const int64_t fit = p.part ? p.part_bytes / (p.M * p.N * 4) : 0;
         splits = fit >= 2 ? (int)fit : 1;
@@ -831,7 +848,7 @@ int launch_mfma(const GemmParams& p, hipStream_t s) {
 
 bool gemm_bf16_nk_supported(int64_t M, int64_t N, int64_t K, const void* a, const void* bt,
                             const void* y) {
-    return M > 0 && (2 * K) % kBK == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(bt, 16) &&
+    return M > 0 && (2 * K) % kBK == 0 && aligned_to(a, 16) && aligned_to(bt, 16) &&
            aligned_to(y, 8) && ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);
 }
 
@@ -918,7 +935,7 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
         return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
                                   workspace, workspace_bytes, s);
     const bool forced_tile = (flags & (kFlagForceSmallTile | kFlagForceLargeTile)) != 0;
-    bool fast = (K % kBK) == 0 && (N % 4) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
+    bool fast = (K % kBK) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
                 (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
                 (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&
                 ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);

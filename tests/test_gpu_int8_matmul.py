@@ -50,7 +50,9 @@ def run_dense_int8(dev, M, K, N, dtype, prepack, exact, seed=0, with_bias=True, 
 SHAPES = [
     (1, 128, 4), (3, 128, 12), (16, 4096, 4096), (17, 256, 260), (64, 512, 1000),
     (255, 384, 256), (256, 1024, 512), (300, 640, 772), (513, 256, 1028),
-    # shapes off the MFMA path (K % 128 != 0 or N % 4 != 0): plain kernel
+    # N % 4 != 0 (a vocabulary of 50257 or 30522): the tiles store those rows element-wise
+    (300, 256, 1001), (129, 384, 50257), (64, 128, 30522), (200, 512, 3), (1000, 128, 130),
+    # K % 128 != 0: plain kernel
     (5, 100, 30), (8, 8, 16), (33, 64, 7), (2, 200, 64),
 ]
 

@@ -217,7 +217,8 @@ def test_unsupported_paths_raise(dev):
                                    (700, 1024, 2048),
                                    # decode sizes: the streaming kernel (1..8 rows, K % 16 == 0)
                                    (1, 4096, 4096), (3, 8192, 1000), (4, 4096, 14336), (8, 1024, 7),
-                                   (7, 16, 33), (1, 16384, 64), (9, 4096, 512)])
+                                   (7, 16, 33), (1, 16384, 64), (9, 4096, 512),
+                                   (300, 256, 1001), (40, 512, 30522)])
 def test_dense_int8_weight_only(dev, policy, M, K, N):
     layer = build_dense(dev, K, N, policy, seed=5)
     kernel_f = layer._kernel.value.cpu()
