@@ -258,30 +258,25 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         // 32-byte K step, i.e. logical chunk 2*ks + g of the row.
         const int fi = lane & 31;
         const int fg = lane >> 5;
-        int a_row[kMBlk], a_swz[kMBlk], b_row[kNBlk], b_swz[kNBlk];
-#pragma unroll
-        for (int mb = 0; mb < kMBlk; ++mb) {
-            const int row = wm * kWM + mb * 32 + fi;
-            a_row[mb] = row * kBK;
-            a_swz[mb] = swz(row);
-        }
-#pragma unroll
-        for (int nb = 0; nb < kNBlk; ++nb) {
-            const int row = wn * kWN + nb * 32 + fi;
-            b_row[nb] = kATileBytes + row * kBK;
-            b_swz[nb] = swz(row);
-        }
+        // Every 32-row block starts at a multiple of 32 rows, so swz(row) = swz(i) for all of
+        // them, and 2*ks + g = (2*ks) ^ g.  The byte address of a fragment is therefore
+        // (row base | ((g ^ swz(i)) << 4)) ^ (32 * ks) + block * 32 rows: one register per
+        // operand, one XOR per K step, the blocks as immediate offsets.  The stage is a bit of
+        // that register, flipped at the hand-over.
+        static_assert((kStageBytes & (kStageBytes - 1)) == 0 && kWM % 32 == 0 && kWN % 32 == 0, "addressing");
+        const int lane_chunk = (fg ^ swz(fi)) << 4;
+        int ra = (wm * kWM + fi) * kBK + lane_chunk;
+        int rb = kATileBytes + (wn * kWN + fi) * kBK + lane_chunk;
         v4i af[2][kMBlk], bf[2][kNBlk];
-        auto read_frags = [&](int fb, int stage, int ks) {
-            const char* st = lds + stage * kStageBytes;
+        auto read_frags = [&](int fb, int ks) {
 #ifndef K3Q_GEMM_PROBE_NO_BREAD
+            const char* pb = lds + (rb ^ (32 * ks));
 #pragma unroll
-            for (int nb = 0; nb < kNBlk; ++nb)
-                bf[fb][nb] = *(const v4i*)(st + b_row[nb] + (((2 * ks + fg) ^ b_swz[nb]) << 4));
+            for (int nb = 0; nb < kNBlk; ++nb) bf[fb][nb] = *(const v4i*)(pb + nb * 32 * kBK);
 #endif
+            const char* pa = lds + (ra ^ (32 * ks));
 #pragma unroll
-            for (int mb = 0; mb < kMBlk; ++mb)
-                af[fb][mb] = *(const v4i*)(st + a_row[mb] + (((2 * ks + fg) ^ a_swz[mb]) << 4));
+            for (int mb = 0; mb < kMBlk; ++mb) af[fb][mb] = *(const v4i*)(pa + mb * 32 * kBK);
         };
 
         typename Mma<kKind>::Acc acc[kNBlk][kMBlk];
@@ -308,7 +303,7 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
             wait_vmcnt0();
         }
         bare_barrier();
-        read_frags(0, 0, 0);
+        read_frags(0, 0);
         // The DMA of a stage is not issued as one burst: the texture unit takes an instruction
         // per ~16 clocks and the workgroup's 64 would hold every wave (an in-order issuer) away
         // from its MFMAs for up to a thousand clocks.  Instead one DMA instruction follows every
@@ -351,7 +346,6 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
             }
         };
         for (int kt = 0; kt < KT; ++kt) {
-            const int cur = kt & 1;
 #pragma unroll
             for (int ks = 0; ks < kKSteps; ++ks) {
                 // first half of this step's MFMAs, then the reads for the next step, then the
@@ -360,11 +354,13 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                 mma_half(ks, 0, kt);
                 __builtin_amdgcn_sched_barrier(0);
                 if (ks + 1 < kKSteps) {
-                    read_frags((ks + 1) & 1, cur, ks + 1);
+                    read_frags((ks + 1) & 1, ks + 1);
                 } else if (kt + 1 < KT) {
                     wait_vmcnt0();  // own DMA of stage kt+1 has landed (own reads of stage kt are done)
                     bare_barrier();
-                    read_frags(0, cur ^ 1, 0);
+                    ra ^= kStageBytes;
+                    rb ^= kStageBytes;
+                    read_frags(0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 mma_half(ks, 1, kt);
