@@ -183,7 +183,24 @@ int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
                 int64_t workspace_bytes, void* stream);
 
 /*
- * Same as k3q_gemv_w4 with the launch plan overridden, for tuning sweeps:
+ * k3q_gemv_w4 with the K split of decode sizes finished in the same launch instead of by a
+ * second kernel (K = N = 8192, one row: one launch less per call).  The workgroups of a column
+ * block count their arrivals in `counters` and the one that comes last sums the partials, in
+ * the order of the split, so results do not depend on which one that is.
+ * counters: k3q_gemv_w4_counters_bytes(N) bytes of device memory, 4-byte aligned, ZERO before
+ * the first call; every call leaves them zero again.  Calls ordered on one stream may share
+ * them; two calls that overlap in time must not.  Null or too small: as k3q_gemv_w4.
+ * No counterpart in the reference (torch's matmul owns its own scratch there).
+ */
+int64_t k3q_gemv_w4_counters_bytes(int64_t N);
+int k3q_gemv_w4_fused(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                      const void* w_packed, const void* scale, const void* zero,
+                      int64_t block_size, const void* bias, void* y, void* workspace,
+                      int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                      void* stream);
+
+/*
+ * Same as k3q_gemv_w4_fused with the launch plan overridden, for tuning sweeps:
  * plan = {dwords per lane per k row (1|2), 16-row steps per chunk (1|2),
  * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null
  * `plan` keep the built-in choice.  The workspace must then hold
@@ -192,7 +209,8 @@ int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
 int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
                      const void* w_packed, const void* scale, const void* zero,
                      int64_t block_size, const void* bias, void* y, void* workspace,
-                     int64_t workspace_bytes, const int* plan, void* stream);
+                     int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                     const int* plan, void* stream);
 
 /*
  * Weight-only int4 matmul for decode-sized M with the kernel stored K-contiguous:

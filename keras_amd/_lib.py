@@ -67,10 +67,16 @@ SIGNATURES = {
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr],
     ),
+    "k3q_gemv_w4_counters_bytes": (_i64, [_i64]),
+    "k3q_gemv_w4_fused": (
+        _int,
+        [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
+         _ptr],
+    ),
     "k3q_gemv_w4_plan": (
         _int,
-        [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr,
-         _ptr],
+        [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
+         _ptr, _ptr],
     ),
 }
 

@@ -57,6 +57,7 @@ struct GemvParams {
     const void* bias;      // T [N] or null
     void* y;               // T [M, N]
     float* part;           // [KS, M, N] fp32 partials (KS > 1)
+    unsigned* sync;        // arrival counters, one per column block, zero between calls (or null)
     int64_t K, N, row_bytes;
     int M;                 // rows of x in this launch
     int m0;                // first row of x handled by this launch
@@ -91,6 +92,76 @@ __device__ __forceinline__ void finish(const GemvParams& p, int m, int64_t n, fl
     }
 }
 
+// Partial sums that another workgroup of the same launch reads go around the caches that are
+// not coherent across the device (agent-scope accesses), as two 8-byte halves.
+__device__ __forceinline__ void store_v4f_device(float* dst, const v4f& v) {
+    const v4u b = __builtin_bit_cast(v4u, v);
+    __hip_atomic_store((uint64_t*)dst, (uint64_t)b[0] | ((uint64_t)b[1] << 32), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store((uint64_t*)dst + 1, (uint64_t)b[2] | ((uint64_t)b[3] << 32), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool kDevice>
+__device__ __forceinline__ v4f load_v4f(const float* src) {
+    if (!kDevice) return *(const v4f*)src;
+    const uint64_t lo = __hip_atomic_load((const uint64_t*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t hi = __hip_atomic_load((const uint64_t*)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const v4u b = {(u32)lo, (u32)(lo >> 32), (u32)hi, (u32)(hi >> 32)};
+    return __builtin_bit_cast(v4f, b);
+}
+
+// Sum of the KS partials of four adjacent outputs, in one fixed order wherever it is
+// computed: four interleaved chains (partial ks goes to chain ks % 4), joined pairwise.
+// Eight loads are in flight before the first add (left alone, the scheduler pairs every load
+// with its add: one memory round trip per partial instead of one per eight).
+template <bool kDevice>
+__device__ __forceinline__ v4f sum_partials(const float* src, int64_t stride, int KS) {
+    v4f s4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) s4[u] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < KS; ks += 8) {
+        v4f t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            t[u] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (ks + u < KS) t[u] = load_v4f<kDevice>(src + (ks + u) * stride);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s4[u & 3] += t[u];
+    }
+    return (s4[0] + s4[1]) + (s4[2] + s4[3]);
+}
+
+// finish for four adjacent outputs with the scale and bias loads issued before `sum` is
+// needed (`sum` is passed as a callable): in the single-launch K split the loads of the
+// partials then overlap them instead of following them.
+template <bool kBF16, bool kGrouped, typename SumFn>
+__device__ __forceinline__ void finish4_prefetched(const GemvParams& p, int m, int64_t n, SumFn sum_fn) {
+    float sc[4] = {1.f, 1.f, 1.f, 1.f}, bi[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (!kGrouped) sc[e] = load_t<kBF16>(p.scale, n + e);
+        if (p.bias) bi[e] = load_t<kBF16>(p.bias, n + e);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const v4f sum = sum_fn();
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v = sum[e];
+        if (kBF16) {
+            v = round_bf16(v);
+            if (!kGrouped) v = round_bf16(v / sc[e]);
+            if (p.bias) v = round_bf16(v + bi[e]);
+            ((uint16_t*)p.y)[(int64_t)(p.m0 + m) * p.N + n + e] = (uint16_t)(__float_as_uint(v) >> 16);
+        } else {
+            if (!kGrouped) v = v / sc[e];
+            if (p.bias) v = v + bi[e];
+            ((float*)p.y)[(int64_t)(p.m0 + m) * p.N + n + e] = v;
+        }
+    }
+}
+
 template <int kVec>
 struct Packed {
     u32 d[kVec];
@@ -122,7 +193,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     // dependent ones spread over the address set-up (0.8 us before the first load otherwise);
     // launch geometry comes with the arguments, not from the dispatch packet.
     asm volatile("" ::"s"(p.x), "s"(p.w), "s"(p.scale), "s"(p.zero), "s"(p.bias), "s"(p.y),
-                 "s"(p.part), "s"(p.K), "s"(p.N), "s"(p.row_bytes), "s"(p.M), "s"(p.m0),
+                 "s"(p.part), "s"(p.sync), "s"(p.K), "s"(p.N), "s"(p.row_bytes), "s"(p.M), "s"(p.m0),
                  "s"(p.block_size), "s"(p.klen), "s"(p.nwaves), "s"(p.per_xcd), "s"(p.ks));
     constexpr bool kBF16 = !kXF32;
     constexpr int kAccSets = kXF32 ? 1 : kSets;
@@ -411,7 +482,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) finish<kBF16, kGrouped>(p, m, n + e, sum[e]);
             } else {
-                *(v4f*)(p.part + ((int64_t)blockIdx.y * M + m) * p.N + n) = sum;
+                float* dst = p.part + ((int64_t)blockIdx.y * M + m) * p.N + n;
+                if (p.sync) store_v4f_device(dst, sum);
+                else *(v4f*)dst = sum;
             }
         }
     }
@@ -422,6 +495,32 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
         d[4] = ts2b; d[5] = ts2c;
     }
 #endif
+    // ---- K split finished in this launch ----
+    // The workgroup that arrives last at its column block's counter sums the KS partials (in
+    // the order of the split, whoever comes last) and applies the epilogue; it leaves the
+    // counter at zero for the next call.
+    if (KS == 1 || p.sync == nullptr) return;
+    // The partials were stored around the non-coherent caches; once the stores are
+    // acknowledged (the wait this fence emits) they are visible device-wide.  A device-scope
+    // release here would write back the whole L2 once per wave (54 us per call instead of 12).
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();  // every thread's stores are out before the arrival is counted
+    int* flag = (int*)red;
+    if (threadIdx.x == 0) flag[0] = atomicAdd(p.sync + cb, 1u) == (unsigned)(KS - 1);
+    __syncthreads();
+    const bool last = flag[0] != 0;
+    if (!last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // no load below moves above the count
+    const int items = M * (kNB / 4);
+    for (int idx = threadIdx.x; idx < items; idx += nwaves * 64) {
+        const int m = idx / (kNB / 4);
+        const int64_t n = nb + (idx % (kNB / 4)) * 4;
+        if (n >= p.N) continue;
+        finish4_prefetched<kBF16, kGrouped>(p, m, n, [&]() {
+            return sum_partials<true>(p.part + (int64_t)m * p.N + n, (int64_t)M * p.N, KS);
+        });
+    }
+    if (threadIdx.x == 0) atomicExch(p.sync + cb, 0u);
 }
 
 // Second pass when K is split over workgroups: sum the KS partials of every output in a
@@ -432,18 +531,7 @@ __global__ __launch_bounds__(256) void gemv_w4_reduce(GemvParams p, int KS) {
     const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const int m = blockIdx.y;
     if (n >= p.N) return;
-    v4f s4[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) s4[u] = v4f{0.f, 0.f, 0.f, 0.f};
-    const float* src = p.part + (int64_t)m * p.N + n;
-    const int64_t stride = (int64_t)p.M * p.N;
-    int ks = 0;
-    for (; ks + 4 <= KS; ks += 4) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) s4[u] += *(const v4f*)(src + (ks + u) * stride);
-    }
-    for (; ks < KS; ++ks) s4[0] += *(const v4f*)(src + ks * stride);
-    const v4f sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    const v4f sum = sum_partials<false>(p.part + (int64_t)m * p.N + n, (int64_t)p.M * p.N, KS);
 #pragma unroll
     for (int e = 0; e < 4; ++e) finish<kBF16, kGrouped>(p, m, n + e, sum[e]);
 }
@@ -665,8 +753,11 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     const int rows_used = (int)(M < pl.rows ? M : pl.rows);
 
     // Measured on MI355X at K = N = 8192: 8 waves per workgroup, 8-byte loads per lane and
-    // one or two workgroups per CU beat wider loads and finer K splits.
+    // one or two workgroups per CU beat wider loads and finer K splits.  Narrow or small
+    // kernels (N <= 4096, or under 2^25 weights) do better with 4-byte loads, i.e. twice the
+    // column blocks and half the K split (Llama-7B-sized decoder step: 4.91 -> 4.76 ms).
     int vec = ((grouped && pl.sets == 2) || pl.sets == 4) ? 1 : 2;
+    if (vec == 2 && (N <= 4096 || N * K < ((int64_t)1 << 25))) vec = 1;
     if (plan_override && plan_override[0] > 0) vec = plan_override[0];
     while (vec > 1 && (N % (8 * vec)) != 0) vec >>= 1;
     if (vec != 1 && vec != 2) vec = vec > 2 ? 2 : 1;  // 16-byte loads per lane lost every sweep
@@ -711,6 +802,19 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
                 frac /= 2;
             klen = frac;
         }
+    }
+    if (target == kTargetWorkgroups) {
+        // a few workgroups more than CUs run as a second round on some CUs and hold the launch
+        // back (weights cold in HBM; K = 4096, N = 11008, groups of 128: 16.4 us, 12.1 us once
+        // the launch fits one round; K = 5120, N = 13824: 21.4 / 18.0): lengthen the slices
+        const int64_t step = grouped ? (klen >= block_size ? block_size : klen) : chunk;
+        auto workgroups = [&](int64_t kl) {
+            const int64_t slices = (K + kl - 1) / kl;
+            return nblocks * ((slices + waves - 1) / waves);
+        };
+        while (workgroups(klen) > kTargetWorkgroups && workgroups(klen) < 7 * kTargetWorkgroups / 4 &&
+               klen + step <= K)
+            klen += step;
     }
     if (plan_override && plan_override[3] > 0) klen = (plan_override[3] + chunk - 1) / chunk * chunk;
     if (klen > K) klen = (K + chunk - 1) / chunk * chunk;
@@ -769,7 +873,8 @@ void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, bool g
 
 int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* w_packed,
                 const void* scale, const void* zero, int64_t block_size, const void* bias, void* y,
-                void* workspace, int64_t workspace_bytes, const int* plan_override, hipStream_t s) {
+                void* workspace, int64_t workspace_bytes, const int* plan_override, void* counters,
+                int64_t counters_bytes, hipStream_t s) {
     if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
     if (M == 0) return K3Q_OK;
@@ -861,6 +966,13 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         if (!workspace || workspace_bytes < need) return K3Q_ERR_WORKSPACE;
         if (!aligned_to(workspace, 16)) return K3Q_ERR_ALIGN;
         p.part = (float*)workspace;
+        // with arrival counters (zero between calls) the K split is summed in the same launch,
+        // while the last workgroup of a column block has one output quad per thread at most
+        // (K = N = 8192, 16 rows, per-channel: 19.0 us with two quads per thread, 17.3 us with the
+        // second kernel; Llama-7B-sized decoder step: 4.67 ms against 4.92 ms)
+        if (counters && counters_bytes >= nblocks * 4 && aligned_to(counters, 4) &&
+            ((pl.sets < 4 && rows_max * (nb_cols / 4) <= pl.waves * 64) || plan_override))
+            p.sync = (unsigned*)counters;
     }
     p.klen = pl.klen;
     for (int64_t m0 = 0; m0 < M; m0 += pl.rows) {
@@ -875,7 +987,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         const size_t lds = (size_t)pl.waves * rows * (nb_cols + kRedPad) * sizeof(float);
         const int sets = f32 ? 2 : (rows > 16 ? 4 : rows > 8 ? 2 : 1);
         launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
-        if (pl.ks > 1) {
+        if (pl.ks > 1 && !p.sync) {
             dim3 rgrid((unsigned)((N / 4 + 255) / 256), rows);
             if (f32) {
                 if (grouped)
@@ -933,13 +1045,27 @@ extern "C" int k3q_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int
                            int64_t block_size, const void* bias, void* y, void* workspace,
                            int64_t workspace_bytes, void* stream) {
     return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
-                       workspace_bytes, nullptr, (hipStream_t)stream);
+                       workspace_bytes, nullptr, nullptr, 0, (hipStream_t)stream);
+}
+
+extern "C" int64_t k3q_gemv_w4_counters_bytes(int64_t N) {
+    return N <= 0 ? 0 : (N + 127) / 128 * 4;
+}
+
+extern "C" int k3q_gemv_w4_fused(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                 const void* w_packed, const void* scale, const void* zero,
+                                 int64_t block_size, const void* bias, void* y, void* workspace,
+                                 int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                                 void* stream) {
+    return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
+                       workspace_bytes, nullptr, counters, counters_bytes, (hipStream_t)stream);
 }
 
 extern "C" int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
                                 const void* w_packed, const void* scale, const void* zero,
                                 int64_t block_size, const void* bias, void* y, void* workspace,
-                                int64_t workspace_bytes, const int* plan, void* stream) {
+                                int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                                const int* plan, void* stream) {
     return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
-                       workspace_bytes, plan, (hipStream_t)stream);
+                       workspace_bytes, plan, counters, counters_bytes, (hipStream_t)stream);
 }

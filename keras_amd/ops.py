@@ -31,8 +31,22 @@ def _workspace(device, nbytes):
     return ws
 
 
+_counters = {}
+
+
+def _arrival_counters(device, nbytes):
+    """Arrival counters of the single-launch K split: zero between calls, one per (device, stream)."""
+    stream = torch.cuda.current_stream(device)
+    key = (device.index, stream.cuda_stream)
+    c = _counters.get(key)
+    if c is None or c.numel() < nbytes:
+        c = torch.zeros(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
+        _counters[key] = c
+    return c
+
+
 def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=None,
-                block_size=None, bias=None, plan=None):
+                block_size=None, bias=None, plan=None, single_launch=True):
     """`x[..., K] . W4[K, N]` for a Dense int4 kernel as the layer stores it.
 
     kernel_packed: int8 [K, ceil(N/2)] (two nibbles per byte along N).
@@ -79,8 +93,10 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
         int(block_size) if grouped else -1, _lib.ptr(bias), _lib.ptr(y),
         _lib.ptr(ws), ws.numel(),
     ]
+    cnt = _arrival_counters(x.device, lib.k3q_gemv_w4_counters_bytes(N)) if single_launch else None
+    args += [_lib.ptr(cnt), cnt.numel() if single_launch else 0]
     if plan is None:
-        rc = lib.k3q_gemv_w4(*args, _lib.stream_ptr(x.device))
+        rc = lib.k3q_gemv_w4_fused(*args, _lib.stream_ptr(x.device))
     else:
         arr = (ctypes.c_int * 4)(*[int(v) for v in plan[:4]])
         rc = lib.k3q_gemv_w4_plan(*args, arr, _lib.stream_ptr(x.device))

@@ -143,3 +143,40 @@ def test_int4_large_m_off_route(dev, M, K, N, block_size, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_int4_mid_rows(dev, M, K, N, block_size, dtype):
     run_case(dev, M, K, N, block_size, dtype, with_bias=(M % 2 == 0))
+
+
+def test_int4_single_launch_split_matches_two_launches(dev):
+    # k3q_gemv_w4_fused (arrival counters, last workgroup sums) against k3q_gemv_w4 (second
+    # kernel sums): same partials, same summation order -> same bits.  One counter buffer is
+    # shared by calls of different shapes in a row and must read zero after each of them.
+    from keras_amd import _lib
+    lib = _lib.load()
+    cases = [(1, 8192, 8192, None, torch.bfloat16), (4, 4096, 14336, 128, torch.bfloat16),
+             (1, 4096, 4096, 128, torch.bfloat16), (8, 14336, 4096, None, torch.float32),
+             (3, 2048, 1024, None, torch.bfloat16), (16, 4096, 4096, 128, torch.bfloat16),
+             (40, 4096, 2048, None, torch.bfloat16), (1, 8192, 8192, None, torch.bfloat16)]
+    counters = torch.zeros(1 << 12, dtype=torch.uint8, device=dev)
+    for i, (M, K, N, bs, dtype) in enumerate(cases):
+        qk, bias = make_layer(K, N, bs, 20 + i, True)
+        grouped = bs is not None
+        x = torch.randn(M, K, generator=torch.Generator().manual_seed(i)).to(dtype).to(dev)
+        w = qk["kernel"].to(dev)
+        sc = qk["kernel_scale"].to(dtype).to(dev)
+        zp = qk["kernel_zero"].to(dev) if grouped else None
+        b = bias.to(dtype).to(dev)
+        nbytes = lib.k3q_gemv_w4_workspace_bytes(M, K, N)
+        assert lib.k3q_gemv_w4_counters_bytes(N) <= counters.numel()
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+        y2 = torch.empty((M, N), dtype=dtype, device=dev)
+        y1 = torch.empty((M, N), dtype=dtype, device=dev)
+        args = [_lib.ptr(x), _lib.dtype_code(dtype), M, K, N, _lib.ptr(w), _lib.ptr(sc), _lib.ptr(zp),
+                bs if grouped else -1, _lib.ptr(b)]
+        s = _lib.stream_ptr(dev)
+        assert lib.k3q_gemv_w4(*args, _lib.ptr(y2), _lib.ptr(ws), ws.numel(), s) == 0
+        for _ in range(2):
+            y1.zero_()
+            assert lib.k3q_gemv_w4_fused(*args, _lib.ptr(y1), _lib.ptr(ws), ws.numel(),
+                                         _lib.ptr(counters), counters.numel(), s) == 0
+            torch.cuda.synchronize()
+            assert torch.equal(y1, y2), (M, K, N, bs, dtype)
+            assert int(counters.count_nonzero()) == 0
