@@ -23,6 +23,18 @@ constexpr int kWave = 64;
 
 __device__ __forceinline__ float bf16_bits_to_f32(u32 h) { return __uint_as_float(h << 16); }
 
+// A float32 / bfloat16 element as raw bits, and back.  Loads issued as raw bits can all be
+// in flight before the first conversion waits for one of them.
+template <bool kBF16>
+__device__ __forceinline__ u32 load_raw(const void* p, int64_t i) {
+    if (kBF16) return (u32)((const uint16_t*)p)[i];
+    return ((const u32*)p)[i];
+}
+template <bool kBF16>
+__device__ __forceinline__ float raw_to_f32(u32 bits) {
+    return __uint_as_float(kBF16 ? bits << 16 : bits);
+}
+
 // float -> bfloat16 bits, round to nearest even (NaN stays NaN): one v_cvt_pk_bf16_f32.
 __device__ __forceinline__ u32 f32_to_bf16_bits(float f) {
     return (u32)__builtin_bit_cast(unsigned short, (__bf16)f);

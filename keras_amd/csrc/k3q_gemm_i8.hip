@@ -716,14 +716,35 @@ __global__ __launch_bounds__(256) void gemm_split_reduce(GemmParams p) {
     const int64_t m = i / quads, n = (i - m * quads) * 4;
     typedef typename std::conditional<kKind == kKindI8, int, float>::type Elem;
     Elem sum[4] = {0, 0, 0, 0};
-    for (int sp = 0; sp < p.splits; ++sp) {
-        const v4u v = *(const v4u*)((const u32*)p.part + ((int64_t)sp * p.M + m) * p.N + n);
+    // scales and bias as raw bits first, then eight partials, all in flight before the first
+    // use (left alone, the scheduler pairs every load with its use: one memory round trip
+    // each); the partials are summed in the order of the split
+    u32 sa_raw = 0, sb_raw[4] = {0, 0, 0, 0}, bi_raw[4] = {0, 0, 0, 0};
+    if (p.y) {
+        if (kKind == kKindI8 && p.a_scale) sa_raw = load_raw<kBF16>(p.a_scale, m);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            Elem t;
-            from_bits(v[e], t);
-            sum[e] += t;
+            if (p.b_scale) sb_raw[e] = load_raw<kBF16>(p.b_scale, n + e);
+            if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, n + e);
         }
+    }
+    for (int sp0 = 0; sp0 < p.splits; sp0 += 8) {
+        v4u v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            v[u] = v4u{0u, 0u, 0u, 0u};  // +0 of either type
+            if (sp0 + u < p.splits)
+                v[u] = *(const v4u*)((const u32*)p.part + ((int64_t)(sp0 + u) * p.M + m) * p.N + n);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Elem t;
+                from_bits(v[u][e], t);
+                sum[e] += t;
+            }
     }
     if constexpr (kKind == kKindI8) {
         if (p.acc_out) {
@@ -736,14 +757,14 @@ __global__ __launch_bounds__(256) void gemm_split_reduce(GemmParams p) {
     const bool has_bias = p.bias != nullptr;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const float bv = has_bias ? load_t<kBF16>(p.bias, n + e) : 0.0f;
+        const float bv = has_bias ? raw_to_f32<kBF16>(bi_raw[e]) : 0.0f;
         if constexpr (kKind == kKindBF16) {
             const bool has_s = p.b_scale != nullptr;
-            r[e] = descale_f<kBF16>((float)sum[e], has_s ? load_t<kBF16>(p.b_scale, n + e) : 1.0f, bv,
+            r[e] = descale_f<kBF16>((float)sum[e], has_s ? raw_to_f32<kBF16>(sb_raw[e]) : 1.0f, bv,
                                     has_s, has_bias);
         } else {
-            float sa = p.a_scale ? load_t<kBF16>(p.a_scale, m) : 1.0f;
-            float sb = p.b_scale ? load_t<kBF16>(p.b_scale, n + e) : 1.0f;
+            float sa = p.a_scale ? raw_to_f32<kBF16>(sa_raw) : 1.0f;
+            float sb = p.b_scale ? raw_to_f32<kBF16>(sb_raw[e]) : 1.0f;
             if (!kExact) {
                 sa = 1.0f / sa;
                 sb = 1.0f / sb;

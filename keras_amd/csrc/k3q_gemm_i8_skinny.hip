@@ -49,25 +49,33 @@ __device__ __forceinline__ float load_t(const void* p, int64_t i) {
     return ((const float*)p)[i];
 }
 
+// epilogue of one output with its scales and bias already in registers (bias 0 without one)
 template <bool kBF16>
-__device__ __forceinline__ void finish(const SkinnyParams& p, int m, int64_t n, int acc) {
+__device__ __forceinline__ void finish_vals(const SkinnyParams& p, int m, int64_t n, int acc, float sa,
+                                            float sb, float bias) {
     const int64_t row = p.m0 + m;
     if (p.acc_out) p.acc_out[row * p.N + n] = acc;
     if (!p.y) return;
-    const float sa = p.a_scale ? load_t<kBF16>(p.a_scale, row) : 1.0f;
-    const float sb = p.b_scale ? load_t<kBF16>(p.b_scale, n) : 1.0f;
     float r;
     if (kBF16) {
         // decode-sized outputs always take the reference's rounding chain
         r = round_bf16(round_bf16((float)acc) / round_bf16(sb * sa));
-        if (p.bias) r = round_bf16(r + load_t<true>(p.bias, n));
+        if (p.bias) r = round_bf16(r + bias);
         ((uint16_t*)p.y)[row * p.N + n] = (uint16_t)f32_to_bf16_bits(r);
     } else {
         const float accf = (p.exact & 4) ? round_bf16((float)acc) : (float)acc;
         r = accf / (sb * sa);
-        if (p.bias) r = r + load_t<false>(p.bias, n);
+        if (p.bias) r = r + bias;
         ((float*)p.y)[row * p.N + n] = r;
     }
+}
+
+template <bool kBF16>
+__device__ __forceinline__ void finish(const SkinnyParams& p, int m, int64_t n, int acc) {
+    const float sa = (p.y && p.a_scale) ? load_t<kBF16>(p.a_scale, p.m0 + m) : 1.0f;
+    const float sb = (p.y && p.b_scale) ? load_t<kBF16>(p.b_scale, n) : 1.0f;
+    const float bias = (p.y && p.bias) ? load_t<kBF16>(p.bias, n) : 0.0f;
+    finish_vals<kBF16>(p, m, n, acc, sa, sb, bias);
 }
 
 // kSteps: 8-row steps per chunk.  kSets: 8-row groups of x handled per pass (1 or 2).
@@ -214,20 +222,36 @@ __global__ __launch_bounds__(256) void gemm_i8_skinny_reduce(SkinnyParams p, int
     const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const int m = blockIdx.y;
     if (n >= p.N) return;
-    v4i s4[4];
+    // scales and bias first, then eight partials in flight before the first add (left alone,
+    // the scheduler pairs every load with its add: one memory round trip per partial)
+    const bool want_y = p.y != nullptr;
+    u32 sa_raw = 0, sb_raw[4] = {0, 0, 0, 0}, bi_raw[4] = {0, 0, 0, 0};
+    if (want_y) {
+        if (p.a_scale) sa_raw = load_raw<kBF16>(p.a_scale, p.m0 + m);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) s4[u] = v4i{0, 0, 0, 0};
+        for (int e = 0; e < 4; ++e) {
+            if (p.b_scale) sb_raw[e] = load_raw<kBF16>(p.b_scale, n + e);
+            if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, n + e);
+        }
+    }
     const int32_t* src = p.part + (int64_t)m * p.N + n;
     const int64_t stride = (int64_t)p.M * p.N;
-    int ks = 0;
-    for (; ks + 4 <= KS; ks += 4) {
+    v4i sum = {0, 0, 0, 0};
+    for (int ks = 0; ks < KS; ks += 8) {
+        v4i t[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) s4[u] += *(const v4i*)(src + (ks + u) * stride);
+        for (int u = 0; u < 8; ++u) {
+            t[u] = v4i{0, 0, 0, 0};
+            if (ks + u < KS) t[u] = *(const v4i*)(src + (ks + u) * stride);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += t[u];
     }
-    for (; ks < KS; ++ks) s4[0] += *(const v4i*)(src + ks * stride);
-    const v4i sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) finish<kBF16>(p, m, n + e, sum[e]);
+    for (int e = 0; e < 4; ++e)
+        finish_vals<kBF16>(p, m, n + e, sum[e], p.a_scale ? raw_to_f32<kBF16>(sa_raw) : 1.0f,
+                           p.b_scale ? raw_to_f32<kBF16>(sb_raw[e]) : 1.0f, raw_to_f32<kBF16>(bi_raw[e]));
 }
 
 // ---- [N, K] kernel layout (K contiguous): tied embedding tables, prepacked kernels ----

@@ -138,11 +138,11 @@ __device__ __forceinline__ v4f sum_partials(const float* src, int64_t stride, in
 // partials then overlap them instead of following them.
 template <bool kBF16, bool kGrouped, typename SumFn>
 __device__ __forceinline__ void finish4_prefetched(const GemvParams& p, int m, int64_t n, SumFn sum_fn) {
-    float sc[4] = {1.f, 1.f, 1.f, 1.f}, bi[4] = {0.f, 0.f, 0.f, 0.f};
+    u32 sc_raw[4] = {0, 0, 0, 0}, bi_raw[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        if (!kGrouped) sc[e] = load_t<kBF16>(p.scale, n + e);
-        if (p.bias) bi[e] = load_t<kBF16>(p.bias, n + e);
+        if (!kGrouped) sc_raw[e] = load_raw<kBF16>(p.scale, n + e);
+        if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, n + e);
     }
     __builtin_amdgcn_sched_barrier(0);
     const v4f sum = sum_fn();
@@ -151,12 +151,12 @@ __device__ __forceinline__ void finish4_prefetched(const GemvParams& p, int m, i
         float v = sum[e];
         if (kBF16) {
             v = round_bf16(v);
-            if (!kGrouped) v = round_bf16(v / sc[e]);
-            if (p.bias) v = round_bf16(v + bi[e]);
+            if (!kGrouped) v = round_bf16(v / raw_to_f32<true>(sc_raw[e]));
+            if (p.bias) v = round_bf16(v + raw_to_f32<true>(bi_raw[e]));
             ((uint16_t*)p.y)[(int64_t)(p.m0 + m) * p.N + n + e] = (uint16_t)(__float_as_uint(v) >> 16);
         } else {
-            if (!kGrouped) v = v / sc[e];
-            if (p.bias) v = v + bi[e];
+            if (!kGrouped) v = v / raw_to_f32<false>(sc_raw[e]);
+            if (p.bias) v = v + raw_to_f32<false>(bi_raw[e]);
             ((float*)p.y)[(int64_t)(p.m0 + m) * p.N + n + e] = v;
         }
     }
@@ -531,9 +531,9 @@ __global__ __launch_bounds__(256) void gemv_w4_reduce(GemvParams p, int KS) {
     const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const int m = blockIdx.y;
     if (n >= p.N) return;
-    const v4f sum = sum_partials<false>(p.part + (int64_t)m * p.N + n, (int64_t)p.M * p.N, KS);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) finish<kBF16, kGrouped>(p, m, n + e, sum[e]);
+    finish4_prefetched<kBF16, kGrouped>(p, m, n, [&]() {
+        return sum_partials<false>(p.part + (int64_t)m * p.N + n, (int64_t)p.M * p.N, KS);
+    });
 }
 
 // Any shape: one thread per output, fp32 FMA chain over K.  Used when N is not a
