@@ -33,14 +33,14 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
 # `--pmc WRITE_SIZE` (KiB per dispatch), each scaled by what the same counter reads for a plain
 # device copy of known size (FETCH_SIZE reads 0.50x, WRITE_SIZE 1.00x):
 # profiles/bench_dense_int8_M4096_K8192_N8192_and_int4_decode.md
-GEMM_HBM_TRAFFIC_BYTES = int((198717.9 * 2.0 + 67607.1) * 1024)
-QUANT_HBM_TRAFFIC_BYTES = int((32840.4 * 2.0 + 32832.0) * 1024)
+GEMM_HBM_TRAFFIC_BYTES = int((201555.1 * 2.0 + 70144.0) * 1024)
+QUANT_HBM_TRAFFIC_BYTES = int((32838.7 * 2.0 + 32832.0) * 1024)
 # int4 decode main kernel, keyed by (M > 8, grouped)
 GEMV_HBM_TRAFFIC_BYTES = {
-    (False, False): int((16601.6 * 2.0 + 1280.0) * 1024),
-    (False, True): int((17419.6 * 2.0 + 640.0) * 1024),
-    (True, False): int((17477.0 * 2.0 + 4096.0) * 1024),
-    (True, True): int((18469.1 * 2.0 + 2048.0) * 1024),
+    (False, False): int((17263.1 * 2.0 + 2617.0) * 1024),
+    (False, True): int((17751.6 * 2.0 + 1329.0) * 1024),
+    (True, False): int(((17474.5 + 2082.0) * 2.0 + 4096.0 + 256.0) * 1024),  # with its second kernel
+    (True, True): int((19431.4 * 2.0 + 4362.0) * 1024),
 }
 
 
