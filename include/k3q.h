@@ -152,6 +152,29 @@ int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_layout, int64
                 int64_t workspace_bytes, void* stream);
 
 /*
+ * Float matmul against a kernel that exists only de-quantised, stored as bfloat16 [N, parts * K]
+ * (K-contiguous rows):  y[m, n] = T(sum_k x[m, k] * w[n, k]) (+ bias[n]).
+ *   x bfloat16:  parts = 1, wt = w.
+ *   x float32:   parts = 3, wt = [wh | wh | wl] with w = wh + wl (the bfloat16 rounding of a
+ *                float32 weight and the rounded remainder); x is split the same way in
+ *                `workspace` and the product runs as one bfloat16 GEMM over 3K with float32
+ *                accumulation (x and w to about 2^-17 relative).  parts = 2, wt = [w | w], for
+ *                weights that are exact in bfloat16.
+ * K % 64 == 0 and 16-byte aligned operands run on the MFMA tile kernel (which splits K over
+ * workgroups while its tiles are few); anything else on a plain kernel.
+ * For EinsumDense int4 kernels whose stored [rows, columns] matrix is a row-major reshape of a
+ * kernel with contracted axes that are not leading (e.g. "btd,ndh->btnh"): there a stored
+ * column's scale does not belong to one output column, so the reference's own order
+ * (de-quantise, reshape, einsum: keras/src/layers/core/einsum_dense.py:1136-1187, :1205-1236)
+ * is the only one, with the de-quantised kernel kept by the layer instead of rebuilt per call.
+ * workspace: k3q_gemm_wbf16_workspace_bytes(M, N, K, parts) bytes, 16-byte aligned.
+ */
+int64_t k3q_gemm_wbf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int parts);
+int k3q_gemm_wbf16(const void* x, int x_dtype, const uint16_t* wt, int parts, int64_t M, int64_t N,
+                   int64_t K, const void* bias, void* y, void* workspace, int64_t workspace_bytes,
+                   void* stream);
+
+/*
  * Weight-only int4 matmul, any M (bandwidth-bound kernel tuned for M <= 16; passes of
  * 32 rows (bfloat16) or 8 rows (float32) below prefill sizes; from 65 (float32: 48 to 80) rows on, for
  * K % 128 == 0 and N % 64 == 0, the kernel is de-quantised once per call into `workspace`

@@ -54,6 +54,11 @@ SIGNATURES = {
         _int,
         [_ptr, _int, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _ptr],
     ),
+    "k3q_gemm_wbf16_workspace_bytes": (_i64, [_i64, _i64, _i64, _int]),
+    "k3q_gemm_wbf16": (
+        _int,
+        [_ptr, _int, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr],
+    ),
     "k3q_gemv_w4_nk": (
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _int, _ptr, _i64, _ptr, _ptr],

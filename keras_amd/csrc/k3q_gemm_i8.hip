@@ -667,6 +667,31 @@ __global__ __launch_bounds__(256) void transpose_widen_i8_to_bf16(const int8_t* 
     }
 }
 
+// Float x against a bfloat16 kernel [N, parts * K] (parts 3: [wh | wh | wl], the weight is
+// wh + wl), any shape: one thread per output, fp32 accumulation.
+template <bool kBF16>
+__global__ __launch_bounds__(256) void gemm_wbf16_simple(const void* x, const uint16_t* wt, int parts,
+                                                         const void* bias, void* y, int64_t N,
+                                                         int64_t K) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t m = blockIdx.y;
+    if (n >= N) return;
+    const uint16_t* w = wt + n * parts * K;
+    float acc = 0.f;
+    for (int64_t k = 0; k < K; ++k) {
+        float wv = bf16_bits_to_f32(w[k]);
+        if (parts == 3) wv += bf16_bits_to_f32(w[2 * K + k]);
+        acc = fmaf(load_t<kBF16>(x, m * K + k), wv, acc);
+    }
+    if (kBF16) {
+        float r = round_bf16(acc);
+        if (bias) r = round_bf16(r + load_t<true>(bias, n));
+        ((uint16_t*)y)[m * N + n] = (uint16_t)f32_to_bf16_bits(r);
+    } else {
+        ((float*)y)[m * N + n] = bias ? acc + load_t<false>(bias, n) : acc;
+    }
+}
+
 // Any shape and dtype: one thread per output, fp32 accumulation.
 template <bool kBF16>
 __global__ __launch_bounds__(256) void gemm_w8_simple(const void* x, const int8_t* b,
@@ -1054,5 +1079,45 @@ extern "C" int k3q_gemm_w8(const void* x, int x_dtype, const int8_t* b, int b_la
         gemm_w8_simple<true><<<grid, 256, 0, s>>>(x, b, sk, sn, b_scale, bias, y, N, K);
     else
         gemm_w8_simple<false><<<grid, 256, 0, s>>>(x, b, sk, sn, b_scale, bias, y, N, K);
+    return launch_status();
+}
+
+extern "C" int64_t k3q_gemm_wbf16_workspace_bytes(int64_t M, int64_t N, int64_t K, int parts) {
+    if (M <= 0 || N <= 0 || K <= 0 || parts < 1 || parts > 3) return 0;
+    // the split rows of float32 x, then the partials of a K split
+    return (parts > 1 ? M * parts * K * 2 : 0) + split_workspace_bytes(M, N, 2 * parts * K);
+}
+
+extern "C" int k3q_gemm_wbf16(const void* x, int x_dtype, const uint16_t* wt, int parts, int64_t M,
+                              int64_t N, int64_t K, const void* bias, void* y, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+    if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || N <= 0 || K <= 0) return K3Q_ERR_SHAPE;
+    const bool bf16 = x_dtype == K3Q_BF16;
+    if (bf16 ? parts != 1 : (parts != 2 && parts != 3)) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (!x || !wt || !y) return K3Q_ERR_NULL;
+    const size_t el = bf16 ? 2 : 4;
+    if (!aligned_to(x, el) || !aligned_to(wt, 2) || !aligned_to(y, el) || (bias && !aligned_to(bias, el)))
+        return K3Q_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t xs_bytes = bf16 ? 0 : M * parts * K * 2;
+    const void* a_op = bf16 ? x : workspace;
+    const bool fast = (K % 64) == 0 && aligned_to(x, 16) && (bf16 || (K % 4) == 0) &&
+                      (bf16 || (workspace && workspace_bytes >= xs_bytes && aligned_to(workspace, 16))) &&
+                      gemm_bf16_nk_supported(M, N, parts * K, a_op, wt, y) &&
+                      aligned_to(y, bf16 ? 8 : 16) && (!bias || aligned_to(bias, 4));
+    if (fast) {
+        if (!bf16) split_f32_rows_launch((const float*)x, (uint16_t*)workspace, M, K, parts, s);
+        char* rest = workspace ? (char*)workspace + xs_bytes : nullptr;
+        return gemm_bf16_nk_run(a_op, wt, M, N, parts * K, nullptr, bias, y, !bf16, rest,
+                                workspace ? workspace_bytes - xs_bytes : 0, s);
+    }
+    if (M > 65535) return K3Q_ERR_SHAPE;
+    dim3 grid((unsigned)((N + 255) / 256), (unsigned)M);
+    if (bf16)
+        gemm_wbf16_simple<true><<<grid, 256, 0, s>>>(x, wt, parts, bias, y, N, K);
+    else
+        gemm_wbf16_simple<false><<<grid, 256, 0, s>>>(x, wt, parts, bias, y, N, K);
     return launch_status();
 }

@@ -470,15 +470,12 @@ class EinsumDense(Layer):
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
         gv = self._gemm_view()
-        if not gv.k_plain:
-            raise NotImplementedError(
-                f"equation '{self.equation}': the stored int4 kernel is a row-major reshape of a kernel "
-                "whose contracted axes are not leading, which the fused int4 kernel cannot consume in place"
-            )
         x2, free_shape = self._input_rows(inputs, gv)
         cd = to_torch_dtype(self.compute_dtype)
         block_size = self._int4_block_size
         grouped = block_size is not None and block_size > 0
+        if not gv.k_plain:
+            return self._int4_call_dequantized(x2, free_shape, gv, cd, grouped)
         bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
         if self.inputs_quantizer:
             if grouped:
@@ -508,6 +505,62 @@ class EinsumDense(Layer):
             block_size=block_size if grouped else None,
             bias=bias,
         )
+        return self._finish(y2, free_shape, gv, fused)
+
+    def _int4_dequantized_kernel(self, gv, cd, grouped):
+        """The float kernel of einsum_dense.py:1143-1150 / :1213-1222 (unpack, divide by the
+        scale | dequantize_with_sz_map, cast, reshape to the kernel's own shape), then laid
+        out as the [N, K] operand of the float GEMM.  Kept until a variable changes."""
+        variables = [self._kernel, self.kernel_scale]
+        if grouped:
+            variables += [self.kernel_zero, self.g_idx]
+        stamp = tuple((id(v), v.version) for v in variables) + (cd,)
+        hit = self._cache.get("int4_dequantized")
+        if hit is not None and hit[0] == stamp:
+            return hit[1], hit[2]
+        unpacked = quantizers.unpack_int4(
+            as_tensor(self._kernel), self._int4_unpacked_column_size, axis=-1)
+        scale = as_tensor(self.kernel_scale).to(cd)
+        if grouped:
+            fk = quantizers.dequantize_with_sz_map(
+                unpacked, scale, as_tensor(self.kernel_zero), as_tensor(self.g_idx), group_axis=0
+            ).to(cd)
+        else:
+            fk = torch.divide(unpacked.to(cd), scale)
+        fk = fk.reshape(self.original_kernel_shape).permute(gv.k_perm)
+        k = 1
+        for c in gv.contracted:
+            k *= self.full_output_shape_of(c)
+        w_nk = fk.reshape(k, -1).t().contiguous()
+        if cd == torch.bfloat16:
+            wt, parts = w_nk, 1
+        else:
+            wt, parts = kops.split_f32_kernel(w_nk.to(torch.float32)), 3
+        self._cache["int4_dequantized"] = (stamp, wt, parts)
+        return wt, parts
+
+    def _int4_call_dequantized(self, x2, free_shape, gv, cd, grouped):
+        """int4 kernels stored as a row-major reshape of a kernel whose contracted axes are not
+        leading (e.g. "btd,ndh->btnh"): a stored column then mixes output columns and rows of
+        K, so its scale cannot be taken out of the sum.  The reference's order is the only
+        one: de-quantise, reshape, contract in the compute dtype."""
+        if x2.dtype not in (torch.bfloat16, torch.float32):
+            raise TypeError(f"int4 EinsumDense computes in bfloat16 or float32, got {x2.dtype}")
+        wt, parts = self._int4_dequantized_kernel(gv, cd, grouped)
+        if self.inputs_quantizer:
+            if grouped:
+                raise NotImplementedError(
+                    "Grouped int4 with an activation quantizer has no counterpart in the "
+                    "reference (einsum_dense.py:1188-1261 ignores the quantizer there)."
+                )
+            # einsum_dense.py:1163-1184: quantised rows, cast back to float, against the float
+            # kernel; then the division by the input scale, then the bias
+            q, scale = self.inputs_quantizer(x2, axis=-1)
+            y2 = kops.float_matmul_nk(q.to(cd), wt, parts)
+            y2 = torch.divide(y2, scale.to(cd))
+            return self._finish(y2, free_shape, gv, False)
+        bias, fused = self._fusable_bias(gv, wt.shape[0])
+        y2 = kops.float_matmul_nk(x2.to(cd), wt, parts, bias=bias)
         return self._finish(y2, free_shape, gv, fused)
 
     # ---- serialization -------------------------------------------------------------------------

@@ -338,3 +338,45 @@ def int8_weight_only_matmul(x, kernel, kernel_scale, bias=None, prepacked=None):
                          _lib.ptr(ws), ws.numel(), _lib.stream_ptr(x.device))
     _lib.check(rc, "k3q_gemm_w8")
     return y.reshape(*lead, N)
+
+
+def split_f32_kernel(w_nk):
+    """float32 [N, K] kernel -> bfloat16 [N, 3K] = [wh | wh | wl], w = wh + wl to 2^-17: the
+    operand `float_matmul_nk` takes for float32 inputs.  Made once per layer."""
+    wh = w_nk.to(torch.bfloat16)
+    wl = (w_nk - wh.to(torch.float32)).to(torch.bfloat16)
+    return torch.cat([wh, wh, wl], dim=1).contiguous()
+
+
+def float_matmul_nk(x, wt, parts=1, bias=None):
+    """`x[M, K] . w[N, K]^T` in x.dtype against a de-quantised kernel kept as bfloat16.
+
+    x bfloat16: wt = w [N, K], parts 1.  x float32: wt = `split_f32_kernel(w)` [N, 3K], parts 3.
+    Reference: the `ops.einsum(self.equation, inputs, float_kernel)` of
+    keras/src/layers/core/einsum_dense.py:1186 and :1236 for kernels the fused int4 kernel
+    cannot consume in place.
+    """
+    _lib.require_device(x, wt, bias)
+    if wt.dtype != torch.bfloat16 or wt.dim() != 2 or not wt.is_contiguous():
+        raise TypeError("the kernel must be a contiguous 2-D bfloat16 tensor")
+    if x.dim() != 2:
+        raise ValueError("x must be [M, K]")
+    want_parts = 1 if x.dtype == torch.bfloat16 else 3
+    if parts not in (want_parts, 2 if want_parts == 3 else want_parts):
+        raise ValueError(f"parts={parts} does not fit inputs of {x.dtype}")
+    M, K = x.shape
+    if wt.shape[1] != parts * K:
+        raise ValueError(f"kernel row length {wt.shape[1]} is not parts * K = {parts * K}")
+    if bias is not None and bias.dtype != x.dtype:
+        raise TypeError("bias must be read in the input's dtype")
+    N = wt.shape[0]
+    x = x if x.is_contiguous() else x.contiguous()
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    ws = _workspace(x.device, lib.k3q_gemm_wbf16_workspace_bytes(M, N, K, parts))
+    rc = lib.k3q_gemm_wbf16(_lib.ptr(x), _lib.dtype_code(x.dtype), _lib.ptr(wt), parts, M, N, K,
+                            _lib.ptr(bias), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
+                            _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemm_wbf16")
+    return y
+

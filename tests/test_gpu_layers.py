@@ -149,6 +149,73 @@ def test_einsum_dense_int8(dev, equation, output_shape, input_shape, policy):
     assert (y_float.float() - y.float()).pow(2).mean().item() < 2e-2
 
 
+# kernels whose contracted axis is not leading ("ndh" contracts d): the stored int4 matrix is a
+# row-major reshape that mixes output columns, so these run de-quantise + float GEMM
+NON_LEADING = [
+    EQUATIONS[1],
+    ("btd,ndh->btnh", (None, 8, 64), (2, 5, 256)),
+    ("btd,ndh->btnh", (None, 4, 40), (1, 3, 72)),   # K % 64 != 0: the plain kernel
+    ("ab,cb->ac", (48,), (7, 128)),
+]
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape", NON_LEADING)
+@pytest.mark.parametrize("block_size", [128, 8, None])
+@pytest.mark.parametrize("policy", ["mixed_bfloat16", "float32"])
+def test_einsum_dense_int4_non_leading_contraction(dev, equation, output_shape, input_shape, block_size, policy):
+    g = torch.Generator().manual_seed(77)
+    layer = EinsumDense(equation, output_shape, dtype=policy, device=dev, bias_axes=None,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    x = torch.rand(input_shape, generator=g) - 0.5
+    y_float = layer(x)
+    layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=block_size))
+    qk = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), block_size)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    assert torch.equal(layer.kernel_scale.value.cpu(), qk["kernel_scale"])
+    y = layer(x)
+    again = layer(x)  # second call: the cached de-quantised kernel
+    want = ref.einsum_dense_int4_call(x.to(cd), qk, equation, compute_dtype=cd, block_size=block_size)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    assert torch.equal(y, again)
+    assert max_rel_err(y, want) <= RTOL[cd]
+    # the float reference evaluated exactly: the kernel is at least about as close as torch's chain
+    uk = ref.unpack_int4(qk["kernel"], qk["cols"], axis=-1)
+    ks = qk["kernel_scale"].to(cd)
+    if block_size is None:
+        fk = torch.divide(uk.to(cd), ks)
+    else:
+        fk = ref.dequantize_with_sz_map(uk, ks, qk["kernel_zero"], qk["g_idx"], group_axis=0).to(cd)
+    exact = torch.einsum(equation, x.to(cd).double(), fk.reshape(qk["original_kernel_shape"]).double())
+    assert max_rel_err(y, exact) <= max(2 * max_rel_err(want, exact), RTOL[cd] / 4)
+    mse = (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item()
+    mse_ref = (y_float.float().cpu() - want.float()).pow(2).mean().item()
+    assert mse <= 1.25 * mse_ref + 1e-5
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape", NON_LEADING[:2])
+@pytest.mark.parametrize("policy", ["mixed_bfloat16", "float32"])
+def test_einsum_dense_int4_non_leading_activation_quantized(dev, equation, output_shape, input_shape, policy):
+    g = torch.Generator().manual_seed(78)
+    layer = EinsumDense(equation, output_shape, dtype=policy, device=dev, bias_axes="h",
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d),
+                        bias_initializer=lambda s, d: (torch.rand(s, generator=g) * 0.1).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    bias = layer.bias.value.cpu()
+    x = torch.rand(input_shape, generator=g)
+    config = ka.Int4QuantizationConfig(block_size=None, activation_quantizer=ka.quantizers.AbsMaxQuantizer())
+    layer.quantize("int4", config=config)
+    qk = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), None)
+    y = layer(x)
+    want = ref.einsum_dense_int4_activation_quantized_call(x.to(cd), qk, equation, bias=bias, compute_dtype=cd)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    assert max_rel_err(y, want) <= RTOL[cd]
+
+
 @pytest.mark.parametrize("equation,output_shape,input_shape", [EQUATIONS[0], EQUATIONS[2], EQUATIONS[4], EQUATIONS[5]])
 @pytest.mark.parametrize("block_size", [128, None])
 def test_einsum_dense_int4(dev, equation, output_shape, input_shape, block_size):
