@@ -368,3 +368,33 @@ def test_einsum_dense_int4_activation_quantized(dev, equation, output_shape, inp
     want = ref.einsum_dense_int4_activation_quantized_call(x.to(cd), qk, equation, compute_dtype=cd)
     assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
     assert max_rel_err(y, want) <= RTOL[cd]
+
+
+@pytest.mark.parametrize("mode,equation,output_shape,input_shape,threshold", [
+    # einsum_dense_test.py:629-677, the reference's own cases and thresholds
+    ("int8", "btnh,nhd->btd", (None, 8), (1, 2, 2, 4), 1e-3),
+    ("int8", "btd,ndh->btnh", (None, 2, 8), (1, 2, 4), 1e-3),
+    ("int8", "btd,df->btf", (None, 4), (1, 2, 4), 1e-3),
+    ("int4", "btnh,nhd->btd", (None, 8), (1, 2, 2, 4), 4e-3),
+    ("int4", "btd,ndh->btnh", (None, 2, 8), (1, 2, 4), 4e-3),
+    ("int4", "btd,df->btf", (None, 4), (1, 2, 4), 4e-3),
+])
+def test_quantize_with_specific_equations(dev, mode, equation, output_shape, input_shape, threshold):
+    # einsum_dense_test.py:678-697: quantize a float layer, the output stays close (MSE)
+    g = torch.Generator().manual_seed(1337)
+    fan = 1
+    for d in input_shape[1:]:
+        fan *= d
+
+    def glorot(shape, dtype):
+        limit = (6.0 / (fan + shape[-1])) ** 0.5
+        return ((torch.rand(shape, generator=g) * 2 - 1) * limit).to(dtype)
+
+    layer = EinsumDense(equation, output_shape, device=dev, kernel_initializer=glorot)
+    layer.build(input_shape)
+    x = torch.rand(input_shape, generator=g)
+    y_float = layer(x)
+    layer.quantize(mode)
+    y_quantized = layer(x)
+    mse = (y_float.float() - y_quantized.float()).pow(2).mean().item()
+    assert mse < threshold
