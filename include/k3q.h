@@ -92,8 +92,11 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  * with one final rounding (differs from the chain by at most the chain's own
  * intermediate roundings).
  * The MFMA kernel needs K % 128 == 0 and 16-byte aligned operands (any N; with
- * N % 4 != 0 the rows of y are stored element by element and K is never split);
- * other shapes run a plain kernel.  With b_layout 0 the MFMA kernel also needs
+ * N % 4 != 0 the rows of y are stored element by element and K is never split).
+ * With K % 128 != 0 (a model width of 1600 or 960) and a `workspace` of
+ * k3q_gemm_i8_workspace_bytes (either b_layout) both operands are first copied into it
+ * with their rows zero-padded to the next multiple of 128: the same accumulators, bit for
+ * bit.  Other shapes run a plain kernel.  With b_layout 0 the MFMA kernel also needs
  * `workspace` (k3q_gemm_i8_workspace_bytes, 16-byte aligned) to hold the [N,K]
  * copy it makes on every call; callers that reuse a kernel should prepack once.
  * flags bit 1 (K3Q_GEMM_ROUND_ACC_BF16, float32 output only): acc is cast to bfloat16

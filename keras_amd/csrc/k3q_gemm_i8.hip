@@ -595,9 +595,11 @@ __global__ __launch_bounds__(256) void gemm_i8_simple(const int8_t* a, const int
     }
 }
 
-// [K, N] -> [N, K] byte transpose through a padded LDS tile (one-time per layer).
+// [K, N] -> [N, out_stride] byte transpose through a padded LDS tile (one-time per layer);
+// bytes [K, out_stride) of every output row are zero.  The grid covers out_stride along y.
 __global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ in,
-                                                    int8_t* __restrict__ out, int64_t K, int64_t N) {
+                                                    int8_t* __restrict__ out, int64_t K, int64_t N,
+                                                    int64_t out_stride) {
     __shared__ int8_t tile[64][64 + 4];
     const int64_t k0 = (int64_t)blockIdx.y * 64;
     const int64_t n0 = (int64_t)blockIdx.x * 64;
@@ -610,8 +612,28 @@ __global__ __launch_bounds__(256) void transpose_i8(const int8_t* __restrict__ i
     __syncthreads();
     for (int e = threadIdx.x; e < 64 * 64; e += 256) {
         const int r = e / 64, c = e % 64;  // r: n within tile, c: k within tile
-        if (n0 + r < N && k0 + c < K) out[(n0 + r) * K + k0 + c] = tile[c][r];
+        if (n0 + r < N && k0 + c < out_stride) out[(n0 + r) * out_stride + k0 + c] = tile[c][r];
     }
+}
+
+// rows of K bytes -> rows of Kpad bytes, zero-filled (Kpad % 16 == 0), 16 output bytes per thread
+__global__ __launch_bounds__(256) void pad_rows_i8(const int8_t* __restrict__ in,
+                                                   int8_t* __restrict__ out, int64_t rows, int64_t K,
+                                                   int64_t Kpad) {
+    const int64_t per_row = Kpad / 16;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * per_row) return;
+    const int64_t r = i / per_row, c = (i - r * per_row) * 16;
+    const int8_t* src = in + r * K + c;
+    v4u v = {0u, 0u, 0u, 0u};
+    if (c + 16 <= K && (((uintptr_t)src) & 15) == 0) {
+        v = *(const v4u*)src;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            if (c + e < K) v[e >> 2] |= (u32)(uint8_t)src[e] << (8 * (e & 3));
+    }
+    *(v4u*)(out + r * Kpad + c) = v;
 }
 
 // ---- weight-only int8: the int8 kernel widened to bfloat16 [N, K] in scratch (exact) ----
@@ -933,6 +955,10 @@ extern "C" int64_t k3q_gemm_i8_workspace_bytes(int64_t M, int64_t N, int64_t K) 
         const int64_t nk = gemm_i8_skinny_nk_workspace_bytes(M, N, K);
         return kn > nk ? kn : nk;
     }
+    // K not a multiple of the tile's K step: zero-padded copies of both operands, then the
+    // partials of a K split
+    const int64_t Kpad = (K + kBK - 1) / kBK * kBK;
+    if (Kpad != K) return (M + N) * Kpad + split_workspace_bytes(M, N, Kpad);
     // the [N,K] copy (16-byte multiple), then the partials of a K split
     return (N * K + 15) / 16 * 16 + split_workspace_bytes(M, N, K);
 }
@@ -942,7 +968,7 @@ extern "C" int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N,
     if (K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
     if (!kernel || !prepacked) return K3Q_ERR_NULL;
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
-    transpose_i8<<<grid, 256, 0, (hipStream_t)stream>>>(kernel, prepacked, K, N);
+    transpose_i8<<<grid, 256, 0, (hipStream_t)stream>>>(kernel, prepacked, K, N, K);
     return launch_status();
 }
 
@@ -977,7 +1003,12 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
         return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
                                   workspace, workspace_bytes, s);
     const bool forced_tile = (flags & (kFlagForceSmallTile | kFlagForceLargeTile)) != 0;
-    bool fast = (K % kBK) == 0 && aligned_to(a, 16) && aligned_to(b, 16) &&
+    // K % 128 != 0 (model widths like 1600 or 960): both operands are copied into scratch with
+    // their rows zero-padded to the tile's K step; zeros add nothing, the result is the same
+    const int64_t Kpad = (K + kBK - 1) / kBK * kBK;
+    const bool padded = Kpad != K;
+    bool fast = (padded ? (workspace && aligned_to(workspace, 16) && workspace_bytes >= (M + N) * Kpad)
+                        : (aligned_to(a, 16) && aligned_to(b, 16))) &&
                 (!y || aligned_to(y, 4 * el)) && (!acc_out || aligned_to(acc_out, 16)) &&
                 (!b_scale || aligned_to(b_scale, 16)) && (!bias || aligned_to(bias, 16)) &&
                 ((M + 127) / 128) * ((N + 127) / 128) < (1 << 28);
@@ -990,7 +1021,22 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
                                      workspace, workspace_bytes, s);
     char* scratch = (workspace && aligned_to(workspace, 16)) ? (char*)workspace : nullptr;
     int64_t scratch_bytes = scratch ? workspace_bytes : 0;
-    if (fast && b_layout == 0) {
+    if (fast && padded) {
+        int8_t* a_pad = (int8_t*)scratch;
+        int8_t* b_pad = a_pad + M * Kpad;
+        pad_rows_i8<<<(unsigned)((M * (Kpad / 16) + 255) / 256), 256, 0, s>>>(a, a_pad, M, K, Kpad);
+        if (b_layout == 0) {
+            dim3 grid((unsigned)((N + 63) / 64), (unsigned)(Kpad / 64));
+            transpose_i8<<<grid, 256, 0, s>>>(b, b_pad, K, N, Kpad);
+        } else {
+            pad_rows_i8<<<(unsigned)((N * (Kpad / 16) + 255) / 256), 256, 0, s>>>(b, b_pad, N, K, Kpad);
+        }
+        p.a = a_pad;
+        p.bt = b_pad;
+        p.row_bytes = Kpad;
+        scratch += (M + N) * Kpad;
+        scratch_bytes -= (M + N) * Kpad;
+    } else if (fast && b_layout == 0) {
         // needs the [N,K] copy: made here per call when the caller supplies scratch for it
         const int64_t copy_bytes = (N * K + 15) / 16 * 16;
         if (scratch && scratch_bytes >= N * K) {

@@ -160,9 +160,11 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
     nbytes = lib.k3q_gemm_i8_workspace_bytes(M, N, K)
     if prepacked is not None and not skinny:
         # no per-call [N,K] copy: only the part of the scratch beyond it (partial sums of a
-        # K split, taken for few-tile problems) is of use
+        # K split, taken for few-tile problems) is of use; a K that is not a multiple of 128
+        # keeps all of it (both operands are zero-padded into it)
         b, layout = prepacked, 1
-        nbytes = max(0, nbytes - (N * K + 15) // 16 * 16)
+        if K % 128 == 0:
+            nbytes = max(0, nbytes - (N * K + 15) // 16 * 16)
     else:
         b = kernel if kernel.is_contiguous() else kernel.contiguous()
         layout = 0
@@ -212,7 +214,9 @@ def int8_matmul_nk(a, kernel_nk, a_scale=None, kernel_scale=None, out_dtype=None
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
     lib = _lib.load()
     ws, ws_bytes = None, 0
-    if M <= 64:  # the decode kernels may split K and then need room for int32 partials
+    if M <= 64 or K % 128 != 0:
+        # the decode kernels may split K and then need room for int32 partials; a K that is not
+        # a multiple of 128 has both operands zero-padded into scratch
         ws = _workspace(a.device, lib.k3q_gemm_i8_workspace_bytes(M, N, K))
         ws_bytes = ws.numel()
     rc = lib.k3q_gemm_i8(

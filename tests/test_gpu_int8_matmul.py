@@ -52,8 +52,10 @@ SHAPES = [
     (255, 384, 256), (256, 1024, 512), (300, 640, 772), (513, 256, 1028),
     # N % 4 != 0 (a vocabulary of 50257 or 30522): the tiles store those rows element-wise
     (300, 256, 1001), (129, 384, 50257), (64, 128, 30522), (200, 512, 3), (1000, 128, 130),
-    # K % 128 != 0: plain kernel
-    (5, 100, 30), (8, 8, 16), (33, 64, 7), (2, 200, 64),
+    # K % 128 != 0: operands zero-padded into scratch, then the tiles (model widths 1600, 960;
+    # odd and unaligned K; with a K split; N % 4 != 0 as well)
+    (5, 100, 30), (8, 8, 16), (33, 64, 7), (2, 200, 64), (300, 1600, 640), (64, 960, 1280),
+    (130, 6400, 1600), (77, 333, 129), (40, 72, 264), (1100, 200, 1001),
 ]
 
 
