@@ -180,3 +180,35 @@ def test_int4_single_launch_split_matches_two_launches(dev):
             torch.cuda.synchronize()
             assert torch.equal(y1, y2), (M, K, N, bs, dtype)
             assert int(counters.count_nonzero()) == 0
+
+
+def test_int4_single_launch_split_repeated(dev):
+    # the last-arriver protocol a few hundred times per shape, other work in between: every
+    # result equals the two-launch one (a lost or stale partial would show as a different sum)
+    from keras_amd import _lib
+    lib = _lib.load()
+    counters = torch.zeros(1 << 12, dtype=torch.uint8, device=dev)
+    noise = torch.randn(1 << 22, device=dev)
+    for (M, K, N, bs) in [(1, 8192, 8192, None), (8, 4096, 14336, 128), (2, 14336, 4096, 128)]:
+        qk, _ = make_layer(K, N, bs, 40, False)
+        grouped = bs is not None
+        w = qk["kernel"].to(dev)
+        sc = qk["kernel_scale"].to(torch.bfloat16).to(dev)
+        zp = qk["kernel_zero"].to(dev) if grouped else None
+        ws = torch.empty(max(lib.k3q_gemv_w4_workspace_bytes(M, K, N), 16), dtype=torch.uint8, device=dev)
+        s = _lib.stream_ptr(dev)
+        bad = torch.zeros((), dtype=torch.int64, device=dev)
+        for it in range(300):
+            x = torch.randn(M, K, device=dev).to(torch.bfloat16)
+            args = [_lib.ptr(x), _lib.dtype_code(torch.bfloat16), M, K, N, _lib.ptr(w), _lib.ptr(sc),
+                    _lib.ptr(zp), bs if grouped else -1, None]
+            y2 = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            y1 = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            assert lib.k3q_gemv_w4(*args, _lib.ptr(y2), _lib.ptr(ws), ws.numel(), s) == 0
+            if it % 3 == 0:
+                noise.mul_(1.0001)  # unrelated traffic through the caches
+            assert lib.k3q_gemv_w4_fused(*args, _lib.ptr(y1), _lib.ptr(ws), ws.numel(),
+                                         _lib.ptr(counters), counters.numel(), s) == 0
+            bad += (y1.view(torch.int16) != y2.view(torch.int16)).sum()
+        assert int(bad) == 0
+        assert int(counters.count_nonzero()) == 0
