@@ -112,23 +112,50 @@ __device__ __forceinline__ v4f load_v4f(const float* src) {
 
 // Sum of the KS partials of four adjacent outputs, in one fixed order wherever it is
 // computed: four interleaved chains (partial ks goes to chain ks % 4), joined pairwise.
-// Eight loads are in flight before the first add (left alone, the scheduler pairs every load
-// with its add: one memory round trip per partial instead of one per eight).
-template <bool kDevice>
+// The loads go out in groups of 16 or 8, then 4 and a remainder, each group in flight as a whole
+// before its first add (left alone, the scheduler pairs every load with its add: one memory
+// round trip per partial).
+template <bool kDevice, int kCount>
+__device__ __forceinline__ void add_partials(v4f (&s4)[4], const float* src, int64_t stride) {
+    v4f t[kCount];
+#pragma unroll
+    for (int u = 0; u < kCount; ++u) t[u] = load_v4f<kDevice>(src + u * stride);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < kCount; ++u) s4[u & 3] += t[u];
+}
+
+// kWide: groups of 16 (64 data and 32 address registers: too many inside the main kernel,
+// where they cost the per-channel variant its fourth wave per SIMD)
+template <bool kDevice, bool kWide>
 __device__ __forceinline__ v4f sum_partials(const float* src, int64_t stride, int KS) {
     v4f s4[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) s4[u] = v4f{0.f, 0.f, 0.f, 0.f};
-    for (int ks = 0; ks < KS; ks += 8) {
-        v4f t[8];
+    int ks = 0;
+    if (kWide) {
+        for (; ks + 16 <= KS; ks += 16) add_partials<kDevice, 16>(s4, src + ks * stride, stride);
+    } else {
+        for (; ks + 16 <= KS; ks += 8) add_partials<kDevice, 8>(s4, src + ks * stride, stride);
+    }
+    if (ks + 8 <= KS) {
+        add_partials<kDevice, 8>(s4, src + ks * stride, stride);
+        ks += 8;
+    }
+    if (ks + 4 <= KS) {
+        add_partials<kDevice, 4>(s4, src + ks * stride, stride);
+        ks += 4;
+    }
+    if (ks < KS) {  // one to three left
+        v4f t[3];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 3; ++u) {
             t[u] = v4f{0.f, 0.f, 0.f, 0.f};
             if (ks + u < KS) t[u] = load_v4f<kDevice>(src + (ks + u) * stride);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s4[u & 3] += t[u];
+        for (int u = 0; u < 3; ++u) s4[u] += t[u];
     }
     return (s4[0] + s4[1]) + (s4[2] + s4[3]);
 }
@@ -517,7 +544,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
         const int64_t n = nb + (idx % (kNB / 4)) * 4;
         if (n >= p.N) continue;
         finish4_prefetched<kBF16, kGrouped>(p, m, n, [&]() {
-            return sum_partials<true>(p.part + (int64_t)m * p.N + n, (int64_t)M * p.N, KS);
+            return sum_partials<true, false>(p.part + (int64_t)m * p.N + n, (int64_t)M * p.N, KS);
         });
     }
     if (threadIdx.x == 0) atomicExch(p.sync + cb, 0u);
@@ -532,7 +559,7 @@ __global__ __launch_bounds__(256) void gemv_w4_reduce(GemvParams p, int KS) {
     const int m = blockIdx.y;
     if (n >= p.N) return;
     finish4_prefetched<kBF16, kGrouped>(p, m, n, [&]() {
-        return sum_partials<false>(p.part + (int64_t)m * p.N + n, (int64_t)p.M * p.N, KS);
+        return sum_partials<false, true>(p.part + (int64_t)m * p.N + n, (int64_t)p.M * p.N, KS);
     });
 }
 
