@@ -226,6 +226,31 @@ int k3q_gemv_w4_fused(const void* x, int x_dtype, int64_t M, int64_t K, int64_t 
                       void* stream);
 
 /*
+ * Several weight-only int4 matmuls against ONE x, each as k3q_gemv_w4_fused computes it (same
+ * bits), in one launch when they are decode-sized (M <= 16) and their launch plans agree
+ * (e.g. kernels of one shape: the query / key / value projections of an attention block, the
+ * gate / up projections of a gated MLP); otherwise one after the other.  A launch costs
+ * several microseconds whatever it does, which is most of a decode-sized matmul.
+ * problems[i]: the operands of k3q_gemv_w4 that differ per kernel (N, w_packed [K, ceil(N/2)],
+ * scale, zero, bias, y [M, N]); block_size is common.  workspace: the sum over i of
+ * k3q_gemv_w4_workspace_bytes(M, K, N_i), each rounded up to a multiple of 256; counters: the
+ * sum of k3q_gemv_w4_counters_bytes(N_i), zero between calls as for k3q_gemv_w4_fused.
+ * No counterpart in the reference, whose layers each call matmul on their own.
+ */
+typedef struct {
+    int64_t N;
+    const void* w_packed;
+    const void* scale;
+    const void* zero;
+    const void* bias;
+    void* y;
+} k3q_gemv_w4_problem;
+int k3q_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
+                      const k3q_gemv_w4_problem* problems, int64_t block_size, void* workspace,
+                      int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                      void* stream);
+
+/*
  * Same as k3q_gemv_w4_fused with the launch plan overridden, for tuning sweeps:
  * plan = {dwords per lane per k row (1|2), 16-row steps per chunk (1|2),
  * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null

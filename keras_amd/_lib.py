@@ -78,12 +78,25 @@ SIGNATURES = {
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
          _ptr],
     ),
+    "k3q_gemv_w4_multi": (
+        _int,
+        [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr],
+    ),
     "k3q_gemv_w4_plan": (
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
          _ptr, _ptr],
     ),
 }
+
+
+
+class GemvW4Problem(ctypes.Structure):
+    """`k3q_gemv_w4_problem` of include/k3q.h."""
+
+    _fields_ = [("N", ctypes.c_int64), ("w_packed", ctypes.c_void_p), ("scale", ctypes.c_void_p),
+                ("zero", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p)]
+
 
 _lib = None
 

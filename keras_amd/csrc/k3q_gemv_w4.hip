@@ -211,7 +211,7 @@ __device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
 // kSteps: 16-row K steps per chunk.  kSets: n -> up to 8n rows of bf16 x (n = 1, 2, 4); 2 -> also
 // rows of bf16 x, or up to 8 rows of f32 x split into two bf16 parts.
 template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
-__global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
+__device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, const int by) {
     extern __shared__ float red[];  // [waves][M][kNB + kRedPad]
 #ifdef K3Q_GEMV_PROBE
     const uint64_t ts0 = __builtin_amdgcn_s_memrealtime();
@@ -240,10 +240,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     // column blocks, so that blocks which share a 128-byte line of a packed row (kVec == 1)
     // meet in one L2 instead of fetching the line twice.
     const int per_xcd = p.per_xcd;
-    const int cb = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int cb = (bx % 8) * per_xcd + bx / 8;
     const int64_t nb = (int64_t)cb * kNB;
     if (nb >= p.N) return;  // grid.x is padded to a multiple of 8
-    const int64_t kw0 = ((int64_t)blockIdx.y * nwaves + wave) * p.klen;
+    const int64_t kw0 = ((int64_t)by * nwaves + wave) * p.klen;
     const int nchunks = p.klen / kChunk;
     const int M = p.M;
 
@@ -509,7 +509,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) finish<kBF16, kGrouped>(p, m, n + e, sum[e]);
             } else {
-                float* dst = p.part + ((int64_t)blockIdx.y * M + m) * p.N + n;
+                float* dst = p.part + ((int64_t)by * M + m) * p.N + n;
                 if (p.sync) store_v4f_device(dst, sum);
                 else *(v4f*)dst = sum;
             }
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
     }
 #ifdef K3Q_GEMV_PROBE
     if (threadIdx.x == 0 && KS > 1) {
-        uint64_t* d = (uint64_t*)(p.part + (int64_t)KS * M * p.N) + 8 * (blockIdx.y * (8 * per_xcd) + blockIdx.x);
+        uint64_t* d = (uint64_t*)(p.part + (int64_t)KS * M * p.N) + 8 * (by * (8 * per_xcd) + bx);
         d[0] = ts0; d[1] = ts1; d[2] = ts2; d[3] = __builtin_amdgcn_s_memrealtime();
         d[4] = ts2b; d[5] = ts2c;
     }
@@ -548,6 +548,32 @@ __global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
         });
     }
     if (threadIdx.x == 0) atomicExch(p.sync + cb, 0u);
+}
+
+template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
+__global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma(GemvParams p) {
+    gemv_w4_body<kVec, kSteps, kSets, kXF32, kGrouped>(p, blockIdx.x, blockIdx.y);
+}
+
+// Several kernels against one x in one launch (the query / key / value projections of an
+// attention block, the gate / up projections of a gated MLP): the column blocks of the
+// problems lie side by side along blockIdx.x, each problem with its own operands, partials
+// and arrival counters; the K split (blockIdx.y) is the largest of theirs.
+constexpr int kMaxProblems = 4;
+struct GemvMulti {
+    GemvParams p[kMaxProblems];
+    int first[kMaxProblems + 1];  // first blockIdx.x of each problem (multiples of 8), then the end
+    int count;
+};
+
+template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
+__global__ __launch_bounds__(kMaxWaves * 64) void gemv_w4_mfma_multi(GemvMulti mp) {
+    const int bx = blockIdx.x;
+    int i = 0;
+    while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
+    const GemvParams& p = mp.p[i];
+    if ((int)blockIdx.y >= p.ks) return;
+    gemv_w4_body<kVec, kSteps, kSets, kXF32, kGrouped>(p, bx - mp.first[i], blockIdx.y);
 }
 
 // Second pass when K is split over workgroups: sum the KS partials of every output in a
@@ -853,48 +879,59 @@ Plan make_plan(int x_dtype, int64_t M, int64_t K, int64_t N, int64_t block_size,
     return pl;
 }
 
+// `multi` (may be null): the multi-problem launch; otherwise `p` alone
 template <int kVec, int kSteps, int kSets, bool kXF32>
-void launch4(const GemvParams& p, bool grouped, dim3 grid, int threads, size_t lds, hipStream_t s) {
+void launch4(const GemvParams& p, const GemvMulti* multi, bool grouped, dim3 grid, int threads,
+             size_t lds, hipStream_t s) {
     // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
     static const bool raised = [] {
-        bool ok = hipFuncSetAttribute((const void*)gemv_w4_mfma<kVec, kSteps, kSets, kXF32, true>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      kLdsBudget) == hipSuccess;
-        ok = hipFuncSetAttribute((const void*)gemv_w4_mfma<kVec, kSteps, kSets, kXF32, false>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 kLdsBudget) == hipSuccess && ok;
+        bool ok = true;
+        const void* kernels[4] = {
+            (const void*)gemv_w4_mfma<kVec, kSteps, kSets, kXF32, true>,
+            (const void*)gemv_w4_mfma<kVec, kSteps, kSets, kXF32, false>,
+            (const void*)gemv_w4_mfma_multi<kVec, kSteps, kSets, kXF32, true>,
+            (const void*)gemv_w4_mfma_multi<kVec, kSteps, kSets, kXF32, false>};
+        for (const void* k : kernels)
+            ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget) ==
+                     hipSuccess && ok;
         return ok;
     }();
     (void)raised;
-    if (grouped)
+    if (multi) {
+        if (grouped)
+            gemv_w4_mfma_multi<kVec, kSteps, kSets, kXF32, true><<<grid, threads, lds, s>>>(*multi);
+        else
+            gemv_w4_mfma_multi<kVec, kSteps, kSets, kXF32, false><<<grid, threads, lds, s>>>(*multi);
+    } else if (grouped) {
         gemv_w4_mfma<kVec, kSteps, kSets, kXF32, true><<<grid, threads, lds, s>>>(p);
-    else
-        gemv_w4_mfma<kVec, kSteps, kSets, kXF32, false><<<grid, threads, lds, s>>>(p);
-}
-
-template <int kVec, int kSteps>
-void launch2(int sets, bool f32, const GemvParams& p, bool grouped, dim3 grid, int threads,
-             size_t lds, hipStream_t s) {
-    if (f32) {
-        launch4<kVec, kSteps, 2, true>(p, grouped, grid, threads, lds, s);
-    } else if (sets == 4) {
-        // four row sets only with 4-byte loads per lane (register budget)
-        if constexpr (kVec == 1) launch4<1, kSteps, 4, false>(p, grouped, grid, threads, lds, s);
-    } else if (sets == 2) {
-        launch4<kVec, kSteps, 2, false>(p, grouped, grid, threads, lds, s);
     } else {
-        launch4<kVec, kSteps, 1, false>(p, grouped, grid, threads, lds, s);
+        gemv_w4_mfma<kVec, kSteps, kSets, kXF32, false><<<grid, threads, lds, s>>>(p);
     }
 }
 
-void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, bool grouped, dim3 grid,
-                 int threads, size_t lds, hipStream_t s) {
+template <int kVec, int kSteps>
+void launch2(int sets, bool f32, const GemvParams& p, const GemvMulti* multi, bool grouped, dim3 grid,
+             int threads, size_t lds, hipStream_t s) {
+    if (f32) {
+        launch4<kVec, kSteps, 2, true>(p, multi, grouped, grid, threads, lds, s);
+    } else if (sets == 4) {
+        // four row sets only with 4-byte loads per lane (register budget)
+        if constexpr (kVec == 1) launch4<1, kSteps, 4, false>(p, multi, grouped, grid, threads, lds, s);
+    } else if (sets == 2) {
+        launch4<kVec, kSteps, 2, false>(p, multi, grouped, grid, threads, lds, s);
+    } else {
+        launch4<kVec, kSteps, 1, false>(p, multi, grouped, grid, threads, lds, s);
+    }
+}
+
+void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, const GemvMulti* multi,
+                 bool grouped, dim3 grid, int threads, size_t lds, hipStream_t s) {
     const int key = pl.vec * 10 + pl.steps;
     switch (key) {
-        case 22: launch2<2, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
-        case 21: launch2<2, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
-        case 12: launch2<1, 2>(sets, f32, p, grouped, grid, threads, lds, s); break;
-        default: launch2<1, 1>(sets, f32, p, grouped, grid, threads, lds, s); break;
+        case 22: launch2<2, 2>(sets, f32, p, multi, grouped, grid, threads, lds, s); break;
+        case 21: launch2<2, 1>(sets, f32, p, multi, grouped, grid, threads, lds, s); break;
+        case 12: launch2<1, 2>(sets, f32, p, multi, grouped, grid, threads, lds, s); break;
+        default: launch2<1, 1>(sets, f32, p, multi, grouped, grid, threads, lds, s); break;
     }
 }
 
@@ -1013,7 +1050,7 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         p.ks = pl.ks;
         const size_t lds = (size_t)pl.waves * rows * (nb_cols + kRedPad) * sizeof(float);
         const int sets = f32 ? 2 : (rows > 16 ? 4 : rows > 8 ? 2 : 1);
-        launch_plan(pl, sets, f32, p, grouped, grid, threads, lds, s);
+        launch_plan(pl, sets, f32, p, nullptr, grouped, grid, threads, lds, s);
         if (pl.ks > 1 && !p.sync) {
             dim3 rgrid((unsigned)((N / 4 + 255) / 256), rows);
             if (f32) {
@@ -1030,6 +1067,80 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
         }
     }
     return launch_status();
+}
+
+// One launch for several decode-sized problems that share x; returns false when their
+// plans do not allow it (the caller then runs them one by one).
+struct MultiProblem {
+    int64_t N;
+    const void* w_packed;
+    const void* scale;
+    const void* zero;
+    const void* bias;
+    void* y;
+};
+
+bool try_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
+                       const MultiProblem* pr, int64_t block_size, char* workspace,
+                       const int64_t* ws_offset, unsigned* counters, const int64_t* cnt_offset,
+                       hipStream_t s, int* rc) {
+    if (count < 2 || count > kMaxProblems) return false;
+    const bool grouped = block_size > 0;
+    const bool f32 = x_dtype == K3Q_F32;
+    // One plan for all of them, made for a kernel as wide as the problems together: the launch
+    // is then cut into about one workgroup per CU overall, not per problem.
+    int64_t n_total = 0;
+    for (int i = 0; i < count; ++i) n_total += pr[i].N;
+    const Plan pl0 = make_plan(x_dtype, M, K, n_total, block_size, nullptr);
+    if (!pl0.fast || M > pl0.rows || pl0.sets >= 4) return false;
+    const int nb_cols = 128 * pl0.vec;
+    // the last workgroup of a column block sums the K split: one output quad per thread
+    if (pl0.ks > 1 && (int)M * (nb_cols / 4) > pl0.waves * 64) return false;
+    GemvMulti mp{};
+    int next_block = 0;
+    const size_t lds = (size_t)pl0.waves * M * (nb_cols + kRedPad) * sizeof(float);
+    for (int i = 0; i < count; ++i) {
+        if ((pr[i].N % (8 * pl0.vec)) != 0) return false;
+        if (!aligned_to(pr[i].w_packed, 16) || !aligned_to(pr[i].scale, 16) ||
+            (pr[i].zero && !aligned_to(pr[i].zero, 4)))
+            return false;
+        const int64_t nblocks = (pr[i].N + nb_cols - 1) / nb_cols;
+        if (pl0.ks > 1 && ((int64_t)pl0.ks * M * pr[i].N * 4 > ws_offset[i + 1] - ws_offset[i] ||
+                           nblocks * 4 > cnt_offset[i + 1] - cnt_offset[i]))
+            return false;
+        GemvParams& p = mp.p[i];
+        p.x = x;
+        p.w = (const uint8_t*)pr[i].w_packed;
+        p.scale = pr[i].scale;
+        p.zero = (const int8_t*)pr[i].zero;
+        p.bias = pr[i].bias;
+        p.y = pr[i].y;
+        p.K = K;
+        p.N = pr[i].N;
+        p.row_bytes = (pr[i].N + 1) / 2;
+        p.block_size = grouped ? (int)block_size : 0;
+        p.M = (int)M;
+        p.m0 = 0;
+        p.klen = pl0.klen;
+        p.nwaves = pl0.waves;
+        p.ks = pl0.ks;
+        const int gx = (int)((nblocks + 7) / 8 * 8);
+        p.per_xcd = gx / 8;
+        if (pl0.ks > 1) {
+            p.part = (float*)(workspace + ws_offset[i]);
+            p.sync = counters + cnt_offset[i] / 4;
+        }
+        mp.first[i] = next_block;
+        next_block += gx;
+    }
+    const int max_ks = pl0.ks;
+    mp.first[count] = next_block;
+    mp.count = count;
+    dim3 grid((unsigned)next_block, (unsigned)max_ks);
+    const int sets = f32 ? 2 : (M > 16 ? 4 : M > 8 ? 2 : 1);
+    launch_plan(pl0, sets, f32, mp.p[0], &mp, grouped, grid, pl0.waves * 64, lds, s);
+    *rc = launch_status();
+    return true;
 }
 
 }  // namespace
@@ -1095,4 +1206,50 @@ extern "C" int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K
                                 const int* plan, void* stream) {
     return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
                        workspace_bytes, plan, counters, counters_bytes, (hipStream_t)stream);
+}
+
+extern "C" int k3q_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
+                                 const k3q_gemv_w4_problem* problems, int64_t block_size,
+                                 void* workspace, int64_t workspace_bytes, void* counters,
+                                 int64_t counters_bytes, void* stream) {
+    if (count < 0) return K3Q_ERR_SHAPE;
+    if (count == 0) return K3Q_OK;
+    if (!problems) return K3Q_ERR_NULL;
+    if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || K <= 0) return K3Q_ERR_SHAPE;
+    // every problem has its own slice of the workspace and of the counters
+    constexpr int kMaxCount = 16;
+    if (count > kMaxCount) return K3Q_ERR_SHAPE;
+    int64_t ws_offset[kMaxCount + 1], cnt_offset[kMaxCount + 1];
+    MultiProblem pr[kMaxCount];
+    ws_offset[0] = cnt_offset[0] = 0;
+    const size_t el = x_dtype == K3Q_F32 ? 4 : 2;
+    for (int i = 0; i < count; ++i) {
+        const k3q_gemv_w4_problem& q = problems[i];
+        if (q.N <= 0) return K3Q_ERR_SHAPE;
+        if (M > 0 && (!x || !q.w_packed || !q.scale || !q.y || (block_size > 0 && !q.zero)))
+            return K3Q_ERR_NULL;
+        if (!aligned_to(q.scale, el) || !aligned_to(q.y, el) || (q.bias && !aligned_to(q.bias, el)))
+            return K3Q_ERR_ALIGN;
+        pr[i] = MultiProblem{q.N, q.w_packed, q.scale, q.zero, q.bias, q.y};
+        ws_offset[i + 1] = ws_offset[i] + (k3q_gemv_w4_workspace_bytes(M, K, q.N) + 255) / 256 * 256;
+        cnt_offset[i + 1] = cnt_offset[i] + k3q_gemv_w4_counters_bytes(q.N);
+    }
+    if (M == 0) return K3Q_OK;
+    const bool ws_ok = workspace && aligned_to(workspace, 16) && workspace_bytes >= ws_offset[count];
+    const bool cnt_ok = counters && aligned_to(counters, 4) && counters_bytes >= cnt_offset[count];
+    hipStream_t s = (hipStream_t)stream;
+    int rc = K3Q_OK;
+    if (ws_ok && cnt_ok && aligned_to(x, 16) &&
+        try_gemv_w4_multi(x, x_dtype, M, K, count, pr, block_size, (char*)workspace, ws_offset,
+                          (unsigned*)counters, cnt_offset, s, &rc))
+        return rc;
+    for (int i = 0; i < count; ++i) {
+        // one after the other on the stream: each may use all of the workspace and counters
+        rc = run_gemv_w4(x, x_dtype, M, K, pr[i].N, pr[i].w_packed, pr[i].scale, pr[i].zero, block_size,
+                         pr[i].bias, pr[i].y, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0,
+                         nullptr, cnt_ok ? counters : nullptr, cnt_ok ? counters_bytes : 0, s);
+        if (rc != K3Q_OK) return rc;
+    }
+    return K3Q_OK;
 }

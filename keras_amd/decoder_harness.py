@@ -16,7 +16,7 @@ import math
 import torch
 
 from keras_amd import dtype_policies
-from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding
+from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding, call_together
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
 from keras_amd.models import Model
 from keras_amd.quantization_config import Int4QuantizationConfig
@@ -83,10 +83,11 @@ class DecoderBlock(Layer):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
         (an int64 device tensor [T]); mask [T, maxT] True where a key may be attended to."""
         h = self.attn_norm(x)
+        # the three projections of h in one launch at decode sizes
+        q, k, v = call_together((self.query, self.key, self.value), h)
         # one rotation over the query and key heads together (half the elementwise launches)
-        qk = apply_rope(torch.cat((self.query(h), self.key(h)), dim=2), cos, sin)
+        qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
         q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
-        v = self.value(h)
         kc, vc = cache
         kc.index_copy_(2, pos, k.transpose(1, 2))
         vc.index_copy_(2, pos, v.transpose(1, 2))
@@ -94,7 +95,8 @@ class DecoderBlock(Layer):
             q.transpose(1, 2), kc, vc, attn_mask=mask[None, None])
         x = x + self.attn_out(a.transpose(1, 2))
         h = self.ffn_norm(x)
-        return x + self.down(torch.nn.functional.silu(self.gate(h)) * self.up(h))
+        gate, up = call_together((self.gate, self.up), h)
+        return x + self.down(torch.nn.functional.silu(gate) * up)
 
 
 class LlamaStyleDecoder(Model):

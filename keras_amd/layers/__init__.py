@@ -1,5 +1,6 @@
 from keras_amd.layers.dense import Dense
 from keras_amd.layers.einsum_dense import EinsumDense
 from keras_amd.layers.embedding import Embedding, ReversibleEmbedding
+from keras_amd.layers.together import call_together
 
-__all__ = ["Dense", "EinsumDense", "Embedding", "ReversibleEmbedding"]
+__all__ = ["Dense", "EinsumDense", "Embedding", "ReversibleEmbedding", "call_together"]

@@ -302,6 +302,31 @@ class Dense(Layer):
             y = self.activation(y)
         return y
 
+    def _int4_together_spec(self, inputs):
+        """What `call_together` needs to run this layer's weight-only int4 forward in a launch
+        shared with other layers: the [M, K] rows, the kernel's operands and the step that
+        turns the [M, N] result into the layer's output.  None when the layer's forward is
+        anything else."""
+        if (not self.built or self.quantization_mode != "int4" or self.inputs_quantizer
+                or self.lora_enabled):
+            return None
+        block_size = getattr(self, "_int4_block_size", None)
+        grouped = block_size is not None and block_size > 0
+        lead = inputs.shape[:-1]
+
+        def finish(y2):
+            y = y2.reshape(*lead, self._orig_output_dim)
+            return self.activation(y) if self.activation is not None else y
+
+        return dict(
+            x2=inputs.reshape(-1, inputs.shape[-1]), block_size=block_size if grouped else None,
+            kernel=dict(kernel_packed=as_tensor(self._kernel),
+                        kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
+                        units=self._orig_output_dim,
+                        kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+                        bias=self._read_cached("bias", self.bias)),
+            finish=finish)
+
     # ---- serialization ---------------------------------------------------------------
     @property
     def variable_serialization_spec(self):

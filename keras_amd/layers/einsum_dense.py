@@ -507,6 +507,29 @@ class EinsumDense(Layer):
         )
         return self._finish(y2, free_shape, gv, fused)
 
+    def _int4_together_spec(self, inputs):
+        """As Dense._int4_together_spec, for equations whose input rows and stored kernel are
+        the GEMM's operands as they lie (e.g. "btd,dnh->btnh")."""
+        if (not self.built or self.quantization_mode != "int4" or self.inputs_quantizer
+                or self.lora_enabled or getattr(self, "_gemm", None) is None):
+            return None
+        gv = self._gemm_view()
+        if not (gv.k_plain and gv.in_is_view):
+            return None
+        cd = to_torch_dtype(self.compute_dtype)
+        block_size = self._int4_block_size
+        grouped = block_size is not None and block_size > 0
+        x2, free_shape = self._input_rows(inputs, gv)
+        bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
+        return dict(
+            x2=x2, block_size=block_size if grouped else None,
+            kernel=dict(kernel_packed=as_tensor(self._kernel),
+                        kernel_scale=self._cached("kernel_scale", self.kernel_scale,
+                                                  lambda t: t.to(cd).contiguous()),
+                        units=self._int4_unpacked_column_size,
+                        kernel_zero=as_tensor(self.kernel_zero) if grouped else None, bias=bias),
+            finish=lambda y2: self._finish(y2, free_shape, gv, fused))
+
     def _int4_dequantized_kernel(self, gv, cd, grouped):
         """The float kernel of einsum_dense.py:1143-1150 / :1213-1222 (unpack, divide by the
         scale | dequantize_with_sz_map, cast, reshape to the kernel's own shape), then laid

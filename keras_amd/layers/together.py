@@ -1,0 +1,50 @@
+"""Several layers on one input.
+
+A decode step calls the query, key and value projections of a block -- and the gate and up
+projections of its MLP -- on the same activations.  Each call is a few microseconds of launch
+and drain around a kernel that streams a few megabytes, so running them as one launch is worth
+more than any tuning of the kernel itself.  The reference has no such call (its layers each run
+their own `matmul`); this one returns exactly what the separate calls return.
+"""
+
+import numpy as np
+import torch
+
+from keras_amd import ops as kops
+from keras_amd.layers.layer import to_torch_dtype
+
+
+def call_together(layers, inputs):
+    """`[layer(inputs) for layer in layers]`.
+
+    Weight-only int4 `Dense` / `EinsumDense` layers with one compute dtype, input width and
+    group size go to `ops.int4_matmul_multi` (one launch at decode sizes); anything else is
+    called layer by layer.
+    """
+    layers = list(layers)
+    if len(layers) < 2:
+        return [layer(inputs) for layer in layers]
+    if not isinstance(inputs, torch.Tensor):
+        inputs = torch.as_tensor(np.asarray(inputs))
+    first = layers[0]
+    for layer in layers:
+        if not layer.built:
+            layer.build(tuple(inputs.shape))
+    if any(l.device != first.device or l.compute_dtype != first.compute_dtype for l in layers):
+        return [layer(inputs) for layer in layers]
+    x = inputs.to(first.device) if inputs.device != first.device else inputs
+    cd = to_torch_dtype(first.compute_dtype)
+    if x.dtype.is_floating_point and x.dtype != cd:
+        x = x.to(cd)
+    specs = []
+    for layer in layers:
+        make = getattr(layer, "_int4_together_spec", None)
+        spec = make(x) if make is not None else None
+        if spec is None:
+            return [layer(inputs) for layer in layers]
+        specs.append(spec)
+    x2 = specs[0]["x2"]
+    if any(s["x2"].shape != x2.shape or s["block_size"] != specs[0]["block_size"] for s in specs):
+        return [layer(inputs) for layer in layers]
+    outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])
+    return [s["finish"](y) for s, y in zip(specs, outs)]

@@ -104,6 +104,60 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
     return y.reshape(*lead, N)
 
 
+def int4_matmul_multi(x, kernels, block_size=None):
+    """`[x . W_i for W_i in kernels]` for int4 Dense kernels that share the input `x[..., K]`:
+    one launch when the calls are decode-sized and the kernels' launch plans agree (kernels of
+    one shape do), otherwise one launch each; the same bits as `int4_matmul` either way.
+
+    kernels: dicts with `kernel_packed` int8 [K, ceil(N/2)], `kernel_scale` ([N] or [G, N], in
+    x.dtype), `units` (N), and optionally `kernel_zero` int8 [G, N] (grouped) and `bias` [N].
+    Reference: each is keras/src/layers/core/dense.py:988-1095; calling several layers on one
+    input in one launch has no counterpart there.
+    """
+    grouped = block_size is not None and block_size > 0
+    code = _lib.dtype_code(x.dtype)
+    K = x.shape[-1]
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    lib = _lib.load()
+    problems = (_lib.GemvW4Problem * len(kernels))()
+    outs, keep = [], []
+    ws_bytes = cnt_bytes = 0
+    for i, k in enumerate(kernels):
+        kp, ks = k["kernel_packed"], k["kernel_scale"]
+        kz, bias = k.get("kernel_zero"), k.get("bias")
+        N = int(k["units"])
+        _lib.require_device(x, kp, ks, kz, bias)
+        if kp.dtype != torch.int8 or kp.shape[0] != K or kp.shape[1] != (N + 1) // 2:
+            raise ValueError("kernel must be int8 of shape [input_dim, ceil(units / 2)]")
+        if ks.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+            raise TypeError("kernel_scale and bias must be read in the input's dtype")
+        if grouped and kz is None:
+            raise ValueError("grouped int4 needs kernel_zero")
+        kp = kp if kp.is_contiguous() else kp.contiguous()
+        ks = ks if ks.is_contiguous() else ks.contiguous()
+        if kz is not None and not kz.is_contiguous():
+            kz = kz.contiguous()
+        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+        keep.append((kp, ks, kz, bias))
+        outs.append(y)
+        problems[i] = _lib.GemvW4Problem(
+            N, kp.data_ptr(), ks.data_ptr(), kz.data_ptr() if grouped else None,
+            bias.data_ptr() if bias is not None else None, y.data_ptr())
+        ws_bytes += (lib.k3q_gemv_w4_workspace_bytes(M, K, N) + 255) // 256 * 256
+        cnt_bytes += lib.k3q_gemv_w4_counters_bytes(N)
+    ws = _workspace(x.device, ws_bytes)
+    cnt = _arrival_counters(x.device, cnt_bytes)
+    rc = lib.k3q_gemv_w4_multi(_lib.ptr(x2), code, M, K, len(kernels), ctypes.byref(problems),
+                               int(block_size) if grouped else -1, _lib.ptr(ws), ws.numel(),
+                               _lib.ptr(cnt), cnt.numel(), _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemv_w4_multi")
+    return [y.reshape(*lead, y.shape[1]) for y in outs]
+
+
 GEMM_EXACT_EPILOGUE = 1
 # up to this many rows the int8 matmul streams the [K, N] kernel in place; above, the prepacked
 # copy on 128-row MFMA tiles (K split over workgroups while the tiles are few) is faster

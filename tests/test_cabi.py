@@ -58,6 +58,10 @@ def test_argument_validation_without_device():
     assert lib.k3q_gemv_w4_workspace_bytes(1, 8192, 8192) >= 8192 * 4
     assert lib.k3q_gemv_w4_fused(one, 0, 1, 0, 8, one, one, null, -1, null, one, null, 0, null, 0, null) == -2
     assert lib.k3q_gemv_w4_counters_bytes(8192) == 64 * 4 and lib.k3q_gemv_w4_counters_bytes(0) == 0
+    assert lib.k3q_gemv_w4_multi(one, 1, 1, 64, -1, one, -1, null, 0, null, 0, null) == -2
+    assert lib.k3q_gemv_w4_multi(one, 1, 1, 64, 2, null, -1, null, 0, null, 0, null) == -1
+    assert lib.k3q_gemv_w4_multi(one, 1, 1, 64, 0, null, -1, null, 0, null, 0, null) == 0
+    assert lib.k3q_gemv_w4_multi(one, 1, 1, 64, 17, one, -1, null, 0, null, 0, null) == -2
     assert lib.k3q_gemm_wbf16(one, 1, one, 3, 4, 8, 64, null, one, null, 0, null) == -2  # bf16 x takes parts == 1
     assert lib.k3q_gemm_wbf16(one, 0, one, 1, 4, 8, 64, null, one, null, 0, null) == -2  # f32 x takes parts 2 | 3
     assert lib.k3q_gemm_wbf16(one, 5, one, 1, 4, 8, 64, null, one, null, 0, null) == -4

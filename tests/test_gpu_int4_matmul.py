@@ -212,3 +212,39 @@ def test_int4_single_launch_split_repeated(dev):
             bad += (y1.view(torch.int16) != y2.view(torch.int16)).sum()
         assert int(bad) == 0
         assert int(counters.count_nonzero()) == 0
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 16, 40])
+@pytest.mark.parametrize("block_size", [None, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_int4_multi_matches_single_calls(dev, M, block_size, dtype):
+    # several kernels against one x in one launch.  The launch is planned for the kernels'
+    # combined width, so its K split (the order of the fp32 sums) differs from a single
+    # call's: equal to the summation order, i.e. far inside the float tolerance; groups that
+    # cannot share a launch (here: 40 rows) run one by one and return the same bits.
+    K = 2048
+    widths = [1024, 1024, 1024, 3072]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).to(dtype).to(dev)
+    kernels, singles = [], []
+    for i, N in enumerate(widths):
+        qk, bias = make_layer(K, N, block_size, 60 + i, i % 2 == 0)
+        grouped = block_size is not None
+        spec = dict(kernel_packed=qk["kernel"].to(dev), kernel_scale=qk["kernel_scale"].to(dtype).to(dev),
+                    units=N, kernel_zero=qk["kernel_zero"].to(dev) if grouped else None,
+                    bias=bias.to(dtype).to(dev) if bias is not None else None)
+        kernels.append(spec)
+        singles.append(kops.int4_matmul(x, spec["kernel_packed"], spec["kernel_scale"], N,
+                                        kernel_zero=spec["kernel_zero"], block_size=block_size,
+                                        bias=spec["bias"]))
+    for base, end in ((0, 3), (0, 4), (2, 4)):
+        first = None
+        for _ in range(2):
+            got = kops.int4_matmul_multi(x, kernels[base:end], block_size=block_size)
+            for j, y in enumerate(got):
+                if M > 32:
+                    assert torch.equal(y, singles[base + j])
+                else:
+                    assert max_rel_err(y, singles[base + j]) <= RTOL[dtype] / 2, (M, block_size, dtype, base + j)
+            if first is not None:  # repeatable: the arrival counters were left at zero
+                assert all(torch.equal(a, b) for a, b in zip(first, got))
+            first = got

@@ -398,3 +398,44 @@ def test_quantize_with_specific_equations(dev, mode, equation, output_shape, inp
     y_quantized = layer(x)
     mse = (y_float.float() - y_quantized.float()).pow(2).mean().item()
     assert mse < threshold
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 100])
+@pytest.mark.parametrize("block_size", [128, None])
+def test_call_together_matches_separate_calls(dev, rows, block_size):
+    # attention-style projections (EinsumDense) and MLP-style ones (Dense, one with a bias and
+    # an activation) on one input: call_together returns what the layers return one by one
+    g = torch.Generator().manual_seed(11)
+    init = lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d)
+    cfg = ka.Int4QuantizationConfig(block_size=block_size)
+    proj = [EinsumDense("btd,dnh->btnh", (None, 4, 64), dtype="mixed_bfloat16", device=dev,
+                        kernel_initializer=init) for _ in range(3)]
+    x = torch.randn((1, rows, 256), generator=g)
+    for layer in proj:
+        layer.build((1, rows, 256))
+        layer.quantize("int4", config=cfg)
+    want = [layer(x) for layer in proj]
+    got = ka.layers.call_together(proj, x)
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and a.dtype == b.dtype
+        assert max_rel_err(a, b) <= RTOL[torch.bfloat16] / 2  # another order of the fp32 sums
+    mlp = [Dense(512, use_bias=False, dtype="mixed_bfloat16", device=dev, kernel_initializer=init),
+           Dense(512, use_bias=True, activation="relu", dtype="mixed_bfloat16", device=dev,
+                 kernel_initializer=init)]
+    x2 = torch.randn((rows, 256), generator=g)
+    for layer in mlp:
+        layer.build((rows, 256))
+        layer.quantize("int4", config=cfg)
+    want = [layer(x2) for layer in mlp]
+    got = ka.layers.call_together(mlp, x2)
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and a.dtype == b.dtype
+        assert max_rel_err(a, b) <= RTOL[torch.bfloat16] / 2
+    # a layer that is not weight-only int4 sends the whole group down the one-by-one road
+    other = Dense(512, dtype="mixed_bfloat16", device=dev, kernel_initializer=init)
+    other.build((rows, 256))
+    other.quantize("int8")
+    want = [layer(x2) for layer in (mlp[0], other)]
+    got = ka.layers.call_together((mlp[0], other), x2)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
