@@ -248,3 +248,31 @@ def test_int4_multi_matches_single_calls(dev, M, block_size, dtype):
             if first is not None:  # repeatable: the arrival counters were left at zero
                 assert all(torch.equal(a, b) for a, b in zip(first, got))
             first = got
+
+
+@pytest.mark.parametrize("M", [65, 128, 300])
+@pytest.mark.parametrize("block_size", [None, 128])
+def test_int4_multi_prefill_sizes(dev, M, block_size):
+    # prefill-sized groups run one kernel after the other on the de-quantise + GEMM route
+    K = 1024
+    widths = [512, 512, 1536]
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).to(torch.bfloat16).to(dev)
+    kernels, singles = [], []
+    for i, N in enumerate(widths):
+        qk, _ = make_layer(K, N, block_size, 80 + i, False)
+        grouped = block_size is not None
+        spec = dict(kernel_packed=qk["kernel"].to(dev), kernel_scale=qk["kernel_scale"].to(torch.bfloat16).to(dev),
+                    units=N, kernel_zero=qk["kernel_zero"].to(dev) if grouped else None, bias=None)
+        kernels.append(spec)
+        singles.append(kops.int4_matmul(x, spec["kernel_packed"], spec["kernel_scale"], N,
+                                        kernel_zero=spec["kernel_zero"], block_size=block_size))
+        # and against the oracle, as for a single call
+        want = ref.dense_int4_call(x.cpu(), qk["kernel"], qk["kernel_scale"], N, kernel_zero=qk["kernel_zero"],
+                                   g_idx=qk["g_idx"], block_size=block_size, bias=None,
+                                   compute_dtype=torch.bfloat16)
+        assert max_rel_err(singles[-1], want) <= 1.5 * RTOL[torch.bfloat16]
+    for _ in range(2):
+        got = kops.int4_matmul_multi(x, kernels, block_size=block_size)
+        for j, y in enumerate(got):
+            assert y.shape == singles[j].shape
+            assert max_rel_err(y, singles[j]) <= RTOL[torch.bfloat16] / 2, (M, block_size, j)
