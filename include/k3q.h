@@ -226,6 +226,25 @@ int k3q_gemv_w4_fused(const void* x, int x_dtype, int64_t M, int64_t K, int64_t 
                       void* stream);
 
 /*
+ * Weight-only int4 matmul for 17 ... 512 bfloat16 rows from a K-contiguous copy of the kernel:
+ * the same result as k3q_gemv_w4 to the order of the fp32 sums, with the kernel read once as
+ * int4 (k3q_gemv_w4's route for these sizes writes it out as bfloat16 first: nine times the
+ * bytes at 128 rows).
+ * w_kmajor: int4 [N, K/2]; dword j of row n holds k = 8j ... 8j+7 of column n, the nibble of
+ * k = 8j + 2p at bits [4p, 4p+4) and of k = 8j + 2p + 1 at bits [16+4p, 16+4p+4), each the low
+ * four bits of the two's-complement value (keras_amd.ops.int4_kmajor_copy builds it from the
+ * stored kernel, once per layer).  scale, zero, block_size, bias, y as for k3q_gemv_w4.
+ * Needs K % 128 == 0, N % 32 == 0, K % block_size == 0 and block_size % 64 == 0 (K3Q_ERR_SHAPE
+ * otherwise); workspace: k3q_gemm_w4_kmajor_workspace_bytes bytes, 16-byte aligned.
+ * Replaces what k3q_gemv_w4 replaces (keras/src/layers/core/dense.py:988-1095).
+ */
+int64_t k3q_gemm_w4_kmajor_workspace_bytes(int64_t M, int64_t K, int64_t N, int64_t block_size);
+int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                       const void* w_kmajor, const void* scale, const void* zero, int64_t block_size,
+                       const void* bias, void* y, void* workspace, int64_t workspace_bytes,
+                       void* stream);
+
+/*
  * Several weight-only int4 matmuls against ONE x, each as k3q_gemv_w4_fused computes it (same
  * bits), in one launch when they are decode-sized (M <= 16) and their launch plans agree
  * (e.g. kernels of one shape: the query / key / value projections of an attention block, the

@@ -1143,6 +1143,284 @@ bool try_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t K, int cou
     return true;
 }
 
+// ---- 33 ... 256 rows from a K-contiguous copy of the int4 kernel --------------------------
+// The stored kernel has N contiguous, an MFMA operand wants K contiguous.  With a copy of the
+// kernel laid out [N, K/2] -- eight consecutive k of a column per dword, the even ones in the
+// low half-word's nibbles and the odd ones in the high half-word's -- a lane's 16-byte load IS
+// its operand of four MFMA steps: `(d >> 4p) & 0x000F000F` is the nibble pair (k = 2p, 2p + 1),
+// and `^ 0x00080008 | 0x43004300` turns it into the bfloat16 pair (136 + q).  Nothing is
+// de-quantised in memory; the kernel is read once, as int4.  The offset, the zero point and
+// the scale are taken out per group of K with the sums of x over that group, as the decode
+// kernel does: tot += scale * (acc - (136 + zero) * sum_k x).
+constexpr int kKmBM = 128, kKmBN = 256, kKmStage = 64;  // tile; values of K per stage
+constexpr int kKmThreads = 512;                        // 8 waves: 2 (M) x 4 (N), 64 x 64 each
+constexpr u32 kKmNibbles = 0x000F000Fu, kKmFlip = 0x00080008u, kKmExp = 0x43004300u;
+
+__device__ __forceinline__ int km_swz(int row) { return (row & 6) | ((row ^ (row >> 3)) & 1); }
+
+struct KmParams {
+    const uint16_t* x;      // [M, K] bf16
+    const uint8_t* shadow;  // [N, K/2]
+    const void* scale;      // bf16 [G, N] (grouped) or unused
+    const int8_t* zero;     // [G, N] (grouped)
+    const float* sx;        // [K / gsize, M] sums of x over each group of K
+    float* part;            // [KS, M, N]
+    int64_t M, N, K;
+    int gsize;              // values of K per group (multiple of kKmStage)
+    int klen;               // values of K per split (multiple of gsize)
+};
+
+// sx[g][m] = sum of x[m, g*gsize .. (g+1)*gsize): one wave per (g, m), fixed order
+__global__ __launch_bounds__(256) void km_group_sums(const uint16_t* __restrict__ x, float* __restrict__ sx,
+                                                     int64_t M, int64_t K, int gsize) {
+    const int lane = threadIdx.x & 63;
+    const int64_t m = (int64_t)blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int64_t g = blockIdx.x;
+    if (m >= M) return;
+    const uint16_t* row = x + m * K + g * gsize;
+    float sum = 0.f;
+    for (int k = lane * 2; k < gsize; k += 128) {
+        const u32 d = *(const u32*)(row + k);
+        sum += bf16_bits_to_f32(d & 0xffffu) + bf16_bits_to_f32(d >> 16);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0) sx[g * M + m] = sum;
+}
+
+// gfx9 s_waitcnt immediate for "at most n vector-memory operations outstanding"
+constexpr int km_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+
+// Everything the loop consumes arrives by LDS-DMA (global_load_lds), nothing through
+// registers: the compiler then places no waits of its own in the loop (a register load there
+// made it wait for every outstanding operation at each use, which serialised the pipeline:
+// 3 us per stage), and the one s_waitcnt per stage is written by hand.
+// kDepth: stages in flight or in use.  Per stage a slot holds the x tile (128 rows x 128 B,
+// chunk-swizzled), the kernel rows (256 rows x 32 B) and the group's parameters (256 scales,
+// 256 zero points, 128 sums of x); every wave issues four DMA instructions per stage.
+constexpr int kKmXBytes = kKmBM * 128, kKmWBytes = kKmBN * 32, kKmParBytes = 2048;
+constexpr int kKmSlotBytes = kKmXBytes + kKmWBytes + kKmParBytes;
+constexpr int kKmParScale = 0, kKmParZero = 512, kKmParSx = 768, kKmParSpare = 1280;
+
+template <bool kGrouped, int kDepth>
+__global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
+    extern __shared__ char km_lds[];
+    constexpr int kOpsPerStage = 4;  // DMA instructions a wave issues per stage
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 2, wn = wave & 3;
+    const int i = lane & 31, g = lane >> 5;
+    const int64_t n0 = (int64_t)blockIdx.x * kKmBN, m0 = (int64_t)blockIdx.y * kKmBM;
+    const int64_t k_begin = (int64_t)blockIdx.z * p.klen;
+    const int64_t k_end = k_begin + p.klen < p.K ? k_begin + p.klen : p.K;
+    const int stages = (int)((k_end - k_begin) / kKmStage);
+
+    // x tile: instruction d of a stage fills LDS bytes [d * 1024, +1024) = 8 rows, the lane's
+    // 16 bytes at lane * 16; the chunk swizzle is applied on the source side.  A wave issues
+    // instructions 2 * wave and 2 * wave + 1.
+    const char* a_src[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int row = (2 * wave + j) * 8 + (lane >> 3);
+        const int ch = (lane & 7) ^ km_swz(row);
+        int64_t grow = m0 + row;
+        if (grow >= p.M) grow = p.M - 1;
+        a_src[j] = (const char*)(p.x + grow * p.K + k_begin) + ch * 16;
+    }
+    // kernel rows: one instruction per wave and stage = 32 rows x 32 bytes, two lanes per row
+    const char* w_src;
+    {
+        int64_t n = n0 + wave * 32 + (lane >> 1);
+        if (n >= p.N) n = p.N - 1;
+        w_src = (const char*)p.shadow + n * (p.K / 2) + k_begin / 2 + (lane & 1) * 16;
+    }
+    // group parameters, four bytes per lane: waves 0, 1 the scales, wave 2 the zero points,
+    // waves 3, 4 the sums of x; the others fetch a spare copy so that every wave counts alike
+    const char* par_base;
+    int64_t par_step;   // bytes from one group to the next
+    int par_dst;
+    {
+        const int w = wave;
+        if (kGrouped && w < 2) {
+            int64_t n = n0 + w * 128 + lane * 2;
+            if (n > p.N - 2) n = p.N - 2;
+            par_base = (const char*)p.scale + n * 2;
+            par_step = p.N * 2;
+            par_dst = kKmParScale + w * 256;
+        } else if (kGrouped && w == 2) {
+            int64_t n = n0 + lane * 4;
+            if (n > p.N - 4) n = p.N - 4;
+            par_base = (const char*)p.zero + n;
+            par_step = p.N;
+            par_dst = kKmParZero;
+        } else {
+            const int h = (w == 3 || w == 4) ? w - 3 : 0;
+            int64_t m = m0 + h * 64 + lane;
+            if (m >= p.M) m = p.M - 1;
+            par_base = (const char*)(p.sx + m);
+            par_step = p.M * 4;
+            par_dst = (w == 3 || w == 4) ? kKmParSx + h * 256 : kKmParSpare + (w > 4 ? w - 5 : w) * 256;
+        }
+    }
+    int a_row[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) a_row[mb] = wm * 64 + mb * 32 + i;
+
+    v16f acc[2][2], tot[2][2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[nb][mb][r] = tot[nb][mb][r] = 0.f;
+
+    auto issue = [&](int st, int slot) {
+        char* base = km_lds + slot * kKmSlotBytes;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(a_src[j] + (int64_t)st * 128),
+                (__attribute__((address_space(3))) void*)(base + (2 * wave + j) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(w_src + (int64_t)st * 32),
+            (__attribute__((address_space(3))) void*)(base + kKmXBytes + wave * 1024), 16, 0, 0);
+        const int64_t gi = (k_begin + (int64_t)st * kKmStage) / p.gsize;
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(par_base + gi * par_step),
+            (__attribute__((address_space(3))) void*)(base + kKmXBytes + kKmWBytes + par_dst), 4, 0, 0);
+    };
+#pragma unroll
+    for (int d = 0; d < kDepth - 1; ++d)
+        if (d < stages) issue(d, d);
+
+    const int group_stages = p.gsize / kKmStage;
+    for (int st0 = 0; st0 < stages; st0 += kDepth) {
+#pragma unroll
+        for (int u = 0; u < kDepth; ++u) {
+            const int st = st0 + u;
+            if (st >= stages) break;
+            // stage st has landed once at most the operations of the stages issued after it are
+            // outstanding; near the end fewer were issued: wait for everything
+            if (st + kDepth - 2 < stages)
+                __builtin_amdgcn_s_waitcnt(km_vmcnt(kOpsPerStage * (kDepth - 2)));
+            else
+                __builtin_amdgcn_s_waitcnt(km_vmcnt(0));
+            // s_barrier without a fence (a fence would drain the DMA of the stages in flight):
+            // every wave's part of the slot is there; slot u - 1 is free
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (st + kDepth - 1 < stages) issue(st + kDepth - 1, (u + kDepth - 1) % kDepth);
+            const char* cur = km_lds + u * kKmSlotBytes;
+            v4u wq[2];  // this lane's 32 values of K of its two kernel rows: chunk 4g + s at step s
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+                wq[nb] = *(const v4u*)(cur + kKmXBytes + (wn * 64 + nb * 32 + i) * 32 + g * 16);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                v4u xa[2], wb[2];
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+                    xa[mb] = *(const v4u*)(cur + a_row[mb] * 128 + (((4 * g + s) ^ km_swz(a_row[mb])) << 4));
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    const u32 d = wq[nb][s];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) wb[nb][q] = (((d >> (4 * q)) & kKmNibbles) ^ kKmFlip) | kKmExp;
+                }
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                    for (int mb = 0; mb < 2; ++mb)
+                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf(wb[nb]), as_bf(xa[mb]),
+                                                                              acc[nb][mb], 0, 0, 0);
+            }
+            // end of a group of K (or of this split): fold offset, zero point and scale
+            if (((st + 1) % group_stages) == 0 || st + 1 == stages) {
+                const char* par = cur + kKmXBytes + kKmWBytes;
+                float sxv[2];
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) sxv[mb] = *(const float*)(par + kKmParSx + a_row[mb] * 4);
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        float sc[4] = {1.f, 1.f, 1.f, 1.f}, off[4] = {kOffset, kOffset, kOffset, kOffset};
+                        if (kGrouped) {
+                            const int nl = wn * 64 + nb * 32 + 8 * rg + 4 * g;
+                            const v2u sraw = *(const v2u*)(par + kKmParScale + nl * 2);
+                            const u32 zraw = *(const u32*)(par + kKmParZero + nl);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const u32 w = sraw[e >> 1];
+                                sc[e] = __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
+                                off[e] = kOffset + (float)(int)(int8_t)(zraw >> (8 * e));
+                            }
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+#pragma unroll
+                            for (int mb = 0; mb < 2; ++mb) {
+                                const int r = 4 * rg + e;
+                                const float t = __builtin_fmaf(-off[e], sxv[mb], acc[nb][mb][r]);
+                                tot[nb][mb][r] = __builtin_fmaf(sc[e], t, tot[nb][mb][r]);
+                                acc[nb][mb][r] = 0.f;
+                            }
+                    }
+                }
+            }
+        }
+    }
+
+    // raw sums of this split; gemv_w4_reduce adds the splits and applies the epilogue
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        const int64_t m = m0 + a_row[mb];
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            if (n0 + wn * 64 + nb * 32 >= p.N) continue;  // N % 32 == 0: a block is in or out as a whole
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const int64_t n = n0 + wn * 64 + nb * 32 + 8 * rg + 4 * g;
+                v4f o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = tot[nb][mb][4 * rg + e];
+                *(v4f*)(p.part + ((int64_t)blockIdx.z * p.M + m) * p.N + n) = o;
+            }
+        }
+    }
+}
+
+// shapes and sizes the K-contiguous route takes
+inline bool kmajor_ok(int64_t M, int64_t K, int64_t N, int64_t block_size) {
+    const int64_t gsize = block_size > 0 ? block_size : 128;
+    return M >= 17 && M <= 512 && (K % 128) == 0 && (N % 32) == 0 && (gsize % kKmStage) == 0 &&
+           (K % gsize) == 0;
+}
+
+struct KmPlan {
+    int ks;
+    int64_t klen;
+};
+
+inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
+    const int64_t tiles = ((M + kKmBM - 1) / kKmBM) * ((N + kKmBN - 1) / kKmBN);
+    // about one workgroup per CU, at most eight splits (every split writes and the reduction
+    // reads M x N floats: at 128 rows one split of a 4096 x 14336 kernel is a quarter of the
+    // kernel's own bytes), at least eight stages per split
+    int64_t ks = (kTargetWorkgroups + tiles - 1) / tiles;
+    if (ks > 8) ks = 8;
+    const int64_t unit = gsize > 2 * kKmStage ? gsize : 2 * kKmStage;  // a split is whole groups
+    int64_t klen = (K / ks + unit - 1) / unit * unit;
+    if (klen < 8 * kKmStage) klen = (8 * kKmStage + unit - 1) / unit * unit;
+    if (klen > K) klen = K;
+    KmPlan pl;
+    pl.klen = klen;
+    pl.ks = (int)((K + klen - 1) / klen);
+    return pl;
+}
+
 }  // namespace
 
 void split_f32_rows_launch(const float* x, uint16_t* out, int64_t M, int64_t K, int parts,
@@ -1252,4 +1530,80 @@ extern "C" int k3q_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t 
         if (rc != K3Q_OK) return rc;
     }
     return K3Q_OK;
+}
+
+extern "C" int64_t k3q_gemm_w4_kmajor_workspace_bytes(int64_t M, int64_t K, int64_t N, int64_t block_size) {
+    if (!kmajor_ok(M, K, N, block_size)) return 0;
+    const int64_t gsize = block_size > 0 ? block_size : 128;
+    const KmPlan pl = kmajor_plan(M, K, N, gsize);
+    return ((K / gsize) * M * 4 + 255) / 256 * 256 + (int64_t)pl.ks * M * N * 4;
+}
+
+extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                  const void* w_kmajor, const void* scale, const void* zero,
+                                  int64_t block_size, const void* bias, void* y, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+    if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (!x || !w_kmajor || !scale || !y) return K3Q_ERR_NULL;
+    const bool grouped = block_size > 0;
+    if (grouped && !zero) return K3Q_ERR_NULL;
+    if (!kmajor_ok(M, K, N, block_size)) return K3Q_ERR_SHAPE;
+    if (!aligned_to(x, 16) || !aligned_to(w_kmajor, 16) || !aligned_to(scale, 8) ||
+        (zero && !aligned_to(zero, 4)) || !aligned_to(y, 8) || (bias && !aligned_to(bias, 2)))
+        return K3Q_ERR_ALIGN;
+    const int64_t need = k3q_gemm_w4_kmajor_workspace_bytes(M, K, N, block_size);
+    if (!workspace || workspace_bytes < need) return K3Q_ERR_WORKSPACE;
+    if (!aligned_to(workspace, 16)) return K3Q_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    int64_t gsize = grouped ? block_size : 128;
+    const KmPlan pl = kmajor_plan(M, K, N, gsize);
+    // per-channel kernels need the offset taken out only once per split
+    if (!grouped && (K % pl.klen) == 0) gsize = pl.klen;
+    float* sx = (float*)workspace;
+    float* part = (float*)((char*)workspace + ((K / gsize) * M * 4 + 255) / 256 * 256);
+    km_group_sums<<<dim3((unsigned)(K / gsize), (unsigned)((M + 3) / 4)), 256, 0, s>>>(
+        (const uint16_t*)x, sx, M, K, (int)gsize);
+    KmParams kp{};
+    kp.x = (const uint16_t*)x;
+    kp.shadow = (const uint8_t*)w_kmajor;
+    kp.scale = scale;
+    kp.zero = (const int8_t*)zero;
+    kp.sx = sx;
+    kp.part = part;
+    kp.M = M;
+    kp.N = N;
+    kp.K = K;
+    kp.gsize = (int)gsize;
+    kp.klen = (int)pl.klen;
+    dim3 grid((unsigned)((N + kKmBN - 1) / kKmBN), (unsigned)((M + kKmBM - 1) / kKmBM), (unsigned)pl.ks);
+    constexpr int kDepth = 4;
+    const size_t lds = (size_t)kDepth * kKmSlotBytes;
+    static const bool raised = [] {
+        bool ok = hipFuncSetAttribute((const void*)gemm_w4_kmajor<true, kDepth>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget) == hipSuccess;
+        return hipFuncSetAttribute((const void*)gemm_w4_kmajor<false, kDepth>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget) == hipSuccess && ok;
+    }();
+    (void)raised;
+    if (grouped)
+        gemm_w4_kmajor<true, kDepth><<<grid, kKmThreads, lds, s>>>(kp);
+    else
+        gemm_w4_kmajor<false, kDepth><<<grid, kKmThreads, lds, s>>>(kp);
+    // the decode kernel's second pass: sums the splits in order, applies scale and bias
+    GemvParams gp{};
+    gp.scale = scale;
+    gp.bias = bias;
+    gp.y = y;
+    gp.part = part;
+    gp.N = N;
+    gp.M = (int)M;
+    gp.m0 = 0;
+    dim3 rgrid((unsigned)((N / 4 + 255) / 256), (unsigned)M);
+    if (grouped)
+        gemv_w4_reduce<true, true><<<rgrid, 256, 0, s>>>(gp, pl.ks);
+    else
+        gemv_w4_reduce<true, false><<<rgrid, 256, 0, s>>>(gp, pl.ks);
+    return launch_status();
 }

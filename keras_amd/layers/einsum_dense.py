@@ -497,10 +497,23 @@ class EinsumDense(Layer):
                                           lambda t: t.to(cd).reshape(-1).contiguous()),
                 bias=bias, out_dtype=cd, exact_epilogue=True)
             return self._finish(y2, free_shape, gv, fused)
+        from keras_amd.layers.dense import KMAJOR_MAX_ROWS, KMAJOR_MIN_ROWS
+
+        units = self._int4_unpacked_column_size
+        if (x2.dtype == torch.bfloat16 and KMAJOR_MIN_ROWS <= x2.shape[0] <= KMAJOR_MAX_ROWS
+                and kops.int4_kmajor_supported(x2.shape[0], x2.shape[1], units,
+                                               block_size if grouped else None)):
+            # as Dense: from the K-contiguous copy of the kernel, read once as int4
+            y2 = kops.int4_matmul_kmajor(
+                x2, self._cached("kmajor", self._kernel, lambda t: kops.int4_kmajor_copy(t, units)),
+                self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).contiguous()),
+                kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+                block_size=block_size if grouped else None, bias=bias)
+            return self._finish(y2, free_shape, gv, fused)
         y2 = kops.int4_matmul(
             x2, as_tensor(self._kernel),
             self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).contiguous()),
-            self._int4_unpacked_column_size,
+            units,
             kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
             block_size=block_size if grouped else None,
             bias=bias,

@@ -44,6 +44,9 @@ def call_together(layers, inputs):
             return [layer(inputs) for layer in layers]
         specs.append(spec)
     x2 = specs[0]["x2"]
+    if x2.shape[0] > 16:
+        # beyond decode sizes nothing is shared: every layer takes its own route for the size
+        return [layer(inputs) for layer in layers]
     if any(s["x2"].shape != x2.shape or s["block_size"] != specs[0]["block_size"] for s in specs):
         return [layer(inputs) for layer in layers]
     outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])

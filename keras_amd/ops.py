@@ -158,6 +158,63 @@ def int4_matmul_multi(x, kernels, block_size=None):
     return [y.reshape(*lead, y.shape[1]) for y in outs]
 
 
+def int4_kmajor_copy(kernel_packed, units):
+    """The K-contiguous copy `int4_matmul_kmajor` reads: int32 [N, K/8], eight consecutive k of
+    a column per dword, even k in the low half-word's nibbles, odd k in the high half-word's
+    (include/k3q.h, k3q_gemm_w4_kmajor).  Made once per layer from the stored
+    `[K, ceil(N/2)]` kernel; K % 8 == 0."""
+    from keras_amd import quantizers
+
+    q = quantizers.unpack_int4(kernel_packed, int(units), axis=-1)      # int8 [K, N]
+    K, N = q.shape
+    if K % 8:
+        raise ValueError("the K-contiguous copy needs K % 8 == 0")
+    u = (q.t().contiguous().to(torch.int64) & 0xF).reshape(N, K // 8, 8)
+    d = torch.zeros((N, K // 8), dtype=torch.int64, device=q.device)
+    for p in range(4):
+        d |= u[..., 2 * p] << (4 * p)
+        d |= u[..., 2 * p + 1] << (16 + 4 * p)
+    d = torch.where(d >= 1 << 31, d - (1 << 32), d)   # as two's-complement int32
+    return d.to(torch.int32).contiguous()
+
+
+def int4_kmajor_supported(M, K, N, block_size=None):
+    lib = _lib.load()
+    bs = int(block_size) if block_size is not None and block_size > 0 else -1
+    return lib.k3q_gemm_w4_kmajor_workspace_bytes(M, K, N, bs) > 0
+
+
+def int4_matmul_kmajor(x, kernel_kmajor, kernel_scale, kernel_zero=None, block_size=None, bias=None):
+    """`x[..., K] . W4` for 17 ... 512 bfloat16 rows from `int4_kmajor_copy(kernel)`; the kernel
+    is read once, as int4.  Reference: keras/src/layers/core/dense.py:988-1095."""
+    _lib.require_device(x, kernel_kmajor, kernel_scale, kernel_zero, bias)
+    if x.dtype != torch.bfloat16 or kernel_scale.dtype != torch.bfloat16:
+        raise TypeError("the K-contiguous route computes in bfloat16")
+    grouped = block_size is not None and block_size > 0
+    N, K8 = kernel_kmajor.shape
+    K = K8 * 8
+    if x.shape[-1] != K:
+        raise ValueError(f"last axis of the input ({x.shape[-1]}) does not match the kernel's input dim ({K})")
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    bs = int(block_size) if grouped else -1
+    nbytes = lib.k3q_gemm_w4_kmajor_workspace_bytes(M, K, N, bs)
+    if nbytes <= 0:
+        raise ValueError(f"the K-contiguous route does not take M={M}, K={K}, N={N}, block_size={block_size}")
+    ws = _workspace(x.device, nbytes)
+    ks = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
+    rc = lib.k3q_gemm_w4_kmajor(_lib.ptr(x2), _lib.dtype_code(x.dtype), M, K, N, _lib.ptr(kernel_kmajor),
+                                _lib.ptr(ks), _lib.ptr(kernel_zero) if grouped else None, bs,
+                                _lib.ptr(bias), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
+                                _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemm_w4_kmajor")
+    return y.reshape(*lead, N)
+
+
 GEMM_EXACT_EPILOGUE = 1
 # up to this many rows the int8 matmul streams the [K, N] kernel in place; above, the prepacked
 # copy on 128-row MFMA tiles (K split over workgroups while the tiles are few) is faster

@@ -276,3 +276,39 @@ def test_int4_multi_prefill_sizes(dev, M, block_size):
         for j, y in enumerate(got):
             assert y.shape == singles[j].shape
             assert max_rel_err(y, singles[j]) <= RTOL[torch.bfloat16] / 2, (M, block_size, j)
+
+
+@pytest.mark.parametrize("M,K,N,block_size", [
+    (17, 128, 32, None), (33, 256, 64, 128), (64, 512, 256, 64), (128, 1024, 512, 128),
+    (130, 2048, 1056, 128), (200, 1024, 288, None), (256, 4096, 4096, 128), (512, 1024, 1024, 256),
+    (100, 4096, 1024, None),
+])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_int4_kmajor_route(dev, M, K, N, block_size, with_bias):
+    # 17 ... 512 bfloat16 rows from the K-contiguous copy of the kernel: against the oracle, the
+    # float64 value, and the other route's result
+    qk, bias = make_layer(K, N, block_size, 90, with_bias)
+    g = torch.Generator().manual_seed(91)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    grouped = block_size is not None
+    dt = torch.bfloat16
+    want = ref.dense_int4_call(x, qk["kernel"], qk["kernel_scale"], N, kernel_zero=qk["kernel_zero"],
+                               g_idx=qk["g_idx"], block_size=block_size, bias=bias, compute_dtype=dt)
+    scale_t = qk["kernel_scale"].to(dt)
+    bias_t = bias.to(dt) if bias is not None else None
+    kernel = qk["kernel"].to(dev)
+    shadow = kops.int4_kmajor_copy(kernel, N)
+    assert shadow.dtype == torch.int32 and tuple(shadow.shape) == (N, K // 8)
+    got = kops.int4_matmul_kmajor(x.to(dev), shadow, scale_t.to(dev),
+                                  kernel_zero=qk["kernel_zero"].to(dev) if grouped else None,
+                                  block_size=block_size, bias=bias_t.to(dev) if with_bias else None)
+    assert got.dtype == dt and tuple(got.shape) == (M, N)
+    exact = c_w4_matmul_f64(x, qk["kernel"], scale_t, qk["kernel_zero"], block_size, bias_t, N)
+    e_ref, e_exact, e_ref_exact = max_rel_err(got, want), max_rel_err(got, exact), max_rel_err(want, exact)
+    tol = RTOL[dt]
+    assert e_ref <= tol or (e_ref <= 1.5 * tol and e_exact <= e_ref_exact), (e_ref, e_exact, e_ref_exact)
+    assert e_exact <= max(2.0 * e_ref_exact, tol / 4), (e_exact, e_ref_exact)
+    other = kops.int4_matmul(x.to(dev), kernel, scale_t.to(dev), N,
+                             kernel_zero=qk["kernel_zero"].to(dev) if grouped else None,
+                             block_size=block_size, bias=bias_t.to(dev) if with_bias else None)
+    assert max_rel_err(got, other) <= 1.5 * tol
