@@ -1274,26 +1274,38 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[nb][mb][r] = tot[nb][mb][r] = 0.f;
 
-    auto issue = [&](int st, int slot) {
+    // stages are issued in order, one after the other: the sources advance by a stage each time
+    // and the parameter source by a group every `group_stages` stages (no per-stage address
+    // arithmetic: a 64-bit division per stage cost more scalar instructions than the MFMAs)
+    const int group_stages = p.gsize / kKmStage;
+    const char* par_src = par_base + (k_begin / p.gsize) * par_step;
+    int issued_in_group = 0;
+    auto issue = [&](int slot) {
         char* base = km_lds + slot * kKmSlotBytes;
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j) {
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(a_src[j] + (int64_t)st * 128),
+                (const __attribute__((address_space(1))) void*)a_src[j],
                 (__attribute__((address_space(3))) void*)(base + (2 * wave + j) * 1024), 16, 0, 0);
+            a_src[j] += 128;
+        }
         __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(w_src + (int64_t)st * 32),
+            (const __attribute__((address_space(1))) void*)w_src,
             (__attribute__((address_space(3))) void*)(base + kKmXBytes + wave * 1024), 16, 0, 0);
-        const int64_t gi = (k_begin + (int64_t)st * kKmStage) / p.gsize;
+        w_src += 32;
         __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(par_base + gi * par_step),
+            (const __attribute__((address_space(1))) void*)par_src,
             (__attribute__((address_space(3))) void*)(base + kKmXBytes + kKmWBytes + par_dst), 4, 0, 0);
+        if (++issued_in_group == group_stages) {
+            issued_in_group = 0;
+            par_src += par_step;
+        }
     };
 #pragma unroll
     for (int d = 0; d < kDepth - 1; ++d)
-        if (d < stages) issue(d, d);
+        if (d < stages) issue(d);
 
-    const int group_stages = p.gsize / kKmStage;
+    int done_in_group = 0;
     for (int st0 = 0; st0 < stages; st0 += kDepth) {
 #pragma unroll
         for (int u = 0; u < kDepth; ++u) {
@@ -1310,7 +1322,7 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (st + kDepth - 1 < stages) issue(st + kDepth - 1, (u + kDepth - 1) % kDepth);
+            if (st + kDepth - 1 < stages) issue((u + kDepth - 1) % kDepth);
             const char* cur = km_lds + u * kKmSlotBytes;
             v4u wq[2];  // this lane's 32 values of K of its two kernel rows: chunk 4g + s at step s
 #pragma unroll
@@ -1336,7 +1348,8 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
                                                                               acc[nb][mb], 0, 0, 0);
             }
             // end of a group of K (or of this split): fold offset, zero point and scale
-            if (((st + 1) % group_stages) == 0 || st + 1 == stages) {
+            if (++done_in_group == group_stages || st + 1 == stages) {
+                done_in_group = 0;
                 const char* par = cur + kKmXBytes + kKmWBytes;
                 float sxv[2];
 #pragma unroll
@@ -1409,7 +1422,9 @@ inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
     // about one workgroup per CU, at most eight splits (every split writes and the reduction
     // reads M x N floats: at 128 rows one split of a 4096 x 14336 kernel is a quarter of the
     // kernel's own bytes), at least eight stages per split
-    int64_t ks = (kTargetWorkgroups + tiles - 1) / tiles;
+    // (one workgroup fits a CU: the launch must not spill into a second round)
+    int64_t ks = kTargetWorkgroups / tiles;
+    if (ks < 1) ks = 1;
     if (ks > 8) ks = 8;
     const int64_t unit = gsize > 2 * kKmStage ? gsize : 2 * kKmStage;  // a split is whole groups
     int64_t klen = (K / ks + unit - 1) / unit * unit;
@@ -1418,7 +1433,7 @@ inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
     KmPlan pl;
     pl.klen = klen;
     pl.ks = (int)((K + klen - 1) / klen);
-    return pl;
+    return pl;  // rounding klen up can only lower the split count
 }
 
 }  // namespace

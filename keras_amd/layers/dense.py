@@ -60,9 +60,10 @@ def glorot_uniform(shape, dtype, generator=None):
 
 
 # rows for which the int4 forward reads the K-contiguous copy of the kernel (measured against
-# the 32-row passes below and the de-quantise + GEMM route above: K=4096, N=14336, groups of
-# 128: 64 rows 41 against 60 us, 128 rows 49 against 65 us, 256 rows 87 against 81 us)
-KMAJOR_MIN_ROWS, KMAJOR_MAX_ROWS = 33, 128
+# the 32-row passes below it and the de-quantise + GEMM route above it, groups of 128, us:
+# K=4096, N=14336: 64 rows 37 against 60, 128 rows 44 against 66, 256 rows 67 against 81,
+# 512 rows 114 against 97; K=N=4096: 64 rows 24 against 32, 128 rows 31 against 30)
+KMAJOR_MIN_ROWS, KMAJOR_MAX_ROWS = 33, 256
 
 
 class Dense(Layer):
