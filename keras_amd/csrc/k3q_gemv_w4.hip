@@ -1163,15 +1163,17 @@ struct KmParams {
     const uint8_t* shadow;  // [N, K/2]
     const void* scale;      // bf16 [G, N] (grouped) or unused
     const int8_t* zero;     // [G, N] (grouped)
-    const float* sx;        // [K / gsize, M] sums of x over each group of K
+    const v2u* sx;          // [K / gsize, M] sums of x over each group of K, as three bfloat16 parts
     float* part;            // [KS, M, N]
     int64_t M, N, K;
     int gsize;              // values of K per group (multiple of kKmStage)
     int klen;               // values of K per split (multiple of gsize)
 };
 
-// sx[g][m] = sum of x[m, g*gsize .. (g+1)*gsize): one wave per (g, m), fixed order
-__global__ __launch_bounds__(256) void km_group_sums(const uint16_t* __restrict__ x, float* __restrict__ sx,
+// sx[g][m] = sum of x[m, g*gsize .. (g+1)*gsize): one wave per (g, m), fixed order.  Stored as
+// three bfloat16 parts {hi, lo, lolo, 0} whose sum is the float32 sum (each part rounds what the
+// ones before left over), so that an MFMA step can multiply it by a kernel-side constant
+__global__ __launch_bounds__(256) void km_group_sums(const uint16_t* __restrict__ x, v2u* __restrict__ sx,
                                                      int64_t M, int64_t K, int gsize) {
     const int lane = threadIdx.x & 63;
     const int64_t m = (int64_t)blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -1185,7 +1187,16 @@ __global__ __launch_bounds__(256) void km_group_sums(const uint16_t* __restrict_
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    if (lane == 0) sx[g * M + m] = sum;
+    if (lane == 0) {
+        const u32 hi = f32_to_bf16_bits(sum);
+        const float r1 = sum - bf16_bits_to_f32(hi);
+        const u32 lo = f32_to_bf16_bits(r1);
+        const u32 lolo = f32_to_bf16_bits(r1 - bf16_bits_to_f32(lo));
+        v2u o;
+        o[0] = hi | (lo << 16);
+        o[1] = lolo;
+        sx[g * M + m] = o;
+    }
 }
 
 // gfx9 s_waitcnt immediate for "at most n vector-memory operations outstanding"
@@ -1197,12 +1208,15 @@ constexpr int km_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 // 3 us per stage), and the one s_waitcnt per stage is written by hand.
 // kDepth: stages in flight or in use.  Per stage a slot holds the x tile (128 rows x 128 B,
 // chunk-swizzled), the kernel rows (256 rows x 32 B) and the group's parameters (256 scales,
-// 256 zero points, 128 sums of x); every wave issues four DMA instructions per stage.
+// 256 zero points, 128 sums of x of 8 bytes); every wave issues four DMA instructions per stage.
 constexpr int kKmXBytes = kKmBM * 128, kKmWBytes = kKmBN * 32, kKmParBytes = 2048;
 constexpr int kKmSlotBytes = kKmXBytes + kKmWBytes + kKmParBytes;
-constexpr int kKmParScale = 0, kKmParZero = 512, kKmParSx = 768, kKmParSpare = 1280;
+constexpr int kKmParScale = 0, kKmParZero = 512, kKmParSx = 768, kKmParSpare = 1792;
 
-template <bool kGrouped, int kDepth>
+// kGroupStages: stages per group of K when that is 1, 2 or 4 (groups of 64, 128, 256), else 0.
+// Known at compile time, the first MFMAs of a group take a zero accumulator operand and the
+// 64 accumulators are never cleared; with 0 the group ends are found at run time.
+template <bool kGrouped, int kDepth, int kGroupStages>
 __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
     extern __shared__ char km_lds[];
     constexpr int kOpsPerStage = 4;  // DMA instructions a wave issues per stage
@@ -1235,7 +1249,8 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
         w_src = (const char*)p.shadow + n * (p.K / 2) + k_begin / 2 + (lane & 1) * 16;
     }
     // group parameters, four bytes per lane: waves 0, 1 the scales, wave 2 the zero points,
-    // waves 3, 4 the sums of x; the others fetch a spare copy so that every wave counts alike
+    // waves 3 ... 6 the sums of x (two dwords per row); the last fetches a spare copy so that
+    // every wave counts alike (per-channel kernels: waves 0 ... 2 as well)
     const char* par_base;
     int64_t par_step;   // bytes from one group to the next
     int par_dst;
@@ -1254,12 +1269,13 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
             par_step = p.N;
             par_dst = kKmParZero;
         } else {
-            const int h = (w == 3 || w == 4) ? w - 3 : 0;
-            int64_t m = m0 + h * 64 + lane;
+            const bool sums = w >= 3 && w <= 6;
+            const int dw = sums ? (w - 3) * 64 + lane : lane;  // dword of the tile's 128 x 2
+            int64_t m = m0 + (dw >> 1);
             if (m >= p.M) m = p.M - 1;
-            par_base = (const char*)(p.sx + m);
-            par_step = p.M * 4;
-            par_dst = (w == 3 || w == 4) ? kKmParSx + h * 256 : kKmParSpare + (w > 4 ? w - 5 : w) * 256;
+            par_base = (const char*)(p.sx + m) + (dw & 1) * 4;
+            par_step = p.M * 8;
+            par_dst = sums ? kKmParSx + (w - 3) * 256 : (w == 7 ? kKmParSpare : w * 256);
         }
     }
     int a_row[2];
@@ -1273,6 +1289,9 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[nb][mb][r] = tot[nb][mb][r] = 0.f;
+    v16f zero16;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
 
     // stages are issued in order, one after the other: the sources advance by a stage each time
     // and the parameter source by a group every `group_stages` stages (no per-stage address
@@ -1328,6 +1347,9 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb)
                 wq[nb] = *(const v4u*)(cur + kKmXBytes + (wn * 64 + nb * 32 + i) * 32 + g * 16);
+            // (kDepth is a multiple of kGroupStages and a split starts on a group: u tells)
+            constexpr bool kStatic = kGroupStages > 0;
+            const bool group_first = kStatic && (u % (kStatic ? kGroupStages : 1)) == 0;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 v4u xa[2], wb[2];
@@ -1344,30 +1366,61 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
                 for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
                     for (int mb = 0; mb < 2; ++mb)
-                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf(wb[nb]), as_bf(xa[mb]),
-                                                                              acc[nb][mb], 0, 0, 0);
+                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            as_bf(wb[nb]), as_bf(xa[mb]), (group_first && s == 0) ? zero16 : acc[nb][mb], 0, 0, 0);
             }
             // end of a group of K (or of this split): fold offset, zero point and scale
-            if (++done_in_group == group_stages || st + 1 == stages) {
-                done_in_group = 0;
+            bool group_last;
+            if (kStatic) {
+                group_last = (u % (kStatic ? kGroupStages : 1)) == (kStatic ? kGroupStages : 1) - 1;
+            } else {
+                group_last = ++done_in_group == group_stages || st + 1 == stages;
+                if (group_last) done_in_group = 0;
+            }
+            if (group_last) {
                 const char* par = cur + kKmXBytes + kKmWBytes;
-                float sxv[2];
+                // acc -= (136 + zero) * sum(x) as one more MFMA step: k = 0 ... 2 carry -128 on the
+                // kernel side, k = 3 ... 5 carry -(8 + zero) (any int8 zero point is exact in
+                // bfloat16), both against the three bfloat16 parts of the sum of x; products of
+                // two bfloat16 are exact in float32, so the cancellation happens in the accumulator
+                v4u xs[2], wz[2];
 #pragma unroll
-                for (int mb = 0; mb < 2; ++mb) sxv[mb] = *(const float*)(par + kKmParSx + a_row[mb] * 4);
+                for (int mb = 0; mb < 2; ++mb) {
+                    v2u raw = *(const v2u*)(par + kKmParSx + a_row[mb] * 8);
+                    if (g) raw[0] = raw[1] = 0;  // lanes 32 ... 63 hold k = 8 ... 15: nothing there
+                    xs[mb][0] = raw[0];                                   // hi, lo
+                    xs[mb][1] = (raw[1] & 0xffffu) | (raw[0] << 16);      // lolo, hi
+                    xs[mb][2] = (raw[0] >> 16) | (raw[1] << 16);          // lo, lolo
+                    xs[mb][3] = 0;
+                }
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    int zp = 0;
+                    if (kGrouped) zp = *(const int8_t*)(par + kKmParZero + wn * 64 + nb * 32 + i);
+                    const u32 cz = __float_as_uint(-(float)(8 + zp)) >> 16;
+                    wz[nb][0] = 0xC300C300u;                              // -128, -128
+                    wz[nb][1] = 0xC300u | (cz << 16);                     // -128, -(8 + zero)
+                    wz[nb][2] = cz | (cz << 16);
+                    wz[nb][3] = 0;
+                }
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                    for (int mb = 0; mb < 2; ++mb)
+                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf(wz[nb]), as_bf(xs[mb]),
+                                                                              acc[nb][mb], 0, 0, 0);
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
                     for (int rg = 0; rg < 4; ++rg) {
-                        float sc[4] = {1.f, 1.f, 1.f, 1.f}, off[4] = {kOffset, kOffset, kOffset, kOffset};
+                        float sc[4] = {1.f, 1.f, 1.f, 1.f};
                         if (kGrouped) {
                             const int nl = wn * 64 + nb * 32 + 8 * rg + 4 * g;
                             const v2u sraw = *(const v2u*)(par + kKmParScale + nl * 2);
-                            const u32 zraw = *(const u32*)(par + kKmParZero + nl);
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
                                 const u32 w = sraw[e >> 1];
                                 sc[e] = __uint_as_float((e & 1) ? (w & 0xffff0000u) : (w << 16));
-                                off[e] = kOffset + (float)(int)(int8_t)(zraw >> (8 * e));
                             }
                         }
 #pragma unroll
@@ -1375,9 +1428,8 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
 #pragma unroll
                             for (int mb = 0; mb < 2; ++mb) {
                                 const int r = 4 * rg + e;
-                                const float t = __builtin_fmaf(-off[e], sxv[mb], acc[nb][mb][r]);
-                                tot[nb][mb][r] = __builtin_fmaf(sc[e], t, tot[nb][mb][r]);
-                                acc[nb][mb][r] = 0.f;
+                                tot[nb][mb][r] = __builtin_fmaf(sc[e], acc[nb][mb][r], tot[nb][mb][r]);
+                                if (!kStatic) acc[nb][mb][r] = 0.f;
                             }
                     }
                 }
@@ -1551,7 +1603,7 @@ extern "C" int64_t k3q_gemm_w4_kmajor_workspace_bytes(int64_t M, int64_t K, int6
     if (!kmajor_ok(M, K, N, block_size)) return 0;
     const int64_t gsize = block_size > 0 ? block_size : 128;
     const KmPlan pl = kmajor_plan(M, K, N, gsize);
-    return ((K / gsize) * M * 4 + 255) / 256 * 256 + (int64_t)pl.ks * M * N * 4;
+    return ((K / gsize) * M * 8 + 255) / 256 * 256 + (int64_t)pl.ks * M * N * 4;
 }
 
 extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
@@ -1576,8 +1628,8 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     const KmPlan pl = kmajor_plan(M, K, N, gsize);
     // per-channel kernels need the offset taken out only once per split
     if (!grouped && (K % pl.klen) == 0) gsize = pl.klen;
-    float* sx = (float*)workspace;
-    float* part = (float*)((char*)workspace + ((K / gsize) * M * 4 + 255) / 256 * 256);
+    v2u* sx = (v2u*)workspace;
+    float* part = (float*)((char*)workspace + ((K / gsize) * M * 8 + 255) / 256 * 256);
     km_group_sums<<<dim3((unsigned)(K / gsize), (unsigned)((M + 3) / 4)), 256, 0, s>>>(
         (const uint16_t*)x, sx, M, K, (int)gsize);
     KmParams kp{};
@@ -1595,17 +1647,24 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     dim3 grid((unsigned)((N + kKmBN - 1) / kKmBN), (unsigned)((M + kKmBM - 1) / kKmBM), (unsigned)pl.ks);
     constexpr int kDepth = 4;
     const size_t lds = (size_t)kDepth * kKmSlotBytes;
+    using KmKernel = void (*)(KmParams);
+    static const KmKernel kernels[2][4] = {
+        {gemm_w4_kmajor<false, kDepth, 0>, gemm_w4_kmajor<false, kDepth, 1>,
+         gemm_w4_kmajor<false, kDepth, 2>, gemm_w4_kmajor<false, kDepth, 4>},
+        {gemm_w4_kmajor<true, kDepth, 0>, gemm_w4_kmajor<true, kDepth, 1>,
+         gemm_w4_kmajor<true, kDepth, 2>, gemm_w4_kmajor<true, kDepth, 4>}};
     static const bool raised = [] {
-        bool ok = hipFuncSetAttribute((const void*)gemm_w4_kmajor<true, kDepth>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget) == hipSuccess;
-        return hipFuncSetAttribute((const void*)gemm_w4_kmajor<false, kDepth>,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget) == hipSuccess && ok;
+        bool ok = true;
+        for (int a = 0; a < 2; ++a)
+            for (int b = 0; b < 4; ++b)
+                ok = hipFuncSetAttribute((const void*)kernels[a][b], hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         kLdsBudget) == hipSuccess && ok;
+        return ok;
     }();
     (void)raised;
-    if (grouped)
-        gemm_w4_kmajor<true, kDepth><<<grid, kKmThreads, lds, s>>>(kp);
-    else
-        gemm_w4_kmajor<false, kDepth><<<grid, kKmThreads, lds, s>>>(kp);
+    const int gs = (int)(gsize / kKmStage);
+    const int variant = gs == 1 ? 1 : gs == 2 ? 2 : gs == 4 ? 3 : 0;
+    kernels[grouped ? 1 : 0][variant]<<<grid, kKmThreads, lds, s>>>(kp);
     // the decode kernel's second pass: sums the splits in order, applies scale and bias
     GemvParams gp{};
     gp.scale = scale;

@@ -281,7 +281,7 @@ def test_int4_multi_prefill_sizes(dev, M, block_size):
 @pytest.mark.parametrize("M,K,N,block_size", [
     (17, 128, 32, None), (33, 256, 64, 128), (64, 512, 256, 64), (128, 1024, 512, 128),
     (130, 2048, 1056, 128), (200, 1024, 288, None), (256, 4096, 4096, 128), (512, 1024, 1024, 256),
-    (100, 4096, 1024, None),
+    (100, 4096, 1024, None), (96, 1536, 256, 192), (40, 2048, 128, 512),
 ])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_int4_kmajor_route(dev, M, K, N, block_size, with_bias):
@@ -312,3 +312,24 @@ def test_int4_kmajor_route(dev, M, K, N, block_size, with_bias):
                              kernel_zero=qk["kernel_zero"].to(dev) if grouped else None,
                              block_size=block_size, bias=bias_t.to(dev) if with_bias else None)
     assert max_rel_err(got, other) <= 1.5 * tol
+
+
+@pytest.mark.parametrize("M,K,N,block_size", [(48, 1024, 256, 128), (130, 1536, 96, 192), (64, 512, 64, 64)])
+def test_int4_kmajor_any_zero_point_and_offset_inputs(dev, M, K, N, block_size):
+    # zero points over the whole int8 range (a stored file may hold any) and inputs with a large
+    # mean, so that (136 + zero) * sum(x), which the kernel takes out per group, is hundreds of
+    # times the result: against the float64 value and the other route
+    qk, _ = make_layer(K, N, block_size, 92, False)
+    g = torch.Generator().manual_seed(93)
+    x = (torch.randn(M, K, generator=g) + 3.0).to(torch.bfloat16)
+    zero = torch.randint(-128, 128, qk["kernel_zero"].shape, generator=g, dtype=torch.int8)
+    dt = torch.bfloat16
+    scale_t = qk["kernel_scale"].to(dt)
+    kernel = qk["kernel"].to(dev)
+    got = kops.int4_matmul_kmajor(x.to(dev), kops.int4_kmajor_copy(kernel, N), scale_t.to(dev),
+                                  kernel_zero=zero.to(dev), block_size=block_size)
+    exact = c_w4_matmul_f64(x, qk["kernel"], scale_t, zero, block_size, None, N)
+    assert max_rel_err(got, exact) <= RTOL[dt] / 2
+    other = kops.int4_matmul(x.to(dev), kernel, scale_t.to(dev), N, kernel_zero=zero.to(dev),
+                             block_size=block_size)
+    assert max_rel_err(got, other) <= RTOL[dt]
