@@ -61,9 +61,10 @@ def glorot_uniform(shape, dtype, generator=None):
 
 # rows for which the int4 forward reads the K-contiguous copy of the kernel (measured against
 # the 32-row passes below it and the de-quantise + GEMM route above it, groups of 128, us:
-# K=4096, N=14336: 64 rows 37 against 60, 128 rows 44 against 66, 256 rows 67 against 81,
-# 512 rows 114 against 97; K=N=4096: 64 rows 24 against 32, 128 rows 31 against 30)
-KMAJOR_MIN_ROWS, KMAJOR_MAX_ROWS = 33, 256
+# K=4096, N=14336: 64 rows 32 against 59, 128 rows 37 against 64, 256 rows 57 against 80,
+# 512 rows 96 against 97; K=N=4096: 64 rows 22 against 32, 128 rows 28 against 30, 512 rows
+# 39 against 44; K=14336, N=4096: 512 rows 93 against 100)
+KMAJOR_MIN_ROWS, KMAJOR_MAX_ROWS = 33, 512
 
 
 class Dense(Layer):
