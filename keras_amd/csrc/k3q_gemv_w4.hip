@@ -1216,15 +1216,18 @@ constexpr int kKmParScale = 0, kKmParZero = 512, kKmParSx = 768, kKmParSpare = 1
 // kGroupStages: stages per group of K when that is 1, 2 or 4 (groups of 64, 128, 256), else 0.
 // Known at compile time, the first MFMAs of a group take a zero accumulator operand and the
 // 64 accumulators are never cleared; with 0 the group ends are found at run time.
-template <bool kGrouped, int kDepth, int kGroupStages>
+// kNB: blocks of 32 kernel rows per wave: 2 (tiles of 128 x 256) or 1 (128 x 128, for kernels so
+// narrow that wide tiles leave CUs idle even at eight splits).
+template <bool kGrouped, int kDepth, int kGroupStages, int kNB>
 __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
+    constexpr int kBN = 128 * kNB, kWaveN = 32 * kNB;
     extern __shared__ char km_lds[];
     constexpr int kOpsPerStage = 4;  // DMA instructions a wave issues per stage
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 2, wn = wave & 3;
     const int i = lane & 31, g = lane >> 5;
-    const int64_t n0 = (int64_t)blockIdx.x * kKmBN, m0 = (int64_t)blockIdx.y * kKmBM;
+    const int64_t n0 = (int64_t)blockIdx.x * kBN, m0 = (int64_t)blockIdx.y * kKmBM;
     const int64_t k_begin = (int64_t)blockIdx.z * p.klen;
     const int64_t k_end = k_begin + p.klen < p.K ? k_begin + p.klen : p.K;
     const int stages = (int)((k_end - k_begin) / kKmStage);
@@ -1244,7 +1247,8 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
     // kernel rows: one instruction per wave and stage = 32 rows x 32 bytes, two lanes per row
     const char* w_src;
     {
-        int64_t n = n0 + wave * 32 + (lane >> 1);
+        // (narrow tiles: waves 4 ... 7 fetch the rows of waves 0 ... 3 again, into the unused half)
+        int64_t n = n0 + (kNB == 1 ? (wave & 3) : wave) * 32 + (lane >> 1);
         if (n >= p.N) n = p.N - 1;
         w_src = (const char*)p.shadow + n * (p.K / 2) + k_begin / 2 + (lane & 1) * 16;
     }
@@ -1282,9 +1286,9 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) a_row[mb] = wm * 64 + mb * 32 + i;
 
-    v16f acc[2][2], tot[2][2];
+    v16f acc[kNB][2], tot[kNB][2];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -1343,27 +1347,27 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
             asm volatile("" ::: "memory");
             if (st + kDepth - 1 < stages) issue((u + kDepth - 1) % kDepth);
             const char* cur = km_lds + u * kKmSlotBytes;
-            v4u wq[2];  // this lane's 32 values of K of its two kernel rows: chunk 4g + s at step s
+            v4u wq[kNB];  // this lane's 32 values of K of its two kernel rows: chunk 4g + s at step s
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb)
-                wq[nb] = *(const v4u*)(cur + kKmXBytes + (wn * 64 + nb * 32 + i) * 32 + g * 16);
+            for (int nb = 0; nb < kNB; ++nb)
+                wq[nb] = *(const v4u*)(cur + kKmXBytes + (wn * kWaveN + nb * 32 + i) * 32 + g * 16);
             // (kDepth is a multiple of kGroupStages and a split starts on a group: u tells)
             constexpr bool kStatic = kGroupStages > 0;
             const bool group_first = kStatic && (u % (kStatic ? kGroupStages : 1)) == 0;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                v4u xa[2], wb[2];
+                v4u xa[2], wb[kNB];
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb)
                     xa[mb] = *(const v4u*)(cur + a_row[mb] * 128 + (((4 * g + s) ^ km_swz(a_row[mb])) << 4));
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
+                for (int nb = 0; nb < kNB; ++nb) {
                     const u32 d = wq[nb][s];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) wb[nb][q] = (((d >> (4 * q)) & kKmNibbles) ^ kKmFlip) | kKmExp;
                 }
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb)
+                for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
                     for (int mb = 0; mb < 2; ++mb)
                         acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -1383,7 +1387,7 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
                 // kernel side, k = 3 ... 5 carry -(8 + zero) (any int8 zero point is exact in
                 // bfloat16), both against the three bfloat16 parts of the sum of x; products of
                 // two bfloat16 are exact in float32, so the cancellation happens in the accumulator
-                v4u xs[2], wz[2];
+                v4u xs[2], wz[kNB];
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) {
                     v2u raw = *(const v2u*)(par + kKmParSx + a_row[mb] * 8);
@@ -1394,9 +1398,9 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
                     xs[mb][3] = 0;
                 }
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
+                for (int nb = 0; nb < kNB; ++nb) {
                     int zp = 0;
-                    if (kGrouped) zp = *(const int8_t*)(par + kKmParZero + wn * 64 + nb * 32 + i);
+                    if (kGrouped) zp = *(const int8_t*)(par + kKmParZero + wn * kWaveN + nb * 32 + i);
                     const u32 cz = __float_as_uint(-(float)(8 + zp)) >> 16;
                     wz[nb][0] = 0xC300C300u;                              // -128, -128
                     wz[nb][1] = 0xC300u | (cz << 16);                     // -128, -(8 + zero)
@@ -1404,18 +1408,18 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
                     wz[nb][3] = 0;
                 }
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb)
+                for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
                     for (int mb = 0; mb < 2; ++mb)
                         acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf(wz[nb]), as_bf(xs[mb]),
                                                                               acc[nb][mb], 0, 0, 0);
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
+                for (int nb = 0; nb < kNB; ++nb) {
 #pragma unroll
                     for (int rg = 0; rg < 4; ++rg) {
                         float sc[4] = {1.f, 1.f, 1.f, 1.f};
                         if (kGrouped) {
-                            const int nl = wn * 64 + nb * 32 + 8 * rg + 4 * g;
+                            const int nl = wn * kWaveN + nb * 32 + 8 * rg + 4 * g;
                             const v2u sraw = *(const v2u*)(par + kKmParScale + nl * 2);
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
@@ -1443,11 +1447,11 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
         const int64_t m = m0 + a_row[mb];
         if (m >= p.M) continue;
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            if (n0 + wn * 64 + nb * 32 >= p.N) continue;  // N % 32 == 0: a block is in or out as a whole
+        for (int nb = 0; nb < kNB; ++nb) {
+            if (n0 + wn * kWaveN + nb * 32 >= p.N) continue;  // N % 32 == 0: a block is in or out as a whole
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
-                const int64_t n = n0 + wn * 64 + nb * 32 + 8 * rg + 4 * g;
+                const int64_t n = n0 + wn * kWaveN + nb * 32 + 8 * rg + 4 * g;
                 v4f o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = tot[nb][mb][4 * rg + e];
@@ -1467,10 +1471,13 @@ inline bool kmajor_ok(int64_t M, int64_t K, int64_t N, int64_t block_size) {
 struct KmPlan {
     int ks;
     int64_t klen;
+    int bn;  // tile width: 256, or 128 where 256 would leave CUs idle even at eight splits
 };
 
 inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
-    const int64_t tiles = ((M + kKmBM - 1) / kKmBM) * ((N + kKmBN - 1) / kKmBN);
+    const int64_t m_tiles = (M + kKmBM - 1) / kKmBM;
+    const int bn = (m_tiles * ((N + kKmBN - 1) / kKmBN) * 8 < kTargetWorkgroups) ? kKmBN / 2 : kKmBN;
+    const int64_t tiles = m_tiles * ((N + bn - 1) / bn);
     // about one workgroup per CU, at most eight splits (every split writes and the reduction
     // reads M x N floats: at 128 rows one split of a 4096 x 14336 kernel is a quarter of the
     // kernel's own bytes), at least eight stages per split
@@ -1483,6 +1490,7 @@ inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
     if (klen < 8 * kKmStage) klen = (8 * kKmStage + unit - 1) / unit * unit;
     if (klen > K) klen = K;
     KmPlan pl;
+    pl.bn = bn;
     pl.klen = klen;
     pl.ks = (int)((K + klen - 1) / klen);
     return pl;  // rounding klen up can only lower the split count
@@ -1644,27 +1652,30 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     kp.K = K;
     kp.gsize = (int)gsize;
     kp.klen = (int)pl.klen;
-    dim3 grid((unsigned)((N + kKmBN - 1) / kKmBN), (unsigned)((M + kKmBM - 1) / kKmBM), (unsigned)pl.ks);
+    dim3 grid((unsigned)((N + pl.bn - 1) / pl.bn), (unsigned)((M + kKmBM - 1) / kKmBM), (unsigned)pl.ks);
     constexpr int kDepth = 4;
     const size_t lds = (size_t)kDepth * kKmSlotBytes;
     using KmKernel = void (*)(KmParams);
-    static const KmKernel kernels[2][4] = {
-        {gemm_w4_kmajor<false, kDepth, 0>, gemm_w4_kmajor<false, kDepth, 1>,
-         gemm_w4_kmajor<false, kDepth, 2>, gemm_w4_kmajor<false, kDepth, 4>},
-        {gemm_w4_kmajor<true, kDepth, 0>, gemm_w4_kmajor<true, kDepth, 1>,
-         gemm_w4_kmajor<true, kDepth, 2>, gemm_w4_kmajor<true, kDepth, 4>}};
+#define K3Q_KM_ROW(G, NB)                                                                   \
+    {gemm_w4_kmajor<G, kDepth, 0, NB>, gemm_w4_kmajor<G, kDepth, 1, NB>,                     \
+     gemm_w4_kmajor<G, kDepth, 2, NB>, gemm_w4_kmajor<G, kDepth, 4, NB>}
+    static const KmKernel kernels[2][2][4] = {{K3Q_KM_ROW(false, 1), K3Q_KM_ROW(false, 2)},
+                                              {K3Q_KM_ROW(true, 1), K3Q_KM_ROW(true, 2)}};
+#undef K3Q_KM_ROW
     static const bool raised = [] {
         bool ok = true;
         for (int a = 0; a < 2; ++a)
-            for (int b = 0; b < 4; ++b)
-                ok = hipFuncSetAttribute((const void*)kernels[a][b], hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         kLdsBudget) == hipSuccess && ok;
+            for (int b = 0; b < 2; ++b)
+                for (int c = 0; c < 4; ++c)
+                    ok = hipFuncSetAttribute((const void*)kernels[a][b][c],
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             kLdsBudget) == hipSuccess && ok;
         return ok;
     }();
     (void)raised;
     const int gs = (int)(gsize / kKmStage);
     const int variant = gs == 1 ? 1 : gs == 2 ? 2 : gs == 4 ? 3 : 0;
-    kernels[grouped ? 1 : 0][variant]<<<grid, kKmThreads, lds, s>>>(kp);
+    kernels[grouped ? 1 : 0][pl.bn == kKmBN ? 1 : 0][variant]<<<grid, kKmThreads, lds, s>>>(kp);
     // the decode kernel's second pass: sums the splits in order, applies scale and bias
     GemvParams gp{};
     gp.scale = scale;
