@@ -1218,27 +1218,29 @@ constexpr int kKmParScale = 0, kKmParZero = 512, kKmParSx = 768, kKmParSpare = 1
 // 64 accumulators are never cleared; with 0 the group ends are found at run time.
 // kNB: blocks of 32 kernel rows per wave: 2 (tiles of 128 x 256) or 1 (128 x 128, for kernels so
 // narrow that wide tiles leave CUs idle even at eight splits).
-template <bool kGrouped, int kDepth, int kGroupStages, int kNB>
+// kWM: waves along M: 2 (tiles of 128 rows) or 1 (64 rows, eight waves side by side, kNB = 1).
+template <bool kGrouped, int kDepth, int kGroupStages, int kWM, int kNB>
 __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
-    constexpr int kBN = 128 * kNB, kWaveN = 32 * kNB;
+    constexpr int kWaveN = 32 * kNB, kBN = kWaveN * (8 / kWM), kBM = 64 * kWM;
     extern __shared__ char km_lds[];
-    constexpr int kOpsPerStage = 4;  // DMA instructions a wave issues per stage
+    constexpr int kXOps = kWM;               // x-tile DMA instructions a wave issues per stage
+    constexpr int kOpsPerStage = kXOps + 2;  // DMA instructions a wave issues per stage
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 2, wn = wave & 3;
+    const int wm = kWM == 2 ? wave >> 2 : 0, wn = kWM == 2 ? (wave & 3) : wave;
     const int i = lane & 31, g = lane >> 5;
-    const int64_t n0 = (int64_t)blockIdx.x * kBN, m0 = (int64_t)blockIdx.y * kKmBM;
+    const int64_t n0 = (int64_t)blockIdx.x * kBN, m0 = (int64_t)blockIdx.y * kBM;
     const int64_t k_begin = (int64_t)blockIdx.z * p.klen;
     const int64_t k_end = k_begin + p.klen < p.K ? k_begin + p.klen : p.K;
     const int stages = (int)((k_end - k_begin) / kKmStage);
 
     // x tile: instruction d of a stage fills LDS bytes [d * 1024, +1024) = 8 rows, the lane's
     // 16 bytes at lane * 16; the chunk swizzle is applied on the source side.  A wave issues
-    // instructions 2 * wave and 2 * wave + 1.
-    const char* a_src[2];
+    // instructions kXOps * wave ... kXOps * wave + kXOps - 1.
+    const char* a_src[kXOps];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int row = (2 * wave + j) * 8 + (lane >> 3);
+    for (int j = 0; j < kXOps; ++j) {
+        const int row = (kXOps * wave + j) * 8 + (lane >> 3);
         const int ch = (lane & 7) ^ km_swz(row);
         int64_t grow = m0 + row;
         if (grow >= p.M) grow = p.M - 1;
@@ -1248,7 +1250,7 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
     const char* w_src;
     {
         // (narrow tiles: waves 4 ... 7 fetch the rows of waves 0 ... 3 again, into the unused half)
-        int64_t n = n0 + (kNB == 1 ? (wave & 3) : wave) * 32 + (lane >> 1);
+        int64_t n = n0 + (kBN == 128 ? (wave & 3) : wave) * 32 + (lane >> 1);
         if (n >= p.N) n = p.N - 1;
         w_src = (const char*)p.shadow + n * (p.K / 2) + k_begin / 2 + (lane & 1) * 16;
     }
@@ -1306,10 +1308,10 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
     auto issue = [&](int slot) {
         char* base = km_lds + slot * kKmSlotBytes;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < kXOps; ++j) {
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)a_src[j],
-                (__attribute__((address_space(3))) void*)(base + (2 * wave + j) * 1024), 16, 0, 0);
+                (__attribute__((address_space(3))) void*)(base + (kXOps * wave + j) * 1024), 16, 0, 0);
             a_src[j] += 128;
         }
         __builtin_amdgcn_global_load_lds(
@@ -1472,11 +1474,14 @@ struct KmPlan {
     int ks;
     int64_t klen;
     int bn;  // tile width: 256, or 128 where 256 would leave CUs idle even at eight splits
+    int bm;  // tile rows: 128, or 64 (with 256 columns) up to 64 rows
 };
 
 inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
-    const int64_t m_tiles = (M + kKmBM - 1) / kKmBM;
-    const int bn = (m_tiles * ((N + kKmBN - 1) / kKmBN) * 8 < kTargetWorkgroups) ? kKmBN / 2 : kKmBN;
+    const int bm = M <= 64 ? 64 : kKmBM;
+    const int64_t m_tiles = (M + bm - 1) / bm;
+    const int bn = (bm == kKmBM && m_tiles * ((N + kKmBN - 1) / kKmBN) * 8 < kTargetWorkgroups) ? kKmBN / 2
+                                                                                               : kKmBN;
     const int64_t tiles = m_tiles * ((N + bn - 1) / bn);
     // about one workgroup per CU, at most eight splits (every split writes and the reduction
     // reads M x N floats: at 128 rows one split of a 4096 x 14336 kernel is a quarter of the
@@ -1491,6 +1496,7 @@ inline KmPlan kmajor_plan(int64_t M, int64_t K, int64_t N, int64_t gsize) {
     if (klen > K) klen = K;
     KmPlan pl;
     pl.bn = bn;
+    pl.bm = bm;
     pl.klen = klen;
     pl.ks = (int)((K + klen - 1) / klen);
     return pl;  // rounding klen up can only lower the split count
@@ -1652,20 +1658,22 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     kp.K = K;
     kp.gsize = (int)gsize;
     kp.klen = (int)pl.klen;
-    dim3 grid((unsigned)((N + pl.bn - 1) / pl.bn), (unsigned)((M + kKmBM - 1) / kKmBM), (unsigned)pl.ks);
+    dim3 grid((unsigned)((N + pl.bn - 1) / pl.bn), (unsigned)((M + pl.bm - 1) / pl.bm), (unsigned)pl.ks);
     constexpr int kDepth = 4;
     const size_t lds = (size_t)kDepth * kKmSlotBytes;
     using KmKernel = void (*)(KmParams);
-#define K3Q_KM_ROW(G, NB)                                                                   \
-    {gemm_w4_kmajor<G, kDepth, 0, NB>, gemm_w4_kmajor<G, kDepth, 1, NB>,                     \
-     gemm_w4_kmajor<G, kDepth, 2, NB>, gemm_w4_kmajor<G, kDepth, 4, NB>}
-    static const KmKernel kernels[2][2][4] = {{K3Q_KM_ROW(false, 1), K3Q_KM_ROW(false, 2)},
-                                              {K3Q_KM_ROW(true, 1), K3Q_KM_ROW(true, 2)}};
+#define K3Q_KM_ROW(G, WM, NB)                                                               \
+    {gemm_w4_kmajor<G, kDepth, 0, WM, NB>, gemm_w4_kmajor<G, kDepth, 1, WM, NB>,             \
+     gemm_w4_kmajor<G, kDepth, 2, WM, NB>, gemm_w4_kmajor<G, kDepth, 4, WM, NB>}
+    // tile shapes: 128 x 128, 128 x 256, 64 x 256
+    static const KmKernel kernels[2][3][4] = {
+        {K3Q_KM_ROW(false, 2, 1), K3Q_KM_ROW(false, 2, 2), K3Q_KM_ROW(false, 1, 1)},
+        {K3Q_KM_ROW(true, 2, 1), K3Q_KM_ROW(true, 2, 2), K3Q_KM_ROW(true, 1, 1)}};
 #undef K3Q_KM_ROW
     static const bool raised = [] {
         bool ok = true;
         for (int a = 0; a < 2; ++a)
-            for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < 3; ++b)
                 for (int c = 0; c < 4; ++c)
                     ok = hipFuncSetAttribute((const void*)kernels[a][b][c],
                                              hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1675,7 +1683,8 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     (void)raised;
     const int gs = (int)(gsize / kKmStage);
     const int variant = gs == 1 ? 1 : gs == 2 ? 2 : gs == 4 ? 3 : 0;
-    kernels[grouped ? 1 : 0][pl.bn == kKmBN ? 1 : 0][variant]<<<grid, kKmThreads, lds, s>>>(kp);
+    const int shape = pl.bm == 64 ? 2 : pl.bn == kKmBN ? 1 : 0;
+    kernels[grouped ? 1 : 0][shape][variant]<<<grid, kKmThreads, lds, s>>>(kp);
     // the decode kernel's second pass: sums the splits in order, applies scale and bias
     GemvParams gp{};
     gp.scale = scale;

@@ -193,16 +193,116 @@ class LlamaStyleDecoder(Model):
             x = x[:, -1:, :]
         return self.token_embedding(self.final_norm(x), reverse=True)
 
+    def _weights_fingerprint(self):
+        """Changes whenever a variable is assigned, replaced or written in place."""
+        fp = []
+        for layer in self._flatten_layers(include_self=True):
+            for v in layer._variables:
+                t = v.value
+                fp.append((id(v), v.version, t.data_ptr(), t._version))
+        return hash(tuple(fp))
+
+    def _session(self, batch):
+        """Static buffers for `batch` sequences (KV cache, token, position, output), the
+        decode-step graph and one prompt graph per prompt length; dropped when a weight
+        changes (the graphs hold the addresses of the layers' derived copies)."""
+        fp = self._weights_fingerprint()
+        if self._graphs.get("weights") != fp:
+            self._graphs = {"weights": fp}
+        sess = self._graphs.get(batch)
+        if sess is None:
+            dev = self.device
+            sess = dict(
+                cache=self.new_cache(batch),
+                out=torch.zeros((batch, self.max_len), dtype=torch.int64, device=dev),
+                tok=torch.zeros((batch, 1), dtype=torch.int64, device=dev),
+                pos=torch.zeros((1,), dtype=torch.int64, device=dev),
+                idx=torch.zeros((1,), dtype=torch.int64, device=dev),
+                stream=torch.cuda.Stream(dev), step_graph=None, prompts={})
+            self._graphs[batch] = sess
+        return sess
+
+    def _graphed_generate(self, prompt, steps, stats):
+        B, P = prompt.shape
+        sess = self._session(B)
+        cache, out_buf, tok_buf, pos_buf, idx_buf = (sess[k] for k in ("cache", "out", "tok", "pos", "idx"))
+        cur = torch.cuda.current_stream(self.device)
+
+        def prefill(ids):
+            # stale cache rows beyond the current position are never attended (the mask keeps
+            # keys <= pos), so the static cache needs no clearing between sequences
+            logits = self.forward(ids, torch.arange(P, device=self.device), cache)
+            token = logits[:, -1, :].argmax(dim=-1, keepdim=True)
+            out_buf[:, :1] = token
+            tok_buf.copy_(token)
+            pos_buf.fill_(P)
+            idx_buf.fill_(1)
+
+        def step():
+            lg = self.forward(tok_buf, pos_buf, cache)
+            nxt = lg[:, -1, :].argmax(dim=-1, keepdim=True)
+            out_buf.index_copy_(1, idx_buf, nxt)
+            tok_buf.copy_(nxt)
+            pos_buf.add_(1)
+            idx_buf.add_(1)
+
+        def capture(fn):
+            # one eager run first (first-call set-up, scratch and derived copies), then the capture
+            side = sess["stream"]
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):
+                fn()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    fn()
+            cur.wait_stream(side)
+            return graph
+
+        entry = sess["prompts"].get(P)
+        if entry is None:
+            ids = torch.zeros((B, P), dtype=torch.int64, device=self.device)
+            ids.copy_(prompt)
+            entry = sess["prompts"][P] = (ids, capture(lambda: prefill(ids)))
+        ids, prompt_graph = entry
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        ev[0].record()
+        ids.copy_(prompt)
+        prompt_graph.replay()
+        ev[1].record()
+        done = 1
+        if sess["step_graph"] is None and steps > 2:
+            # (the eager run inside capture() is a real step of this sequence)
+            sess["step_graph"] = capture(step)
+            done += 1
+        ev[2].record()
+        timed = steps - done
+        for _ in range(timed):
+            if sess["step_graph"] is not None:
+                sess["step_graph"].replay()
+            else:
+                step()
+        ev[3].record()
+        result = out_buf[:, :steps].clone()
+        if stats is not None:
+            torch.cuda.synchronize(self.device)
+            stats.update(prefill_ms=ev[0].elapsed_time(ev[1]), decode_ms=ev[2].elapsed_time(ev[3]),
+                         decode_steps=timed, batch=B)
+        return result
+
     def generate(self, prompt, steps, use_graph=True, stats=None):
         """Greedy decode: prompt [B, P] -> generated ids [B, steps].  The prompt is one
         forward over P positions; each later step is one forward over one position that also
-        feeds its token back, replayed from a HIP graph when use_graph is set (shapes and
-        buffers are static, the position lives on the device).  `stats` (a dict) receives
-        prefill_ms, decode_ms, decode_steps as measured with device events."""
+        feeds its token back.  With use_graph both are replayed from HIP graphs (shapes and
+        buffers are static, the position lives on the device) that the model keeps per batch
+        size and prompt length: the first call for a shape captures them (untimed), later
+        calls only replay.  `stats` (a dict) receives prefill_ms, decode_ms, decode_steps as
+        measured with device events."""
         prompt = prompt.to(self.device)
         B, P = prompt.shape
         if P + steps > self.max_len:
             raise ValueError(f"prompt {P} + steps {steps} exceeds max_len {self.max_len}")
+        if use_graph:
+            return self._graphed_generate(prompt, steps, stats)
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         cache = self.new_cache(B)
         ev[0].record()
@@ -224,24 +324,10 @@ class LlamaStyleDecoder(Model):
             idx_buf.add_(1)
 
         done = 1
-        graph = None
-        if use_graph and steps > 2:
-            side = torch.cuda.Stream(self.device)
-            side.wait_stream(torch.cuda.current_stream(self.device))
-            with torch.cuda.stream(side):
-                step()  # a real step, run eagerly: first-call set-up and scratch allocation
-                done += 1
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, stream=side):
-                    step()
-            torch.cuda.current_stream(self.device).wait_stream(side)
         ev[2].record()
         timed = steps - done
         for _ in range(timed):
-            if graph is not None:
-                graph.replay()
-            else:
-                step()
+            step()
         ev[3].record()
         if stats is not None:
             torch.cuda.synchronize(self.device)

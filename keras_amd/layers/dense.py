@@ -61,10 +61,18 @@ def glorot_uniform(shape, dtype, generator=None):
 
 # rows for which the int4 forward reads the K-contiguous copy of the kernel (measured against
 # the 32-row passes below it and the de-quantise + GEMM route above it, groups of 128, us:
-# K=4096, N=14336: 64 rows 32 against 59, 128 rows 37 against 64, 256 rows 57 against 80,
-# 512 rows 96 against 97; K=N=4096: 64 rows 22 against 32, 128 rows 28 against 30, 512 rows
-# 39 against 44; K=14336, N=4096: 512 rows 93 against 100)
+# K=4096, N=14336: 17 rows 22 against 27, 32 rows 23 against 31, 64 rows 26 against 60, 128 rows
+# 38 against 65, 256 rows 58 against 81, 512 rows 98 against 98; K=N=4096: 17 rows 14.5 against
+# 13.4, 32 rows 16 against 17, 64 rows 19 against 32, 128 rows 24 against 30, 512 rows 40
+# against 45; K=14336, N=4096: 17 rows 29 against 27, 512 rows 96 against 102)
 KMAJOR_MIN_ROWS, KMAJOR_MAX_ROWS = 33, 512
+KMAJOR_MIN_ROWS_WIDE, KMAJOR_WIDE_UNITS = 17, 8192   # kernels at least this wide: from 17 rows
+
+
+def kmajor_rows(rows, units):
+    """Whether `rows` bfloat16 rows into `units` outputs take the K-contiguous int4 route."""
+    low = KMAJOR_MIN_ROWS_WIDE if units >= KMAJOR_WIDE_UNITS else KMAJOR_MIN_ROWS
+    return low <= rows <= KMAJOR_MAX_ROWS
 
 
 class Dense(Layer):
@@ -300,7 +308,7 @@ class Dense(Layer):
                 y = self.activation(y)
             return y
         rows = inputs.numel() // inputs.shape[-1] if inputs.shape[-1] else 0
-        if (inputs.dtype == torch.bfloat16 and KMAJOR_MIN_ROWS <= rows <= KMAJOR_MAX_ROWS
+        if (inputs.dtype == torch.bfloat16 and kmajor_rows(rows, self._orig_output_dim)
                 and kops.int4_kmajor_supported(rows, inputs.shape[-1], self._orig_output_dim,
                                                block_size if grouped else None)):
             # a few dozen to a hundred-odd rows: from the K-contiguous copy of the kernel (made

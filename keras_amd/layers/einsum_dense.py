@@ -497,10 +497,10 @@ class EinsumDense(Layer):
                                           lambda t: t.to(cd).reshape(-1).contiguous()),
                 bias=bias, out_dtype=cd, exact_epilogue=True)
             return self._finish(y2, free_shape, gv, fused)
-        from keras_amd.layers.dense import KMAJOR_MAX_ROWS, KMAJOR_MIN_ROWS
+        from keras_amd.layers.dense import kmajor_rows
 
         units = self._int4_unpacked_column_size
-        if (x2.dtype == torch.bfloat16 and KMAJOR_MIN_ROWS <= x2.shape[0] <= KMAJOR_MAX_ROWS
+        if (x2.dtype == torch.bfloat16 and kmajor_rows(x2.shape[0], units)
                 and kops.int4_kmajor_supported(x2.shape[0], x2.shape[1], units,
                                                block_size if grouped else None)):
             # as Dense: from the K-contiguous copy of the kernel, read once as int4

@@ -162,6 +162,32 @@ def test_generate_graph_equals_eager(dev, mode, dtype):
     assert torch.equal(eager.cpu(), graphed.cpu())
     again = model.generate(prompt, 12, use_graph=True)
     assert torch.equal(graphed.cpu(), again.cpu())
+    # the prompt graph and the step graph are kept by the model and only replayed from here on:
+    # other prompts of the same shape, another prompt length and fewer steps, with eager work
+    # and synchronisations between the replays, each against the eager result
+    for seed, shape, steps in [(5, (3, 8), 12), (6, (3, 8), 7), (7, (3, 20), 9), (8, (3, 8), 12),
+                               (9, (3, 20), 9), (3, (3, 8), 12)]:
+        other = torch.randint(0, CFG["vocab"], shape, generator=torch.Generator().manual_seed(seed))
+        want = model.generate(other, steps, use_graph=False)
+        torch.cuda.synchronize()
+        got = model.generate(other, steps, use_graph=True)
+        assert tuple(got.shape) == (3, steps)
+        assert torch.equal(want.cpu(), got.cpu()), (seed, shape, steps)
+    assert torch.equal(model.generate(prompt, 12, use_graph=True).cpu(), eager.cpu())
+
+
+def test_generate_graphs_follow_weight_changes(dev):
+    model = LlamaStyleDecoder(dtype="bfloat16", device=dev, layer_policy="int4/128_from_bfloat16",
+                              **{**CFG, "d_model": 256, "ffn_dim": 512})
+    model.randomize_quantized_weights(seed=1)
+    prompt = torch.randint(0, CFG["vocab"], (2, 20), generator=torch.Generator().manual_seed(4))
+    first = model.generate(prompt, 8, use_graph=True)
+    assert torch.equal(first.cpu(), model.generate(prompt, 8, use_graph=False).cpu())
+    model.randomize_quantized_weights(seed=2)   # the kept graphs point at the old derived copies
+    want = model.generate(prompt, 8, use_graph=False)
+    got = model.generate(prompt, 8, use_graph=True)
+    assert torch.equal(want.cpu(), got.cpu())
+    assert not torch.equal(first.cpu(), got.cpu())
 
 
 @pytest.mark.parametrize("policy", ["int4/128_from_bfloat16", "int4/-1_from_bfloat16", "int8_from_bfloat16"])
