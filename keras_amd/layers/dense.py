@@ -16,6 +16,7 @@ import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.layers.together import quantize_rows
 from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
 
 _ACTIVATIONS = {
@@ -260,7 +261,7 @@ class Dense(Layer):
             return y
         lead = inputs.shape[:-1]
         x2 = inputs.reshape(-1, inputs.shape[-1])
-        q, scale = self.inputs_quantizer(x2, axis=-1)
+        q, scale = quantize_rows(self.inputs_quantizer, x2)
         M, N = x2.shape[0], self.units
         exact = self.exact_epilogue
         if exact is None:
@@ -295,7 +296,7 @@ class Dense(Layer):
             # nibbles unpacked to int8 in scratch, exact int32 accumulation, one de-scale
             lead = inputs.shape[:-1]
             x2 = inputs.reshape(-1, inputs.shape[-1])
-            q, scale = self.inputs_quantizer(x2, axis=-1)
+            q, scale = quantize_rows(self.inputs_quantizer, x2)
             unpacked = quantizers.unpack_int4(as_tensor(self._kernel), self._orig_output_dim, axis=-1)
             y = kops.int8_matmul(
                 q, unpacked, a_scale=scale,

@@ -21,6 +21,7 @@ from keras_amd import dtype_policies, ops as kops, quantizers
 from keras_amd.layers.dense import (_ACTIVATIONS, activation_name, glorot_uniform,
                                     serialize_quantization_config)
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.layers.together import quantize_rows
 from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
 
 
@@ -453,7 +454,7 @@ class EinsumDense(Layer):
                              lambda t: t.to(cd).reshape(-1).contiguous()),
                 bias=bias, prepacked=pre)
             return self._finish(y2, free_shape, gv, fused)
-        q, scale = self.inputs_quantizer(x2, axis=-1)
+        q, scale = quantize_rows(self.inputs_quantizer, x2)
         exact = self.exact_epilogue
         if exact is None:
             exact = True
@@ -488,7 +489,7 @@ class EinsumDense(Layer):
             # divided by its scale weight by weight; here the contraction is the exact int32
             # one and both scales divide the result -- the same quantity without the
             # per-weight rounding.
-            q, scale = self.inputs_quantizer(x2, axis=-1)
+            q, scale = quantize_rows(self.inputs_quantizer, x2)
             unpacked = quantizers.unpack_int4(
                 as_tensor(self._kernel), self._int4_unpacked_column_size, axis=-1)
             y2 = kops.int8_matmul(
@@ -591,7 +592,7 @@ class EinsumDense(Layer):
                 )
             # einsum_dense.py:1163-1184: quantised rows, cast back to float, against the float
             # kernel; then the division by the input scale, then the bias
-            q, scale = self.inputs_quantizer(x2, axis=-1)
+            q, scale = quantize_rows(self.inputs_quantizer, x2)
             y2 = kops.float_matmul_nk(q.to(cd), wt, parts)
             y2 = torch.divide(y2, scale.to(cd))
             return self._finish(y2, free_shape, gv, False)

@@ -7,11 +7,45 @@ more than any tuning of the kernel itself.  The reference has no such call (its 
 their own `matmul`); this one returns exactly what the separate calls return.
 """
 
+import contextlib
+import threading
+
 import numpy as np
 import torch
 
 from keras_amd import ops as kops
 from keras_amd.layers.layer import to_torch_dtype
+
+_state = threading.local()
+
+
+@contextlib.contextmanager
+def shared_input_rows():
+    """While active, layers whose activation quantizers are configured alike and that are
+    called on the same rows quantise them once (the quantizer is a function of the rows
+    alone: keras/src/quantizers/quantizers.py:307-373)."""
+    prev = getattr(_state, "memo", None)
+    _state.memo = {}
+    try:
+        yield
+    finally:
+        _state.memo = prev
+
+
+def quantize_rows(quantizer, x2):
+    """`quantizer(x2, axis=-1)`, taken from the enclosing `shared_input_rows()` when another
+    layer has already quantised these very rows with the same settings."""
+    memo = getattr(_state, "memo", None)
+    config = getattr(quantizer, "get_config", None)
+    if memo is None or config is None:
+        return quantizer(x2, axis=-1)
+    key = (type(quantizer), repr(sorted(config().items())), x2.data_ptr(), tuple(x2.shape),
+           tuple(x2.stride()), x2.dtype, x2._version)
+    hit = memo.get(key)
+    if hit is None:
+        # the memo keeps x2 alive, so its address cannot be handed to another tensor meanwhile
+        hit = memo[key] = (quantizer(x2, axis=-1), x2)
+    return hit[0]
 
 
 def call_together(layers, inputs):
@@ -19,8 +53,14 @@ def call_together(layers, inputs):
 
     Weight-only int4 `Dense` / `EinsumDense` layers with one compute dtype, input width and
     group size go to `ops.int4_matmul_multi` (one launch at decode sizes); anything else is
-    called layer by layer.
+    called layer by layer, with the input rows quantised once for the layers that quantise
+    them alike (int8 layers: one quantizer launch instead of one per layer).
     """
+    with shared_input_rows():
+        return _call_together(layers, inputs)
+
+
+def _call_together(layers, inputs):
     layers = list(layers)
     if len(layers) < 2:
         return [layer(inputs) for layer in layers]
@@ -36,18 +76,21 @@ def call_together(layers, inputs):
     cd = to_torch_dtype(first.compute_dtype)
     if x.dtype.is_floating_point and x.dtype != cd:
         x = x.to(cd)
+    x = x.contiguous()
+    # (from here on the layers are handed x: moved and cast once, and the same tensor for all,
+    # which is what lets them share its quantised rows)
     specs = []
     for layer in layers:
         make = getattr(layer, "_int4_together_spec", None)
         spec = make(x) if make is not None else None
         if spec is None:
-            return [layer(inputs) for layer in layers]
+            return [layer(x) for layer in layers]
         specs.append(spec)
     x2 = specs[0]["x2"]
     if x2.shape[0] > 16:
         # beyond decode sizes nothing is shared: every layer takes its own route for the size
-        return [layer(inputs) for layer in layers]
+        return [layer(x) for layer in layers]
     if any(s["x2"].shape != x2.shape or s["block_size"] != specs[0]["block_size"] for s in specs):
-        return [layer(inputs) for layer in layers]
+        return [layer(x) for layer in layers]
     outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])
     return [s["finish"](y) for s, y in zip(specs, outs)]

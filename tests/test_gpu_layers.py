@@ -4,6 +4,7 @@ import pytest
 import torch
 
 import keras_amd as ka
+from keras_amd import quantizers as kq
 from keras_amd.layers import Dense, EinsumDense
 from oracle import keras_cpu_path as ref
 from tests.helpers import RTOL, max_rel_err
@@ -437,5 +438,45 @@ def test_call_together_matches_separate_calls(dev, rows, block_size):
     other.quantize("int8")
     want = [layer(x2) for layer in (mlp[0], other)]
     got = ka.layers.call_together((mlp[0], other), x2)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("rows", [1, 8, 40])
+@pytest.mark.parametrize("dtype", ["mixed_bfloat16", "float32"])
+def test_call_together_int8_quantises_shared_rows_once(dev, rows, dtype, monkeypatch):
+    # int8 layers on one input: the rows are quantised by one call, the results are the bits
+    # of the separate calls; a layer with another value range quantises for itself
+    g = torch.Generator().manual_seed(12)
+    init = lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d)
+    proj = [EinsumDense("btd,dnh->btnh", (None, 4, 64), dtype=dtype, device=dev, kernel_initializer=init)
+            for _ in range(3)]
+    mlp = [Dense(512, use_bias=(j == 1), dtype=dtype, device=dev, kernel_initializer=init) for j in range(2)]
+    x = torch.randn((1, rows, 256), generator=g)
+    for layer in proj + mlp:
+        layer.build((1, rows, 256))
+        layer.quantize("int8")
+    calls = []
+    real = kq.abs_max_quantize
+    monkeypatch.setattr(kq, "abs_max_quantize", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    want = [layer(x) for layer in proj + mlp]
+    assert len(calls) == 5
+    del calls[:]
+    got = ka.layers.call_together(proj + mlp, x)
+    assert len(calls) == 1
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and torch.equal(a, b)
+    # outside call_together nothing is remembered
+    del calls[:]
+    proj[0](x)
+    proj[1](x)
+    assert len(calls) == 2
+    # another quantizer configuration is not served from the shared rows
+    mlp[1].inputs_quantizer = kq.AbsMaxQuantizer(axis=-1, value_range=(-100, 100))
+    del calls[:]
+    want = [mlp[0](x), mlp[1](x)]
+    del calls[:]
+    got = ka.layers.call_together(mlp, x)
+    assert len(calls) == 2
     for a, b in zip(got, want):
         assert torch.equal(a, b)
