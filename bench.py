@@ -9,7 +9,8 @@ activations (inputs and weights already resident in HBM).  `value` is
 2*M*N*K / step time in TOP/s.  The int4 decode GEMV (K=N=8192, M in {1,4,16}),
 the second half of the headline metric, is reported under `int4_gemv` with its own
 HBM roofline; `llama_decode_int4` is the end-to-end greedy decode of a 32-layer
-Llama-style decoder whose weight matrices are all int4 (tokens/s at batch 1 and 8).
+Llama-style decoder whose weight matrices are all int4 (tokens/s at batch 1 and 8),
+`llama_decode_int8` the same with int8 layers.
 The CPU oracle (a restatement of the reference's torch-CPU op sequence) is timed
 on the host cores on a bounded sample as `cpu_baseline`.
 
@@ -206,33 +207,40 @@ def main():
     # ------------------------------------------------------------------ end-to-end decode
     # Llama-style 32-layer decoder (d_model 4096, 32 heads, SwiGLU 14336, vocab 32000), every
     # weight matrix int4 (grouped, block 128) with synthetic values written on the device;
-    # prompt of 128 random ids, greedy decode of 128 steps, decode steps replayed from a HIP
-    # graph.  Matmuls, embedding lookup and LM head run the k3q kernels; norms, RoPE,
+    # prompt of 128 random ids, greedy decode of 128 steps, prompt and decode steps replayed from
+    # HIP graphs.  Matmuls, embedding lookup and LM head run the k3q kernels; norms, RoPE,
     # attention and the gating are torch ops.
     decode = None
+    decode_int8 = None
     if not args.no_decode:
         from keras_amd.decoder_harness import LlamaStyleDecoder
 
         w4_host = packs[0].cpu()
         del packs
         torch.cuda.empty_cache()
-        model = LlamaStyleDecoder(max_len=256, dtype="bfloat16", device=dev,
-                                  layer_policy="int4/128_from_bfloat16")
-        model.randomize_quantized_weights()
-        decode = []
-        for batch in (1, 8):
-            prompt = torch.randint(0, model.vocab, (batch, 128), generator=g)
-            model.generate(prompt, 8)  # first-call set-up
-            st = {}
-            model.generate(prompt, 128, stats=st)
-            decode.append({
-                "batch": batch, "prompt": 128, "steps": 128,
-                "prefill_ms": round(st["prefill_ms"], 2),
-                "decode_ms_per_step": round(st["decode_ms"] / st["decode_steps"], 3),
-                "tokens_per_s": round(batch * st["decode_steps"] / st["decode_ms"] * 1e3, 1),
-            })
-        del model
-        torch.cuda.empty_cache()
+
+        def decode_figures(policy):
+            model = LlamaStyleDecoder(max_len=256, dtype="bfloat16", device=dev, layer_policy=policy)
+            model.randomize_quantized_weights()
+            out = []
+            for batch in (1, 8):
+                prompt = torch.randint(0, model.vocab, (batch, 128), generator=g)
+                model.generate(prompt, 8)  # first-call set-up: the graphs of this shape are captured
+                st = {}
+                model.generate(prompt, 128, stats=st)
+                out.append({
+                    "batch": batch, "prompt": 128, "steps": 128,
+                    "prefill_ms": round(st["prefill_ms"], 2),
+                    "decode_ms_per_step": round(st["decode_ms"] / st["decode_steps"], 3),
+                    "tokens_per_s": round(batch * st["decode_steps"] / st["decode_ms"] * 1e3, 1),
+                })
+            del model
+            torch.cuda.empty_cache()
+            return out
+
+        decode = decode_figures("int4/128_from_bfloat16")
+        # the same decoder with int8 layers (dynamic per-row activation quantisation)
+        decode_int8 = decode_figures("int8_from_bfloat16")
 
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None
@@ -291,6 +299,7 @@ def main():
                                    "traffic": QUANT_HBM_TRAFFIC_BYTES}},
         "int4_gemv": gemv,
         "llama_decode_int4": decode,
+        "llama_decode_int8": decode_int8,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
