@@ -285,10 +285,14 @@ def test_int4_multi_prefill_sizes(dev, M, block_size):
 ])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_int4_kmajor_route(dev, M, K, N, block_size, with_bias):
+    run_kmajor_case(dev, M, K, N, block_size, with_bias)
+
+
+def run_kmajor_case(dev, M, K, N, block_size, with_bias, seed=90):
     # 17 ... 512 bfloat16 rows from the K-contiguous copy of the kernel: against the oracle, the
     # float64 value, and the other route's result
-    qk, bias = make_layer(K, N, block_size, 90, with_bias)
-    g = torch.Generator().manual_seed(91)
+    qk, bias = make_layer(K, N, block_size, seed, with_bias)
+    g = torch.Generator().manual_seed(seed + 1)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     grouped = block_size is not None
     dt = torch.bfloat16
