@@ -81,7 +81,7 @@ class DecoderBlock(Layer):
 
     def forward(self, x, cos, sin, cache, pos, mask):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
-        (an int64 device tensor [T]); mask [T, maxT] True where a key may be attended to."""
+        (an int64 device tensor [T]); mask [T, maxT]: 0 where a key may be attended to, -inf elsewhere."""
         h = self.attn_norm(x)
         # the three projections of h in one launch at decode sizes
         q, k, v = call_together((self.query, self.key, self.value), h)
@@ -186,7 +186,9 @@ class LlamaStyleDecoder(Model):
         cos = self.cos.index_select(0, pos)
         sin = self.sin.index_select(0, pos)
         keys = torch.arange(self.max_len, device=self.device)
-        mask = keys[None, :] <= pos[:, None]
+        # additive form once per forward (a boolean mask is converted by every attention call)
+        mask = torch.zeros((pos.shape[0], self.max_len), dtype=cd, device=self.device).masked_fill_(
+            keys[None, :] > pos[:, None], float("-inf"))
         for block, kv in zip(self.blocks, cache):
             x = block.forward(x, cos, sin, kv, pos, mask)
         if last_only:
