@@ -38,19 +38,22 @@ class RMSNorm(Layer):
 
 
 def rope_tables(head_dim, max_len, device, base=10000.0, dtype=torch.float32):
-    """cos / sin [max_len, head_dim] for the rotate-half form: the half-width table repeated."""
+    """cos / sin [max_len, head_dim] for the rotate-half form: the half-width table repeated,
+    the first half of sin negated (the sign of the rotated half lives in the table, so
+    applying it costs no negation)."""
     inv = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
     ang = torch.outer(torch.arange(max_len, dtype=torch.float32), inv)
-    ang = torch.cat((ang, ang), dim=-1)
-    return torch.cos(ang).to(device=device, dtype=dtype), torch.sin(ang).to(device=device, dtype=dtype)
+    cos = torch.cos(torch.cat((ang, ang), dim=-1))
+    sin = torch.cat((-torch.sin(ang), torch.sin(ang)), dim=-1)
+    return cos.to(device=device, dtype=dtype), sin.to(device=device, dtype=dtype)
 
 
 def apply_rope(x, cos, sin):
-    """x [B, T, H, hd]; cos / sin [T, hd] for the positions of these T tokens
-    (rotate-half: pairs are (i, i + hd/2))."""
+    """x [B, T, H, hd]; cos / sin [T, hd] from `rope_tables` for the positions of these T
+    tokens (rotate-half: pairs are (i, i + hd/2); x * cos + (-x2, x1) * |sin|)."""
     half = x.shape[-1] // 2
-    rot = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
-    return x * cos[None, :, None, :] + rot * sin[None, :, None, :]
+    swapped = torch.cat((x[..., half:], x[..., :half]), dim=-1)
+    return x * cos[None, :, None, :] + swapped * sin[None, :, None, :]
 
 
 class DecoderBlock(Layer):
