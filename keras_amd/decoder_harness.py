@@ -16,7 +16,7 @@ import math
 import torch
 
 from keras_amd import dtype_policies
-from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding, call_together
+from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding, call_add, call_together
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
 from keras_amd.models import Model
 from keras_amd.quantization_config import Int4QuantizationConfig
@@ -96,10 +96,11 @@ class DecoderBlock(Layer):
         vc.index_copy_(2, pos, v.transpose(1, 2))
         a = torch.nn.functional.scaled_dot_product_attention(
             q.transpose(1, 2), kc, vc, attn_mask=mask[None, None])
-        x = x + self.attn_out(a.transpose(1, 2))
+        # (one row: the residual rides in the projection's bias slot, same bits as the add)
+        x = call_add(self.attn_out, a.transpose(1, 2), x)
         h = self.ffn_norm(x)
         gate, up = call_together((self.gate, self.up), h)
-        return x + self.down(torch.nn.functional.silu(gate) * up)
+        return call_add(self.down, torch.nn.functional.silu(gate) * up, x)
 
 
 class LlamaStyleDecoder(Model):

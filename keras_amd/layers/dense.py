@@ -253,7 +253,7 @@ class Dense(Layer):
             y = kops.int8_weight_only_matmul(
                 inputs, as_tensor(self._kernel),
                 self._read_cached("kernel_scale", self.kernel_scale),
-                bias=self._read_cached("bias", self.bias),
+                bias=self._call_bias(),
                 prepacked=self._cached("prepacked", self._kernel, kops.prepack_int8_kernel),
             )
             if self.activation is not None:
@@ -269,7 +269,7 @@ class Dense(Layer):
         y = kops.int8_matmul(
             q, as_tensor(self._kernel), a_scale=scale,
             kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
-            bias=self._read_cached("bias", self.bias),
+            bias=self._call_bias(),
             out_dtype=to_torch_dtype(self.compute_dtype),
             prepacked=self._cached("prepacked", self._kernel, kops.prepack_int8_kernel),
             exact_epilogue=exact,
@@ -301,7 +301,7 @@ class Dense(Layer):
             y = kops.int8_matmul(
                 q, unpacked, a_scale=scale,
                 kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
-                bias=self._read_cached("bias", self.bias),
+                bias=self._call_bias(),
                 out_dtype=to_torch_dtype(self.compute_dtype), exact_epilogue=True,
             )
             y = y.reshape(*lead, self._orig_output_dim)
@@ -320,7 +320,7 @@ class Dense(Layer):
                 self._read_cached("kernel_scale", self.kernel_scale),
                 kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
                 block_size=block_size if grouped else None,
-                bias=self._read_cached("bias", self.bias),
+                bias=self._call_bias(),
             )
         else:
             y = kops.int4_matmul(
@@ -328,11 +328,24 @@ class Dense(Layer):
                 self._read_cached("kernel_scale", self.kernel_scale), self._orig_output_dim,
                 kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
                 block_size=block_size if grouped else None,
-                bias=self._read_cached("bias", self.bias),
+                bias=self._call_bias(),
             )
         if self.activation is not None:
             y = self.activation(y)
         return y
+
+    def _call_bias(self):
+        """The bias of this call: the layer's own, or -- for a layer without one -- the row
+        that `call_add` lends for the duration of a one-row call."""
+        if self.bias is None:
+            return getattr(self, "_row_bias", None)
+        return self._read_cached("bias", self.bias)
+
+    def _row_bias_ok(self):
+        return self.bias is None and self.activation is None
+
+    def _rows_of(self, inputs):
+        return inputs.numel() // inputs.shape[-1]
 
     def _int4_together_spec(self, inputs):
         """What `call_together` needs to run this layer's weight-only int4 forward in a launch
@@ -356,7 +369,7 @@ class Dense(Layer):
                         kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
                         units=self._orig_output_dim,
                         kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
-                        bias=self._read_cached("bias", self.bias)),
+                        bias=self._call_bias()),
             finish=finish)
 
     # ---- serialization ---------------------------------------------------------------

@@ -416,15 +416,26 @@ class EinsumDense(Layer):
     def _fusable_bias(self, gv, n):
         """The bias as an [N] vector when it spans exactly the kept (kernel) axes, which
         are then the trailing output axes; otherwise None and the bias is added after."""
-        if self.bias is None:
-            return None, True
         o_spec = self._quant_info["specs"][2]
         trailing = list(o_spec[len(o_spec) - len(gv.kept):]) == gv.kept
+        if self.bias is None:
+            # (a row lent by `call_add` for a one-row call stands in for the bias)
+            return (getattr(self, "_row_bias", None) if trailing else None), True
         kept_shape = tuple(self.full_output_shape_of(c) for c in gv.kept)
         if trailing and self.bias.shape == kept_shape:
             cd = to_torch_dtype(self.compute_dtype)
             return self._cached("bias", self.bias, lambda t: t.to(cd).reshape(-1).contiguous()), True
         return None, False
+
+    def _row_bias_ok(self):
+        if self.bias is not None or self.activation is not None or not self.built:
+            return False
+        gv = self._gemm_view()
+        o_spec = self._quant_info["specs"][2]
+        return list(o_spec[len(o_spec) - len(gv.kept):]) == gv.kept
+
+    def _rows_of(self, inputs):
+        return self._input_rows(inputs, self._gemm_view())[0].shape[0]
 
     # ---- quantized forward -----------------------------------------------------------------
     def _int8_call(self, inputs, training=None):

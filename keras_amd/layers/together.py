@@ -94,3 +94,31 @@ def _call_together(layers, inputs):
         return [layer(x) for layer in layers]
     outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])
     return [s["finish"](y) for s, y in zip(specs, outs)]
+
+
+def call_add(layer, inputs, residual):
+    """`residual + layer(inputs)`.
+
+    On ONE row of a quantized `Dense` / `EinsumDense` that has neither bias nor activation the
+    add rides in the matmul's bias slot: the kernels add a bias to the rounded product,
+    `T(T(x . W) + b)`, which is what the separate add computes with `b` = the residual row --
+    the same bits, one launch less.  Anything else is the plain sum.
+    """
+    ok = getattr(layer, "_row_bias_ok", None)
+    if (isinstance(inputs, torch.Tensor) and isinstance(residual, torch.Tensor) and ok is not None
+            and layer.built and layer.quantization_mode in ("int8", "int4") and not layer.lora_enabled
+            and inputs.numel() > 0 and layer._rows_of(inputs) == 1
+            and residual.device == layer.device and inputs.device == layer.device
+            and residual.dtype == to_torch_dtype(layer.compute_dtype) and ok()):
+        row = residual.reshape(-1)
+        layer._row_bias = row if row.is_contiguous() else row.contiguous()
+        try:
+            out = layer(inputs)
+        finally:
+            layer._row_bias = None
+        if out.numel() == row.numel():
+            return out.reshape(residual.shape)
+        # (the layer's output is not one row of the residual's size: nothing was added that
+        # should have been; fall through to the plain sum)
+        raise ValueError(f"residual of {tuple(residual.shape)} does not match the layer's output {tuple(out.shape)}")
+    return residual + layer(inputs)

@@ -480,3 +480,37 @@ def test_call_together_int8_quantises_shared_rows_once(dev, rows, dtype, monkeyp
     assert len(calls) == 2
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("mode", ["int8", "int4"])
+@pytest.mark.parametrize("dtype", ["mixed_bfloat16", "float32"])
+def test_call_add_is_the_separate_add(dev, mode, dtype):
+    # residual + layer(x): one row goes through the matmul's bias slot (same bits as the add
+    # after it), more rows, a layer with a bias or an activation take the plain sum
+    g = torch.Generator().manual_seed(13)
+    init = lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d)
+    cd = torch.bfloat16 if dtype == "mixed_bfloat16" else torch.float32
+    out = EinsumDense("btnh,nhd->btd", (None, 256), dtype=dtype, device=dev, kernel_initializer=init)
+    down = Dense(256, use_bias=False, dtype=dtype, device=dev, kernel_initializer=init)
+    biased = Dense(256, use_bias=True, dtype=dtype, device=dev, kernel_initializer=init,
+                   bias_initializer=init)
+    out.build((1, 1, 4, 64))
+    for layer in (down, biased):
+        layer.build((1, 1, 512))
+    for layer in (out, down, biased):
+        layer.quantize(mode)
+    for rows in (1, 3):
+        res = torch.randn((1, rows, 256), generator=g).to(cd).to(dev)
+        a = torch.randn((1, rows, 4, 64), generator=g).to(cd).to(dev)
+        h = torch.randn((1, rows, 512), generator=g).to(cd).to(dev)
+        for layer, x in ((out, a), (down, h), (biased, h)):
+            want = res + layer(x)
+            got = ka.layers.call_add(layer, x, res)
+            assert got.shape == want.shape and got.dtype == want.dtype
+            assert torch.equal(got, want), (rows, layer.name)
+            assert getattr(layer, "_row_bias", None) is None
+    # the lent row is gone afterwards: the layer alone gives its own result again
+    h = torch.randn((1, 1, 512), generator=g).to(cd).to(dev)
+    plain = down(h)
+    ka.layers.call_add(down, h, torch.ones((1, 1, 256), dtype=cd, device=dev))
+    assert torch.equal(down(h), plain)
