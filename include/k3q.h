@@ -226,6 +226,20 @@ int k3q_gemv_w4_fused(const void* x, int x_dtype, int64_t M, int64_t K, int64_t 
                       void* stream);
 
 /*
+ * k3q_gemv_w4_fused for a layer without bias, with an [M, N] addend (same dtype as x,
+ * row-major, may be y itself) that is added to the rounded product the way a bias is:
+ *     y[m, n] = T(T(x . W)[m, n] + addend[m, n])
+ * which is what `residual + layer(x)` computes in the reference's op sequence
+ * (keras/src/layers/core/dense.py:1088-1095 followed by the caller's add), in one launch.
+ * Decode sizes only: M <= 64 (K3Q_ERR_SHAPE beyond); runs the decode kernels in passes.
+ */
+int k3q_gemv_w4_addend(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                       const void* w_packed, const void* scale, const void* zero,
+                       int64_t block_size, const void* addend, void* y, void* workspace,
+                       int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                       void* stream);
+
+/*
  * Weight-only int4 matmul for 17 ... 512 bfloat16 rows from a K-contiguous copy of the kernel:
  * the same result as k3q_gemv_w4 to the order of the fp32 sums, with the kernel read once as
  * int4 (k3q_gemv_w4's route for these sizes writes it out as bfloat16 first: nine times the

@@ -55,6 +55,8 @@ struct GemvParams {
     const void* scale;     // T [N] or [G, N]
     const int8_t* zero;    // [G, N] or null
     const void* bias;      // T [N] or null
+    int64_t bias_stride;   // elements from one row's bias to the next: 0 (one bias for all rows)
+                           // or N (an [M, N] addend, e.g. a residual)
     void* y;               // T [M, N]
     float* part;           // [KS, M, N] fp32 partials (KS > 1)
     unsigned* sync;        // arrival counters, one per column block, zero between calls (or null)
@@ -83,11 +85,11 @@ __device__ __forceinline__ void finish(const GemvParams& p, int m, int64_t n, fl
     if (kBF16) {
         v = round_bf16(v);
         if (!kGrouped) v = round_bf16(v / load_t<true>(p.scale, n));
-        if (p.bias) v = round_bf16(v + load_t<true>(p.bias, n));
+        if (p.bias) v = round_bf16(v + load_t<true>(p.bias, (int64_t)(p.m0 + m) * p.bias_stride + n));
         ((uint16_t*)p.y)[(int64_t)(p.m0 + m) * p.N + n] = (uint16_t)(__float_as_uint(v) >> 16);
     } else {
         if (!kGrouped) v = v / load_t<false>(p.scale, n);
-        if (p.bias) v = v + load_t<false>(p.bias, n);
+        if (p.bias) v = v + load_t<false>(p.bias, (int64_t)(p.m0 + m) * p.bias_stride + n);
         ((float*)p.y)[(int64_t)(p.m0 + m) * p.N + n] = v;
     }
 }
@@ -169,7 +171,7 @@ __device__ __forceinline__ void finish4_prefetched(const GemvParams& p, int m, i
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         if (!kGrouped) sc_raw[e] = load_raw<kBF16>(p.scale, n + e);
-        if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, n + e);
+        if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, (int64_t)(p.m0 + m) * p.bias_stride + n + e);
     }
     __builtin_amdgcn_sched_barrier(0);
     const v4f sum = sum_fn();
@@ -938,7 +940,7 @@ void launch_plan(const Plan& pl, int sets, bool f32, const GemvParams& p, const 
 int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* w_packed,
                 const void* scale, const void* zero, int64_t block_size, const void* bias, void* y,
                 void* workspace, int64_t workspace_bytes, const int* plan_override, void* counters,
-                int64_t counters_bytes, hipStream_t s) {
+                int64_t counters_bytes, hipStream_t s, bool bias_per_row = false) {
     if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
     if (M == 0) return K3Q_OK;
@@ -957,13 +959,16 @@ int run_gemv_w4(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, con
     p.scale = scale;
     p.zero = (const int8_t*)zero;
     p.bias = bias;
+    p.bias_stride = (bias && bias_per_row) ? N : 0;
     p.y = y;
     p.K = K;
     p.N = N;
     p.row_bytes = (N + 1) / 2;
     p.block_size = grouped ? (int)block_size : 0;
 
-    if (!plan_override && gemm_route_ok(f32, M, K, N) && workspace &&
+    // (the tile GEMM's epilogue knows one bias row only: a per-row addend stays on the decode
+    // kernels, whose entry point admits decode sizes only)
+    if (!plan_override && !bias_per_row && gemm_route_ok(f32, M, K, N) && workspace &&
         workspace_bytes >= gemm_route_bytes(f32, grouped, M, K, N) && aligned_to(workspace, 16) &&
         aligned_to(w_packed, 16) && aligned_to(scale, 16) && (!zero || aligned_to(zero, 16)) &&
         aligned_to(x, 16) && aligned_to(y, 16)) {
@@ -1556,6 +1561,17 @@ extern "C" int k3q_gemv_w4_fused(const void* x, int x_dtype, int64_t M, int64_t 
                                  void* stream) {
     return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y, workspace,
                        workspace_bytes, nullptr, counters, counters_bytes, (hipStream_t)stream);
+}
+
+extern "C" int k3q_gemv_w4_addend(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                  const void* w_packed, const void* scale, const void* zero,
+                                  int64_t block_size, const void* addend, void* y, void* workspace,
+                                  int64_t workspace_bytes, void* counters, int64_t counters_bytes,
+                                  void* stream) {
+    if (M > 64) return K3Q_ERR_SHAPE;
+    if (M > 0 && !addend) return K3Q_ERR_NULL;
+    return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, addend, y, workspace,
+                       workspace_bytes, nullptr, counters, counters_bytes, (hipStream_t)stream, true);
 }
 
 extern "C" int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,

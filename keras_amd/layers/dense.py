@@ -335,8 +335,9 @@ class Dense(Layer):
         return y
 
     def _call_bias(self):
-        """The bias of this call: the layer's own, or -- for a layer without one -- the row
-        that `call_add` lends for the duration of a one-row call."""
+        """The bias of this call: the layer's own, or -- for a layer without one -- the rows
+        that `call_add` lends for the duration of a call (one row: a bias; a row per row of the
+        input: the int4 decode kernel's addend)."""
         if self.bias is None:
             return getattr(self, "_row_bias", None)
         return self._read_cached("bias", self.bias)

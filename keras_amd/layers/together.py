@@ -18,6 +18,9 @@ from keras_amd.layers.layer import to_torch_dtype
 
 _state = threading.local()
 
+# rows up to which a weight-only int4 layer runs the decode kernel proper (above, other routes)
+ADDEND_MAX_ROWS = 16
+
 
 @contextlib.contextmanager
 def shared_input_rows():
@@ -99,26 +102,29 @@ def _call_together(layers, inputs):
 def call_add(layer, inputs, residual):
     """`residual + layer(inputs)`.
 
-    On ONE row of a quantized `Dense` / `EinsumDense` that has neither bias nor activation the
-    add rides in the matmul's bias slot: the kernels add a bias to the rounded product,
-    `T(T(x . W) + b)`, which is what the separate add computes with `b` = the residual row --
-    the same bits, one launch less.  Anything else is the plain sum.
+    For a quantized `Dense` / `EinsumDense` that has neither bias nor activation the add rides
+    in the matmul's bias slot: the kernels add a bias to the rounded product,
+    `T(T(x . W) + b)`, which is what the separate add computes with `b` = the residual -- the
+    same bits, one launch less.  One row: any quantized layer (the residual IS a bias row).
+    Up to 16 rows: weight-only int4 layers, whose decode kernel takes a row of addends per row
+    of x.  Anything else is the plain sum.
     """
     ok = getattr(layer, "_row_bias_ok", None)
     if (isinstance(inputs, torch.Tensor) and isinstance(residual, torch.Tensor) and ok is not None
             and layer.built and layer.quantization_mode in ("int8", "int4") and not layer.lora_enabled
-            and inputs.numel() > 0 and layer._rows_of(inputs) == 1
-            and residual.device == layer.device and inputs.device == layer.device
+            and inputs.numel() > 0 and residual.device == layer.device and inputs.device == layer.device
             and residual.dtype == to_torch_dtype(layer.compute_dtype) and ok()):
-        row = residual.reshape(-1)
-        layer._row_bias = row if row.is_contiguous() else row.contiguous()
-        try:
-            out = layer(inputs)
-        finally:
-            layer._row_bias = None
-        if out.numel() == row.numel():
+        rows = layer._rows_of(inputs)
+        if rows == 1 or (rows <= ADDEND_MAX_ROWS and residual.numel() % rows == 0
+                         and layer._int4_together_spec(inputs) is not None):
+            lent = residual.reshape(-1)
+            layer._row_bias = lent if lent.is_contiguous() else lent.contiguous()
+            try:
+                out = layer(inputs)
+            finally:
+                layer._row_bias = None
+            if out.numel() != lent.numel():
+                raise ValueError(f"residual of {tuple(residual.shape)} does not match the layer's "
+                                 f"output {tuple(out.shape)}")
             return out.reshape(residual.shape)
-        # (the layer's output is not one row of the residual's size: nothing was added that
-        # should have been; fall through to the plain sum)
-        raise ValueError(f"residual of {tuple(residual.shape)} does not match the layer's output {tuple(out.shape)}")
     return residual + layer(inputs)

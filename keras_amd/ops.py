@@ -45,8 +45,11 @@ def _arrival_counters(device, nbytes):
     return c
 
 
+INT4_ADDEND_MAX_ROWS = 64
+
+
 def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=None,
-                block_size=None, bias=None, plan=None, single_launch=True):
+                block_size=None, bias=None, plan=None, single_launch=True, addend=None):
     """`x[..., K] . W4[K, N]` for a Dense int4 kernel as the layer stores it.
 
     kernel_packed: int8 [K, ceil(N/2)] (two nibbles per byte along N).
@@ -95,7 +98,19 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
     ]
     cnt = _arrival_counters(x.device, lib.k3q_gemv_w4_counters_bytes(N)) if single_launch else None
     args += [_lib.ptr(cnt), cnt.numel() if single_launch else 0]
-    if plan is None:
+    if addend is None and bias is not None and M > 1 and bias.numel() == M * N:
+        addend, bias = bias, None  # a bias with a row per row of x is an addend
+    if addend is not None:
+        # [M, N] rows added to the rounded product the way a bias is (a residual), decode sizes
+        if bias is not None or plan is not None or M > INT4_ADDEND_MAX_ROWS:
+            raise ValueError("addend: at most %d rows, no bias, no plan" % INT4_ADDEND_MAX_ROWS)
+        _lib.require_device(addend)
+        if addend.dtype != x.dtype or addend.numel() != M * N:
+            raise ValueError("addend must hold M x N values of the input's dtype")
+        ad = addend.reshape(M, N)
+        args[9] = _lib.ptr(ad if ad.is_contiguous() else ad.contiguous())
+        rc = lib.k3q_gemv_w4_addend(*args, _lib.stream_ptr(x.device))
+    elif plan is None:
         rc = lib.k3q_gemv_w4_fused(*args, _lib.stream_ptr(x.device))
     else:
         arr = (ctypes.c_int * 4)(*[int(v) for v in plan[:4]])

@@ -58,6 +58,9 @@ def test_argument_validation_without_device():
     assert lib.k3q_gemv_w4_workspace_bytes(1, 8192, 8192) >= 8192 * 4
     assert lib.k3q_gemv_w4_fused(one, 0, 1, 0, 8, one, one, null, -1, null, one, null, 0, null, 0, null) == -2
     assert lib.k3q_gemv_w4_counters_bytes(8192) == 64 * 4 and lib.k3q_gemv_w4_counters_bytes(0) == 0
+    assert lib.k3q_gemv_w4_addend(one, 0, 65, 16, 8, one, one, null, -1, one, one, null, 0, null, 0, null) == -2
+    assert lib.k3q_gemv_w4_addend(one, 0, 4, 16, 8, one, one, null, -1, null, one, null, 0, null, 0, null) == -1
+    assert lib.k3q_gemv_w4_addend(one, 0, 0, 16, 8, one, one, null, -1, null, one, null, 0, null, 0, null) == 0
     assert lib.k3q_gemm_w4_kmajor(one, 0, 64, 128, 64, one, one, null, -1, null, one, one, 1 << 20, null) == -4  # bf16 only
     assert lib.k3q_gemm_w4_kmajor(one, 1, 64, 100, 64, one, one, null, -1, null, one, one, 1 << 20, null) == -2  # K % 128
     assert lib.k3q_gemm_w4_kmajor(one, 1, 64, 128, 64, one, one, null, 128, null, one, one, 1 << 20, null) == -1  # zero missing

@@ -337,3 +337,31 @@ def test_int4_kmajor_any_zero_point_and_offset_inputs(dev, M, K, N, block_size):
     other = kops.int4_matmul(x.to(dev), kernel, scale_t.to(dev), N, kernel_zero=zero.to(dev),
                              block_size=block_size)
     assert max_rel_err(got, other) <= RTOL[dt]
+
+
+@pytest.mark.parametrize("M,K,N,block_size", [
+    (1, 4096, 4096, 128), (2, 512, 256, None), (8, 4096, 4096, 128), (8, 14336, 4096, 128),
+    (16, 1024, 2048, None), (16, 4096, 4096, 128), (5, 96, 40, 32), (3, 100, 30, None),
+    (33, 256, 512, 128), (64, 512, 264, None),
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_int4_addend_is_the_add_after(dev, M, K, N, block_size, dtype):
+    # an [M, N] addend (a residual) added in the kernel's epilogue the way a bias is: the bits
+    # of `addend + int4_matmul(x)`, through the single-launch K split, the second pass, the
+    # row passes and the plain kernel alike
+    qk, _ = make_layer(K, N, block_size, 70, False)
+    g = torch.Generator().manual_seed(71)
+    x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+    res = torch.randn(M, N, generator=g).to(dtype).to(dev)
+    grouped = block_size is not None
+    kw = dict(kernel_zero=qk["kernel_zero"].to(dev) if grouped else None, block_size=block_size)
+    kernel, scale = qk["kernel"].to(dev), qk["kernel_scale"].to(dtype).to(dev)
+    want = res + kops.int4_matmul(x, kernel, scale, N, **kw)
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    for single in (True, False):
+        got = kops.int4_matmul(x, kernel, scale, N, addend=res, single_launch=single, **kw)
+        assert got.dtype == dtype and torch.equal(got.view(bits), want.view(bits)), single
+    # in place: the addend may be the output of an earlier call and is not modified
+    keep = res.clone()
+    kops.int4_matmul(x, kernel, scale, N, addend=res, **kw)
+    assert torch.equal(res, keep)

@@ -485,8 +485,9 @@ def test_call_together_int8_quantises_shared_rows_once(dev, rows, dtype, monkeyp
 @pytest.mark.parametrize("mode", ["int8", "int4"])
 @pytest.mark.parametrize("dtype", ["mixed_bfloat16", "float32"])
 def test_call_add_is_the_separate_add(dev, mode, dtype):
-    # residual + layer(x): one row goes through the matmul's bias slot (same bits as the add
-    # after it), more rows, a layer with a bias or an activation take the plain sum
+    # residual + layer(x): one row goes through the matmul's bias slot, up to 16 rows of a
+    # weight-only int4 layer through the decode kernel's addend (same bits as the add after
+    # it); more rows, int8 beyond one row, a layer with a bias or an activation take the plain sum
     g = torch.Generator().manual_seed(13)
     init = lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d)
     cd = torch.bfloat16 if dtype == "mixed_bfloat16" else torch.float32
@@ -499,7 +500,7 @@ def test_call_add_is_the_separate_add(dev, mode, dtype):
         layer.build((1, 1, 512))
     for layer in (out, down, biased):
         layer.quantize(mode)
-    for rows in (1, 3):
+    for rows in (1, 3, 8, 16, 17, 40):
         res = torch.randn((1, rows, 256), generator=g).to(cd).to(dev)
         a = torch.randn((1, rows, 4, 64), generator=g).to(cd).to(dev)
         h = torch.randn((1, rows, 512), generator=g).to(cd).to(dev)
