@@ -67,12 +67,17 @@ def glorot_uniform(shape, dtype, generator=None):
 # 13.4, 32 rows 16 against 17, 64 rows 19 against 32, 128 rows 24 against 30, 512 rows 40
 # against 45; K=14336, N=4096: 17 rows 29 against 27, 512 rows 96 against 102)
 KMAJOR_MIN_ROWS, KMAJOR_MAX_ROWS = 33, 512
-KMAJOR_MIN_ROWS_WIDE, KMAJOR_WIDE_UNITS = 17, 8192   # kernels at least this wide: from 17 rows
+# from 17 rows on kernels at least this wide or this large (17 rows, groups of 128, us:
+# K=5120, N=13824: 26 against 36; K=13824, N=5120: 29 against 37; K=11008, N=4096: 25 against
+# 27; K=8192, N=28672: 59 against 129; K=N=5120: 18 against 18.5 and K=N=4096: 14.5 against
+# 13.4, both left on the decode kernel)
+KMAJOR_MIN_ROWS_WIDE, KMAJOR_WIDE_UNITS, KMAJOR_LARGE_WEIGHTS = 17, 8192, 40 << 20
 
 
-def kmajor_rows(rows, units):
+def kmajor_rows(rows, units, input_dim=0):
     """Whether `rows` bfloat16 rows into `units` outputs take the K-contiguous int4 route."""
-    low = KMAJOR_MIN_ROWS_WIDE if units >= KMAJOR_WIDE_UNITS else KMAJOR_MIN_ROWS
+    wide = units >= KMAJOR_WIDE_UNITS or units * input_dim >= KMAJOR_LARGE_WEIGHTS
+    low = KMAJOR_MIN_ROWS_WIDE if wide else KMAJOR_MIN_ROWS
     return low <= rows <= KMAJOR_MAX_ROWS
 
 
@@ -309,7 +314,7 @@ class Dense(Layer):
                 y = self.activation(y)
             return y
         rows = inputs.numel() // inputs.shape[-1] if inputs.shape[-1] else 0
-        if (inputs.dtype == torch.bfloat16 and kmajor_rows(rows, self._orig_output_dim)
+        if (inputs.dtype == torch.bfloat16 and kmajor_rows(rows, self._orig_output_dim, inputs.shape[-1])
                 and kops.int4_kmajor_supported(rows, inputs.shape[-1], self._orig_output_dim,
                                                block_size if grouped else None)):
             # a few dozen to a hundred-odd rows: from the K-contiguous copy of the kernel (made

@@ -512,7 +512,7 @@ class EinsumDense(Layer):
         from keras_amd.layers.dense import kmajor_rows
 
         units = self._int4_unpacked_column_size
-        if (x2.dtype == torch.bfloat16 and kmajor_rows(x2.shape[0], units)
+        if (x2.dtype == torch.bfloat16 and kmajor_rows(x2.shape[0], units, x2.shape[1])
                 and kops.int4_kmajor_supported(x2.shape[0], x2.shape[1], units,
                                                block_size if grouped else None)):
             # as Dense: from the K-contiguous copy of the kernel, read once as int4
