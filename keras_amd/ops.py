@@ -25,10 +25,18 @@ def _workspace(device, nbytes):
     key = (device.index, stream.cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        size = max(int(nbytes), 1 << 20)
+        # A captured HIP graph keeps the address of the buffer its kernels were recorded with:
+        # an outgrown buffer is retired, never freed (sizes at least double, so the retired
+        # ones together stay below the live one).
+        if ws is not None:
+            _retired.append(ws)
+        size = max(int(nbytes), 1 << 20, 2 * (ws.numel() if ws is not None else 0))
         ws = torch.zeros(size, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+_retired = []
 
 
 _counters = {}
@@ -40,6 +48,8 @@ def _arrival_counters(device, nbytes):
     key = (device.index, stream.cuda_stream)
     c = _counters.get(key)
     if c is None or c.numel() < nbytes:
+        if c is not None:
+            _retired.append(c)  # a captured graph may still count in it
         c = torch.zeros(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
         _counters[key] = c
     return c
