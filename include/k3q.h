@@ -133,6 +133,18 @@ int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64
                 void* stream);
 
 /*
+ * k3q_gemm_i8 at decode sizes (M <= 64, b as [K, N], N % 16 == 0, K % 8 == 0; anything else
+ * K3Q_ERR_SHAPE) for a layer without bias, with an [M, N] addend (the output dtype,
+ * row-major, may be y itself) added to the de-scaled product the way a bias is:
+ *     y[m, n] = T(T(acc / scales)[m, n] + addend[m, n])
+ * which is `residual + layer(x)` of the reference's op sequence
+ * (keras/src/layers/core/dense.py:961-983 followed by the caller's add) in the same launch.
+ */
+int k3q_gemm_i8_addend(const int8_t* a, const int8_t* b, int64_t M, int64_t N, int64_t K,
+                       const void* a_scale, const void* b_scale, const void* addend, int out_dtype,
+                       int flags, void* y, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Weight-only int8 matmul: float activations, int8 kernel (a Dense int8 layer whose
  * config has no activation quantizer):
  *     y = T(T(x . b) / b_scale[n]) (+ bias)

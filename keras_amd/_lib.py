@@ -49,6 +49,10 @@ SIGNATURES = {
         [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _int, _int, _ptr, _ptr, _ptr,
          _i64, _ptr],
     ),
+    "k3q_gemm_i8_addend": (
+        _int,
+        [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _int, _int, _ptr, _ptr, _i64, _ptr],
+    ),
     "k3q_gemm_w8_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "k3q_gemm_w8": (
         _int,

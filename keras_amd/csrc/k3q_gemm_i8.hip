@@ -978,6 +978,19 @@ extern "C" int k3q_prepack_kernel_i8(const int8_t* kernel, int64_t K, int64_t N,
     return launch_status();
 }
 
+extern "C" int k3q_gemm_i8_addend(const int8_t* a, const int8_t* b, int64_t M, int64_t N, int64_t K,
+                                  const void* a_scale, const void* b_scale, const void* addend,
+                                  int out_dtype, int flags, void* y, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+    if (out_dtype != K3Q_F32 && out_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || N <= 0 || K <= 0) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (!a || !b || !y || !addend) return K3Q_ERR_NULL;
+    if (!gemm_i8_skinny_supported(M, N, K, a, b)) return K3Q_ERR_SHAPE;
+    return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, addend, out_dtype == K3Q_BF16, flags, y,
+                              nullptr, workspace, workspace_bytes, (hipStream_t)stream, true);
+}
+
 extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64_t M, int64_t N,
                            int64_t K, const void* a_scale, const void* b_scale, const void* bias,
                            int out_dtype, int flags, void* y, int32_t* acc_out, void* workspace,

@@ -33,6 +33,8 @@ struct SkinnyParams {
     const void* a_scale;   // T [M] or null
     const void* b_scale;   // T [N] or null
     const void* bias;      // T [N] or null
+    int64_t bias_stride;   // elements from one row's bias to the next: 0 (one bias for all rows)
+                           // or N (an [M, N] addend, e.g. a residual)
     void* y;               // T [M, N] or null
     int32_t* acc_out;      // [M, N] or null
     int32_t* part;         // [KS, M, N]
@@ -74,7 +76,7 @@ template <bool kBF16>
 __device__ __forceinline__ void finish(const SkinnyParams& p, int m, int64_t n, int acc) {
     const float sa = (p.y && p.a_scale) ? load_t<kBF16>(p.a_scale, p.m0 + m) : 1.0f;
     const float sb = (p.y && p.b_scale) ? load_t<kBF16>(p.b_scale, n) : 1.0f;
-    const float bias = (p.y && p.bias) ? load_t<kBF16>(p.bias, n) : 0.0f;
+    const float bias = (p.y && p.bias) ? load_t<kBF16>(p.bias, (int64_t)(p.m0 + m) * p.bias_stride + n) : 0.0f;
     finish_vals<kBF16>(p, m, n, acc, sa, sb, bias);
 }
 
@@ -231,7 +233,7 @@ __global__ __launch_bounds__(256) void gemm_i8_skinny_reduce(SkinnyParams p, int
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if (p.b_scale) sb_raw[e] = load_raw<kBF16>(p.b_scale, n + e);
-            if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, n + e);
+            if (p.bias) bi_raw[e] = load_raw<kBF16>(p.bias, (int64_t)(p.m0 + m) * p.bias_stride + n + e);
         }
     }
     const int32_t* src = p.part + (int64_t)m * p.N + n;
@@ -495,13 +497,14 @@ int gemm_i8_skinny_nk_run(const int8_t* a, const int8_t* b, int64_t M, int64_t N
 int gemm_i8_skinny_run(const int8_t* a, const int8_t* b, int64_t M, int64_t N, int64_t K,
                        const void* a_scale, const void* b_scale, const void* bias, bool bf16, int flags,
                        void* y, int32_t* acc_out, void* workspace, int64_t workspace_bytes,
-                       hipStream_t s) {
+                       hipStream_t s, bool bias_per_row) {
     SkinnyParams p{};
     p.xq = a;
     p.w = b;
     p.a_scale = a_scale;
     p.b_scale = b_scale;
     p.bias = bias;
+    p.bias_stride = (bias && bias_per_row) ? N : 0;
     p.y = y;
     p.acc_out = acc_out;
     p.K = K;

@@ -99,6 +99,17 @@ def _call_together(layers, inputs):
     return [s["finish"](y) for s, y in zip(specs, outs)]
 
 
+def _int8_addend_ok(layer, rows, residual):
+    """Activation-quantized int8 layer at the rows and widths its decode kernel takes."""
+    if layer.quantization_mode != "int8" or not layer.inputs_quantizer or rows > kops.SKINNY_MAX_ROWS:
+        return False
+    if residual.numel() % rows:
+        return False
+    units = residual.numel() // rows
+    kernel = layer._kernel
+    return units % 16 == 0 and (kernel.value.numel() // units) % 8 == 0
+
+
 def call_add(layer, inputs, residual):
     """`residual + layer(inputs)`.
 
@@ -106,8 +117,9 @@ def call_add(layer, inputs, residual):
     in the matmul's bias slot: the kernels add a bias to the rounded product,
     `T(T(x . W) + b)`, which is what the separate add computes with `b` = the residual -- the
     same bits, one launch less.  One row: any quantized layer (the residual IS a bias row).
-    Up to 16 rows: weight-only int4 layers, whose decode kernel takes a row of addends per row
-    of x.  Anything else is the plain sum.
+    Up to 16 rows: weight-only int4 layers, up to 8 rows: int8 layers with an activation
+    quantizer; their decode kernels take a row of addends per row of x.  Anything else is the
+    plain sum.
     """
     ok = getattr(layer, "_row_bias_ok", None)
     if (isinstance(inputs, torch.Tensor) and isinstance(residual, torch.Tensor) and ok is not None
@@ -115,8 +127,9 @@ def call_add(layer, inputs, residual):
             and inputs.numel() > 0 and residual.device == layer.device and inputs.device == layer.device
             and residual.dtype == to_torch_dtype(layer.compute_dtype) and ok()):
         rows = layer._rows_of(inputs)
-        if rows == 1 or (rows <= ADDEND_MAX_ROWS and residual.numel() % rows == 0
-                         and layer._int4_together_spec(inputs) is not None):
+        if (rows == 1 or (rows <= ADDEND_MAX_ROWS and residual.numel() % rows == 0
+                          and layer._int4_together_spec(inputs) is not None)
+                or _int8_addend_ok(layer, rows, residual)):
             lent = residual.reshape(-1)
             layer._row_bias = lent if lent.is_contiguous() else lent.contiguous()
             try:

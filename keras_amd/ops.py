@@ -306,6 +306,19 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
         layout = 0
     ws = _workspace(a.device, nbytes) if nbytes > 0 else None
     ws_bytes = nbytes if ws is not None else 0
+    if bias is not None and M > 1 and bias.numel() == M * N:
+        # a bias with a row per row of a: an addend (a residual), decode sizes only
+        if not skinny or want_acc or not want_y:
+            raise ValueError("a per-row addend takes at most %d rows, N %% 16 == 0, K %% 8 == 0 "
+                             "and returns y only" % SKINNY_MAX_ROWS)
+        ad = bias.reshape(M, N)
+        rc = lib.k3q_gemm_i8_addend(
+            _lib.ptr(a), _lib.ptr(b), M, N, K, _lib.ptr(sa), _lib.ptr(sb),
+            _lib.ptr(ad if ad.is_contiguous() else ad.contiguous()), code,
+            GEMM_EXACT_EPILOGUE if exact_epilogue else 0, _lib.ptr(y), _lib.ptr(ws), ws_bytes,
+            _lib.stream_ptr(a.device))
+        _lib.check(rc, "k3q_gemm_i8_addend")
+        return y
     rc = lib.k3q_gemm_i8(
         _lib.ptr(a), _lib.ptr(b), layout, M, N, K, _lib.ptr(sa), _lib.ptr(sb), _lib.ptr(bias),
         code, GEMM_EXACT_EPILOGUE if exact_epilogue else 0, _lib.ptr(y), _lib.ptr(acc),

@@ -52,6 +52,11 @@ def test_argument_validation_without_device():
     assert lib.k3q_gemm_i8(one, one, 0, 4, 4, 4, null, null, null, 5, 0, one, null, null, 0, null) == -4
     assert lib.k3q_gemm_i8(one, one, 3, 4, 4, 4, null, null, null, 0, 0, one, null, null, 0, null) == -2
     assert lib.k3q_gemm_i8(one, one, 0, 4, 4, 4, null, null, null, 0, 0, null, null, null, 0, null) == -1
+    assert lib.k3q_gemm_i8_addend(one, one, 4, 16, 8, null, null, one, 5, 0, one, null, 0, null) == -4
+    assert lib.k3q_gemm_i8_addend(one, one, 4, 16, 8, null, null, null, 0, 0, one, null, 0, null) == -1
+    assert lib.k3q_gemm_i8_addend(one, one, 4, 12, 8, null, null, one, 0, 0, one, null, 0, null) == -2  # N % 16
+    assert lib.k3q_gemm_i8_addend(one, one, 65, 16, 8, null, null, one, 0, 0, one, null, 0, null) == -2
+    assert lib.k3q_gemm_i8_addend(one, one, 0, 16, 8, null, null, null, 0, 0, one, null, 0, null) == 0
     assert lib.k3q_gemv_w4(one, 0, 1, 0, 8, one, one, null, -1, null, one, null, 0, null) == -2
     assert lib.k3q_gemv_w4(one, 9, 1, 16, 8, one, one, null, -1, null, one, null, 0, null) == -4
     assert lib.k3q_gemv_w4(one, 0, 1, 16, 8, one, one, null, 128, null, one, null, 0, null) == -1  # zero missing

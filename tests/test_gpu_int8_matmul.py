@@ -177,3 +177,23 @@ def test_dense_int8_decode_sizes(dev, M, K, N, dtype):
     # and the layer-level route (prepacked given, still routed by M) agrees bit for bit
     y2 = run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True, seed=M + K)
     assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("M,K,N", [(2, 4096, 4096), (8, 4096, 4096), (8, 14336, 4096), (5, 64, 48),
+                                   (3, 512, 1040), (8, 8, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_int8_addend_is_the_add_after(dev, M, K, N, dtype):
+    # an [M, N] addend (a residual) in the decode kernel's epilogue, where a bias would be
+    # added: the bits of `addend + int8_matmul(...)`, with and without a K split
+    x, qk, ks, _ = make_case(M, K, N, dtype, seed=M + N, with_bias=False)
+    res = torch.randn(M, N, generator=torch.Generator().manual_seed(5)).to(dtype).to(dev)
+    q, s = kq.abs_max_quantize(x.to(dev), axis=-1)
+    args = dict(a_scale=s, kernel_scale=ks.to(dtype).to(dev), out_dtype=dtype, exact_epilogue=True)
+    want = res + kops.int8_matmul(q, qk.to(dev), **args)
+    keep = res.clone()
+    got = kops.int8_matmul(q, qk.to(dev), bias=res, **args)
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    assert torch.equal(got.view(bits), want.view(bits))
+    assert torch.equal(res, keep)
+    with pytest.raises(ValueError):
+        kops.int8_matmul(q, qk.to(dev), bias=res, want_acc=True, **args)
