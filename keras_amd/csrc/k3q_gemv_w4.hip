@@ -31,10 +31,16 @@
 // chunks of kSteps * 16 rows.  Waves of a workgroup are reduced through LDS,
 // workgroups through fp32 partials in `workspace` that a second, tiny kernel
 // adds in a fixed order before applying the epilogue: the result does not
-// depend on scheduling.  (A single-kernel variant in which the last workgroup
-// to arrive sums the partials needs a device-scope release/acquire per
-// workgroup, which on this multi-XCD part means an L2 write-back and
-// invalidate each: measured 2-5x slower than the second launch.)
+// depend on scheduling.  With arrival counters from the caller the second
+// kernel is not launched: the workgroup that arrives last at its column
+// block's counter sums the partials itself, in the same order (same bits).
+// That variant does NOT use device-scope fences -- on this multi-XCD part an
+// agent-scope release / acquire is a write-back / invalidate of a whole L2 per
+// wave, measured 4-7x slower than the second launch.  It orders the data by
+// hand instead: partials are written with write-through stores (sc1), every
+// thread waits for the acknowledgement of its own stores (s_waitcnt vmcnt(0)),
+// the workgroup's barrier collects those waits, and only then is the arrival
+// counted; the last workgroup reads the partials with L2-bypassing loads (sc1).
 #include "k3q_common.h"
 #include "k3q_gemm_bf16.h"
 
@@ -48,6 +54,10 @@ constexpr float kOffset = 136.0f;  // 128 (bf16 magic exponent) + 8 (nibble ^ 8)
 constexpr int kMaxWaves = 8;
 constexpr int kRedPad = 8;
 constexpr int kLdsBudget = 144 * 1024;  // of the 160 KiB a workgroup may use
+
+// gfx9 s_waitcnt immediate for "at most n vector-memory operations outstanding" (loads AND
+// stores count in vmcnt on this ISA; expcnt and lgkmcnt are left alone)
+constexpr int km_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 
 struct GemvParams {
     const void* x;         // [M, K] bf16 or f32
@@ -529,11 +539,16 @@ __device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, 
     // the order of the split, whoever comes last) and applies the epilogue; it leaves the
     // counter at zero for the next call.
     if (KS == 1 || p.sync == nullptr) return;
-    // The partials were stored around the non-coherent caches; once the stores are
-    // acknowledged (the wait this fence emits) they are visible device-wide.  A device-scope
-    // release here would write back the whole L2 once per wave (54 us per call instead of 12).
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();  // every thread's stores are out before the arrival is counted
+    // The partials were stored write-through (sc1), around the caches that are not coherent
+    // across the device; a store leaves vmcnt only when the memory side has acknowledged it.
+    // Every thread waits for its own stores here, explicitly: a workgroup-scope release fence
+    // does NOT wait for vector-memory stores on this target (it only orders LDS), and a
+    // device-scope release would write back the whole L2 once per wave (54 us per call
+    // instead of 12).  The barrier then joins the waits of all threads, and only after it is
+    // the arrival counted, so the counter cannot run ahead of any partial of this workgroup.
+    __builtin_amdgcn_s_waitcnt(km_vmcnt(0));
+    asm volatile("" ::: "memory");
+    __syncthreads();
     int* flag = (int*)red;
     if (threadIdx.x == 0) flag[0] = atomicAdd(p.sync + cb, 1u) == (unsigned)(KS - 1);
     __syncthreads();
@@ -1203,9 +1218,6 @@ __global__ __launch_bounds__(256) void km_group_sums(const uint16_t* __restrict_
         sx[g * M + m] = o;
     }
 }
-
-// gfx9 s_waitcnt immediate for "at most n vector-memory operations outstanding"
-constexpr int km_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 
 // Everything the loop consumes arrives by LDS-DMA (global_load_lds), nothing through
 // registers: the compiler then places no waits of its own in the loop (a register load there

@@ -15,7 +15,7 @@ import math
 import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
-from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.layers.layer import Layer, as_tensor, require_default_g_idx, to_torch_dtype
 from keras_amd.layers.together import quantize_rows
 from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
 
@@ -313,6 +313,8 @@ class Dense(Layer):
             if self.activation is not None:
                 y = self.activation(y)
             return y
+        if grouped:
+            require_default_g_idx(self, block_size)
         rows = inputs.numel() // inputs.shape[-1] if inputs.shape[-1] else 0
         if (inputs.dtype == torch.bfloat16 and kmajor_rows(rows, self._orig_output_dim, inputs.shape[-1])
                 and kops.int4_kmajor_supported(rows, inputs.shape[-1], self._orig_output_dim,
@@ -363,6 +365,8 @@ class Dense(Layer):
             return None
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
+        if grouped:
+            require_default_g_idx(self, block_size)
         lead = inputs.shape[:-1]
 
         def finish(y2):

@@ -20,7 +20,7 @@ import torch
 from keras_amd import dtype_policies, ops as kops, quantizers
 from keras_amd.layers.dense import (_ACTIVATIONS, activation_name, glorot_uniform,
                                     serialize_quantization_config)
-from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.layers.layer import Layer, as_tensor, require_default_g_idx, to_torch_dtype
 from keras_amd.layers.together import quantize_rows
 from keras_amd.quantization_config import QuantizationConfig, get_block_size_for_layer
 
@@ -489,6 +489,8 @@ class EinsumDense(Layer):
         if not gv.k_plain:
             return self._int4_call_dequantized(x2, free_shape, gv, cd, grouped)
         bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
+        if grouped:
+            require_default_g_idx(self, block_size)  # (the de-quantised route above reads g_idx)
         if self.inputs_quantizer:
             if grouped:
                 raise NotImplementedError(
@@ -544,6 +546,8 @@ class EinsumDense(Layer):
         cd = to_torch_dtype(self.compute_dtype)
         block_size = self._int4_block_size
         grouped = block_size is not None and block_size > 0
+        if grouped:
+            require_default_g_idx(self, block_size)
         x2, free_shape = self._input_rows(inputs, gv)
         bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
         return dict(

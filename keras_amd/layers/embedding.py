@@ -20,7 +20,7 @@ import math
 import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
-from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
+from keras_amd.layers.layer import Layer, as_tensor, require_default_g_idx, to_torch_dtype
 from keras_amd.quantization_config import (
     Int4QuantizationConfig,
     QuantizationConfig,
@@ -189,6 +189,8 @@ class Embedding(Layer):
             raise NotImplementedError("LoRA on a quantized Embedding is outside this inference path.")
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
+        if grouped:
+            require_default_g_idx(self, block_size)
         return kops.embedding_lookup(
             inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
             self._orig_output_dim, bits=4,
@@ -504,6 +506,8 @@ class ReversibleEmbedding(Embedding):
         cd = to_torch_dtype(self.compute_dtype)
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
+        if grouped:
+            require_default_g_idx(self, block_size)
         lead = inputs.shape[:-1]
         x2 = inputs.reshape(-1, inputs.shape[-1])
         in_scale = None

@@ -92,6 +92,29 @@ def as_tensor(x):
     return x.value if isinstance(x, Variable) else x
 
 
+def require_default_g_idx(layer, block_size):
+    """The grouped int4 kernels take the group of row k to be `k // block_size`; the reference
+    looks it up in the `g_idx` variable (keras/src/quantizers/quantizers.py:1659-1668), which
+    `quantize()` fills with exactly that (keras/src/layers/core/dense.py:868-889).  A stored
+    `g_idx` holding any other map would silently compute something else here, so it is
+    rejected: checked once per value of the variable (one small device-to-host read)."""
+    var = getattr(layer, "g_idx", None)
+    if var is None:
+        return
+    stamp = (id(var), var.version)
+    if getattr(layer, "_g_idx_checked", None) == stamp:
+        return
+    g = as_tensor(var)
+    want = torch.floor_divide(torch.arange(g.numel(), dtype=torch.float32, device=g.device),
+                              float(block_size))
+    if g.shape != want.shape or not bool(torch.equal(g.to(torch.float32), want)):
+        raise ValueError(
+            f"{type(layer).__name__} '{layer.name}': g_idx is not floor(arange(n) / {block_size}); "
+            "group maps other than the one quantize() writes are not supported by the fused "
+            "int4 kernels")
+    layer._g_idx_checked = stamp
+
+
 class Layer:
     def __init__(self, dtype=None, name=None, device=None):
         # default name: the snake-cased class name (keras/src/utils/naming.py; the reference

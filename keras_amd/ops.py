@@ -58,6 +58,14 @@ def _arrival_counters(device, nbytes):
 INT4_ADDEND_MAX_ROWS = 64
 
 
+def _check_bias_size(bias, M, N):
+    """A bias is N values, or M x N (a row per row of the input: an addend).  Checked before
+    anything is launched: the kernels read bias[0 .. N) or [0 .. M * N) unconditionally."""
+    if bias is not None and bias.numel() != N and bias.numel() != M * N:
+        raise ValueError(f"bias holds {bias.numel()} values; the output is [{M}, {N}]: "
+                         f"expected {N} (one row) or {M * N} (a row per input row)")
+
+
 def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=None,
                 block_size=None, bias=None, plan=None, single_launch=True, addend=None):
     """`x[..., K] . W4[K, N]` for a Dense int4 kernel as the layer stores it.
@@ -87,6 +95,7 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
     if not x2.is_contiguous():
         x2 = x2.contiguous()
     M = x2.shape[0]
+    _check_bias_size(bias, M, N)
     kp = kernel_packed if kernel_packed.is_contiguous() else kernel_packed.contiguous()
     ks = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
     kz = None
@@ -162,6 +171,8 @@ def int4_matmul_multi(x, kernels, block_size=None):
             raise TypeError("kernel_scale and bias must be read in the input's dtype")
         if grouped and kz is None:
             raise ValueError("grouped int4 needs kernel_zero")
+        if bias is not None and bias.numel() != N:
+            raise ValueError(f"bias holds {bias.numel()} values, the layer has {N} units")
         kp = kp if kp.is_contiguous() else kp.contiguous()
         ks = ks if ks.is_contiguous() else ks.contiguous()
         if kz is not None and not kz.is_contiguous():
@@ -224,6 +235,8 @@ def int4_matmul_kmajor(x, kernel_kmajor, kernel_scale, kernel_zero=None, block_s
     x2 = x.reshape(-1, K)
     x2 = x2 if x2.is_contiguous() else x2.contiguous()
     M = x2.shape[0]
+    if bias is not None and bias.numel() != N:
+        raise ValueError(f"bias holds {bias.numel()} values, the layer has {N} units")
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     lib = _lib.load()
     bs = int(block_size) if grouped else -1
@@ -289,6 +302,7 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
     a = a if a.is_contiguous() else a.contiguous()
     sa = a_scale.reshape(-1).contiguous() if a_scale is not None else None
     sb = kernel_scale.reshape(-1).contiguous() if kernel_scale is not None else None
+    _check_bias_size(bias, M, N)
     y = torch.empty((M, N), dtype=out_dtype, device=a.device) if want_y else None
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if want_acc else None
     lib = _lib.load()
@@ -479,6 +493,8 @@ def int8_weight_only_matmul(x, kernel, kernel_scale, bias=None, prepacked=None):
     x2 = x.reshape(-1, K)
     x2 = x2 if x2.is_contiguous() else x2.contiguous()
     M = x2.shape[0]
+    if bias is not None and bias.numel() != N:
+        raise ValueError(f"bias holds {bias.numel()} values, the layer has {N} units")
     if prepacked is not None:
         b, layout = prepacked, 1
     else:

@@ -167,6 +167,9 @@ def test_int4_single_launch_split_matches_two_launches(dev):
         nbytes = lib.k3q_gemv_w4_workspace_bytes(M, K, N)
         assert lib.k3q_gemv_w4_counters_bytes(N) <= counters.numel()
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
+        # the fused call gets a workspace of its own, poisoned before every call: a partial it
+        # read before the store had landed would be 3.4e38, not the value the other call left
+        ws1 = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
         y2 = torch.empty((M, N), dtype=dtype, device=dev)
         y1 = torch.empty((M, N), dtype=dtype, device=dev)
         args = [_lib.ptr(x), _lib.dtype_code(dtype), M, K, N, _lib.ptr(w), _lib.ptr(sc), _lib.ptr(zp),
@@ -175,7 +178,8 @@ def test_int4_single_launch_split_matches_two_launches(dev):
         assert lib.k3q_gemv_w4(*args, _lib.ptr(y2), _lib.ptr(ws), ws.numel(), s) == 0
         for _ in range(2):
             y1.zero_()
-            assert lib.k3q_gemv_w4_fused(*args, _lib.ptr(y1), _lib.ptr(ws), ws.numel(),
+            ws1.fill_(0x7f)
+            assert lib.k3q_gemv_w4_fused(*args, _lib.ptr(y1), _lib.ptr(ws1), ws1.numel(),
                                          _lib.ptr(counters), counters.numel(), s) == 0
             torch.cuda.synchronize()
             assert torch.equal(y1, y2), (M, K, N, bs, dtype)
@@ -183,8 +187,9 @@ def test_int4_single_launch_split_matches_two_launches(dev):
 
 
 def test_int4_single_launch_split_repeated(dev):
-    # the last-arriver protocol a few hundred times per shape, other work in between: every
-    # result equals the two-launch one (a lost or stale partial would show as a different sum)
+    # the last-arriver protocol a few hundred times per shape, other work in between, a new x
+    # every time and the fused call's own workspace poisoned before each call: every result
+    # equals the two-launch one (a partial read before it landed would be 3.4e38)
     from keras_amd import _lib
     lib = _lib.load()
     counters = torch.zeros(1 << 12, dtype=torch.uint8, device=dev)
@@ -196,6 +201,7 @@ def test_int4_single_launch_split_repeated(dev):
         sc = qk["kernel_scale"].to(torch.bfloat16).to(dev)
         zp = qk["kernel_zero"].to(dev) if grouped else None
         ws = torch.empty(max(lib.k3q_gemv_w4_workspace_bytes(M, K, N), 16), dtype=torch.uint8, device=dev)
+        ws1 = torch.empty_like(ws)
         s = _lib.stream_ptr(dev)
         bad = torch.zeros((), dtype=torch.int64, device=dev)
         for it in range(300):
@@ -207,7 +213,8 @@ def test_int4_single_launch_split_repeated(dev):
             assert lib.k3q_gemv_w4(*args, _lib.ptr(y2), _lib.ptr(ws), ws.numel(), s) == 0
             if it % 3 == 0:
                 noise.mul_(1.0001)  # unrelated traffic through the caches
-            assert lib.k3q_gemv_w4_fused(*args, _lib.ptr(y1), _lib.ptr(ws), ws.numel(),
+            ws1.fill_(0x7f)
+            assert lib.k3q_gemv_w4_fused(*args, _lib.ptr(y1), _lib.ptr(ws1), ws1.numel(),
                                          _lib.ptr(counters), counters.numel(), s) == 0
             bad += (y1.view(torch.int16) != y2.view(torch.int16)).sum()
         assert int(bad) == 0
