@@ -252,6 +252,24 @@ int k3q_gemv_w4_addend(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
                        void* stream);
 
 /*
+ * k3q_gemv_w4_fused at decode sizes (M <= 16; K3Q_ERR_SHAPE beyond) for callers that cannot
+ * allocate device memory or hand a workspace in: code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc.  It calls no allocating routine.  The partial sums of
+ * the K split and the arrival counters live in a device array inside the library (16 MiB +
+ * 64 KiB per GPU the library runs on, held until the process ends) instead of `workspace` /
+ * `counters`; the same kernels, the same partials, the same summation order, the same bits.
+ * A shape whose K split needs more than k3q_gemv_w4_static_max_bytes() of partials
+ * (K split x min(M, 16) x N floats) is rejected with K3Q_ERR_WORKSPACE and nothing is launched.
+ * Every call on a GPU shares that GPU's array: calls ordered on one stream are fine, calls
+ * that overlap in time on one GPU (two streams, two host threads) race on it.
+ * No counterpart in the reference (torch's matmul owns its own scratch there).
+ */
+int64_t k3q_gemv_w4_static_max_bytes(void);
+int k3q_gemv_w4_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                       const void* w_packed, const void* scale, const void* zero,
+                       int64_t block_size, const void* bias, void* y, void* stream);
+
+/*
  * Weight-only int4 matmul for 17 ... 512 bfloat16 rows from a K-contiguous copy of the kernel:
  * the same result as k3q_gemv_w4 to the order of the fp32 sums, with the kernel read once as
  * int4 (k3q_gemv_w4's route for these sizes writes it out as bfloat16 first: nine times the

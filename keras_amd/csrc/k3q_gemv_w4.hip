@@ -44,6 +44,8 @@
 #include "k3q_common.h"
 #include "k3q_gemm_bf16.h"
 
+#include <mutex>
+
 namespace k3q {
 namespace {
 
@@ -1728,4 +1730,71 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     else
         gemv_w4_reduce<true, false><<<rgrid, 256, 0, s>>>(gp, pl.ks);
     return launch_status();
+}
+
+// ---- the decode-sized call for callers that cannot allocate -----------------------------
+// The K split's partial sums and arrival counters live in a file-scope device array instead
+// of a caller's workspace.  Every device the library runs on holds its own copy of the array
+// (until the process ends); its address on a device comes from hipGetSymbolAddress, asked
+// once per device with that device current -- the array's name is a host-side stand-in in
+// host code, not a device address.
+namespace k3q {
+namespace {
+constexpr int64_t kStaticCounterBytes = 64 * 1024;          // column blocks of N <= 2^21
+constexpr int64_t kStaticPartialBytes = 16 * 1024 * 1024;   // K split x rows x N floats
+static __device__ __align__(256) unsigned char scratch[kStaticCounterBytes + kStaticPartialBytes];
+
+constexpr int kStaticMaxDevices = 64;
+unsigned char* g_scratch_ptr[kStaticMaxDevices];  // per device, null until asked for
+std::mutex g_scratch_mutex;
+
+__global__ void clear_words(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// Address of this device's copy of `scratch`; on the first call on a device its counters are
+// also cleared on `s` (a fill kernel, not a memset node: the call may be under graph capture).
+int static_scratch(hipStream_t s, unsigned char** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) return K3Q_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        unsigned char* ptr = nullptr;
+        if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)
+            return K3Q_ERR_LAUNCH;
+        const int words = (int)(kStaticCounterBytes / 4);
+        clear_words<<<(words + 255) / 256, 256, 0, s>>>((unsigned*)ptr, words);
+        if (hipGetLastError() != hipSuccess) return K3Q_ERR_LAUNCH;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return K3Q_OK;
+}
+}  // namespace
+}  // namespace k3q
+
+extern "C" int64_t k3q_gemv_w4_static_max_bytes(void) { return kStaticPartialBytes; }
+
+extern "C" int k3q_gemv_w4_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                  const void* w_packed, const void* scale, const void* zero,
+                                  int64_t block_size, const void* bias, void* y, void* stream) {
+    if (x_dtype != K3Q_F32 && x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (M > 16) return K3Q_ERR_SHAPE;  // decode sizes only: larger M needs scratch that scales with N * K
+    if (M == 0) return K3Q_OK;
+    if (!x || !w_packed || !scale || !y) return K3Q_ERR_NULL;
+    if (block_size > 0 && !zero) return K3Q_ERR_NULL;
+    // the plan is the one k3q_gemv_w4_fused makes: same kernels, same partials, same order
+    const Plan pl = make_plan(x_dtype, M, K, N, block_size, nullptr);
+    const int64_t rows = M < pl.rows ? M : pl.rows;
+    const int64_t need = (pl.fast && pl.ks > 1) ? (int64_t)pl.ks * rows * N * 4 : 0;
+    if (need > kStaticPartialBytes || k3q_gemv_w4_counters_bytes(N) > kStaticCounterBytes)
+        return K3Q_ERR_WORKSPACE;
+    unsigned char* base = nullptr;
+    const int rc = static_scratch((hipStream_t)stream, &base);
+    if (rc != K3Q_OK) return rc;
+    return run_gemv_w4(x, x_dtype, M, K, N, w_packed, scale, zero, block_size, bias, y,
+                       base + kStaticCounterBytes, kStaticPartialBytes, nullptr, base,
+                       kStaticCounterBytes, (hipStream_t)stream);
 }
