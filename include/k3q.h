@@ -270,6 +270,49 @@ int k3q_gemv_w4_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
                        int64_t block_size, const void* bias, void* y, void* stream);
 
 /*
+ * Weight-only int4 matmul for up to 8 bfloat16 rows from a strip-linear copy of the kernel: what
+ * k3q_gemv_w4 computes (to the order of the fp32 sums), with the kernel streamed as contiguous
+ * 1 KiB pieces, all of K inside a workgroup -- no partial sums, no workspace, no counters, and
+ * nothing allocated: one launch that reads the copy once.
+ *   shadow:  k3q_w4s_shadow_bytes(K, N) bytes made by k3q_w4s_pack from the stored kernel
+ *            ([K, ceil(N/2)], low nibble = even column), once per layer.  Layout:
+ *            [strip = n / 16][unit = k / 128][lane = 64][dword = 4]; lane i + 16 g holds column
+ *            16 strip + i, its dword s the nibbles of k = 128 unit + 32 s + 8 g + e: e = 2t at bits
+ *            [4t, 4t + 4), e = 2t + 1 at bits [16 + 4t, 16 + 4t + 4) (two's-complement low four bits);
+ *            the strip count is rounded up to an even number with zero strips.
+ *   per-channel (block_size <= 0): scale = bfloat16 [N];          y = T(T(x . W) / scale[n]) (+ bias)
+ *   grouped (block_size == 128):   gparams = k3q_w4s_params_bytes bytes made by k3q_w4s_pack_params
+ *            from scale, zero [K / 128, N]: per (strip, unit) four records {4 bfloat16 scales,
+ *            4 bytes zero + 128};                                  y = T(x . ((W - zero) * scale)) (+ bias)
+ *   bias: bfloat16 [N] (bias_stride 0) or an [M, N] addend (bias_stride N), or null.
+ * Takes (k3q_gemv_w4s_supported): bfloat16 x, 1 <= M <= 8 with M * K <= 65536, K % 256 == 0,
+ * K >= 2048, N % 16 == 0, N >= 3072, block_size <= 0 or == 128; anything else K3Q_ERR_SHAPE (callers
+ * keep k3q_gemv_w4 for those).  k3q_gemv_w4s_multi: several kernels against one x (same M, K,
+ * block_size), one launch for those whose launch plans agree.
+ * Replaces what k3q_gemv_w4 replaces (keras/src/layers/core/dense.py:988-1095,
+ * keras/src/layers/core/einsum_dense.py:1120-1261).
+ */
+typedef struct {
+    int64_t N;
+    const void* shadow;
+    const void* scale;
+    const void* gparams;
+    const void* bias;
+    void* y;
+} k3q_gemv_w4s_problem;
+int64_t k3q_w4s_shadow_bytes(int64_t K, int64_t N);
+int64_t k3q_w4s_params_bytes(int64_t K, int64_t N, int64_t block_size);
+int k3q_w4s_pack(const int8_t* w_packed, int64_t K, int64_t N, void* shadow, void* stream);
+int k3q_w4s_pack_params(const void* scale, int scale_dtype, const int8_t* zero, int64_t K, int64_t N,
+                        int64_t block_size, void* params, void* stream);
+int k3q_gemv_w4s_supported(int64_t M, int64_t K, int64_t N, int64_t block_size);
+int k3q_gemv_w4s(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* shadow,
+                 const void* scale, const void* gparams, int64_t block_size, const void* bias,
+                 int64_t bias_stride, void* y, void* stream);
+int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
+                       const k3q_gemv_w4s_problem* problems, int64_t block_size, void* stream);
+
+/*
  * Weight-only int4 matmul for 17 ... 512 bfloat16 rows from a K-contiguous copy of the kernel:
  * the same result as k3q_gemv_w4 to the order of the fp32 sums, with the kernel read once as
  * int4 (k3q_gemv_w4's route for these sizes writes it out as bfloat16 first: nine times the

@@ -92,6 +92,16 @@ SIGNATURES = {
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr],
     ),
+    "k3q_w4s_shadow_bytes": (_i64, [_i64, _i64]),
+    "k3q_w4s_params_bytes": (_i64, [_i64, _i64, _i64]),
+    "k3q_w4s_pack": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "k3q_w4s_pack_params": (_int, [_ptr, _int, _ptr, _i64, _i64, _i64, _ptr, _ptr]),
+    "k3q_gemv_w4s_supported": (_int, [_i64, _i64, _i64, _i64]),
+    "k3q_gemv_w4s": (
+        _int,
+        [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr],
+    ),
+    "k3q_gemv_w4s_multi": (_int, [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr]),
     "k3q_gemm_w4_kmajor_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "k3q_gemm_w4_kmajor": (
         _int,
@@ -115,6 +125,13 @@ class GemvW4Problem(ctypes.Structure):
 
     _fields_ = [("N", ctypes.c_int64), ("w_packed", ctypes.c_void_p), ("scale", ctypes.c_void_p),
                 ("zero", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p)]
+
+
+class GemvW4sProblem(ctypes.Structure):
+    """`k3q_gemv_w4s_problem` of include/k3q.h."""
+
+    _fields_ = [("N", ctypes.c_int64), ("shadow", ctypes.c_void_p), ("scale", ctypes.c_void_p),
+                ("gparams", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p)]
 
 
 _lib = None

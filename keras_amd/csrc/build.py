@@ -18,6 +18,7 @@ SOURCES = [
     "k3q_pack.hip",
     "k3q_quantize.hip",
     "k3q_gemv_w4.hip",
+    "k3q_gemv_w4s.hip",
     "k3q_gemv_w4_nk.hip",
     "k3q_gemv_w8.hip",
     "k3q_gemm_i8.hip",

@@ -1,0 +1,635 @@
+// Weight-only int4 decode matmul from a strip-linear copy of the kernel: y[M,N] = x[M,K] . W4[K,N], M <= 8.
+//
+// The layer's stored kernel ([K, ceil(N/2)] bytes, two output columns per byte) makes a workgroup
+// read 128-byte pieces at a 4 KiB stride and needs a split of K over workgroups to fill the chip.
+// This kernel reads a second copy, laid out for the decode access pattern and made once per layer
+// (k3q_w4s_pack):
+//
+//   [strip = n / 16][unit = k / 128][lane = 64][dword = 4]            1 KiB per (strip, unit)
+//   lane = i + 16 g holds column n = 16 strip + i; its dword s holds the 8 nibbles of
+//   k = 128 unit + 32 s + 8 g + e, e = 2t at bits [4t, 4t + 4), e = 2t + 1 at bits [16 + 4t, ...).
+//
+// A wave's 16-byte-per-lane load of one unit is then 1 KiB of contiguous memory AND, dword by
+// dword, the A operand of four v_mfma_f32_16x16x32_bf16 steps: ((d >> 4t) & 0x000F000F) ^ 0x43084308
+// is the bfloat16 pair (136 + w[k = ..2t], 136 + w[k = ..2t+1]) of column i.  A strip's units follow
+// each other in memory, so a wave streams a contiguous run and a workgroup (one or two strips, all
+// of K) a contiguous region; nothing is exchanged between workgroups, no partial sums leave the CU.
+//
+// x is staged once per workgroup in LDS (rows padded by 16 bytes: the sixteen lanes of a B-operand
+// read then hit disjoint banks) and read back as MFMA B operands, reused for both strips of a wave.
+// An all-ones A operand accumulates the sum of x over the same k, which removes the +136 offset
+// (grouped: the zero point as well, per group of 128 = one unit).
+//
+// Scheduling facts this kernel is built on (measured on MI355X):
+//  * the waits the compiler places around loads that are issued conditionally, or around LDS-DMA
+//    mixed with register loads, drain the whole queue: every load here is unconditional (addresses
+//    clamped instead) and goes through registers;
+//  * a slot of the weight ring is refilled right after its conversion, which is interleaved with the
+//    previous unit's MFMAs (sched_group_barrier), so that the request stream never waits for the
+//    matrix pipe;
+//  * x is requested before any weight: requested after them it would arrive behind the whole first
+//    burst of weights (the memory system serves a launch's first requests roughly in order).
+#include "k3q_common.h"
+
+#include <mutex>
+#include <set>
+#include <type_traits>
+
+namespace k3q {
+namespace {
+
+constexpr int kQ = 8;            // waves per workgroup = slices of K
+constexpr int kT = kQ * 64;      // threads
+constexpr int kMaxRows = 8;      // rows of x
+constexpr int kMaxPieces = 16;   // 16-byte pieces of x a thread stages: M * K <= 16 * 8 * kT
+constexpr int kRedStride = 20;   // floats per (row, strip) line of the cross-wave reduction
+constexpr int kMaxProblems = 4;
+
+struct W4sParams {
+    const uint16_t* x;       // [M, K] bf16
+    const v4u* w;            // strip-linear copy
+    const uint16_t* scale;   // per-channel: bf16 [N]
+    const uint8_t* gparams;  // grouped/128: [strip][unit][4][{4 bf16 scales, 4 (zero + 128)}] = 48 B
+    const uint16_t* bias;    // bf16 [N] or [M, N], or null
+    uint16_t* y;             // [M, N] bf16
+    int64_t bias_stride;     // 0 or N
+    int M, K, N, units;      // units = K / 128
+    int row_magic;           // ceil(2^32 / (K / 8)): piece -> row without a division
+};
+
+struct W4sMulti {
+    W4sParams p[kMaxProblems];
+    int first[kMaxProblems + 1];  // first blockIdx.x of each problem, then the end
+    int count;
+};
+
+__device__ __forceinline__ v8bf as_bf8(const v4u& v) { return __builtin_bit_cast(v8bf, v); }
+__device__ __forceinline__ float bf_lo(u32 d) { return __uint_as_float(d << 16); }
+__device__ __forceinline__ float bf_hi(u32 d) { return __uint_as_float(d & 0xffff0000u); }
+
+// kSW strips per wave (2: the x fragments serve two strips), ring of kD units (2 or 4), kNP staged
+// pieces of x per thread, kGrouped: groups of 128 with zero points.
+// A workgroup takes strip groups `block`, `block + stride`, ... one after the other as ONE stream of
+// units: the ring runs across the boundary (the last bodies of a group convert and request the
+// first units of the next), so that a workgroup pays the memory latency once, not once per group.
+template <int kSW, int kD, int kNP, bool kGrouped>
+__device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int block, const int stride) {
+    extern __shared__ __attribute__((aligned(16))) char w4s_lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int q = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int units = p.units;
+    const int M = p.M, K = p.K;
+    const int j = lane & 15, g = lane >> 4;
+    const int jj = j < M ? j : M - 1;
+    const int groups = (p.N / 16 + kSW - 1) / kSW;
+    // slices of K: whole blocks of kD units, the first (blocks % kQ) waves take one more
+    const int blocks = units / kD;
+    const int base = blocks / kQ, extra = blocks - base * kQ;
+    const int U = (base + (q < extra ? 1 : 0)) * kD;
+    const int u0 = (q * base + (q < extra ? q : extra)) * kD;
+    const int R = U / kD;  // >= 2 (the launch plan sees to it)
+    const int pitch = K * 2 + 16;
+    float* red = (float*)(w4s_lds + ((M * pitch + 255) & ~255));  // two buffers, one per parity of the turn
+
+    // ---- x into registers first (every load unconditional: pieces past the end re-read piece 0) ----
+    const int per_row = K >> 3;
+    const int pieces = M * per_row;
+    v4u xst[kNP];
+#pragma unroll
+    for (int i = 0; i < kNP; ++i) {
+        const int pi = i * kT + tid;
+        xst[i] = *(const v4u*)(p.x + (int64_t)(pi < pieces ? pi : 0) * 8);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // weights and grouped parameters of a strip group at this wave's slice: wave-uniform bases (scalar
+    // registers), the lane's part is added at the load
+    auto w_base = [&](const int grp, const int t) {
+        return (const char*)p.w + ((int64_t)(grp * kSW + t) * units + u0) * 1024;
+    };
+    auto z_base = [&](const int grp, const int t) {
+        return (const char*)p.gparams + ((int64_t)(grp * kSW + t) * units + u0) * 48;
+    };
+    const int lane_w = lane * 16, lane_z = 12 * g;
+    const char* wp[kSW];   // the group being computed
+    const char* wn[kSW];   // the group after it (the last group: itself)
+    const char* zp[kSW];
+    const char* zn[kSW];
+#pragma unroll
+    for (int t = 0; t < kSW; ++t) {
+        wp[t] = w_base(block, t);
+        zp[t] = z_base(block, t);
+    }
+    v4u W[kD][kSW];
+    u32 Z[kGrouped ? kD : 1][kSW][3];
+    // unit u of the group being computed, or (u >= U) unit u - U of the one after it: one
+    // unconditional load either way, the base chosen by a select
+    auto fetch = [&](const int d, const int u) {
+        const bool own = u < U;
+        const int64_t uu = own ? u : u - U;
+#pragma unroll
+        for (int t = 0; t < kSW; ++t)
+            W[d][t] = __builtin_nontemporal_load((const v4u*)((own ? wp[t] : wn[t]) + uu * 1024 + lane_w));
+        if constexpr (kGrouped) {
+#pragma unroll
+            for (int t = 0; t < kSW; ++t) {
+                const u32* z = (const u32*)((own ? zp[t] : zn[t]) + uu * 48 + lane_z);
+                Z[d][t][0] = z[0];
+                Z[d][t][1] = z[1];
+                Z[d][t][2] = z[2];
+            }
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < kSW; ++t) {
+        wn[t] = wp[t];
+        zn[t] = zp[t];
+    }
+#pragma unroll
+    for (int d = 0; d < kD; ++d) fetch(d, d);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- x into LDS: the stores wait for the x loads only (they are the older ones) ----
+#pragma unroll
+    for (int i = 0; i < kNP; ++i) {
+        const int pi = i * kT + tid;
+        if (pi < pieces) {
+            const int m = (int)__umulhi((unsigned)pi, (unsigned)p.row_magic);
+            const int c = pi - m * per_row;
+            *(v4u*)(w4s_lds + m * pitch + c * 16) = xst[i];
+        }
+    }
+    __syncthreads();
+
+    const char* xrow = w4s_lds + jj * pitch + u0 * 256 + g * 16;
+    const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
+    v4f acc[2][kSW][2], accs[2], tot[kSW];
+    u32 Zk[2][kSW][3];
+    v4u av[2][kSW][4], xf[2][4];
+
+    auto cvt1 = [&](const u32 w, v4u& out) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = ((w >> (4 * e)) & 0x000F000Fu) ^ 0x43084308u;
+    };
+    auto read_x = [&](const int b, const int i) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) xf[b][s] = *(const v4u*)(xrow + i * 256 + s * 64);
+    };
+    // grouped: tot += scale * (acc - (136 + zero) * sum(x)) for the unit in buffers a
+    auto fold = [&](const int a) {
+#pragma unroll
+        for (int t = 0; t < kSW; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float sc = (r & 1) ? bf_hi(Zk[a][t][r >> 1]) : bf_lo(Zk[a][t][r >> 1]);
+                const float zf = (float)((Zk[a][t][2] >> (8 * r)) & 0xffu) + 8.0f;
+                tot[t][r] += sc * ((acc[a][t][0][r] + acc[a][t][1][r]) - zf * accs[a][r]);
+            }
+    };
+    // Unit i of the group (slot d, buffers b = d & 1): its MFMAs, interleaved with the conversion of
+    // the unit after it (slot dn; after the group's last unit: the next group's first).  Halfway, the
+    // fold of unit i - 1, whose MFMAs are long done; after it that unit's parameter buffer takes those
+    // of the unit after.  Then slot dn is requested again: unit i + 1 + kD, from the next group if past
+    // the end of this one.
+    auto body = [&](auto d_c, const int i, auto has_next_c, auto do_refill_c, const bool fold_prev) {
+        constexpr int d = decltype(d_c)::value;
+        constexpr bool has_next = decltype(has_next_c)::value, do_refill = decltype(do_refill_c)::value;
+        constexpr int b = d & 1, dn = (d + 1) % kD;
+        constexpr int ab = kGrouped ? b : 0;
+        if (has_next) read_x(b ^ 1, i + 1 < U ? i + 1 : 0);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const bool fresh_s = kGrouped && s == 0, fresh_a = kGrouped && s < 2;  // (constant once unrolled)
+            accs[ab] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf8(ones), as_bf8(xf[b][s]),
+                                                               fresh_s ? zero4 : accs[ab], 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < kSW; ++t)
+                acc[ab][t][s & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    as_bf8(av[b][t][s]), as_bf8(xf[b][s]), fresh_a ? zero4 : acc[ab][t][s & 1], 0, 0, 0);
+            if (has_next) {
+#pragma unroll
+                for (int t = 0; t < kSW; ++t) cvt1(W[dn][t][s], av[b ^ 1][t][s]);
+            }
+            if (s == 1) {
+                if (kGrouped && fold_prev) fold(b ^ 1);
+                if constexpr (kGrouped && has_next) {
+#pragma unroll
+                    for (int t = 0; t < kSW; ++t)
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) Zk[b ^ 1][t][c] = Z[dn][t][c];
+                }
+            }
+        }
+        if (has_next) {
+            // per step: (1 + kSW) MFMAs against 7 kSW conversions
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kSW == 2 ? 5 : 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kSW == 2 ? 5 : 3, 0);
+                if (kSW == 2) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (do_refill) fetch(dn, i + 1 + kD);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::bool_constant;
+    using std::integral_constant;
+    auto round = [&](auto last_c, const int r) {
+        constexpr bool last = decltype(last_c)::value;  // last round of the last group: nothing follows
+        const int i0 = r * kD;
+        body(integral_constant<int, 0>{}, i0, bool_constant<true>{}, bool_constant<!last>{}, r > 0);
+        if constexpr (kD == 2) {
+            body(integral_constant<int, 1>{}, i0 + 1, bool_constant<!last>{}, bool_constant<!last>{}, true);
+        } else {
+            body(integral_constant<int, 1>{}, i0 + 1, bool_constant<true>{}, bool_constant<!last>{}, true);
+            body(integral_constant<int, 2>{}, i0 + 2, bool_constant<true>{}, bool_constant<!last>{}, true);
+            body(integral_constant<int, 3>{}, i0 + 3, bool_constant<!last>{}, bool_constant<!last>{}, true);
+        }
+    };
+
+    // prologue: unit 0 converted, its x fragments read, its slot requested again
+    read_x(0, 0);
+#pragma unroll
+    for (int t = 0; t < kSW; ++t)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) cvt1(W[0][t][s], av[0][t][s]);
+    if constexpr (kGrouped) {
+#pragma unroll
+        for (int t = 0; t < kSW; ++t)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) Zk[0][t][c] = Z[0][t][c];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(0, kD);  // (U >= 2 kD)
+    __builtin_amdgcn_sched_barrier(0);
+
+    u32 esc[kSW][2], ebi[kSW][2];
+    // a group's set-up: where the group after it lies, fresh sums, and the epilogue's operands
+    // requested now rather than at the end of the group's stream
+    auto begin = [&](const int grp, const int nxt_grp) {
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) {
+            wn[t] = w_base(nxt_grp, t);
+            zn[t] = z_base(nxt_grp, t);
+            tot[t] = zero4;
+        }
+        if (!kGrouped) {  // (grouped: every unit starts its own accumulators)
+            accs[0] = zero4;
+#pragma unroll
+            for (int t = 0; t < kSW; ++t) acc[0][t][0] = acc[0][t][1] = zero4;
+        }
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) {
+            int n = (grp * kSW + t) * 16 + 4 * g;
+            n = n < p.N ? n : p.N - 4;  // N % 16 == 0: a valid stand-in, never stored
+            esc[t][0] = esc[t][1] = 0;
+            if (!kGrouped) {
+                const v2u v = *(const v2u*)(p.scale + n);
+                esc[t][0] = v[0];
+                esc[t][1] = v[1];
+            }
+            // (no bias: the load still happens, from x, and is ignored -- a branch around a load costs
+            // the loads behind it their place in the compiler's wait counts)
+            const uint16_t* src = p.bias ? p.bias + (int64_t)jj * p.bias_stride + n : p.x;
+            const v2u v = *(const v2u*)src;
+            ebi[t][0] = v[0];
+            ebi[t][1] = v[1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // a group's end: the slices of K meet in LDS (fixed order), wave 0 applies the layer's epilogue
+    auto finish = [&](const int grp, const int turn) {
+        if (kGrouped) {
+            fold((kD - 1) & 1);
+        } else {
+#pragma unroll
+            for (int t = 0; t < kSW; ++t)
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr)
+                    tot[t][rr] = (acc[0][t][0][rr] + acc[0][t][1][rr]) - 136.0f * accs[0][rr];
+        }
+        float* rbuf = red + (turn & 1) * ((kQ - 1) * kSW * M * kRedStride);  // rows of x only
+        if (q > 0 && j < M) {
+#pragma unroll
+            for (int t = 0; t < kSW; ++t)
+                *(v4f*)(rbuf + (((q - 1) * kSW + t) * M + j) * kRedStride + 4 * g) = tot[t];
+        }
+        __syncthreads();
+        if (q == 0 && j < M) {
+#pragma unroll
+            for (int t = 0; t < kSW; ++t) {
+#pragma unroll
+                for (int qq = 1; qq < kQ; ++qq)
+                    tot[t] += *(const v4f*)(rbuf + (((qq - 1) * kSW + t) * M + j) * kRedStride + 4 * g);
+                const int n = (grp * kSW + t) * 16 + 4 * g;
+                if (n >= p.N) continue;
+                u32 o[4];
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    float v = round_bf16(tot[t][rr]);
+                    if (!kGrouped)
+                        v = round_bf16(v / ((rr & 1) ? bf_hi(esc[t][rr >> 1]) : bf_lo(esc[t][rr >> 1])));
+                    if (p.bias) v = round_bf16(v + ((rr & 1) ? bf_hi(ebi[t][rr >> 1]) : bf_lo(ebi[t][rr >> 1])));
+                    o[rr] = f32_to_bf16_bits(v);
+                }
+                const v2u ov = {o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+                *(v2u*)(p.y + (int64_t)j * p.N + n) = ov;
+            }
+        }
+    };
+
+    int turn = 0;
+    int grp = block;
+    // every group but the workgroup's last: all rounds request and convert ahead, into the next group
+    for (; grp + stride < groups; grp += stride, ++turn) {
+        begin(grp, grp + stride);
+        for (int r = 0; r < R; ++r) round(bool_constant<false>{}, r);
+        finish(grp, turn);
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) {
+            wp[t] = wn[t];
+            zp[t] = zn[t];
+        }
+    }
+    // the last group: its last round has nothing to request or convert (the one request before it that
+    // falls past the end re-reads the group's first unit: never used)
+    begin(grp, grp);
+    for (int r = 0; r < R - 1; ++r) round(bool_constant<false>{}, r);
+    round(bool_constant<true>{}, R - 1);
+    finish(grp, turn);
+}
+
+template <int kSW, int kD, int kNP, bool kGrouped>
+__global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
+    const int bx = blockIdx.x;
+    int i = 0;
+    while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
+    gemv_w4s_body<kSW, kD, kNP, kGrouped>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
+}
+
+// ---- the strip-linear copy ---------------------------------------------------------------
+// One thread per dword of the copy; strips past N (the copy holds an even number of strips) are zero.
+__global__ __launch_bounds__(256) void w4s_pack(const uint8_t* __restrict__ w, u32* __restrict__ out,
+                                                int64_t K, int64_t N, int64_t strips_padded) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t units = K / 128;
+    if (idx >= strips_padded * units * 256) return;
+    const int s = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
+    const int64_t su = idx >> 8, unit = su % units, strip = su / units;
+    const int i = lane & 15, g = lane >> 4;
+    const int64_t n = strip * 16 + i;
+    u32 d = 0;
+    if (n < N) {
+        const int64_t row_bytes = (N + 1) / 2;
+        const int shift = (n & 1) ? 4 : 0;
+        const int64_t k0 = unit * 128 + 32 * s + 8 * g;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const u32 nib = (w[(k0 + e) * row_bytes + (n >> 1)] >> shift) & 0xFu;
+            d |= nib << ((e & 1) ? 16 + 4 * (e >> 1) : 4 * (e >> 1));
+        }
+    }
+    out[idx] = d;
+}
+
+// grouped parameters: [strip][unit][c = 4]{scale[4 c .. 4 c + 3] bf16, (zero + 128)[4 c .. 4 c + 3]}
+template <bool kBF16>
+__global__ __launch_bounds__(256) void w4s_pack_params(const void* __restrict__ scale,
+                                                       const int8_t* __restrict__ zero,
+                                                       uint8_t* __restrict__ out, int64_t units, int64_t N,
+                                                       int64_t strips_padded) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (strip, unit, c)
+    if (idx >= strips_padded * units * 4) return;
+    const int c = (int)(idx & 3);
+    const int64_t su = idx >> 2, unit = su % units, strip = su / units;
+    u32 rec[3] = {0, 0, 0x80808080u};
+    const int64_t n = strip * 16 + 4 * c;
+    if (n < N) {  // N % 16 == 0: four columns in or out together
+        u32 h[4], z = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int64_t o = unit * N + n + e;
+            h[e] = kBF16 ? (u32)((const uint16_t*)scale)[o] : f32_to_bf16_bits(((const float*)scale)[o]);
+            z |= ((u32)(uint8_t)(zero[o] ^ 0x80)) << (8 * e);  // zero + 128 as an unsigned byte
+        }
+        rec[0] = h[0] | (h[1] << 16);
+        rec[1] = h[2] | (h[3] << 16);
+        rec[2] = z;
+    }
+    u32* dst = (u32*)(out + idx * 12);
+    dst[0] = rec[0];
+    dst[1] = rec[1];
+    dst[2] = rec[2];
+}
+
+inline int64_t strips_padded(int64_t N) { return ((N + 15) / 16 + 1) / 2 * 2; }
+
+struct W4sPlan {
+    bool ok;
+    int sw, d, np;
+    int64_t groups;  // strip groups (kSW strips each)
+    int64_t blocks;  // workgroups: each takes groups block, block + blocks, ...
+    size_t lds;
+};
+
+constexpr int kResident = 256;  // workgroups the chip holds at once: one per CU (registers)
+
+W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
+    W4sPlan pl{};
+    const bool grouped = block_size > 0;
+    if (M < 1 || M > kMaxRows || (K % 128) != 0 || (N % 16) != 0) return pl;
+    if (grouped && block_size != 128) return pl;
+    const int64_t units = K / 128, strips = N / 16;
+    if (M * K > (int64_t)kMaxPieces * 8 * kT) return pl;
+    // all of K stays inside a workgroup, so the strips alone have to fill the chip
+    if (strips < 192) return pl;
+    // every wave walks at least two rounds of the ring
+    if ((units % 4) == 0 && units / 4 >= 2 * kQ) pl.d = 4;
+    else if ((units % 2) == 0 && units / 2 >= 2 * kQ) pl.d = 2;
+    else return pl;
+    pl.sw = strips >= 2 * kResident ? 2 : 1;
+    const int64_t pieces = M * K / 8;
+    pl.np = pieces <= 2 * kT ? 2 : pieces <= 4 * kT ? 4 : pieces <= 8 * kT ? 8 : 16;
+    pl.groups = (strips + pl.sw - 1) / pl.sw;
+    // more groups than the chip holds workgroups: each workgroup takes several, one after the other
+    const int64_t turns = (pl.groups + kResident - 1) / kResident;
+    pl.blocks = (pl.groups + turns - 1) / turns;
+    pl.lds = (size_t)((M * (K * 2 + 16) + 255) & ~255) + (size_t)2 * (kQ - 1) * pl.sw * M * kRedStride * 4;
+    pl.ok = pl.lds <= 160 * 1024;
+    return pl;
+}
+
+using W4sKernel = void (*)(W4sMulti);
+
+template <int kSW, int kD, bool kGrouped>
+W4sKernel pick_np(int np) {
+    switch (np) {
+        case 2: return gemv_w4s<kSW, kD, 2, kGrouped>;
+        case 4: return gemv_w4s<kSW, kD, 4, kGrouped>;
+        case 8: return gemv_w4s<kSW, kD, 8, kGrouped>;
+        default: return gemv_w4s<kSW, kD, 16, kGrouped>;
+    }
+}
+
+W4sKernel pick_kernel(const W4sPlan& pl, bool grouped) {
+    if (pl.sw == 2) {
+        if (pl.d == 4) return grouped ? pick_np<2, 4, true>(pl.np) : pick_np<2, 4, false>(pl.np);
+        return grouped ? pick_np<2, 2, true>(pl.np) : pick_np<2, 2, false>(pl.np);
+    }
+    if (pl.d == 4) return grouped ? pick_np<1, 4, true>(pl.np) : pick_np<1, 4, false>(pl.np);
+    return grouped ? pick_np<1, 2, true>(pl.np) : pick_np<1, 2, false>(pl.np);
+}
+
+int fill_params(W4sParams& p, const void* x, int64_t M, int64_t K, int64_t N, const void* shadow,
+                const void* scale, const void* gparams, int64_t block_size, const void* bias,
+                int64_t bias_stride, void* y) {
+    const bool grouped = block_size > 0;
+    if (!x || !shadow || !y || (grouped ? !gparams : !scale)) return K3Q_ERR_NULL;
+    if (!aligned_to(x, 16) || !aligned_to(shadow, 16) || !aligned_to(y, 8) || (scale && !aligned_to(scale, 8)) ||
+        (gparams && !aligned_to(gparams, 4)) || (bias && !aligned_to(bias, 8)))
+        return K3Q_ERR_ALIGN;
+    p.x = (const uint16_t*)x;
+    p.w = (const v4u*)shadow;
+    p.scale = (const uint16_t*)scale;
+    p.gparams = (const uint8_t*)gparams;
+    p.bias = (const uint16_t*)bias;
+    p.y = (uint16_t*)y;
+    p.bias_stride = bias ? bias_stride : 0;
+    p.M = (int)M;
+    p.K = (int)K;
+    p.N = (int)N;
+    p.units = (int)(K / 128);
+    const uint64_t per_row = (uint64_t)K / 8;
+    p.row_magic = (int)(uint32_t)((((uint64_t)1 << 32) + per_row - 1) / per_row);
+    return K3Q_OK;
+}
+
+int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_blocks, hipStream_t s) {
+    const W4sKernel kernel = pick_kernel(pl, grouped);
+    // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+    {
+        static std::mutex mu;
+        static std::set<const void*> raised;
+        std::lock_guard<std::mutex> lock(mu);
+        if (!raised.count((const void*)kernel)) {
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    160 * 1024) != hipSuccess)
+                return K3Q_ERR_LAUNCH;
+            raised.insert((const void*)kernel);
+        }
+    }
+    kernel<<<(unsigned)total_blocks, kT, pl.lds, s>>>(mp);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace k3q
+
+using namespace k3q;
+
+extern "C" int64_t k3q_w4s_shadow_bytes(int64_t K, int64_t N) {
+    if (K <= 0 || N <= 0 || (K % 128) != 0) return 0;
+    return strips_padded(N) * (K / 128) * 1024;
+}
+
+extern "C" int64_t k3q_w4s_params_bytes(int64_t K, int64_t N, int64_t block_size) {
+    if (K <= 0 || N <= 0 || (K % 128) != 0 || block_size != 128) return 0;
+    return strips_padded(N) * (K / 128) * 48;
+}
+
+extern "C" int k3q_w4s_pack(const int8_t* w_packed, int64_t K, int64_t N, void* shadow, void* stream) {
+    if (K <= 0 || N <= 0 || (K % 128) != 0) return K3Q_ERR_SHAPE;
+    if (!w_packed || !shadow) return K3Q_ERR_NULL;
+    if (!aligned_to(shadow, 16)) return K3Q_ERR_ALIGN;
+    const int64_t dwords = k3q_w4s_shadow_bytes(K, N) / 4;
+    w4s_pack<<<(unsigned)((dwords + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint8_t*)w_packed, (u32*)shadow, K, N, strips_padded(N));
+    return launch_status();
+}
+
+extern "C" int k3q_w4s_pack_params(const void* scale, int scale_dtype, const int8_t* zero, int64_t K,
+                                   int64_t N, int64_t block_size, void* params, void* stream) {
+    if (K <= 0 || N <= 0 || (K % 128) != 0 || (N % 16) != 0 || block_size != 128) return K3Q_ERR_SHAPE;
+    if (scale_dtype != K3Q_F32 && scale_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (!scale || !zero || !params) return K3Q_ERR_NULL;
+    if (!aligned_to(params, 4)) return K3Q_ERR_ALIGN;
+    const int64_t recs = strips_padded(N) * (K / 128) * 4;
+    const unsigned grid = (unsigned)((recs + 255) / 256);
+    if (scale_dtype == K3Q_BF16)
+        w4s_pack_params<true><<<grid, 256, 0, (hipStream_t)stream>>>(scale, zero, (uint8_t*)params, K / 128, N,
+                                                                      strips_padded(N));
+    else
+        w4s_pack_params<false><<<grid, 256, 0, (hipStream_t)stream>>>(scale, zero, (uint8_t*)params, K / 128, N,
+                                                                       strips_padded(N));
+    return launch_status();
+}
+
+extern "C" int k3q_gemv_w4s_supported(int64_t M, int64_t K, int64_t N, int64_t block_size) {
+    return w4s_plan(M, K, N, block_size).ok ? 1 : 0;
+}
+
+extern "C" int k3q_gemv_w4s(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* shadow,
+                            const void* scale, const void* gparams, int64_t block_size, const void* bias,
+                            int64_t bias_stride, void* y, void* stream) {
+    if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (bias_stride != 0 && bias_stride != N) return K3Q_ERR_SHAPE;
+    const W4sPlan pl = w4s_plan(M, K, N, block_size);
+    if (!pl.ok) return K3Q_ERR_SHAPE;
+    W4sMulti mp{};
+    const int rc = fill_params(mp.p[0], x, M, K, N, shadow, scale, gparams, block_size, bias, bias_stride, y);
+    if (rc != K3Q_OK) return rc;
+    mp.first[0] = 0;
+    mp.first[1] = (int)pl.blocks;
+    mp.count = 1;
+    return launch_w4s(pl, block_size > 0, mp, (int)pl.blocks, (hipStream_t)stream);
+}
+
+extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
+                                  const k3q_gemv_w4s_problem* problems, int64_t block_size, void* stream) {
+    if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (count < 0 || M < 0 || K <= 0) return K3Q_ERR_SHAPE;
+    if (count == 0 || M == 0) return K3Q_OK;
+    if (!problems) return K3Q_ERR_NULL;
+    hipStream_t s = (hipStream_t)stream;
+    int at = 0;
+    while (at < count) {
+        // problems whose plans agree share a launch, up to kMaxProblems at a time
+        W4sMulti mp{};
+        W4sPlan pl0{};
+        int64_t groups[kMaxProblems], total = 0;
+        int n = 0;
+        for (; at + n < count && n < kMaxProblems; ++n) {
+            const k3q_gemv_w4s_problem& q = problems[at + n];
+            if (q.N <= 0) return K3Q_ERR_SHAPE;
+            const W4sPlan pl = w4s_plan(M, K, q.N, block_size);
+            if (!pl.ok) return K3Q_ERR_SHAPE;
+            if (n == 0) pl0 = pl;
+            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np) break;
+            const int rc = fill_params(mp.p[n], x, M, K, q.N, q.shadow, q.scale, q.gparams, block_size, q.bias,
+                                       0, q.y);
+            if (rc != K3Q_OK) return rc;
+            groups[n] = pl.groups;
+            total += pl.groups;
+        }
+        // the launch as a whole is cut for the chip: about kResident workgroups, each problem its share
+        const int64_t turns = (total + kResident - 1) / kResident;
+        int next_block = 0;
+        for (int i = 0; i < n; ++i) {
+            mp.first[i] = next_block;
+            next_block += (int)((groups[i] + turns - 1) / turns);
+        }
+        mp.first[n] = next_block;
+        mp.count = n;
+        const int rc = launch_w4s(pl0, block_size > 0, mp, next_block, s);
+        if (rc != K3Q_OK) return rc;
+        at += n;
+    }
+    return K3Q_OK;
+}

@@ -248,6 +248,28 @@ class Dense(Layer):
         cd = to_torch_dtype(self.compute_dtype)
         return self._cached(key, var, lambda t: t.to(cd).contiguous())
 
+    def _strip_operands(self, rows, input_dim, units, grouped, block_size):
+        """The operands of the strip-linear decode route (`ops.int4_matmul_strip`) when it takes
+        `rows` bfloat16 rows of this layer, else None: the copy of the kernel it streams and, for
+        grouped kernels, the re-ordered scales / zero points -- made on first use, kept while the
+        variables they come from do not change."""
+        if not (0 < rows <= kops.STRIP_MAX_ROWS and to_torch_dtype(self.compute_dtype) == torch.bfloat16
+                and kops.int4_strip_supported(rows, input_dim, units, block_size if grouped else None)):
+            return None
+        spec = dict(units=units,
+                    shadow=self._cached("w4s", self._kernel, lambda t: kops.int4_strip_copy(t, units)))
+        if grouped:
+            scale, zero = self.kernel_scale, self.kernel_zero
+            stamp = (id(scale), scale.version, id(zero), zero.version)
+            hit = self._cache.get("w4s_params")
+            if hit is None or hit[0] != stamp:
+                value = kops.int4_strip_params(as_tensor(scale), as_tensor(zero), input_dim, units, block_size)
+                hit = self._cache["w4s_params"] = (stamp, None, value)
+            spec["gparams"] = hit[2]
+        else:
+            spec["kernel_scale"] = self._read_cached("kernel_scale", self.kernel_scale)
+        return spec
+
     # ---- quantized forward --------------------------------------------------------
     def _int8_call(self, inputs, training=None):
         """keras/src/layers/core/dense.py:938-986: quantise rows, int8 GEMM, de-scale, bias."""
@@ -316,7 +338,18 @@ class Dense(Layer):
         if grouped:
             require_default_g_idx(self, block_size)
         rows = inputs.numel() // inputs.shape[-1] if inputs.shape[-1] else 0
-        if (inputs.dtype == torch.bfloat16 and kmajor_rows(rows, self._orig_output_dim, inputs.shape[-1])
+        strip = (self._strip_operands(rows, inputs.shape[-1], self._orig_output_dim, grouped, block_size)
+                 if inputs.dtype == torch.bfloat16 else None)
+        if strip is not None:
+            # decode sizes: the strip-linear copy of the kernel, streamed once, all of K inside a
+            # workgroup (one launch, no scratch)
+            bias = self._call_bias()
+            per_row = bias is not None and rows > 1 and bias.numel() == rows * self._orig_output_dim
+            y = kops.int4_matmul_strip(
+                inputs, strip["shadow"], self._orig_output_dim, kernel_scale=strip.get("kernel_scale"),
+                gparams=strip.get("gparams"), block_size=block_size if grouped else None,
+                bias=None if per_row else bias, addend=bias if per_row else None)
+        elif (inputs.dtype == torch.bfloat16 and kmajor_rows(rows, self._orig_output_dim, inputs.shape[-1])
                 and kops.int4_kmajor_supported(rows, inputs.shape[-1], self._orig_output_dim,
                                                block_size if grouped else None)):
             # a few dozen to a hundred-odd rows: from the K-contiguous copy of the kernel (made
@@ -373,8 +406,13 @@ class Dense(Layer):
             y = y2.reshape(*lead, self._orig_output_dim)
             return self.activation(y) if self.activation is not None else y
 
+        x2 = inputs.reshape(-1, inputs.shape[-1])
+        strip = (self._strip_operands(x2.shape[0], x2.shape[1], self._orig_output_dim, grouped, block_size)
+                 if x2.dtype == torch.bfloat16 else None)
+        if strip is not None:
+            strip["bias"] = self._call_bias()
         return dict(
-            x2=inputs.reshape(-1, inputs.shape[-1]), block_size=block_size if grouped else None,
+            x2=x2, block_size=block_size if grouped else None, strip=strip,
             kernel=dict(kernel_packed=as_tensor(self._kernel),
                         kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
                         units=self._orig_output_dim,

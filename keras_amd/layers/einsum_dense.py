@@ -390,6 +390,27 @@ class EinsumDense(Layer):
             raise self._gemm_error
         return self._gemm
 
+    def _strip_operands(self, rows, input_dim, units, grouped, block_size):
+        """As Dense._strip_operands: the operands of the strip-linear decode route, or None."""
+        cd = to_torch_dtype(self.compute_dtype)
+        if not (0 < rows <= kops.STRIP_MAX_ROWS and cd == torch.bfloat16
+                and kops.int4_strip_supported(rows, input_dim, units, block_size if grouped else None)):
+            return None
+        spec = dict(units=units,
+                    shadow=self._cached("w4s", self._kernel, lambda t: kops.int4_strip_copy(t, units)))
+        if grouped:
+            scale, zero = self.kernel_scale, self.kernel_zero
+            stamp = (id(scale), scale.version, id(zero), zero.version)
+            hit = self._cache.get("w4s_params")
+            if hit is None or hit[0] != stamp:
+                value = kops.int4_strip_params(as_tensor(scale), as_tensor(zero), input_dim, units, block_size)
+                hit = self._cache["w4s_params"] = (stamp, None, value)
+            spec["gparams"] = hit[2]
+        else:
+            spec["kernel_scale"] = self._cached("kernel_scale", self.kernel_scale,
+                                                lambda t: t.to(cd).reshape(-1).contiguous())
+        return spec
+
     def _input_rows(self, inputs, gv):
         x = inputs if gv.in_is_view else inputs.permute(gv.in_perm)
         k = 1
@@ -514,6 +535,16 @@ class EinsumDense(Layer):
         from keras_amd.layers.dense import kmajor_rows
 
         units = self._int4_unpacked_column_size
+        strip = (self._strip_operands(x2.shape[0], x2.shape[1], units, grouped, block_size)
+                 if x2.dtype == torch.bfloat16 else None)
+        if strip is not None:
+            # decode sizes: the strip-linear copy of the kernel (one launch, no scratch)
+            per_row = bias is not None and x2.shape[0] > 1 and bias.numel() == x2.shape[0] * units
+            y2 = kops.int4_matmul_strip(
+                x2, strip["shadow"], units, kernel_scale=strip.get("kernel_scale"),
+                gparams=strip.get("gparams"), block_size=block_size if grouped else None,
+                bias=None if per_row else bias, addend=bias if per_row else None)
+            return self._finish(y2, free_shape, gv, fused)
         if (x2.dtype == torch.bfloat16 and kmajor_rows(x2.shape[0], units, x2.shape[1])
                 and kops.int4_kmajor_supported(x2.shape[0], x2.shape[1], units,
                                                block_size if grouped else None)):
@@ -550,8 +581,12 @@ class EinsumDense(Layer):
             require_default_g_idx(self, block_size)
         x2, free_shape = self._input_rows(inputs, gv)
         bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
+        strip = (self._strip_operands(x2.shape[0], x2.shape[1], self._int4_unpacked_column_size, grouped,
+                                      block_size) if x2.dtype == torch.bfloat16 else None)
+        if strip is not None:
+            strip["bias"] = bias
         return dict(
-            x2=x2, block_size=block_size if grouped else None,
+            x2=x2, block_size=block_size if grouped else None, strip=strip,
             kernel=dict(kernel_packed=as_tensor(self._kernel),
                         kernel_scale=self._cached("kernel_scale", self.kernel_scale,
                                                   lambda t: t.to(cd).contiguous()),

@@ -95,7 +95,11 @@ def _call_together(layers, inputs):
         return [layer(x) for layer in layers]
     if any(s["x2"].shape != x2.shape or s["block_size"] != specs[0]["block_size"] for s in specs):
         return [layer(x) for layer in layers]
-    outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])
+    if all(s.get("strip") is not None for s in specs):
+        # every kernel has its strip-linear copy for these rows: one launch, no scratch
+        outs = kops.int4_matmul_strip_multi(x2, [s["strip"] for s in specs], block_size=specs[0]["block_size"])
+    else:
+        outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])
     return [s["finish"](y) for s, y in zip(specs, outs)]
 
 

@@ -194,6 +194,133 @@ def int4_matmul_multi(x, kernels, block_size=None):
     return [y.reshape(*lead, y.shape[1]) for y in outs]
 
 
+STRIP_MAX_ROWS = 8
+
+
+def int4_strip_supported(M, K, N, block_size=None):
+    """Whether `int4_matmul_strip` takes M bfloat16 rows against a [K, N] int4 kernel."""
+    bs = int(block_size) if block_size is not None and block_size > 0 else -1
+    return bool(_lib.load().k3q_gemv_w4s_supported(int(M), int(K), int(N), bs))
+
+
+def int4_strip_copy(kernel_packed, units):
+    """The strip-linear copy of an int4 kernel that `int4_matmul_strip` streams (layout:
+    include/k3q.h, k3q_gemv_w4s).  Made once per layer from the stored `[K, ceil(N/2)]` kernel
+    by a device kernel; the same number of bytes as the kernel (an odd strip count is padded)."""
+    _lib.require_device(kernel_packed)
+    K, N = kernel_packed.shape[0], int(units)
+    if kernel_packed.dtype != torch.int8 or kernel_packed.shape[1] != (N + 1) // 2:
+        raise ValueError("kernel must be int8 of shape [input_dim, ceil(units / 2)]")
+    lib = _lib.load()
+    nbytes = lib.k3q_w4s_shadow_bytes(K, N)
+    if nbytes <= 0:
+        raise ValueError("the strip-linear copy needs K % 128 == 0")
+    kp = kernel_packed if kernel_packed.is_contiguous() else kernel_packed.contiguous()
+    out = torch.empty(nbytes, dtype=torch.uint8, device=kp.device)
+    _lib.check(lib.k3q_w4s_pack(_lib.ptr(kp), K, N, _lib.ptr(out), _lib.stream_ptr(kp.device)), "k3q_w4s_pack")
+    return out
+
+
+def int4_strip_params(kernel_scale, kernel_zero, K, units, block_size):
+    """Scales and zero points of a grouped (block 128) int4 kernel in the order the strip kernel
+    reads them: per (strip, group) four records of four bfloat16 scales and four `zero + 128` bytes."""
+    _lib.require_device(kernel_scale, kernel_zero)
+    lib = _lib.load()
+    N = int(units)
+    nbytes = lib.k3q_w4s_params_bytes(int(K), N, int(block_size))
+    if nbytes <= 0:
+        raise ValueError("strip parameters: groups of 128 and K % 128 == 0 only")
+    sc = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
+    zp = kernel_zero if kernel_zero.is_contiguous() else kernel_zero.contiguous()
+    if tuple(sc.shape) != (K // 128, N) or tuple(zp.shape) != (K // 128, N) or zp.dtype != torch.int8:
+        raise ValueError("scale / zero must be [K / 128, N], zero int8")
+    out = torch.empty(nbytes, dtype=torch.uint8, device=sc.device)
+    rc = lib.k3q_w4s_pack_params(_lib.ptr(sc), _lib.dtype_code(sc.dtype), _lib.ptr(zp), int(K), N,
+                                 int(block_size), _lib.ptr(out), _lib.stream_ptr(sc.device))
+    _lib.check(rc, "k3q_w4s_pack_params")
+    return out
+
+
+def int4_matmul_strip(x, shadow, units, kernel_scale=None, gparams=None, block_size=None, bias=None,
+                      addend=None):
+    """`x[..., K] . W4[K, N]` for up to 8 bfloat16 rows from `int4_strip_copy(kernel)`: one launch,
+    no scratch.  Per-channel: `kernel_scale` bfloat16 [N]; grouped (block 128): `gparams` from
+    `int4_strip_params`.  `bias` [N], or `addend` [M, N] added the way a bias is.
+    Reference: keras/src/layers/core/dense.py:988-1095."""
+    _lib.require_device(x, shadow, kernel_scale, gparams, bias, addend)
+    if x.dtype != torch.bfloat16:
+        raise TypeError("the strip route computes in bfloat16")
+    grouped = block_size is not None and block_size > 0
+    N = int(units)
+    K = x.shape[-1]
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    lib = _lib.load()
+    if shadow.numel() != lib.k3q_w4s_shadow_bytes(K, N):
+        raise ValueError("the strip-linear copy does not belong to a [%d, %d] kernel" % (K, N))
+    stride = 0
+    b = bias
+    if addend is not None:
+        if bias is not None:
+            raise ValueError("addend and bias exclude each other")
+        if addend.numel() != M * N:
+            raise ValueError(f"addend holds {addend.numel()} values; the output is [{M}, {N}]")
+        b = addend.reshape(M, N)
+        b = b if b.is_contiguous() else b.contiguous()
+        stride = N
+    elif bias is not None and bias.numel() != N:
+        raise ValueError(f"bias holds {bias.numel()} values, the layer has {N} units")
+    if b is not None and b.dtype != torch.bfloat16:
+        raise TypeError("bias must be read in the input's dtype")
+    if grouped:
+        if gparams is None or gparams.numel() != lib.k3q_w4s_params_bytes(K, N, int(block_size)):
+            raise ValueError("grouped int4 needs the strip parameters of this kernel")
+    elif kernel_scale is None or kernel_scale.dtype != torch.bfloat16 or kernel_scale.numel() != N:
+        raise ValueError("per-channel int4 needs bfloat16 scales [N]")
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    rc = lib.k3q_gemv_w4s(_lib.ptr(x2), _lib.K3Q_BF16, M, K, N, _lib.ptr(shadow),
+                          None if grouped else _lib.ptr(kernel_scale), _lib.ptr(gparams) if grouped else None,
+                          int(block_size) if grouped else -1, _lib.ptr(b), stride, _lib.ptr(y),
+                          _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemv_w4s")
+    return y.reshape(*lead, N)
+
+
+def int4_matmul_strip_multi(x, kernels, block_size=None):
+    """`[x . W_i]` for kernels that share `x[..., K]` (up to 8 bfloat16 rows): one launch for those
+    whose launch plans agree.  kernels: dicts with `shadow`, `units`, `kernel_scale` (per-channel)
+    or `gparams` (grouped), and optionally `bias` [N]."""
+    grouped = block_size is not None and block_size > 0
+    K = x.shape[-1]
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    lib = _lib.load()
+    problems = (_lib.GemvW4sProblem * len(kernels))()
+    outs = []
+    for i, k in enumerate(kernels):
+        N = int(k["units"])
+        bias = k.get("bias")
+        _lib.require_device(x, k["shadow"], k.get("kernel_scale"), k.get("gparams"), bias)
+        if bias is not None and (bias.numel() != N or bias.dtype != torch.bfloat16):
+            raise ValueError(f"bias must hold {N} bfloat16 values")
+        if k["shadow"].numel() != lib.k3q_w4s_shadow_bytes(K, N):
+            raise ValueError("the strip-linear copy does not belong to a [%d, %d] kernel" % (K, N))
+        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+        outs.append(y)
+        problems[i] = _lib.GemvW4sProblem(
+            N, k["shadow"].data_ptr(), None if grouped else k["kernel_scale"].data_ptr(),
+            k["gparams"].data_ptr() if grouped else None,
+            bias.data_ptr() if bias is not None else None, y.data_ptr())
+    rc = lib.k3q_gemv_w4s_multi(_lib.ptr(x2), _lib.K3Q_BF16, M, K, len(kernels), ctypes.byref(problems),
+                                int(block_size) if grouped else -1, _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemv_w4s_multi")
+    return [y.reshape(*lead, y.shape[1]) for y in outs]
+
+
 def int4_kmajor_copy(kernel_packed, units):
     """The K-contiguous copy `int4_matmul_kmajor` reads: int32 [N, K/8], eight consecutive k of
     a column per dword, even k in the low half-word's nibbles, odd k in the high half-word's
