@@ -8,9 +8,13 @@ de-scale epilogue, at the target shape M=4096, K=N=8192, bfloat16
 activations (inputs and weights already resident in HBM).  `value` is
 2*M*N*K / step time in TOP/s.  The int4 decode GEMV (K=N=8192, M in {1,4,16}),
 the second half of the headline metric, is reported under `int4_gemv` with its own
-HBM roofline; `llama_decode_int4` is the end-to-end greedy decode of a 32-layer
-Llama-style decoder whose weight matrices are all int4 (tokens/s at batch 1 and 8),
-`llama_decode_int8` the same with int8 layers.
+HBM roofline (the layer's route: up to 8 rows the strip-linear copy of the kernel, made once
+per layer; 16 rows the stored kernel).  `int8_gemm_sweep` holds the GEMM kernel's time over the
+large-M sweep (M in {512, 2048, 4096, 8192} x K=N in {4096, 8192}, plus K=8192, N=28672),
+`einsum_int8` the EinsumDense attention projections (batch 8, t in {1, 512});
+`llama_decode_int4` is the end-to-end greedy decode of a 32-layer Llama-style decoder whose
+weight matrices are all int4 (tokens/s at batch 1 and 8), `llama_decode_int8` the same with
+int8 layers.
 The CPU oracle (a restatement of the reference's torch-CPU op sequence) is timed
 on the host cores on a bounded sample as `cpu_baseline`.
 
@@ -30,19 +34,22 @@ if ROOT not in sys.path:
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8, published (5.0 POP/s)
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
 
-# Bytes crossing the L2 <-> memory boundary per launch, from `rocprofv3 --pmc FETCH_SIZE` and
-# `--pmc WRITE_SIZE` (KiB per dispatch), each scaled by what the same counter reads for a plain
-# device copy of known size (FETCH_SIZE reads 0.50x, WRITE_SIZE 1.00x):
-# profiles/bench_dense_int8_M4096_K8192_N8192_and_int4_decode.md
-GEMM_HBM_TRAFFIC_BYTES = int((201555.1 * 2.0 + 70144.0) * 1024)
-QUANT_HBM_TRAFFIC_BYTES = int((32838.7 * 2.0 + 32832.0) * 1024)
-# int4 decode main kernel, keyed by (M > 8, grouped)
-GEMV_HBM_TRAFFIC_BYTES = {
-    (False, False): int((17263.1 * 2.0 + 2617.0) * 1024),
-    (False, True): int((17751.6 * 2.0 + 1329.0) * 1024),
-    (True, False): int(((17474.5 + 2082.0) * 2.0 + 4096.0 + 256.0) * 1024),  # with its second kernel
-    (True, True): int((19431.4 * 2.0 + 4362.0) * 1024),
-}
+# Bytes crossing the L2 <-> memory boundary per launch: `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` (KiB per dispatch) of this same command, each scaled by what the counter
+# reads for a plain device copy of known size (FETCH_SIZE 0.50x, WRITE_SIZE 1.00x).  The
+# figures are measured offline and kept in profiles/ with the command that produced them; this
+# file reads them from there (kernel name -> bytes), so that a line never carries a number
+# from another build than the one profiled.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_bytes.json")
+
+
+def measured_traffic(key):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+
 
 
 def gemv_algorithmic_bytes(M, K, N, grouped, block=128):
@@ -154,19 +161,100 @@ def main():
     quant_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
     quant_bytes = M * K * 2 + M * K + M * 2
 
+    # ------------------------------------------------------------------ int8 GEMM sweep
+    # the GEMM kernel alone (quantised activations given), bit-exact bfloat16 epilogue, HIP events
+    # around bursts of launches on the stream they are issued on
+    def kernel_us(fn, reps):
+        spin_up(torch, lambda: [fn() for _ in range(10)], 0.05)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e3
+
+    sweep = []
+    for (Ks, Ns) in ((4096, 4096), (8192, 8192), (8192, 28672)):
+        if (Ks, Ns) == (K, N):
+            ws_, wp_, sc_ = wq, prepacked, wscale_t
+        else:
+            ws_ = torch.randint(-127, 128, (Ks, Ns), device=dev, dtype=torch.int8)
+            wp_ = kops.prepack_int8_kernel(ws_)
+            sc_ = (torch.rand(Ns, device=dev) * 100 + 100).to(torch.bfloat16)
+        for Ms in (512, 2048, 4096, 8192):
+            xs = torch.randn(Ms, Ks, device=dev).to(torch.bfloat16)
+            qs, ss = kq.abs_max_quantize(xs, axis=-1)
+            us_ = kernel_us(lambda: kops.int8_matmul(qs, ws_, a_scale=ss, kernel_scale=sc_,
+                                                     out_dtype=torch.bfloat16, prepacked=wp_,
+                                                     exact_epilogue=True), 10 if Ms * Ns > 1 << 27 else 30)
+            tops_ = 2.0 * Ms * Ns * Ks / us_ / 1e6
+            sweep.append({"M": Ms, "K": Ks, "N": Ns, "us_per_launch": round(us_, 1),
+                          "tops": round(tops_, 1), "frac": round(tops_ / INT8_PEAK_TOPS, 4)})
+            del xs, qs, ss
+        if (Ks, Ns) != (K, N):
+            del ws_, wp_, sc_
+            torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ EinsumDense int8
+    # attention projections, d_model 4096, 32 heads x 128, batch 8, bfloat16; one layer call
+    # (quantizer + matmul + de-scale) replayed from a HIP graph
+    from keras_amd.layers import EinsumDense
+
+    einsum = []
+    for t_ in (1, 512):
+        for eq, oshape, ishape in (("btd,dnh->btnh", (None, 32, 128), (8, t_, 4096)),
+                                   ("btnh,nhd->btd", (None, 4096), (8, t_, 32, 128))):
+            layer = EinsumDense(eq, oshape, dtype="bfloat16", device=dev)
+            layer.build((None,) + ishape[1:])
+            layer.quantize("int8")
+            xe = torch.randn(*ishape, device=dev).to(torch.bfloat16)
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                layer(xe)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for _ in range(20):
+                        layer(xe)
+            torch.cuda.synchronize()
+            us_ = kernel_us(graph.replay, 5) / 20
+            Me = 8 * t_
+            tops_ = 2.0 * Me * 4096 * 4096 / us_ / 1e6
+            row = {"equation": eq, "batch": 8, "t": t_, "M": Me, "K": 4096, "N": 4096,
+                   "us_per_call": round(us_, 2), "tops": round(tops_, 1)}
+            if t_ == 1:  # decode-sized: bound by the int8 kernel's bytes
+                row["roofline"] = {"bound": "hbm", "achieved": round(4096 * 4096 / us_ / 1e3, 1),
+                                   "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(4096 * 4096 / us_ / 1e3 / HBM_PEAK_GBS, 4)}
+            else:
+                row["roofline"] = {"bound": "mfma", "achieved": round(tops_, 1), "peak": INT8_PEAK_TOPS,
+                                   "unit": "TOP/s", "frac": round(tops_ / INT8_PEAK_TOPS, 4)}
+            einsum.append(row)
+            del graph, layer, xe
+
     # ------------------------------------------------------------------ int4 decode GEMV
     Kg = Ng = 8192
     n_rot = 12  # 12 x 32 MiB packed kernels: more than the 256 MiB last-level cache
     packs = [torch.randint(-128, 128, (Kg, Ng // 2), generator=g, dtype=torch.int8).to(dev)
              for _ in range(n_rot)]
+    # what a layer keeps per kernel for decode-sized calls, made once: the strip-linear copy
+    strips = [kops.int4_strip_copy(pk, Ng) for pk in packs]
     pc_scale = (torch.rand(Ng, generator=g) + 0.5).to(torch.bfloat16).to(dev)
     gr_scale = (torch.rand(Kg // 128, Ng, generator=g) * 0.01 + 0.001).to(torch.bfloat16).to(dev)
     gr_zero = torch.randint(-8, 8, (Kg // 128, Ng), generator=g, dtype=torch.int8).to(dev)
+    gr_params = kops.int4_strip_params(gr_scale, gr_zero, Kg, Ng, 128)
     gemv = []
     for Mg in (1, 4, 16):
         xg = torch.randn(Mg, Kg, generator=g).to(torch.bfloat16).to(dev)
         for grouped in (False, True):
+            strip = kops.int4_strip_supported(Mg, Kg, Ng, 128 if grouped else None)
+
             def call(i):
+                if strip:  # the route Dense._int4_call takes for these rows
+                    return kops.int4_matmul_strip(xg, strips[i % n_rot], Ng,
+                                                  kernel_scale=None if grouped else pc_scale,
+                                                  gparams=gr_params if grouped else None,
+                                                  block_size=128 if grouped else None)
                 if grouped:
                     return kops.int4_matmul(xg, packs[i % n_rot], gr_scale, Ng, kernel_zero=gr_zero,
                                             block_size=128)
@@ -196,10 +284,13 @@ def main():
             gemv.append({
                 "M": Mg, "K": Kg, "N": Ng,
                 "scheme": "grouped/128+zero" if grouped else "per-channel",
+                "kernel": "gemv_w4s (strip-linear copy)" if strip else "gemv_w4_mfma (stored kernel)",
                 "us_per_call": round(us, 2), "algorithmic_bytes": nbytes,
                 "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                              "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                             "traffic": GEMV_HBM_TRAFFIC_BYTES[(Mg > 8, grouped)]},
+                             "traffic": measured_traffic(
+                                 ("gemv_w4s" if strip else "gemv_w4_mfma") + f"_M{Mg}_"
+                                 + ("grouped" if grouped else "per_channel"))},
             })
             del graph
         del xg
@@ -216,7 +307,7 @@ def main():
         from keras_amd.decoder_harness import LlamaStyleDecoder
 
         w4_host = packs[0].cpu()
-        del packs
+        del packs, strips
         torch.cuda.empty_cache()
 
         def decode_figures(policy):
@@ -288,15 +379,17 @@ def main():
         "config": {"workload": f"Dense int8 forward M={M} K={K} N={N}, bf16 activations ~N(0,1), "
                                "glorot-uniform kernel quantized per channel, kernel prepacked once"},
         "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": INT8_PEAK_TOPS,
-                     "unit": "TFLOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 4),
-                     "traffic": GEMM_HBM_TRAFFIC_BYTES, "kernel": "gemm_mfma<int8>",
+                     "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 4),
+                     "traffic": measured_traffic("gemm_mfma_i8_M4096_K8192_N8192"), "kernel": "gemm_mfma<int8>",
                      "avg_launch_us": round(gemm_ms * 1e3, 1), "ops_per_launch": ops_per_step,
                      "note": "int8 multiply-accumulate counted as 2 ops; peak is the published dense int8 figure"},
         "quantizer": {"kernel": "quantize_rows_vec", "avg_launch_us": round(quant_ms * 1e3, 1),
                       "roofline": {"bound": "hbm", "achieved": round(quant_bytes / (quant_ms * 1e-3) / 1e9, 1),
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(quant_bytes / (quant_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                   "traffic": QUANT_HBM_TRAFFIC_BYTES}},
+                                   "traffic": measured_traffic("quantize_rows_vec_bf16_4096x8192")}},
+        "int8_gemm_sweep": sweep,
+        "einsum_int8": einsum,
         "int4_gemv": gemv,
         "llama_decode_int4": decode,
         "llama_decode_int8": decode_int8,

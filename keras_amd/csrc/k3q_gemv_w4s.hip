@@ -162,7 +162,9 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     const char* xrow = w4s_lds + jj * pitch + u0 * 256 + g * 16;
     const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
-    v4f acc[2][kSW][2], accs[2], tot[kSW];
+    // (three MFMAs per step with kSW = 2, two with one strip: a strip's own chain has the others between
+    // its links, which is enough for the matrix pipe's latency)
+    v4f acc[2][kSW], accs[2], tot[kSW];
     u32 Zk[2][kSW][3];
     v4u av[2][kSW][4], xf[2][4];
 
@@ -180,9 +182,11 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         for (int t = 0; t < kSW; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
+                // (136 + zero) * sum(x) = (zero + 128) * sum(x) + 8 * sum(x); the byte converts in one operation
                 const float sc = (r & 1) ? bf_hi(Zk[a][t][r >> 1]) : bf_lo(Zk[a][t][r >> 1]);
-                const float zf = (float)((Zk[a][t][2] >> (8 * r)) & 0xffu) + 8.0f;
-                tot[t][r] += sc * ((acc[a][t][0][r] + acc[a][t][1][r]) - zf * accs[a][r]);
+                const float zu = (float)((Zk[a][t][2] >> (8 * r)) & 0xffu);
+                const float d = __builtin_fmaf(-zu, accs[a][r], acc[a][t][r] - 8.0f * accs[a][r]);
+                tot[t][r] = __builtin_fmaf(sc, d, tot[t][r]);
             }
     };
     // Unit i of the group (slot d, buffers b = d & 1): its MFMAs, interleaved with the conversion of
@@ -198,13 +202,13 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         if (has_next) read_x(b ^ 1, i + 1 < U ? i + 1 : 0);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const bool fresh_s = kGrouped && s == 0, fresh_a = kGrouped && s < 2;  // (constant once unrolled)
+            const bool fresh = kGrouped && s == 0;  // (constant once unrolled)
             accs[ab] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf8(ones), as_bf8(xf[b][s]),
-                                                               fresh_s ? zero4 : accs[ab], 0, 0, 0);
+                                                               fresh ? zero4 : accs[ab], 0, 0, 0);
 #pragma unroll
             for (int t = 0; t < kSW; ++t)
-                acc[ab][t][s & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    as_bf8(av[b][t][s]), as_bf8(xf[b][s]), fresh_a ? zero4 : acc[ab][t][s & 1], 0, 0, 0);
+                acc[ab][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    as_bf8(av[b][t][s]), as_bf8(xf[b][s]), fresh ? zero4 : acc[ab][t], 0, 0, 0);
             if (has_next) {
 #pragma unroll
                 for (int t = 0; t < kSW; ++t) cvt1(W[dn][t][s], av[b ^ 1][t][s]);
@@ -281,7 +285,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         if (!kGrouped) {  // (grouped: every unit starts its own accumulators)
             accs[0] = zero4;
 #pragma unroll
-            for (int t = 0; t < kSW; ++t) acc[0][t][0] = acc[0][t][1] = zero4;
+            for (int t = 0; t < kSW; ++t) acc[0][t] = zero4;
         }
 #pragma unroll
         for (int t = 0; t < kSW; ++t) {
@@ -311,7 +315,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
             for (int t = 0; t < kSW; ++t)
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr)
-                    tot[t][rr] = (acc[0][t][0][rr] + acc[0][t][1][rr]) - 136.0f * accs[0][rr];
+                    tot[t][rr] = acc[0][t][rr] - 136.0f * accs[0][rr];
         }
         float* rbuf = red + (turn & 1) * ((kQ - 1) * kSW * M * kRedStride);  // rows of x only
         if (q > 0 && j < M) {
@@ -370,6 +374,14 @@ __global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
     int i = 0;
     while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
     gemv_w4s_body<kSW, kD, kNP, kGrouped>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
+}
+
+// One problem per launch: its parameters ARE the kernel arguments, fetched in one scalar round trip
+// (the several-problem kernel first finds its problem, then fetches that problem's parameters: two
+// dependent round trips more before the first vector load can be issued).
+template <int kSW, int kD, int kNP, bool kGrouped>
+__global__ __launch_bounds__(kT) void gemv_w4s_one(W4sParams p) {
+    gemv_w4s_body<kSW, kD, kNP, kGrouped>(p, blockIdx.x, gridDim.x);
 }
 
 // ---- the strip-linear copy ---------------------------------------------------------------
@@ -464,19 +476,22 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
     return pl;
 }
 
-using W4sKernel = void (*)(W4sMulti);
+struct W4sKernels {
+    void (*multi)(W4sMulti);
+    void (*one)(W4sParams);
+};
 
 template <int kSW, int kD, bool kGrouped>
-W4sKernel pick_np(int np) {
+W4sKernels pick_np(int np) {
     switch (np) {
-        case 2: return gemv_w4s<kSW, kD, 2, kGrouped>;
-        case 4: return gemv_w4s<kSW, kD, 4, kGrouped>;
-        case 8: return gemv_w4s<kSW, kD, 8, kGrouped>;
-        default: return gemv_w4s<kSW, kD, 16, kGrouped>;
+        case 2: return {gemv_w4s<kSW, kD, 2, kGrouped>, gemv_w4s_one<kSW, kD, 2, kGrouped>};
+        case 4: return {gemv_w4s<kSW, kD, 4, kGrouped>, gemv_w4s_one<kSW, kD, 4, kGrouped>};
+        case 8: return {gemv_w4s<kSW, kD, 8, kGrouped>, gemv_w4s_one<kSW, kD, 8, kGrouped>};
+        default: return {gemv_w4s<kSW, kD, 16, kGrouped>, gemv_w4s_one<kSW, kD, 16, kGrouped>};
     }
 }
 
-W4sKernel pick_kernel(const W4sPlan& pl, bool grouped) {
+W4sKernels pick_kernel(const W4sPlan& pl, bool grouped) {
     if (pl.sw == 2) {
         if (pl.d == 4) return grouped ? pick_np<2, 4, true>(pl.np) : pick_np<2, 4, false>(pl.np);
         return grouped ? pick_np<2, 2, true>(pl.np) : pick_np<2, 2, false>(pl.np);
@@ -510,20 +525,21 @@ int fill_params(W4sParams& p, const void* x, int64_t M, int64_t K, int64_t N, co
 }
 
 int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_blocks, hipStream_t s) {
-    const W4sKernel kernel = pick_kernel(pl, grouped);
+    const W4sKernels ks = pick_kernel(pl, grouped);
+    const void* kernel = mp.count == 1 ? (const void*)ks.one : (const void*)ks.multi;
     // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
     {
         static std::mutex mu;
         static std::set<const void*> raised;
         std::lock_guard<std::mutex> lock(mu);
-        if (!raised.count((const void*)kernel)) {
-            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    160 * 1024) != hipSuccess)
+        if (!raised.count(kernel)) {
+            if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
                 return K3Q_ERR_LAUNCH;
-            raised.insert((const void*)kernel);
+            raised.insert(kernel);
         }
     }
-    kernel<<<(unsigned)total_blocks, kT, pl.lds, s>>>(mp);
+    if (mp.count == 1) ks.one<<<(unsigned)total_blocks, kT, pl.lds, s>>>(mp.p[0]);
+    else ks.multi<<<(unsigned)total_blocks, kT, pl.lds, s>>>(mp);
     return launch_status();
 }
 
