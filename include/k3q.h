@@ -270,7 +270,7 @@ int k3q_gemv_w4_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
                        int64_t block_size, const void* bias, void* y, void* stream);
 
 /*
- * Weight-only int4 matmul for up to 8 bfloat16 rows from a strip-linear copy of the kernel: what
+ * Weight-only int4 matmul for up to 16 bfloat16 rows from a strip-linear copy of the kernel: what
  * k3q_gemv_w4 computes (to the order of the fp32 sums), with the kernel streamed as contiguous
  * 1 KiB pieces, all of K inside a workgroup -- no partial sums, no workspace, no counters, and
  * nothing allocated: one launch that reads the copy once.
@@ -285,9 +285,10 @@ int k3q_gemv_w4_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
  *            from scale, zero [K / 128, N]: per (strip, unit) four records {4 bfloat16 scales,
  *            4 bytes zero + 128};                                  y = T(x . ((W - zero) * scale)) (+ bias)
  *   bias: bfloat16 [N] (bias_stride 0) or an [M, N] addend (bias_stride N), or null.
- * Takes (k3q_gemv_w4s_supported): bfloat16 x, 1 <= M <= 8 with M * K <= 65536, K % 256 == 0,
- * K >= 2048, N % 16 == 0, N >= 3072, block_size <= 0 or == 128; anything else K3Q_ERR_SHAPE (callers
- * keep k3q_gemv_w4 for those).  k3q_gemv_w4s_multi: several kernels against one x (same M, K,
+ * Takes (k3q_gemv_w4s_supported): bfloat16 x, 1 <= M <= 16 while the rows fit a workgroup's LDS
+ * (M * K <= 65536; up to twice that, staged in two halves, when K % 4096 == 0 and N <= 8192),
+ * K % 256 == 0, K >= 4096, N % 16 == 0, N >= 3072, block_size <= 0 or == 128; anything else
+ * K3Q_ERR_SHAPE (callers keep k3q_gemv_w4 for those).  k3q_gemv_w4s_multi: several kernels against one x (same M, K,
  * block_size), one launch for those whose launch plans agree.
  * Replaces what k3q_gemv_w4 replaces (keras/src/layers/core/dense.py:988-1095,
  * keras/src/layers/core/einsum_dense.py:1120-1261).

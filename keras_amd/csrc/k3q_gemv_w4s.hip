@@ -40,7 +40,7 @@ namespace {
 
 constexpr int kQ = 8;            // waves per workgroup = slices of K
 constexpr int kT = kQ * 64;      // threads
-constexpr int kMaxRows = 8;      // rows of x
+constexpr int kMaxRows = 16;     // rows of x
 constexpr int kMaxPieces = 16;   // 16-byte pieces of x a thread stages: M * K <= 16 * 8 * kT
 constexpr int kRedStride = 20;   // floats per (row, strip) line of the cross-wave reduction
 constexpr int kMaxProblems = 4;
@@ -54,7 +54,8 @@ struct W4sParams {
     uint16_t* y;             // [M, N] bf16
     int64_t bias_stride;     // 0 or N
     int M, K, N, units;      // units = K / 128
-    int row_magic;           // ceil(2^32 / (K / 8)): piece -> row without a division
+    int row_magic;           // ceil(2^32 / pieces per staged row): piece -> row without a division
+    int slice_magic;         // (x staged in halves) ceil(2^32 / pieces per half slice)
 };
 
 struct W4sMulti {
@@ -72,7 +73,10 @@ __device__ __forceinline__ float bf_hi(u32 d) { return __uint_as_float(d & 0xfff
 // A workgroup takes strip groups `block`, `block + stride`, ... one after the other as ONE stream of
 // units: the ring runs across the boundary (the last bodies of a group convert and request the
 // first units of the next), so that a workgroup pays the memory latency once, not once per group.
-template <int kSW, int kD, int kNP, bool kGrouped>
+// kHalves: x does not fit LDS as a whole (9 ... 16 rows of a long K): every wave's slice is cut in two,
+// LDS holds the first halves, then -- once every wave is through with them -- the second halves
+// (one turn per workgroup only: the launch plan sees to it).
+template <int kSW, int kD, int kNP, bool kGrouped, bool kHalves>
 __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int block, const int stride) {
     extern __shared__ __attribute__((aligned(16))) char w4s_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -88,18 +92,44 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     const int U = (base + (q < extra ? 1 : 0)) * kD;
     const int u0 = (q * base + (q < extra ? q : extra)) * kD;
     const int R = U / kD;  // >= 2 (the launch plan sees to it)
-    const int pitch = K * 2 + 16;
-    float* red = (float*)(w4s_lds + ((M * pitch + 255) & ~255));  // two buffers, one per parity of the turn
+    const int Uh = kHalves ? U / 2 : U;  // units of a slice whose x is in LDS at a time
+    const int pitch = (kHalves ? K : K * 2) + 16;
+    // (two buffers, one per parity of the turn, when a workgroup takes several turns)
+    float* red = (float*)(w4s_lds + ((M * pitch + 255) & ~255));
 
     // ---- x into registers first (every load unconditional: pieces past the end re-read piece 0) ----
-    const int per_row = K >> 3;
+    // whole rows, or (kHalves) half h of every wave's slice: row m = [slice 0 | slice 1 | ...]
+    const int per_row = kHalves ? K >> 4 : K >> 3;
     const int pieces = M * per_row;
     v4u xst[kNP];
+    auto stage_load = [&](const int h) {
 #pragma unroll
-    for (int i = 0; i < kNP; ++i) {
-        const int pi = i * kT + tid;
-        xst[i] = *(const v4u*)(p.x + (int64_t)(pi < pieces ? pi : 0) * 8);
-    }
+        for (int i = 0; i < kNP; ++i) {
+            int pi = i * kT + tid;
+            pi = pi < pieces ? pi : 0;
+            if (kHalves) {
+                const int m = (int)__umulhi((unsigned)pi, (unsigned)p.row_magic);
+                const int c = pi - m * per_row;
+                const int qq = (int)__umulhi((unsigned)c, (unsigned)p.slice_magic);  // c / (Uh * 16)
+                const int cc = c - qq * (Uh * 16);
+                xst[i] = *(const v4u*)(p.x + (int64_t)m * K + (int64_t)(qq * U + h * Uh) * 128 + cc * 8);
+            } else {
+                xst[i] = *(const v4u*)(p.x + (int64_t)pi * 8);
+            }
+        }
+    };
+    auto stage_store = [&]() {
+#pragma unroll
+        for (int i = 0; i < kNP; ++i) {
+            const int pi = i * kT + tid;
+            if (pi < pieces) {
+                const int m = (int)__umulhi((unsigned)pi, (unsigned)p.row_magic);
+                const int c = pi - m * per_row;
+                *(v4u*)(w4s_lds + m * pitch + c * 16) = xst[i];
+            }
+        }
+    };
+    stage_load(0);
     __builtin_amdgcn_sched_barrier(0);
     // weights and grouped parameters of a strip group at this wave's slice: wave-uniform bases (scalar
     // registers), the lane's part is added at the load
@@ -148,18 +178,10 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     for (int d = 0; d < kD; ++d) fetch(d, d);
     __builtin_amdgcn_sched_barrier(0);
     // ---- x into LDS: the stores wait for the x loads only (they are the older ones) ----
-#pragma unroll
-    for (int i = 0; i < kNP; ++i) {
-        const int pi = i * kT + tid;
-        if (pi < pieces) {
-            const int m = (int)__umulhi((unsigned)pi, (unsigned)p.row_magic);
-            const int c = pi - m * per_row;
-            *(v4u*)(w4s_lds + m * pitch + c * 16) = xst[i];
-        }
-    }
+    stage_store();
     __syncthreads();
 
-    const char* xrow = w4s_lds + jj * pitch + u0 * 256 + g * 16;
+    const char* xrow = w4s_lds + jj * pitch + (kHalves ? q * Uh : u0) * 256 + g * 16;
     const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
     // (three MFMAs per step with kSW = 2, two with one strip: a strip's own chain has the others between
@@ -194,12 +216,19 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // fold of unit i - 1, whose MFMAs are long done; after it that unit's parameter buffer takes those
     // of the unit after.  Then slot dn is requested again: unit i + 1 + kD, from the next group if past
     // the end of this one.
-    auto body = [&](auto d_c, const int i, auto has_next_c, auto do_refill_c, const bool fold_prev) {
+    // x_later: the unit after this one needs the other half of x: its fragments are read by the caller
+    auto body = [&](auto d_c, const int i, auto has_next_c, auto do_refill_c, const bool fold_prev,
+                    auto x_later_c) {
         constexpr int d = decltype(d_c)::value;
         constexpr bool has_next = decltype(has_next_c)::value, do_refill = decltype(do_refill_c)::value;
+        constexpr bool x_later = decltype(x_later_c)::value;
         constexpr int b = d & 1, dn = (d + 1) % kD;
         constexpr int ab = kGrouped ? b : 0;
-        if (has_next) read_x(b ^ 1, i + 1 < U ? i + 1 : 0);
+        if (has_next && !x_later) {
+            int nx = i + 1 < U ? i + 1 : 0;
+            if (kHalves) nx = nx >= Uh ? nx - Uh : nx;
+            read_x(b ^ 1, nx);
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const bool fresh = kGrouped && s == 0;  // (constant once unrolled)
@@ -243,16 +272,18 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     };
     using std::bool_constant;
     using std::integral_constant;
-    auto round = [&](auto last_c, const int r) {
-        constexpr bool last = decltype(last_c)::value;  // last round of the last group: nothing follows
+    // last: last round of the last group, nothing follows; turn_c: last round on the first half of x
+    auto round = [&](auto last_c, const int r, auto turn_c) {
+        constexpr bool last = decltype(last_c)::value;
+        const bool_constant<false> no{};
         const int i0 = r * kD;
-        body(integral_constant<int, 0>{}, i0, bool_constant<true>{}, bool_constant<!last>{}, r > 0);
+        body(integral_constant<int, 0>{}, i0, bool_constant<true>{}, bool_constant<!last>{}, r > 0, no);
         if constexpr (kD == 2) {
-            body(integral_constant<int, 1>{}, i0 + 1, bool_constant<!last>{}, bool_constant<!last>{}, true);
+            body(integral_constant<int, 1>{}, i0 + 1, bool_constant<!last>{}, bool_constant<!last>{}, true, turn_c);
         } else {
-            body(integral_constant<int, 1>{}, i0 + 1, bool_constant<true>{}, bool_constant<!last>{}, true);
-            body(integral_constant<int, 2>{}, i0 + 2, bool_constant<true>{}, bool_constant<!last>{}, true);
-            body(integral_constant<int, 3>{}, i0 + 3, bool_constant<!last>{}, bool_constant<!last>{}, true);
+            body(integral_constant<int, 1>{}, i0 + 1, bool_constant<true>{}, bool_constant<!last>{}, true, no);
+            body(integral_constant<int, 2>{}, i0 + 2, bool_constant<true>{}, bool_constant<!last>{}, true, no);
+            body(integral_constant<int, 3>{}, i0 + 3, bool_constant<!last>{}, bool_constant<!last>{}, true, turn_c);
         }
     };
 
@@ -352,7 +383,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // every group but the workgroup's last: all rounds request and convert ahead, into the next group
     for (; grp + stride < groups; grp += stride, ++turn) {
         begin(grp, grp + stride);
-        for (int r = 0; r < R; ++r) round(bool_constant<false>{}, r);
+        for (int r = 0; r < R; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
         finish(grp, turn);
 #pragma unroll
         for (int t = 0; t < kSW; ++t) {
@@ -363,8 +394,23 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // the last group: its last round has nothing to request or convert (the one request before it that
     // falls past the end re-reads the group's first unit: never used)
     begin(grp, grp);
-    for (int r = 0; r < R - 1; ++r) round(bool_constant<false>{}, r);
-    round(bool_constant<true>{}, R - 1);
+    if constexpr (kHalves) {
+        const int Rh = R / 2;
+        for (int r = 0; r < Rh - 1; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
+        // the last round on the first halves: the second halves are requested now and written once
+        // every wave has read its last fragments of the first (its MFMAs hold them in registers)
+        stage_load(1);
+        __builtin_amdgcn_sched_barrier(0);
+        round(bool_constant<false>{}, Rh - 1, bool_constant<true>{});
+        __syncthreads();
+        stage_store();
+        __syncthreads();
+        read_x(0, 0);  // unit U / 2, the first of the second half (buffer 0: kD is even)
+        for (int r = Rh; r < R - 1; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
+    } else {
+        for (int r = 0; r < R - 1; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
+    }
+    round(bool_constant<true>{}, R - 1, bool_constant<false>{});
     finish(grp, turn);
 }
 
@@ -373,7 +419,7 @@ __global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
     const int bx = blockIdx.x;
     int i = 0;
     while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
-    gemv_w4s_body<kSW, kD, kNP, kGrouped>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
+    gemv_w4s_body<kSW, kD, kNP, kGrouped, false>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
 }
 
 // One problem per launch: its parameters ARE the kernel arguments, fetched in one scalar round trip
@@ -381,7 +427,13 @@ __global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
 // dependent round trips more before the first vector load can be issued).
 template <int kSW, int kD, int kNP, bool kGrouped>
 __global__ __launch_bounds__(kT) void gemv_w4s_one(W4sParams p) {
-    gemv_w4s_body<kSW, kD, kNP, kGrouped>(p, blockIdx.x, gridDim.x);
+    gemv_w4s_body<kSW, kD, kNP, kGrouped, false>(p, blockIdx.x, gridDim.x);
+}
+
+// 9 ... 16 rows of a K too long for LDS: x in two halves (two strips per wave, ring of two, one turn)
+template <int kSW, bool kGrouped>
+__global__ __launch_bounds__(kT) void gemv_w4s_halves(W4sParams p) {
+    gemv_w4s_body<kSW, 2, 16, kGrouped, true>(p, blockIdx.x, gridDim.x);
 }
 
 // ---- the strip-linear copy ---------------------------------------------------------------
@@ -443,10 +495,12 @@ inline int64_t strips_padded(int64_t N) { return ((N + 15) / 16 + 1) / 2 * 2; }
 
 struct W4sPlan {
     bool ok;
+    bool halves;  // x staged in two halves (9 ... 16 rows of a long K)
     int sw, d, np;
     int64_t groups;  // strip groups (kSW strips each)
     int64_t blocks;  // workgroups: each takes groups block, block + blocks, ...
-    size_t lds;
+    size_t lds;      // dynamic LDS of a launch of this problem alone
+    size_t lds_two;  // the same with both reduction buffers: what a launch needs whose workgroups take turns
 };
 
 constexpr int kResident = 256;  // workgroups the chip holds at once: one per CU (registers)
@@ -457,7 +511,6 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
     if (M < 1 || M > kMaxRows || (K % 128) != 0 || (N % 16) != 0) return pl;
     if (grouped && block_size != 128) return pl;
     const int64_t units = K / 128, strips = N / 16;
-    if (M * K > (int64_t)kMaxPieces * 8 * kT) return pl;
     // all of K stays inside a workgroup, so the strips alone have to fill the chip
     if (strips < 192) return pl;
     // every wave walks at least two rounds of the ring
@@ -465,14 +518,34 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
     else if ((units % 2) == 0 && units / 2 >= 2 * kQ) pl.d = 2;
     else return pl;
     pl.sw = strips >= 2 * kResident ? 2 : 1;
-    const int64_t pieces = M * K / 8;
-    pl.np = pieces <= 2 * kT ? 2 : pieces <= 4 * kT ? 4 : pieces <= 8 * kT ? 8 : 16;
     pl.groups = (strips + pl.sw - 1) / pl.sw;
     // more groups than the chip holds workgroups: each workgroup takes several, one after the other
     const int64_t turns = (pl.groups + kResident - 1) / kResident;
     pl.blocks = (pl.groups + turns - 1) / turns;
-    pl.lds = (size_t)((M * (K * 2 + 16) + 255) & ~255) + (size_t)2 * (kQ - 1) * pl.sw * M * kRedStride * 4;
-    pl.ok = pl.lds <= 160 * 1024;
+    const size_t red = (size_t)(turns > 1 ? 2 : 1) * (kQ - 1) * pl.sw * M * kRedStride * 4;
+    const int64_t stage_max = (int64_t)kMaxPieces * 8 * kT;  // elements of x a workgroup stages at a time
+    const size_t lds_limit = 160 * 1024;
+    // x whole in LDS ...
+    const size_t red_one = (size_t)(kQ - 1) * pl.sw * M * kRedStride * 4;
+    pl.lds = (size_t)((M * (K * 2 + 16) + 255) & ~255) + red;
+    pl.lds_two = pl.lds - red + 2 * red_one;
+    if (M * K <= stage_max && pl.lds <= lds_limit) {
+        const int64_t pieces = M * K / 8;
+        pl.np = pieces <= 2 * kT ? 2 : pieces <= 4 * kT ? 4 : pieces <= 8 * kT ? 8 : 16;
+        pl.ok = true;
+        return pl;
+    }
+    // ... or in two halves: equal slices of whole ring rounds per half, one turn per workgroup
+    pl.lds = (size_t)((M * (K + 16) + 255) & ~255) + red;
+    // (grouped kernels with two strips per wave do not fit the register file next to the staged
+    // half of x: those calls stay with k3q_gemv_w4)
+    if (M * K / 2 <= stage_max && pl.lds <= lds_limit && turns == 1 && (units % (4 * kQ)) == 0 &&
+        !(grouped && pl.sw == 2)) {
+        pl.halves = true;
+        pl.d = 2;
+        pl.np = 16;
+        pl.ok = true;
+    }
     return pl;
 }
 
@@ -500,9 +573,9 @@ W4sKernels pick_kernel(const W4sPlan& pl, bool grouped) {
     return grouped ? pick_np<1, 2, true>(pl.np) : pick_np<1, 2, false>(pl.np);
 }
 
-int fill_params(W4sParams& p, const void* x, int64_t M, int64_t K, int64_t N, const void* shadow,
-                const void* scale, const void* gparams, int64_t block_size, const void* bias,
-                int64_t bias_stride, void* y) {
+int fill_params(W4sParams& p, const W4sPlan& pl, const void* x, int64_t M, int64_t K, int64_t N,
+                const void* shadow, const void* scale, const void* gparams, int64_t block_size,
+                const void* bias, int64_t bias_stride, void* y) {
     const bool grouped = block_size > 0;
     if (!x || !shadow || !y || (grouped ? !gparams : !scale)) return K3Q_ERR_NULL;
     if (!aligned_to(x, 16) || !aligned_to(shadow, 16) || !aligned_to(y, 8) || (scale && !aligned_to(scale, 8)) ||
@@ -519,13 +592,20 @@ int fill_params(W4sParams& p, const void* x, int64_t M, int64_t K, int64_t N, co
     p.K = (int)K;
     p.N = (int)N;
     p.units = (int)(K / 128);
-    const uint64_t per_row = (uint64_t)K / 8;
+    const uint64_t per_row = (uint64_t)K / (pl.halves ? 16 : 8);
     p.row_magic = (int)(uint32_t)((((uint64_t)1 << 32) + per_row - 1) / per_row);
+    const uint64_t per_half_slice = (uint64_t)(K / 128 / kQ / 2) * 16;
+    p.slice_magic = pl.halves ? (int)(uint32_t)((((uint64_t)1 << 32) + per_half_slice - 1) / per_half_slice) : 0;
     return K3Q_OK;
 }
 
-int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_blocks, hipStream_t s) {
-    const W4sKernels ks = pick_kernel(pl, grouped);
+int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_blocks, size_t lds, hipStream_t s) {
+    W4sKernels ks = pick_kernel(pl, grouped);
+    if (pl.halves) {
+        if (mp.count != 1) return K3Q_ERR_SHAPE;
+        ks.one = pl.sw == 2 ? (grouped ? gemv_w4s_halves<2, true> : gemv_w4s_halves<2, false>)
+                            : (grouped ? gemv_w4s_halves<1, true> : gemv_w4s_halves<1, false>);
+    }
     const void* kernel = mp.count == 1 ? (const void*)ks.one : (const void*)ks.multi;
     // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
     {
@@ -538,8 +618,8 @@ int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_bl
             raised.insert(kernel);
         }
     }
-    if (mp.count == 1) ks.one<<<(unsigned)total_blocks, kT, pl.lds, s>>>(mp.p[0]);
-    else ks.multi<<<(unsigned)total_blocks, kT, pl.lds, s>>>(mp);
+    if (mp.count == 1) ks.one<<<(unsigned)total_blocks, kT, lds, s>>>(mp.p[0]);
+    else ks.multi<<<(unsigned)total_blocks, kT, lds, s>>>(mp);
     return launch_status();
 }
 
@@ -599,12 +679,12 @@ extern "C" int k3q_gemv_w4s(const void* x, int x_dtype, int64_t M, int64_t K, in
     const W4sPlan pl = w4s_plan(M, K, N, block_size);
     if (!pl.ok) return K3Q_ERR_SHAPE;
     W4sMulti mp{};
-    const int rc = fill_params(mp.p[0], x, M, K, N, shadow, scale, gparams, block_size, bias, bias_stride, y);
+    const int rc = fill_params(mp.p[0], pl, x, M, K, N, shadow, scale, gparams, block_size, bias, bias_stride, y);
     if (rc != K3Q_OK) return rc;
     mp.first[0] = 0;
     mp.first[1] = (int)pl.blocks;
     mp.count = 1;
-    return launch_w4s(pl, block_size > 0, mp, (int)pl.blocks, (hipStream_t)stream);
+    return launch_w4s(pl, block_size > 0, mp, (int)pl.blocks, pl.lds, (hipStream_t)stream);
 }
 
 extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
@@ -627,15 +707,23 @@ extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t
             const W4sPlan pl = w4s_plan(M, K, q.N, block_size);
             if (!pl.ok) return K3Q_ERR_SHAPE;
             if (n == 0) pl0 = pl;
-            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np) break;
-            const int rc = fill_params(mp.p[n], x, M, K, q.N, q.shadow, q.scale, q.gparams, block_size, q.bias,
-                                       0, q.y);
+            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np || pl.halves || pl0.halves) break;
+            const int rc = fill_params(mp.p[n], pl, x, M, K, q.N, q.shadow, q.scale, q.gparams, block_size,
+                                       q.bias, 0, q.y);
             if (rc != K3Q_OK) return rc;
             groups[n] = pl.groups;
             total += pl.groups;
         }
-        // the launch as a whole is cut for the chip: about kResident workgroups, each problem its share
-        const int64_t turns = (total + kResident - 1) / kResident;
+        // the launch as a whole is cut for the chip: about kResident workgroups, each problem its share;
+        // workgroups that take turns need both reduction buffers, and where those do not fit beside x
+        // the first problem goes alone
+        int64_t turns = (total + kResident - 1) / kResident;
+        size_t lds = turns > 1 ? pl0.lds_two : pl0.lds;
+        if (lds > (size_t)160 * 1024) {
+            n = 1;
+            turns = (groups[0] + kResident - 1) / kResident;
+            lds = pl0.lds;
+        }
         int next_block = 0;
         for (int i = 0; i < n; ++i) {
             mp.first[i] = next_block;
@@ -643,7 +731,7 @@ extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t
         }
         mp.first[n] = next_block;
         mp.count = n;
-        const int rc = launch_w4s(pl0, block_size > 0, mp, next_block, s);
+        const int rc = launch_w4s(pl0, block_size > 0, mp, next_block, lds, s);
         if (rc != K3Q_OK) return rc;
         at += n;
     }

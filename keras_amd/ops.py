@@ -194,7 +194,7 @@ def int4_matmul_multi(x, kernels, block_size=None):
     return [y.reshape(*lead, y.shape[1]) for y in outs]
 
 
-STRIP_MAX_ROWS = 8
+STRIP_MAX_ROWS = 16
 
 
 def int4_strip_supported(M, K, N, block_size=None):
@@ -243,7 +243,7 @@ def int4_strip_params(kernel_scale, kernel_zero, K, units, block_size):
 
 def int4_matmul_strip(x, shadow, units, kernel_scale=None, gparams=None, block_size=None, bias=None,
                       addend=None):
-    """`x[..., K] . W4[K, N]` for up to 8 bfloat16 rows from `int4_strip_copy(kernel)`: one launch,
+    """`x[..., K] . W4[K, N]` for up to 16 bfloat16 rows from `int4_strip_copy(kernel)`: one launch,
     no scratch.  Per-channel: `kernel_scale` bfloat16 [N]; grouped (block 128): `gparams` from
     `int4_strip_params`.  `bias` [N], or `addend` [M, N] added the way a bias is.
     Reference: keras/src/layers/core/dense.py:988-1095."""

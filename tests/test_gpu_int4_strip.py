@@ -72,10 +72,13 @@ def run_strip_case(dev, M, K, N, block_size, with_bias, seed=0):
     return got
 
 
-@pytest.mark.parametrize("M", [1, 4, 8])
+@pytest.mark.parametrize("M", [1, 4, 8, 9, 16])
 @pytest.mark.parametrize("block_size", [None, 128])
 def test_strip_decode_config(dev, M, block_size):
-    # target configuration 2: K = N = 8192
+    # target configuration 2: K = N = 8192 (grouped kernels above 8 rows stay on the stored-kernel route)
+    if block_size and M > 8:
+        assert not kops.int4_strip_supported(M, 8192, 8192, block_size)
+        return
     run_strip_case(dev, M, 8192, 8192, block_size, with_bias=False)
 
 
@@ -83,20 +86,23 @@ def test_strip_decode_config(dev, M, block_size):
     (1, 4096, 4096, 128), (3, 4096, 14336, 128), (2, 14336, 4096, 128), (1, 4096, 32000, 128),
     (8, 4096, 4096, None), (5, 4096, 3072, 128), (1, 5120, 5120, None), (7, 8192, 3088, 128),
     (1, 28672, 4096, None), (4, 5120, 13824, 128), (2, 6144, 6144, None),
+    (16, 4096, 4096, 128), (12, 4096, 14336, None), (16, 8192, 4096, 128), (10, 12288, 3072, None),
+    (16, 8192, 8192, None), (16, 8192, 4096, 128),
 ])
 def test_strip_shapes(dev, M, K, N, block_size):
     run_strip_case(dev, M, K, N, block_size, with_bias=(M % 2 == 1), seed=M)
 
 
 def test_strip_rejects_what_it_does_not_take(dev):
-    for M, K, N, bs in [(9, 4096, 4096, None), (1, 4096, 4096, 64), (1, 4000, 4096, None),
+    for M, K, N, bs in [(17, 4096, 4096, None), (16, 14336, 4096, 128), (9, 8192, 16384, None), (1, 4096, 4096, 64),
+                        (16, 4096, 32000, 128), (1, 4000, 4096, None),
                         (1, 4096, 1024, None), (1, 4096, 4104, None), (8, 14336, 4096, 128),
                         (1, 1024, 4096, None), (1, 128 * 33, 4096, None), (1, 2048, 4096, None)]:
         assert not kops.int4_strip_supported(M, K, N, bs), (M, K, N, bs)
     lib = _lib.load()
     one = torch.zeros(64, dtype=torch.uint8, device=dev)
     p, s = _lib.ptr(one), _lib.stream_ptr(dev)
-    assert lib.k3q_gemv_w4s(p, 1, 9, 4096, 4096, p, p, None, -1, None, 0, p, s) == -2
+    assert lib.k3q_gemv_w4s(p, 1, 17, 4096, 4096, p, p, None, -1, None, 0, p, s) == -2
     assert lib.k3q_gemv_w4s(p, 0, 1, 4096, 4096, p, p, None, -1, None, 0, p, s) == -4
     assert lib.k3q_gemv_w4s(p, 1, 1, 4096, 4096, p, None, None, -1, None, 0, p, s) == -1
     assert lib.k3q_gemv_w4s(p, 1, 1, 4096, 4096, p, p, None, -1, p, 7, p, s) == -2
