@@ -78,7 +78,18 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
+    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,decode,cpu: run the headline "
+                    "step and only these further sections (for profiler runs); default: all")
     args = ap.parse_args()
+    only = set(filter(None, args.only.split(",")))
+    unknown = only - {"none", "ceiling", "sweep", "einsum", "gemv", "decode", "cpu"}
+    if unknown:
+        sys.exit(f"bench.py: unknown section(s) {sorted(unknown)}")
+    want = (lambda name: not only or name in only)
+    if args.no_decode:
+        want = (lambda name, w=want: name != "decode" and w(name))
+    if args.no_cpu_baseline:
+        want = (lambda name, w=want: name != "cpu" and w(name))
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the quantized Dense path has no multi-GPU leg "
                  f"(got --gpus {args.gpus}); its column-sharded form needs no exchange step")
@@ -161,6 +172,39 @@ def main():
     quant_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
     quant_bytes = M * K * 2 + M * K + M * 2
 
+    # ------------------------------------------------------------------ matrix cores alone
+    # What the int8 matrix cores sustain on this board with nothing else running: a loop of
+    # v_mfma_i32_32x32x32_i8 on register-resident operands (libk3q_probe.so, a measurement aid
+    # built beside the product library), about 50 ms per operand kind, clock read in-kernel.
+    ceiling = None
+    if want("ceiling"):
+        import ctypes
+
+        probe_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "keras_amd", "libk3q_probe.so")
+        if os.path.exists(probe_path):
+            probe = ctypes.CDLL(probe_path)
+            probe.k3q_probe_mfma_i8_only.restype = ctypes.c_double
+            probe.k3q_probe_mfma_i8_only.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+            pout = torch.zeros(4, dtype=torch.int64, device=dev)
+            stream_h = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            ceiling = []
+            for kind, label in ((0, "all-zero operands"), (1, "uniform random bytes"),
+                                (2, "activation-like A (|a| < 32), uniform random B")):
+                iters = 160000
+                probe.k3q_probe_mfma_i8_only(kind, iters // 4, ctypes.c_void_p(pout.data_ptr()), stream_h)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                n_ops = probe.k3q_probe_mfma_i8_only(kind, iters, ctypes.c_void_p(pout.data_ptr()), stream_h)
+                e1.record()
+                torch.cuda.synchronize()
+                if n_ops <= 0:
+                    sys.exit("bench.py: the MFMA-only probe did not launch")
+                clk = pout.cpu().tolist()
+                ceiling.append({"operands": label, "ms": round(e0.elapsed_time(e1), 2),
+                                "tops": round(n_ops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1),
+                                "clock_ghz": round(clk[0] / (clk[1] / 100e6) / 1e9, 3)})
+
     # ------------------------------------------------------------------ int8 GEMM sweep
     # the GEMM kernel alone (quantised activations given), bit-exact bfloat16 epilogue, HIP events
     # around bursts of launches on the stream they are issued on
@@ -175,7 +219,7 @@ def main():
         return e0.elapsed_time(e1) / reps * 1e3
 
     sweep = []
-    for (Ks, Ns) in ((4096, 4096), (8192, 8192), (8192, 28672)):
+    for (Ks, Ns) in ((4096, 4096), (8192, 8192), (8192, 28672)) if want("sweep") else ():
         if (Ks, Ns) == (K, N):
             ws_, wp_, sc_ = wq, prepacked, wscale_t
         else:
@@ -202,7 +246,7 @@ def main():
     from keras_amd.layers import EinsumDense
 
     einsum = []
-    for t_ in (1, 512):
+    for t_ in (1, 512) if want("einsum") else ():
         for eq, oshape, ishape in (("btd,dnh->btnh", (None, 32, 128), (8, t_, 4096)),
                                    ("btnh,nhd->btd", (None, 4096), (8, t_, 32, 128))):
             layer = EinsumDense(eq, oshape, dtype="bfloat16", device=dev)
@@ -234,7 +278,8 @@ def main():
 
     # ------------------------------------------------------------------ int4 decode GEMV
     Kg = Ng = 8192
-    n_rot = 12  # 12 x 32 MiB packed kernels: more than the 256 MiB last-level cache
+    # 12 x 32 MiB packed kernels: more than the 256 MiB last-level cache
+    n_rot = 12 if want("gemv") else 1
     packs = [torch.randint(-128, 128, (Kg, Ng // 2), generator=g, dtype=torch.int8).to(dev)
              for _ in range(n_rot)]
     # what a layer keeps per kernel for decode-sized calls, made once: the strip-linear copy
@@ -244,7 +289,7 @@ def main():
     gr_zero = torch.randint(-8, 8, (Kg // 128, Ng), generator=g, dtype=torch.int8).to(dev)
     gr_params = kops.int4_strip_params(gr_scale, gr_zero, Kg, Ng, 128)
     gemv = []
-    for Mg in (1, 4, 16):
+    for Mg in (1, 4, 16) if want("gemv") else ():
         xg = torch.randn(Mg, Kg, generator=g).to(torch.bfloat16).to(dev)
         for grouped in (False, True):
             strip = kops.int4_strip_supported(Mg, Kg, Ng, 128 if grouped else None)
@@ -303,7 +348,7 @@ def main():
     # attention and the gating are torch ops.
     decode = None
     decode_int8 = None
-    if not args.no_decode:
+    if want("decode"):
         from keras_amd.decoder_harness import LlamaStyleDecoder
 
         w4_host = packs[0].cpu()
@@ -335,7 +380,7 @@ def main():
 
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None
-    if not args.no_cpu_baseline:
+    if want("cpu"):
         from oracle import keras_cpu_path as ref
 
         Mc = 2048  # bounded sample (about 10 s): 2048 rows of the same K = N = 8192 layer
@@ -382,12 +427,15 @@ def main():
                      "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 4),
                      "traffic": measured_traffic("gemm_mfma_i8_M4096_K8192_N8192"), "kernel": "gemm_mfma<int8>",
                      "avg_launch_us": round(gemm_ms * 1e3, 1), "ops_per_launch": ops_per_step,
+                     # share of what the matrix cores alone sustain on this board with random operands
+                     "frac_of_mfma_only_random": (round(gemm_tops / ceiling[1]["tops"], 4) if ceiling else None),
                      "note": "int8 multiply-accumulate counted as 2 ops; peak is the published dense int8 figure"},
         "quantizer": {"kernel": "quantize_rows_vec", "avg_launch_us": round(quant_ms * 1e3, 1),
                       "roofline": {"bound": "hbm", "achieved": round(quant_bytes / (quant_ms * 1e-3) / 1e9, 1),
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(quant_bytes / (quant_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                                    "traffic": measured_traffic("quantize_rows_vec_bf16_4096x8192")}},
+        "mfma_i8_only": ceiling,
         "int8_gemm_sweep": sweep,
         "einsum_int8": einsum,
         "int4_gemv": gemv,

@@ -116,7 +116,9 @@ def test_gemm_extreme_values(dev):
     assert want.abs().max().item() == K * 127 * 127
 
 
-@pytest.mark.parametrize("M,K,N", [(4096, 8192, 8192), (2048, 4096, 4096), (512, 8192, 28672)])
+@pytest.mark.parametrize("M,K,N", [(4096, 8192, 8192), (2048, 4096, 4096), (512, 8192, 28672),
+                                   (8192, 8192, 8192), (2048, 8192, 28672), (8192, 8192, 28672),
+                                   (8192, 4096, 4096)])
 def test_gemm_full_size_accumulators(dev, M, K, N):
     # full target sizes: sampled rows against the CPU oracle (bit-exact) plus two
     # size-independent integer identities over the whole output

@@ -279,6 +279,23 @@ def test_unsupported_paths_raise(dev):
         cpu_layer(torch.randn(2, 32))  # no CPU fallback
 
 
+def test_non_default_g_idx_is_rejected(dev):
+    # the reference looks the group of row k up in g_idx (quantizers.py:1659-1668); the fused kernels
+    # take k // block_size, so a stored map that says anything else has to raise, not compute
+    for make in (lambda: Dense(64, device=dev), lambda: EinsumDense("ab,bc->ac", (64,), device=dev)):
+        layer = make()
+        layer.build((None, 256))
+        layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=128))
+        x = torch.randn(3, 256, generator=torch.Generator().manual_seed(1))
+        layer(x)  # the map quantize() wrote is fine
+        g = layer.g_idx.value.clone()
+        layer.g_idx.assign(g.flip(0))
+        with pytest.raises(ValueError, match="g_idx"):
+            layer(x)
+        layer.g_idx.assign(g)
+        layer(x)
+
+
 # ---- non-default configs: weight-only int8, activation-quantized int4 --------------------
 @pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16", "bfloat16"])
 @pytest.mark.parametrize("M,K,N", [(16, 4096, 4096), (5, 128, 48), (300, 256, 512), (2, 100, 30),
