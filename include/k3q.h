@@ -320,12 +320,13 @@ int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int cou
  * bytes at 128 rows).
  * w_kmajor: int4 [N, K/2]; dword j of row n holds k = 8j ... 8j+7 of column n, the nibble of
  * k = 8j + 2p at bits [4p, 4p+4) and of k = 8j + 2p + 1 at bits [16+4p, 16+4p+4), each the low
- * four bits of the two's-complement value (keras_amd.ops.int4_kmajor_copy builds it from the
- * stored kernel, once per layer).  scale, zero, block_size, bias, y as for k3q_gemv_w4.
+ * four bits of the two's-complement value (k3q_w4_kmajor_pack builds it from the stored
+ * [K, ceil(N/2)] kernel, once per layer; K % 8 == 0).  scale, zero, block_size, bias, y as for k3q_gemv_w4.
  * Needs K % 128 == 0, N % 32 == 0, K % block_size == 0 and block_size % 64 == 0 (K3Q_ERR_SHAPE
  * otherwise); workspace: k3q_gemm_w4_kmajor_workspace_bytes bytes, 16-byte aligned.
  * Replaces what k3q_gemv_w4 replaces (keras/src/layers/core/dense.py:988-1095).
  */
+int k3q_w4_kmajor_pack(const int8_t* w_packed, int64_t K, int64_t N, int32_t* w_kmajor, void* stream);
 int64_t k3q_gemm_w4_kmajor_workspace_bytes(int64_t M, int64_t K, int64_t N, int64_t block_size);
 int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
                        const void* w_kmajor, const void* scale, const void* zero, int64_t block_size,
@@ -358,7 +359,9 @@ int k3q_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t K, int coun
                       void* stream);
 
 /*
- * Same as k3q_gemv_w4_fused with the launch plan overridden, for tuning sweeps:
+ * TEST HOOK, not for callers: k3q_gemv_w4_fused with the launch plan overridden, so that the
+ * parity tests can run every variant of the kernel (dwords per lane, rows per chunk, waves,
+ * slice length) at one shape instead of relying on the shapes that select them:
  * plan = {dwords per lane per k row (1|2), 16-row steps per chunk (1|2),
  * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null
  * `plan` keep the built-in choice.  The workspace must then hold

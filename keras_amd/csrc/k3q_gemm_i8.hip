@@ -31,10 +31,6 @@ constexpr int kBK = 128;  // bytes of K per stage: one full 128-byte line per ro
 constexpr int kStages = 2;
 constexpr int kKSteps = kBK / 32;  // MFMA K steps per stage
 constexpr int kRowChunks = kBK / 16;  // 16-byte chunks per LDS row
-#ifndef K3Q_GEMM_WAVES_N
-#define K3Q_GEMM_WAVES_N 4
-#define K3Q_GEMM_WAVES_M 2
-#endif
 
 // Tile shape of a workgroup: BM rows of a / y, BN rows of the prepacked weight (= columns of
 // y), waves laid out WN (along N) x WM (along M).
@@ -55,16 +51,13 @@ struct Tile {
     static constexpr int kDmaPerWave = (kDmaA + kDmaB) / (kThreads / 64);
 };
 // 256 x 256, 8 waves, 128 KiB of LDS: one workgroup per CU; the shape for large problems.
-typedef Tile<256, 256, K3Q_GEMM_WAVES_N, K3Q_GEMM_WAVES_M> TileLarge;
+typedef Tile<256, 256, 4, 2> TileLarge;
 // 128 x 128, 4 waves, 64 KiB of LDS: two workgroups per CU; used while the large tile would
 // leave CUs without work.
 typedef Tile<128, 128, 2, 2> TileSmall;
 
 constexpr int kFlagExactEpilogue = 1;
 constexpr int kFlagRoundAccBF16 = 2;   // float32 output of a bfloat16 layer: acc is cast to bfloat16 first
-constexpr int kFlagSkipEpilogue = 1024;  // undocumented timing aid
-constexpr int kFlagForceSmallTile = 2048;  // undocumented tuning aids
-constexpr int kFlagForceLargeTile = 4096;
 
 struct GemmParams {
     const int8_t* a;        // [M, K]
@@ -190,10 +183,6 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
     constexpr int kATileBytes = T::kATileBytes, kStageBytes = T::kStageBytes;
     constexpr int kDmaA = T::kDmaA, kDmaPerWave = T::kDmaPerWave;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
-#ifdef K3Q_GEMM_PROBE_CLOCK
-    const uint64_t clk0 = __builtin_readcyclecounter();
-    const uint64_t rt0 = __builtin_amdgcn_s_memrealtime();
-#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -244,9 +233,6 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
             char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
 #pragma unroll
             for (int d = 0; d < kDmaPerWave; ++d) {
-#ifdef K3Q_GEMM_PROBE_NO_BDMA
-                if (wave * kDmaPerWave + d >= kDmaA) continue;
-#endif
                 __builtin_amdgcn_global_load_lds(
                     (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
                     (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
@@ -269,11 +255,9 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         int rb = kATileBytes + (wn * kWN + fi) * kBK + lane_chunk;
         v4i af[2][kMBlk], bf[2][kNBlk];
         auto read_frags = [&](int fb, int ks) {
-#ifndef K3Q_GEMM_PROBE_NO_BREAD
             const char* pb = lds + (rb ^ (32 * ks));
 #pragma unroll
             for (int nb = 0; nb < kNBlk; ++nb) bf[fb][nb] = *(const v4i*)(pb + nb * 32 * kBK);
-#endif
             const char* pa = lds + (ra ^ (32 * ks));
 #pragma unroll
             for (int mb = 0; mb < kMBlk; ++mb) af[fb][mb] = *(const v4i*)(pa + mb * 32 * kBK);
@@ -314,9 +298,6 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         constexpr int kDmaStride = 5 * kHalfMmas / kDmaPerWave >= 2 ? 2 : 1;
         static_assert(kKSteps == 4 && 5 * kHalfMmas / kDmaStride >= kDmaPerWave, "DMA slots");
         auto issue_one = [&](int kt, int d) {
-#ifdef K3Q_GEMM_PROBE_NO_BDMA
-            if (wave * kDmaPerWave + d >= kDmaA) return;
-#endif
             char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
@@ -329,10 +310,7 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
 #pragma unroll
             for (int j = 0; j < kHalfMmas; ++j) {
                 const int nb = half * (kNBlk / 2) + j / kMBlk, mb = j % kMBlk;
-#ifndef K3Q_GEMM_PROBE_NO_MMA
                 acc[nb][mb] = Mma<kKind>::run(bf[ks & 1][nb], af[ks & 1][mb], acc[nb][mb]);
-#endif
-#ifndef K3Q_GEMM_PROBE_NO_DMA
                 const int pos = hh * kHalfMmas + j;
                 if (hh >= 0 && pos % kDmaStride == kDmaStride - 1 && pos / kDmaStride < kDmaPerWave) {
                     const int target = hh == 0 ? kt + 2 : kt + 1;
@@ -342,7 +320,6 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
-#endif
             }
         };
         for (int kt = 0; kt < KT; ++kt) {
@@ -370,23 +347,10 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
                 __builtin_amdgcn_sched_barrier(0);
                 mma_half(ks, 1, kt);
                 __builtin_amdgcn_s_setprio(0);
-#ifdef K3Q_GEMM_PROBE_NO_MMA
-                // probe build: consume the fragments so that the reads stay
-#pragma unroll
-                for (int mb = 0; mb < kMBlk; ++mb) acc[0][mb][0] += (af[ks & 1][mb][0] ^ bf[ks & 1][mb & 1][1]);
-#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
 
-#ifdef K3Q_GEMM_PROBE_CLOCK
-        if (p.acc_out && tid == 0 && blockIdx.x < 64) {
-            uint64_t* d = (uint64_t*)p.acc_out + 2 * blockIdx.x;
-            d[0] = __builtin_readcyclecounter() - clk0;
-            d[1] = __builtin_amdgcn_s_memrealtime() - rt0;
-        }
-        if (p.acc_out) return;
-#endif
         if (p.splits > 1) {
             // raw accumulators of this split, as they lie (16 bytes per lane and column group)
 #pragma unroll
@@ -410,17 +374,6 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         // acc[nb][mb][r] is output (m, n) with m = m0 + wm*kWM + mb*32 + lane%32 and
         // n = n0 + wn*kWN + nb*32 + 8*(r/4) + 4*(lane/32) + r%4: a lane owns one row of y per mb
         // and groups of four consecutive columns.
-        if (p.flags & kFlagSkipEpilogue) {  // timing aid: main loop only
-            int sink = 0;
-#pragma unroll
-            for (int nb = 0; nb < kNBlk; ++nb)
-#pragma unroll
-                for (int mb = 0; mb < kMBlk; ++mb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) sink ^= (int)acc[nb][mb][r];
-            if (sink == 0x7fffffff && p.y) ((char*)p.y)[0] = 1;
-            continue;
-        }
         // Stage the tile's scales and bias in LDS as floats (the main loop is done with it): the
         // per-lane reads below are then cheap and need no large register arrays.
         float* ep = (float*)lds;  // [0,256) b_scale or its reciprocal, [256,512) bias, [512,768) a_scale or reciprocal
@@ -842,8 +795,7 @@ __global__ __launch_bounds__(256) void gemm_split_reduce(GemmParams p) {
 // writing and reading its 64 KiB of partials, and is taken while tiles * sp still fit on the
 // chip at once.  E.g. 32 tiles x 32 stages: 4; 64 x 64: 4; 32 x 112: 8; 128 x 64: 3;
 // 128 x 16 or 96 x 32: none.
-inline int choose_splits(int64_t tiles, int64_t stages, int resident, int forced) {
-    if (forced > 0) return (int)(forced < stages ? forced : stages);
+inline int choose_splits(int64_t tiles, int64_t stages, int resident) {
     int best = 1;
     int64_t best_gain_ns = 0;
     for (int sp = 2; sp <= 8; ++sp) {
@@ -857,14 +809,13 @@ inline int choose_splits(int64_t tiles, int64_t stages, int resident, int forced
     return best;
 }
 
-constexpr int kFlagSplitShift = 16;  // undocumented tuning aid: bits 16..20 force the split count
 
 // Room for the partials of the largest split the launch may choose (sized for a chip of up
 // to 256 CUs; a launch that finds less room splits less).
 inline int64_t split_workspace_bytes(int64_t M, int64_t N, int64_t row_bytes) {
     if (M <= 0 || (row_bytes % kBK) != 0 || (N % 4) != 0) return 0;
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
-    const int splits = choose_splits(tiles, row_bytes / kBK, 512, 0);
+    const int splits = choose_splits(tiles, row_bytes / kBK, 512);
     return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
 }
 
@@ -882,7 +833,7 @@ int launch_tile(GemmParams p, hipStream_t s) {
     const int resident = cu_count() * (T::kLdsBytes <= 64 * 1024 ? 2 : 1) / 8 * 8;
     const int stages = (int)(p.row_bytes / kBK);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
-    int splits = (p.N % 4) ? 1 : choose_splits(tiles, stages, resident, (p.flags >> kFlagSplitShift) & 31);
+    int splits = (p.N % 4) ? 1 : choose_splits(tiles, stages, resident);
     // partials need room and 16-byte rows (no split for N % 4 != 0, above)
     if (splits > 1 && (!p.part || p.part_bytes < (int64_t)splits * p.M * p.N * 4)) {
         const int64_t fit = p.part ? p.part_bytes / (p.M * p.N * 4) : 0;
@@ -908,8 +859,7 @@ constexpr int64_t kLargeTileMinTiles = 224;
 template <int kKind, bool kBF16, bool kExact>
 int launch_mfma(const GemmParams& p, hipStream_t s) {
     const int64_t large_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
-    const bool large = (p.flags & kFlagForceLargeTile) ||
-                       (large_tiles >= kLargeTileMinTiles && !(p.flags & kFlagForceSmallTile));
+    const bool large = large_tiles >= kLargeTileMinTiles;
     if (large) return launch_tile<TileLarge, kKind, kBF16, kExact>(p, s);
     return launch_tile<TileSmall, kKind, kBF16, kExact>(p, s);
 }
@@ -1021,7 +971,6 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     if (b_layout == 0 && gemm_i8_skinny_supported(M, N, K, a, b))
         return gemm_i8_skinny_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
                                   workspace, workspace_bytes, s);
-    const bool forced_tile = (flags & (kFlagForceSmallTile | kFlagForceLargeTile)) != 0;
     // K % 128 != 0 (model widths like 1600 or 960): both operands are copied into scratch with
     // their rows zero-padded to the tile's K step; zeros add nothing, the result is the same
     const int64_t Kpad = (K + kBK - 1) / kBK * kBK;
@@ -1034,7 +983,7 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
     // [N,K] kernel at decode sizes: the streaming kernel up to 8 rows; beyond that the 128-row
     // tiles (which split K while they are few) are as fast or faster (K = N = 8192, 16 rows:
     // 24 us streamed, 19 us tiled; vocabulary 32000 x 4096, 64 rows: 176 us in passes, 41 us tiled)
-    if (b_layout == 1 && !forced_tile && gemm_i8_skinny_nk_supported(M, N, K, a, b) &&
+    if (b_layout == 1 && gemm_i8_skinny_nk_supported(M, N, K, a, b) &&
         (M <= 8 || !fast))
         return gemm_i8_skinny_nk_run(a, b, M, N, K, a_scale, b_scale, bias, bf16, flags, y, acc_out,
                                      workspace, workspace_bytes, s);

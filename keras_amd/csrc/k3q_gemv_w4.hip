@@ -227,9 +227,6 @@ __device__ __forceinline__ Packed<kVec> load_packed(const uint8_t* p) {
 template <int kVec, int kSteps, int kSets, bool kXF32, bool kGrouped>
 __device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, const int by) {
     extern __shared__ float red[];  // [waves][M][kNB + kRedPad]
-#ifdef K3Q_GEMV_PROBE
-    const uint64_t ts0 = __builtin_amdgcn_s_memrealtime();
-#endif
     // Every kernel argument is fetched now, in one scalar round trip, instead of in four
     // dependent ones spread over the address set-up (0.8 us before the first load otherwise);
     // launch geometry comes with the arguments, not from the dispatch packet.
@@ -464,9 +461,6 @@ __device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, 
 
     load_chunk(0, 0);
     if (kGrouped) load_group((kw0 < p.K ? kw0 : p.K - 1) / p.block_size);
-#ifdef K3Q_GEMV_PROBE
-    const uint64_t ts1 = __builtin_amdgcn_s_memrealtime();
-#endif
 #pragma unroll 1
     for (int c = 0; c < nchunks; c += 2) {
         if (c + 1 < nchunks) load_chunk(1, c + 1);
@@ -479,9 +473,6 @@ __device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, 
         }
     }
 
-#ifdef K3Q_GEMV_PROBE
-    const uint64_t ts2 = __builtin_amdgcn_s_memrealtime();
-#endif
     // ---- remove the +136 offset (per-channel) and park this wave's partial in LDS ----
 #pragma unroll
     for (int a = 0; a < kAccSets; ++a) {
@@ -502,13 +493,7 @@ __device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, 
             }
         }
     }
-#ifdef K3Q_GEMV_PROBE
-    const uint64_t ts2b = __builtin_amdgcn_s_memrealtime();
-#endif
     __syncthreads();
-#ifdef K3Q_GEMV_PROBE
-    const uint64_t ts2c = __builtin_amdgcn_s_memrealtime();
-#endif
 
     // ---- reduce the waves of this workgroup, four columns per thread ----
     const int KS = p.ks;
@@ -529,13 +514,6 @@ __device__ __forceinline__ void gemv_w4_body(const GemvParams& p, const int bx, 
             }
         }
     }
-#ifdef K3Q_GEMV_PROBE
-    if (threadIdx.x == 0 && KS > 1) {
-        uint64_t* d = (uint64_t*)(p.part + (int64_t)KS * M * p.N) + 8 * (by * (8 * per_xcd) + bx);
-        d[0] = ts0; d[1] = ts1; d[2] = ts2; d[3] = __builtin_amdgcn_s_memrealtime();
-        d[4] = ts2b; d[5] = ts2c;
-    }
-#endif
     // ---- K split finished in this launch ----
     // The workgroup that arrives last at its column block's counter sums the KS partials (in
     // the order of the split, whoever comes last) and applies the epilogue; it leaves the
@@ -1641,6 +1619,38 @@ extern "C" int k3q_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t 
         if (rc != K3Q_OK) return rc;
     }
     return K3Q_OK;
+}
+
+namespace k3q {
+namespace {
+// One thread per dword of the K-contiguous copy; threads of a wave take neighbouring columns,
+// so the reads of the stored kernel (row-major [K, ceil(N/2)]) are contiguous per row.
+__global__ __launch_bounds__(256) void w4_kmajor_pack(const uint8_t* __restrict__ w, u32* __restrict__ out,
+                                                     int64_t K8, int64_t N) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= K8 * N) return;
+    const int64_t n = t % N, j = t / N;
+    const int64_t row_bytes = (N + 1) / 2;
+    const int shift = (int)(n & 1) * 4;
+    u32 d = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const u32 nib = (w[(8 * j + e) * row_bytes + n / 2] >> shift) & 0xFu;
+        d |= nib << ((e & 1) * 16 + (e >> 1) * 4);
+    }
+    out[n * K8 + j] = d;
+}
+}  // namespace
+}  // namespace k3q
+
+extern "C" int k3q_w4_kmajor_pack(const int8_t* w_packed, int64_t K, int64_t N, int32_t* w_kmajor, void* stream) {
+    if (K <= 0 || N <= 0 || (K % 8) != 0 || (K / 8) * N >= ((int64_t)1 << 39)) return K3Q_ERR_SHAPE;
+    if (!w_packed || !w_kmajor) return K3Q_ERR_NULL;
+    if (!aligned_to(w_kmajor, 4)) return K3Q_ERR_ALIGN;
+    const int64_t dwords = (K / 8) * N;
+    k3q::w4_kmajor_pack<<<(unsigned)((dwords + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint8_t*)w_packed, (u32*)w_kmajor, K / 8, N);
+    return launch_status();
 }
 
 extern "C" int64_t k3q_gemm_w4_kmajor_workspace_bytes(int64_t M, int64_t K, int64_t N, int64_t block_size) {

@@ -195,6 +195,30 @@ class _GemmView:
         self.k_plain = self.k_is_view
 
 
+class _BatchedView:
+    """An einsum `X,Y->Z` that `_GemmView` does not take, as a stack of `[M, K] x [K, N]`
+    products: labels that the input, the kernel and the output share count the products,
+    a label the input alone carries is summed by giving the kernel a copy per value, and an
+    einsum without a shared summed label has K = 1."""
+
+    def __init__(self, i_spec, k_spec, o_spec):
+        si, sk, so = set(i_spec), set(k_spec), set(o_spec)
+        if sk - si - so:
+            raise NotImplementedError(
+                f"labels {sorted(sk - si - so)} are summed out of the kernel alone: not lowered to "
+                "the quantized GEMM")
+        self.i_spec, self.k_spec, self.o_spec = i_spec, k_spec, o_spec
+        self.batch = [c for c in i_spec if c in sk and c in so]
+        self.free = [c for c in i_spec if c in so and c not in sk]
+        self.kept = [c for c in k_spec if c in so and c not in si]
+        self.contracted = [c for c in i_spec if c in sk and c not in so]
+        self.input_only = [c for c in i_spec if c not in sk and c not in so]
+        # the quantizer reduces the labels the output lacks; the rows it sees keep the others in
+        # input order, so that its scales reshape into the keepdims shape the reference adjusts
+        self.rows = [c for c in i_spec if c in so]
+        self.reduced = [c for c in i_spec if c not in so]
+
+
 class EinsumDense(Layer):
     def __init__(self, equation, output_shape, activation=None, bias_axes=None,
                  kernel_initializer=None, bias_initializer="zeros", dtype=None, name=None,
@@ -263,10 +287,15 @@ class EinsumDense(Layer):
         self._kernel_reduced_axes = info["kernel"]["reduced"]
         self._custom_gradient_equation = info["custom_gradient_equation"]
         self._gemm = None
+        self._batched = None
         try:
             self._gemm = _GemmView(*info["specs"])
         except NotImplementedError as e:
             self._gemm_error = e
+            try:
+                self._batched = _BatchedView(*info["specs"])
+            except NotImplementedError as e2:
+                self._gemm_error = e2
 
     def quantized_build(self, kernel_shape, mode, config=None):
         if mode == "int8":
@@ -451,6 +480,8 @@ class EinsumDense(Layer):
     def _row_bias_ok(self):
         if self.bias is not None or self.activation is not None or not self.built:
             return False
+        if getattr(self, "_gemm", None) is None:
+            return False
         gv = self._gemm_view()
         o_spec = self._quant_info["specs"][2]
         return list(o_spec[len(o_spec) - len(gv.kept):]) == gv.kept
@@ -463,6 +494,8 @@ class EinsumDense(Layer):
         """keras/src/layers/core/einsum_dense.py:1030-1118 as quantise-rows + int8 GEMM."""
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
+        if self._gemm is None and self._batched is not None:
+            return self._int8_call_batched(inputs)
         gv = self._gemm_view()
         x2, free_shape = self._input_rows(inputs, gv)
         cd = to_torch_dtype(self.compute_dtype)
@@ -498,10 +531,105 @@ class EinsumDense(Layer):
         )
         return self._finish(y2, free_shape, gv, fused)
 
+    def _int8_call_batched(self, inputs):
+        """keras/src/layers/core/einsum_dense.py:1030-1118 for equations with labels shared by
+        input, kernel and output, without a summed label, or with one the input alone carries
+        (e.g. "abcde,afce->acdbf", "a,b->ab", "ab,ab->a", einsum_dense_test.py:598-629).
+
+        The integer einsum runs as one exact int8 GEMM per value of the shared labels (raw int32
+        accumulators); the de-scale is then the reference's own broadcast, `acc / (inputs_scale *
+        kernel_scale)` with both scales in the shapes its transpose / expand / squeeze
+        bookkeeping gives them, so results (and result shapes) are the reference's for every
+        equation it accepts."""
+        bv = self._batched
+        cd = to_torch_dtype(self.compute_dtype)
+        if not self.inputs_quantizer:
+            # weight-only (einsum_dense.py:1085-1101): every weight divided by its scale, float einsum
+            ks = as_tensor(self.kernel_scale).to(cd)
+            part = self._quant_info["kernel"]
+            for ax in sorted(part["squeeze"]):
+                ks = ks.unsqueeze(ax)
+            for ax in sorted(part["expand"], reverse=True):
+                ks = ks.squeeze(ax)
+            if part["transpose"]:
+                perm = part["transpose"]
+                ks = ks.permute(sorted(range(len(perm)), key=perm.__getitem__))
+            y = torch.einsum(self.equation, inputs.to(cd), torch.divide(as_tensor(self._kernel).to(cd), ks))
+        else:
+            size = dict(zip(bv.i_spec, inputs.shape))
+            size.update(zip(bv.k_spec, self._kernel.shape))
+            prod = lambda labels: math.prod(size[c] for c in labels)
+            # quantise over the labels the output lacks: rows in input order, those labels last
+            x2 = inputs.permute([bv.i_spec.index(c) for c in bv.rows + bv.reduced]).reshape(
+                prod(bv.rows), prod(bv.reduced))
+            q2, scale = quantize_rows(self.inputs_quantizer, x2.contiguous())
+            s_in = scale.reshape([1 if c in bv.reduced else size[c] for c in bv.i_spec])
+            s_adj = _adjust_scale(s_in, self._quant_info["input"])
+            # [batch, M, K] rows against [batch, K, N] kernels
+            q_labels = bv.rows + bv.reduced
+            q = q2.reshape([size[c] for c in q_labels])
+            order = bv.batch + bv.free + bv.contracted + bv.input_only
+            q3 = q.permute([q_labels.index(c) for c in order]).reshape(
+                prod(bv.batch), prod(bv.free), prod(bv.contracted + bv.input_only)).contiguous()
+
+            def kernel_stack(t):
+                k = t.permute([bv.k_spec.index(c) for c in bv.batch + bv.contracted + bv.kept])
+                k = k.reshape(prod(bv.batch), prod(bv.contracted), 1, prod(bv.kept))
+                k = k.expand(-1, -1, prod(bv.input_only), -1)  # a copy per value of an input-only label
+                return k.reshape(prod(bv.batch), -1, prod(bv.kept)).contiguous()
+
+            shape_key = tuple(size[c] for c in bv.input_only)
+            hit = self._cache.get("kernel_stack")
+            if hit is None or hit[0] != (self._kernel.version, shape_key) or hit[1] is not self._kernel:
+                hit = self._cache["kernel_stack"] = ((self._kernel.version, shape_key), self._kernel,
+                                                     kernel_stack(as_tensor(self._kernel)))
+            k3 = hit[2]
+            acc = torch.stack([kops.int8_matmul(q3[b], k3[b], want_acc=True, want_y=False)
+                               for b in range(q3.shape[0])])
+            acc = acc.reshape([size[c] for c in bv.batch + bv.free + bv.kept])
+            have = bv.batch + bv.free + bv.kept
+            acc = acc.permute([have.index(c) for c in bv.o_spec])
+            y = torch.divide(acc.to(cd), torch.multiply(s_adj, as_tensor(self.kernel_scale).to(cd)))
+        if self.bias is not None:
+            y = torch.add(y, self.read(self.bias))
+        if self.activation is not None:
+            y = self.activation(y)
+        return y
+
+    def _int4_call_batched(self, inputs):
+        """keras/src/layers/core/einsum_dense.py:1120-1261 for the equations `_int8_call_batched`
+        takes: the kernel is de-quantised once (kept until a variable changes), reshaped to its own
+        shape and contracted in the compute dtype, as the reference does on every call."""
+        cd = to_torch_dtype(self.compute_dtype)
+        block_size = self._int4_block_size
+        grouped = block_size is not None and block_size > 0
+        if self.inputs_quantizer:
+            raise NotImplementedError("activation-quantized int4 is built for GEMM-shaped equations only")
+        variables = [self._kernel, self.kernel_scale] + ([self.kernel_zero, self.g_idx] if grouped else [])
+        stamp = tuple((id(v), v.version) for v in variables) + (cd,)
+        hit = self._cache.get("int4_float_kernel")
+        if hit is None or hit[0] != stamp:
+            unpacked = quantizers.unpack_int4(as_tensor(self._kernel), self._int4_unpacked_column_size, axis=-1)
+            scale = as_tensor(self.kernel_scale).to(cd)
+            if grouped:
+                fk = quantizers.dequantize_with_sz_map(
+                    unpacked, scale, as_tensor(self.kernel_zero), as_tensor(self.g_idx), group_axis=0).to(cd)
+            else:
+                fk = torch.divide(unpacked.to(cd), scale)
+            hit = self._cache["int4_float_kernel"] = (stamp, fk.reshape(self.original_kernel_shape))
+        y = torch.einsum(self.equation, inputs.to(cd), hit[1])
+        if self.bias is not None:
+            y = torch.add(y, self.read(self.bias))
+        if self.activation is not None:
+            y = self.activation(y)
+        return y
+
     def _int4_call(self, inputs, training=None):
         """keras/src/layers/core/einsum_dense.py:1120-1261, weight-only."""
         if self.lora_enabled:
             raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
+        if self._gemm is None and self._batched is not None:
+            return self._int4_call_batched(inputs)
         gv = self._gemm_view()
         x2, free_shape = self._input_rows(inputs, gv)
         cd = to_torch_dtype(self.compute_dtype)

@@ -7,32 +7,36 @@ device and stream for the split-K kernels).
 """
 
 import ctypes
+import threading
 
 import torch
 
 from keras_amd import _lib
 
 _workspaces = {}
+_scratch_lock = threading.Lock()
 
 
 def _workspace(device, nbytes):
     """Scratch for split-K partial sums and the per-call [N, K] weight copy.
 
-    One buffer per (device, stream): calls on one stream are ordered, so they
-    can share it; calls on different streams may overlap and must not.
+    One buffer per (device, stream, host thread): the calls one thread makes on one stream are
+    ordered, so they can share it; calls on different streams may overlap, and two threads on
+    one stream may interleave the launches of a two-kernel call, so neither shares.
     """
     stream = torch.cuda.current_stream(device)
-    key = (device.index, stream.cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        # A captured HIP graph keeps the address of the buffer its kernels were recorded with:
-        # an outgrown buffer is retired, never freed (sizes at least double, so the retired
-        # ones together stay below the live one).
-        if ws is not None:
-            _retired.append(ws)
-        size = max(int(nbytes), 1 << 20, 2 * (ws.numel() if ws is not None else 0))
-        ws = torch.zeros(size, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+    key = (device.index, stream.cuda_stream, threading.get_ident())
+    with _scratch_lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            # A captured HIP graph keeps the address of the buffer its kernels were recorded with:
+            # an outgrown buffer is retired, never freed (sizes at least double, so the retired
+            # ones together stay below the live one).
+            if ws is not None:
+                _retired.append(ws)
+            size = max(int(nbytes), 1 << 20, 2 * (ws.numel() if ws is not None else 0))
+            ws = torch.zeros(size, dtype=torch.uint8, device=device)
+            _workspaces[key] = ws
     return ws
 
 
@@ -43,15 +47,17 @@ _counters = {}
 
 
 def _arrival_counters(device, nbytes):
-    """Arrival counters of the single-launch K split: zero between calls, one per (device, stream)."""
+    """Arrival counters of the single-launch K split: zero between calls, one set per
+    (device, stream, host thread), like the workspace they go with."""
     stream = torch.cuda.current_stream(device)
-    key = (device.index, stream.cuda_stream)
-    c = _counters.get(key)
-    if c is None or c.numel() < nbytes:
-        if c is not None:
-            _retired.append(c)  # a captured graph may still count in it
-        c = torch.zeros(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
-        _counters[key] = c
+    key = (device.index, stream.cuda_stream, threading.get_ident())
+    with _scratch_lock:
+        c = _counters.get(key)
+        if c is None or c.numel() < nbytes:
+            if c is not None:
+                _retired.append(c)  # a captured graph may still count in it
+            c = torch.zeros(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
+            _counters[key] = c
     return c
 
 
@@ -326,19 +332,18 @@ def int4_kmajor_copy(kernel_packed, units):
     a column per dword, even k in the low half-word's nibbles, odd k in the high half-word's
     (include/k3q.h, k3q_gemm_w4_kmajor).  Made once per layer from the stored
     `[K, ceil(N/2)]` kernel; K % 8 == 0."""
-    from keras_amd import quantizers
-
-    q = quantizers.unpack_int4(kernel_packed, int(units), axis=-1)      # int8 [K, N]
-    K, N = q.shape
+    _lib.require_device(kernel_packed)
+    lib = _lib.load()
+    K, N = int(kernel_packed.shape[0]), int(units)
+    if kernel_packed.dtype != torch.int8 or kernel_packed.dim() != 2 or kernel_packed.shape[1] != (N + 1) // 2:
+        raise ValueError(f"expected the stored int8 kernel [K, ceil({N}/2)], got {tuple(kernel_packed.shape)}")
     if K % 8:
         raise ValueError("the K-contiguous copy needs K % 8 == 0")
-    u = (q.t().contiguous().to(torch.int64) & 0xF).reshape(N, K // 8, 8)
-    d = torch.zeros((N, K // 8), dtype=torch.int64, device=q.device)
-    for p in range(4):
-        d |= u[..., 2 * p] << (4 * p)
-        d |= u[..., 2 * p + 1] << (16 + 4 * p)
-    d = torch.where(d >= 1 << 31, d - (1 << 32), d)   # as two's-complement int32
-    return d.to(torch.int32).contiguous()
+    src = kernel_packed if kernel_packed.is_contiguous() else kernel_packed.contiguous()
+    out = torch.empty((N, K // 8), dtype=torch.int32, device=src.device)
+    _lib.check(lib.k3q_w4_kmajor_pack(_lib.ptr(src), K, N, _lib.ptr(out), _lib.stream_ptr(src.device)),
+               "k3q_w4_kmajor_pack")
+    return out
 
 
 def int4_kmajor_supported(M, K, N, block_size=None):

@@ -87,7 +87,11 @@ def abs_max_quantize(
     x = inputs if isinstance(inputs, torch.Tensor) else torch.as_tensor(inputs)
     if isinstance(axis, list):
         axis = tuple(axis)
-    amax = torch.amax(torch.abs(x), dim=axis, keepdim=True)  # numpy.py:298-305
+    if axis == ():
+        # numpy.py:302-304: an empty axis tuple reduces nothing (torch.amax would reduce everything)
+        amax = torch.abs(x)
+    else:
+        amax = torch.amax(torch.abs(x), dim=axis, keepdim=True)  # numpy.py:298-305
     denom = torch.add(amax, _scalar_tensor(float(epsilon)))  # numpy.py:68-71
     scale = torch.divide(value_range[1], denom)  # numpy.py:2192-2197
     scale = scale.to(x.dtype)

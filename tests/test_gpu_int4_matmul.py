@@ -295,6 +295,26 @@ def test_int4_kmajor_route(dev, M, K, N, block_size, with_bias):
     run_kmajor_case(dev, M, K, N, block_size, with_bias)
 
 
+@pytest.mark.parametrize("K,N", [(128, 32), (256, 96), (8, 1), (64, 33), (4096, 4096)])
+def test_kmajor_copy_layout(dev, K, N):
+    # dword j of row n: the nibble of k = 8j + 2p at bits [4p, 4p+4), of k = 8j + 2p + 1 at bits
+    # [16+4p, 16+4p+4), each the low four bits of the stored value; built here from the
+    # oracle's unpack, value by value
+    g = torch.Generator().manual_seed(K + N)
+    q = torch.randint(-8, 8, (K, N), generator=g, dtype=torch.int8)
+    packed, _, _ = ref.pack_int4(q, axis=-1)
+    got = kops.int4_kmajor_copy(packed.to(dev), N).cpu()
+    u = (q.t().contiguous().to(torch.int64) & 0xF).reshape(N, K // 8, 8)
+    want = torch.zeros((N, K // 8), dtype=torch.int64)
+    for p in range(4):
+        want |= u[..., 2 * p] << (4 * p)
+        want |= u[..., 2 * p + 1] << (16 + 4 * p)
+    assert got.dtype == torch.int32 and tuple(got.shape) == (N, K // 8)
+    assert torch.equal(got.to(torch.int64) & 0xFFFFFFFF, want)
+    with pytest.raises(ValueError):
+        kops.int4_kmajor_copy(packed[: K - 1].to(dev), N)
+
+
 def run_kmajor_case(dev, M, K, N, block_size, with_bias, seed=90):
     # 17 ... 512 bfloat16 rows from the K-contiguous copy of the kernel: against the oracle, the
     # float64 value, and the other route's result

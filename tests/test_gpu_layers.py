@@ -150,6 +150,81 @@ def test_einsum_dense_int8(dev, equation, output_shape, input_shape, policy):
     assert (y_float.float() - y.float()).pow(2).mean().item() < 2e-2
 
 
+# equations outside the plain GEMM view: labels shared by input, kernel and output, no summed
+# label, a label the input alone carries; the first three are the reference's own
+# (einsum_dense_test.py:598-629: "reduce and transpose", "expand", "squeeze")
+GENERAL = [
+    ("abcde,afce->acdbf", (2, 4, 8, 16), (1, 8, 2, 4, 32), "d"),
+    ("a,b->ab", (4,), (5,), None),
+    ("ab,ab->a", (2,), (2, 4), None),
+    ("ab,c->ac", (5,), (3, 4), "c"),
+    ("bhqd,hdk->bhqk", (8, 16, 96), (3, 8, 16, 64), "k"),
+    ("abcde,afce->acdbf", (3, 4, 40, 48), (2, 40, 3, 4, 256), None),
+]
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape,bias_axes", GENERAL)
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_einsum_dense_int8_general_equations(dev, equation, output_shape, input_shape, bias_axes, policy):
+    g = torch.Generator().manual_seed(99)
+    layer = EinsumDense(equation, output_shape, bias_axes=bias_axes, dtype=policy, device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d),
+                        bias_initializer=lambda s, d: torch.randn(s, generator=g).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu() if layer.bias is not None else None
+    x = torch.rand(input_shape, generator=g) - 0.3
+    y_float = layer(x)
+    layer.quantize("int8")
+    assert layer.dtype_policy.name == f"int8_from_{policy}"
+    qk, ks, _ = ref.einsum_dense_quantize_int8(kernel_f, equation, len(input_shape))
+    assert layer._kernel.dtype == "int8" and layer.kernel_scale.dtype == "float32"
+    assert torch.equal(layer._kernel.value.cpu(), qk)
+    assert tuple(layer.kernel_scale.shape) == tuple(ks.shape)
+    assert torch.equal(layer.kernel_scale.value.cpu(), ks)
+    y = layer(x)
+    want = ref.einsum_dense_int8_call(x.to(cd), qk, ks, equation, bias=bias_f, compute_dtype=cd)
+    # (the reference's scale bookkeeping gives "ab,ab->a" a [1, a] result: kept as it is)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    assert torch.equal(bits(y.cpu().contiguous()), bits(want.contiguous()))
+    assert (y_float.float().cpu() - y.float().cpu()).pow(2).mean().item() < 2e-2
+    # the same layer built from its quantized policy (as the reference's test does), variables loaded
+    twin = EinsumDense(equation, output_shape, bias_axes=bias_axes, dtype=f"int8_from_{policy}", device=dev)
+    twin.build(input_shape)
+    assert twin._kernel.dtype == "int8" and twin.kernel_scale.dtype == "float32"
+    store = {}
+    layer.save_own_variables(store)
+    twin.load_own_variables(store)
+    assert torch.equal(bits(twin(x).cpu().contiguous()), bits(want.contiguous()))
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape,bias_axes", GENERAL)
+@pytest.mark.parametrize("block_size", [8, None])
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_einsum_dense_int4_general_equations(dev, equation, output_shape, input_shape, bias_axes, block_size, policy):
+    g = torch.Generator().manual_seed(98)
+    layer = EinsumDense(equation, output_shape, bias_axes=bias_axes, dtype=policy, device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d),
+                        bias_initializer=lambda s, d: torch.randn(s, generator=g).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu() if layer.bias is not None else None
+    x = torch.rand(input_shape, generator=g) - 0.3
+    layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=block_size))
+    qk = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), block_size)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    assert torch.equal(layer.kernel_scale.value.cpu(), qk["kernel_scale"])
+    y = layer(x)
+    want = ref.einsum_dense_int4_call(x.to(cd), qk, equation, bias=bias_f, compute_dtype=cd,
+                                      block_size=block_size)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    # the same op sequence as the reference on the device (de-quantise, reshape, float einsum):
+    # only the order of the sums inside the einsum differs
+    assert max_rel_err(y, want) <= RTOL[cd]
+
+
 # kernels whose contracted axis is not leading ("ndh" contracts d): the stored int4 matrix is a
 # row-major reshape that mixes output columns, so these run de-quantise + float GEMM
 NON_LEADING = [

@@ -116,6 +116,21 @@ def test_abs_max_closed_form_rows():
     assert q[2].tolist() == [round(v) for v in (x[2] * s[2, 0]).tolist()]
 
 
+def test_abs_max_empty_axis_reduces_nothing():
+    # keras/src/backend/torch/numpy.py:302-304: amax over axis=() returns x itself (as numpy's
+    # max over an empty axis tuple does), so every element gets its own scale 127 / (|x| + eps)
+    # and every element that is not tiny lands on +-127
+    x = torch.tensor([[0.5, -3.0, 0.0], [1e-3, 7.25, -1.0]])
+    q, s = ref.abs_max_quantize(x, axis=())
+    assert tuple(s.shape) == tuple(x.shape)
+    assert torch.allclose(s, 127.0 / (x.abs() + 1e-7), rtol=1e-6, atol=0)
+    assert q.tolist() == [[127, -127, 0], [127, 127, -127]]
+    qn, sn = ref.abs_max_quantize(x, axis=(), to_numpy=True)
+    assert torch.equal(qn, q) and torch.allclose(sn, s, rtol=1e-6, atol=0)
+    q2, s2 = ref.AbsMaxQuantizer()(x, axis=())
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
 @pytest.mark.parametrize("dtype_code,dtype", [(0, torch.float32), (1, torch.bfloat16)])
 def test_abs_max_c_restatement_agrees(dtype_code, dtype):
     g = torch.Generator().manual_seed(1)
@@ -254,10 +269,42 @@ def test_einsum_info_hand_derived_rows():
     assert tuple(s2.shape) == (1, 1, 16)
 
 
+def test_einsum_info_shared_label_and_stale_index_rows():
+    # hand-derived from keras/src/layers/core/einsum_dense.py:1995-2040 for the equations of
+    # einsum_dense_test.py:598-629.  "abcde,afce->acdbf": input keeps a,b,c,d (transpose to
+    # a,c,d,b), e is reduced and takes the place of f (the one output label the input lacks);
+    # kernel a,f,c,e: e is reduced and takes the place of d, the place of b is left to expand
+    a = ref.einsum_quantization_info("abcde,afce->acdbf", 5)
+    assert a["input"] == dict(reduced=[4], expand=[], transpose=[0, 2, 3, 1, 4], squeeze=[])
+    assert a["kernel"] == dict(reduced=[3], expand=[3], transpose=[0, 2, 3, 1], squeeze=[])
+    _, s, _ = ref.einsum_dense_quantize_int8(torch.randn(1, 16, 2, 32), "abcde,afce->acdbf", 5)
+    assert tuple(s.shape) == (1, 2, 1, 1, 16)   # broadcasts against a,c,d,b,f
+    # "ab,ab->a": b is reduced on both sides and the output lacks no label, so the reduced axis
+    # is marked for squeezing and inserted at the stale index, output_spec.find("b") == -1, i.e.
+    # before the last entry: transpose [1, 0].  A [a, 1] scale becomes [1, a]; the squeeze of
+    # axis 1 (size a) is a no-op on the torch backend.  The de-scaled result is therefore [1, a].
+    b = ref.einsum_quantization_info("ab,ab->a", 2)
+    assert b["input"] == dict(reduced=[1], expand=[], transpose=[1, 0], squeeze=[1])
+    assert b["kernel"] == dict(reduced=[1], expand=[], transpose=[1, 0], squeeze=[1])
+    g = torch.Generator().manual_seed(5)
+    k, x = torch.rand(3, 8, generator=g) - 0.5, torch.rand(3, 8, generator=g)
+    qk, ks, _ = ref.einsum_dense_quantize_int8(k, "ab,ab->a", 2)
+    assert tuple(ks.shape) == (1, 3)
+    y = ref.einsum_dense_int8_call(x, qk, ks, "ab,ab->a")
+    assert tuple(y.shape) == (1, 3)
+    assert (y.reshape(-1) - torch.einsum("ab,ab->a", x, k)).abs().max().item() < 2e-2
+    # "a,b->ab": nothing is reduced; each operand's scale is per element and gains the other's axis
+    c = ref.einsum_quantization_info("a,b->ab", 1)
+    assert c["input"] == dict(reduced=[], expand=[1], transpose=[0], squeeze=[])
+    assert c["kernel"] == dict(reduced=[], expand=[0], transpose=[0], squeeze=[])
+
+
 @pytest.mark.parametrize("equation,kshape,xshape", [
     ("btnh,nhd->btd", (2, 4, 8), (1, 2, 2, 4)), ("btd,ndh->btnh", (2, 4, 8), (1, 2, 4)),
     ("btd,df->btf", (4, 4), (1, 2, 4)), ("ab,bcd->acd", (3, 8, 32), (2, 3)),
     ("...b,bc->...c", (7, 5), (2, 3, 7)), ("abc,cd->abd", (6, 9), (2, 3, 6)),
+    ("abcde,afce->acdbf", (1, 16, 2, 32), (1, 8, 2, 4, 32)), ("a,b->ab", (4,), (5,)),
+    ("ab,c->ac", (5,), (3, 4)), ("bhqd,hdk->bhqk", (4, 8, 6), (2, 4, 3, 8)),
 ])
 def test_einsum_int8_descale_approximates_float(equation, kshape, xshape):
     # the scales must broadcast against the einsum output such that the de-scaled integer
