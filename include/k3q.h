@@ -412,6 +412,22 @@ int k3q_embedding_lookup(const void* ids, int ids_dtype, int64_t count, const in
                          int scale_dtype, const int8_t* zero, int64_t block_size, int out_dtype,
                          void* out, int* oob_flag, void* stream);
 
+/*
+ * One new position of causal self-attention against a key / value cache (the decoder
+ * harness's step between the quantized projections): rotate-half RoPE of the new query and
+ * key with the table rows of *pos, the new key and value rows written into the caches at
+ * *pos, softmax(q . K^T / sqrt(128)) . V over cache rows 0 ... *pos.  bfloat16, head width 128.
+ * q, k, v, out: [B, H, 128]; cos_table, sin_table: [max_len, 128] (sin with the sign of the
+ * rotated half folded in); k_cache, v_cache: [B, H, max_len, 128]; pos: one int64 in device
+ * memory, read by the kernel (a captured graph replays with the value it then holds).
+ * No counterpart in the reference's quantized layers: it stands for the torch ops (two
+ * multiplies and an add per rotation, two index_copy, scaled_dot_product_attention) that a
+ * Keras decoder runs between its Dense / EinsumDense calls.
+ */
+int k3q_decode_attention(const void* q, const void* k, const void* v, int dtype, int64_t B, int64_t H,
+                         int64_t head_dim, int64_t max_len, const void* cos_table, const void* sin_table,
+                         const int64_t* pos, void* k_cache, void* v_cache, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -103,6 +103,10 @@ SIGNATURES = {
     ),
     "k3q_gemv_w4s_multi": (_int, [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr]),
     "k3q_w4_kmajor_pack": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "k3q_decode_attention": (
+        _int,
+        [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr],
+    ),
     "k3q_gemm_w4_kmajor_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "k3q_gemm_w4_kmajor": (
         _int,

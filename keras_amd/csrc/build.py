@@ -25,6 +25,7 @@ SOURCES = [
     "k3q_gemm_i8.hip",
     "k3q_gemm_i8_skinny.hip",
     "k3q_embedding.hip",
+    "k3q_decode_attn.hip",
 ]
 
 FLAGS = [

@@ -1,0 +1,188 @@
+// One new position of causal self-attention against a key / value cache, bfloat16, head
+// width 128: rotate the new query and key (rotate-half RoPE, tables indexed by the position),
+// write the new key and value rows into the cache at the position, attend over rows
+// 0 ... position.  One launch where the decoder step otherwise runs a dozen small ones.
+//
+// One workgroup per (sequence, head), 8 waves.  A wave instruction covers 4 cache rows
+// (16 lanes x 16 bytes per 256-byte row), waves take blocks of 4 rows round-robin; scores go
+// through LDS (one float per cache row), softmax in float32, the value sum is reduced over
+// the 4 row slots of a wave by lane exchange and over the waves through LDS.
+// The position is read from device memory, so a captured graph replays with a new one.
+#include "k3q_common.h"
+
+namespace k3q {
+namespace {
+
+constexpr int kHd = 128;
+constexpr int kAW = 8;           // waves per workgroup
+constexpr int kAT = 64 * kAW;
+
+struct AttnParams {
+    const uint16_t *q, *k, *v;      // [B, H, 128] bfloat16 (one position)
+    const uint16_t *cos_t, *sin_t;  // [max_len, 128] bfloat16
+    const int64_t* pos;             // device: the position of this step
+    uint16_t *kc, *vc;              // [B, H, max_len, 128]
+    uint16_t* out;                  // [B, H, 128]
+    int H, max_len;
+    float scale;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+__global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
+    extern __shared__ __attribute__((aligned(16))) float attn_lds[];
+    float* qs = attn_lds;                   // [128] rotated query, pre-scaled
+    float* red = qs + kHd;                  // [2 * kAW]
+    float* oacc = red + 2 * kAW;            // [kAW][128]
+    float* sc = oacc + kAW * kHd;           // [max_len]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int bh = blockIdx.x;
+    int pos = (int)p.pos[0];
+    pos = pos < 0 ? 0 : (pos >= p.max_len ? p.max_len - 1 : pos);
+    const int64_t row0 = (int64_t)bh * p.max_len;  // first cache row of this (sequence, head)
+
+    // ---- rotate q and k, write the new cache rows ----
+    if (tid < 2 * kHd) {
+        const int d = tid & (kHd - 1);
+        const uint16_t* src = (tid < kHd ? p.q : p.k) + (int64_t)bh * kHd;
+        const float x = bf16_bits_to_f32(src[d]), sw = bf16_bits_to_f32(src[d ^ (kHd / 2)]);
+        const float c = bf16_bits_to_f32(p.cos_t[(int64_t)pos * kHd + d]);
+        const float s = bf16_bits_to_f32(p.sin_t[(int64_t)pos * kHd + d]);
+        // the rounding steps of x * cos + swapped * sin evaluated in bfloat16
+        const float r = round_bf16(round_bf16(x * c) + round_bf16(sw * s));
+        if (tid < kHd) qs[d] = r * p.scale;
+        else p.kc[(row0 + pos) * kHd + d] = (uint16_t)f32_to_bf16_bits(r);
+    } else if (tid < 2 * kHd + 16) {
+        const int c = tid - 2 * kHd;
+        ((v4u*)(p.vc + (row0 + pos) * kHd))[c] = ((const v4u*)(p.v + (int64_t)bh * kHd))[c];
+    }
+    __syncthreads();  // the new rows are written (and acknowledged) before any wave reads the cache
+
+    // ---- scores ----
+    const int n = pos + 1;
+    const int nblk = (n + 3) >> 2;
+    const int sub = lane >> 4, dl = (lane & 15) * 8;
+    float qv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[e] = qs[dl + e];
+    float mx = -INFINITY;
+#pragma unroll 4
+    for (int kb = wave; kb < nblk; kb += kAW) {
+        const int j = 4 * kb + sub;
+        const int jj = j < n ? j : pos;
+        const v4u kk = *(const v4u*)(p.kc + (row0 + jj) * kHd + dl);
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            dot += qv[2 * e] * __uint_as_float(kk[e] << 16);
+            dot += qv[2 * e + 1] * __uint_as_float(kk[e] & 0xffff0000u);
+        }
+        dot += __shfl_xor(dot, 1, kWave);
+        dot += __shfl_xor(dot, 2, kWave);
+        dot += __shfl_xor(dot, 4, kWave);
+        dot += __shfl_xor(dot, 8, kWave);
+        if (j < n) {
+            mx = fmaxf(mx, dot);
+            if ((lane & 15) == 0) sc[j] = dot;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    float gmx = red[0];
+#pragma unroll
+    for (int w = 1; w < kAW; ++w) gmx = fmaxf(gmx, red[w]);
+
+    // ---- softmax numerators ----
+    float part = 0.f;
+    for (int j = tid; j < n; j += kAT) {
+        const float e = __expf(sc[j] - gmx);
+        sc[j] = e;
+        part += e;
+    }
+    part = wave_sum(part);
+    if (lane == 0) red[kAW + wave] = part;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < kAW; ++w) total += red[kAW + w];
+
+    // ---- weighted sum of the value rows ----
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll 4
+    for (int kb = wave; kb < nblk; kb += kAW) {
+        const int j = 4 * kb + sub;
+        const int jj = j < n ? j : pos;
+        const v4u vv = *(const v4u*)(p.vc + (row0 + jj) * kHd + dl);
+        const float w = j < n ? sc[j] : 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            acc[2 * e] += w * __uint_as_float(vv[e] << 16);
+            acc[2 * e + 1] += w * __uint_as_float(vv[e] & 0xffff0000u);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        acc[e] += __shfl_xor(acc[e], 16, kWave);
+        acc[e] += __shfl_xor(acc[e], 32, kWave);
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) oacc[wave * kHd + dl + e] = acc[e];
+    }
+    __syncthreads();
+    if (tid < kHd) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAW; ++w) o += oacc[w * kHd + tid];
+        p.out[(int64_t)bh * kHd + tid] = (uint16_t)f32_to_bf16_bits(o / total);
+    }
+}
+
+}  // namespace
+}  // namespace k3q
+
+using namespace k3q;
+
+extern "C" int k3q_decode_attention(const void* q, const void* k, const void* v, int dtype, int64_t B,
+                                    int64_t H, int64_t head_dim, int64_t max_len, const void* cos_table,
+                                    const void* sin_table, const int64_t* pos, void* k_cache,
+                                    void* v_cache, void* out, void* stream) {
+    if (dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (B < 0 || H <= 0 || head_dim != kHd || max_len <= 0 || max_len > 32768 || B * H >= (1 << 30))
+        return K3Q_ERR_SHAPE;
+    if (B == 0) return K3Q_OK;
+    if (!q || !k || !v || !cos_table || !sin_table || !pos || !k_cache || !v_cache || !out) return K3Q_ERR_NULL;
+    if (!aligned_to(v, 16) || !aligned_to(k_cache, 16) || !aligned_to(v_cache, 16) || !aligned_to(pos, 8))
+        return K3Q_ERR_ALIGN;
+    AttnParams p;
+    p.q = (const uint16_t*)q;
+    p.k = (const uint16_t*)k;
+    p.v = (const uint16_t*)v;
+    p.cos_t = (const uint16_t*)cos_table;
+    p.sin_t = (const uint16_t*)sin_table;
+    p.pos = pos;
+    p.kc = (uint16_t*)k_cache;
+    p.vc = (uint16_t*)v_cache;
+    p.out = (uint16_t*)out;
+    p.H = (int)H;
+    p.max_len = (int)max_len;
+    p.scale = 0.08838834764831845f;  // 1 / sqrt(128)
+    const size_t lds = (size_t)(kHd + 2 * kAW + kAW * kHd + max_len) * sizeof(float);
+    if (lds > 64 * 1024) {
+        static const bool raised = hipFuncSetAttribute((const void*)decode_attention,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       160 * 1024) == hipSuccess;
+        if (!raised) return K3Q_ERR_LAUNCH;
+    }
+    decode_attention<<<(unsigned)(B * H), kAT, lds, (hipStream_t)stream>>>(p);
+    return launch_status();
+}

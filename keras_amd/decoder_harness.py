@@ -15,7 +15,7 @@ import math
 
 import torch
 
-from keras_amd import dtype_policies
+from keras_amd import dtype_policies, ops as kops
 from keras_amd.layers import Dense, EinsumDense, ReversibleEmbedding, call_add, call_together
 from keras_amd.layers.layer import Layer, as_tensor, to_torch_dtype
 from keras_amd.models import Model
@@ -82,12 +82,20 @@ class DecoderBlock(Layer):
         self.down.build((None, ffn_dim))
         self.built = True
 
-    def forward(self, x, cos, sin, cache, pos, mask):
+    def forward(self, x, cos, sin, cache, pos, mask, tables=None):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
-        (an int64 device tensor [T]); mask [T, maxT]: 0 where a key may be attended to, -inf elsewhere."""
+        (an int64 device tensor [T]); mask [T, maxT]: 0 where a key may be attended to, -inf
+        elsewhere; tables: the whole (cos, sin) tables, for the one-position kernel."""
         h = self.attn_norm(x)
         # the three projections of h in one launch at decode sizes
         q, k, v = call_together((self.query, self.key, self.value), h)
+        if tables is not None and q.shape[1] == 1 and kops.decode_attention_supported(q, cache[0]):
+            # one position: rotation, cache update and attention in one launch
+            a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
+            x = call_add(self.attn_out, a, x)
+            h = self.ffn_norm(x)
+            gate, up = call_together((self.gate, self.up), h)
+            return call_add(self.down, torch.nn.functional.silu(gate) * up, x)
         # one rotation over the query and key heads together (half the elementwise launches)
         qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
         q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
@@ -194,7 +202,7 @@ class LlamaStyleDecoder(Model):
         mask = torch.zeros((pos.shape[0], self.max_len), dtype=cd, device=self.device).masked_fill_(
             keys[None, :] > pos[:, None], float("-inf"))
         for block, kv in zip(self.blocks, cache):
-            x = block.forward(x, cos, sin, kv, pos, mask)
+            x = block.forward(x, cos, sin, kv, pos, mask, tables=(self.cos, self.sin))
         if last_only:
             x = x[:, -1:, :]
         return self.token_embedding(self.final_norm(x), reverse=True)

@@ -681,3 +681,45 @@ def float_matmul_nk(x, wt, parts=1, bias=None):
     _lib.check(rc, "k3q_gemm_wbf16")
     return y
 
+
+
+def decode_attention_supported(q, cache_k):
+    """bfloat16, head width 128, one new position."""
+    return (q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 4 and q.shape[1] == 1
+            and q.shape[-1] == 128 and cache_k.dtype == torch.bfloat16 and cache_k.shape[2] <= 32768)
+
+
+def decode_attention(q, k, v, cos_table, sin_table, pos, cache_k, cache_v):
+    """One decode position of causal self-attention: q, k, v `[B, 1, H, 128]` bfloat16 (as the
+    projections give them), `cos_table` / `sin_table` `[max_len, 128]`, `pos` an int64 device
+    tensor holding the position, the caches `[B, H, max_len, 128]` (row `pos` is written).
+    Returns `[B, 1, H, 128]`.  What it replaces in a decoder step: the rotation of q and k,
+    two `index_copy_` into the caches and `scaled_dot_product_attention` under a mask that
+    admits keys `<= pos`."""
+    _lib.require_device(q, k, v, cos_table, sin_table, pos, cache_k, cache_v)
+    lib = _lib.load()
+    B, T, H, hd = q.shape
+    if T != 1 or k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(f"decode_attention takes one position: q, k, v [B, 1, H, hd], got {tuple(q.shape)}")
+    max_len = cache_k.shape[2]
+    if tuple(cache_k.shape) != (B, H, max_len, hd) or cache_v.shape != cache_k.shape:
+        raise ValueError(f"caches must be [B, H, max_len, hd], got {tuple(cache_k.shape)}")
+    if tuple(cos_table.shape) != (max_len, hd) or tuple(sin_table.shape) != (max_len, hd):
+        raise ValueError(f"rotation tables must be [max_len, hd] = [{max_len}, {hd}]")
+    if pos.dtype != torch.int64 or pos.numel() != 1:
+        raise ValueError("pos must be one int64 value on the device")
+    for t in (q, k, v, cos_table, sin_table, cache_k, cache_v):
+        if t.dtype != torch.bfloat16:
+            raise TypeError("decode_attention computes in bfloat16")
+    if not (cache_k.is_contiguous() and cache_v.is_contiguous()):
+        raise ValueError("the caches are written in place and must be contiguous")
+    q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
+    cos_table = cos_table if cos_table.is_contiguous() else cos_table.contiguous()
+    sin_table = sin_table if sin_table.is_contiguous() else sin_table.contiguous()
+    out = torch.empty((B, 1, H, hd), dtype=torch.bfloat16, device=q.device)
+    rc = lib.k3q_decode_attention(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.dtype_code(q.dtype), B, H, hd,
+                                  max_len, _lib.ptr(cos_table), _lib.ptr(sin_table), _lib.ptr(pos),
+                                  _lib.ptr(cache_k), _lib.ptr(cache_v), _lib.ptr(out),
+                                  _lib.stream_ptr(q.device))
+    _lib.check(rc, "k3q_decode_attention")
+    return out

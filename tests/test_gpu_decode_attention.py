@@ -1,0 +1,115 @@
+"""GPU: the one-position attention kernel of the decoder harness against the torch ops it
+replaces (rotation, cache update, masked scaled-dot-product attention)."""
+
+import pytest
+import torch
+
+from keras_amd import ops as kops
+from keras_amd.decoder_harness import apply_rope, rope_tables
+
+pytestmark = pytest.mark.gpu
+
+
+def torch_step(q, k, v, cos_t, sin_t, pos, kc, vc):
+    """The harness's own op sequence for one position (decoder_harness.DecoderBlock.forward)."""
+    cos, sin = cos_t.index_select(0, pos), sin_t.index_select(0, pos)
+    H = q.shape[2]
+    qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
+    qr, kr = qk[:, :, :H], qk[:, :, H:]
+    kc.index_copy_(2, pos, kr.transpose(1, 2))
+    vc.index_copy_(2, pos, v.transpose(1, 2))
+    keys = torch.arange(kc.shape[2], device=q.device)
+    mask = torch.zeros((1, kc.shape[2]), dtype=q.dtype, device=q.device).masked_fill_(
+        keys[None, :] > pos[:, None], float("-inf"))
+    a = torch.nn.functional.scaled_dot_product_attention(qr.transpose(1, 2), kc, vc, attn_mask=mask[None, None])
+    return a.transpose(1, 2)
+
+
+def exact_step(q, k, v, cos_t, sin_t, pos, kc, vc):
+    """float64 attention over the bfloat16 cache as the kernel leaves it."""
+    p = int(pos.item())
+    cos, sin = cos_t[p].double(), sin_t[p].double()
+    half = q.shape[-1] // 2
+    rot = lambda x: (x.double() * cos).to(torch.bfloat16).double() + \
+        (torch.cat((x[..., half:], x[..., :half]), -1).double() * sin).to(torch.bfloat16).double()
+    qr = rot(q).to(torch.bfloat16).double()[:, 0]                       # [B, H, hd]
+    K, V = kc[:, :, : p + 1].double(), vc[:, :, : p + 1].double()       # [B, H, n, hd]
+    s = torch.einsum("bhd,bhnd->bhn", qr, K) / (q.shape[-1] ** 0.5)
+    return torch.einsum("bhn,bhnd->bhd", torch.softmax(s, -1), V)[:, None]
+
+
+@pytest.mark.parametrize("B,H,max_len,pos", [(1, 32, 256, 0), (1, 32, 256, 130), (8, 32, 256, 255),
+                                             (2, 5, 64, 17), (3, 8, 1024, 1000), (1, 32, 4096, 4095),
+                                             (1, 2, 20000, 19999)])
+def test_decode_attention_matches_torch_ops(dev, B, H, max_len, pos):
+    g = torch.Generator().manual_seed(B * 1000 + pos)
+    hd = 128
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v = mk(B, 1, H, hd), mk(B, 1, H, hd), mk(B, 1, H, hd)
+    kc0, vc0 = mk(B, H, max_len, hd), mk(B, H, max_len, hd)
+    cos_t, sin_t = rope_tables(hd, max_len, dev, dtype=torch.bfloat16)
+    pos_t = torch.tensor([pos], dtype=torch.int64, device=dev)
+    kc_a, vc_a, kc_b, vc_b = kc0.clone(), vc0.clone(), kc0.clone(), vc0.clone()
+    want = torch_step(q, k, v, cos_t, sin_t, pos_t, kc_a, vc_a)
+    assert kops.decode_attention_supported(q, kc_b)
+    got = kops.decode_attention(q, k, v, cos_t, sin_t, pos_t, kc_b, vc_b)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (B, 1, H, hd)
+    # the caches: the new rows are the torch ops' rows bit for bit, every other row untouched
+    assert torch.equal(kc_a.view(torch.int16), kc_b.view(torch.int16))
+    assert torch.equal(vc_a.view(torch.int16), vc_b.view(torch.int16))
+    exact = exact_step(q, k, v, cos_t, sin_t, pos_t, kc_b, vc_b)
+    denom = exact.abs().max().item()
+    err_kernel = (got.double() - exact).abs().max().item() / denom
+    err_torch = (want.double() - exact).abs().max().item() / denom
+    # one bfloat16 rounding of the result: half an ulp of the largest magnitudes
+    assert err_kernel <= 4e-3, (err_kernel, err_torch)
+    assert err_kernel <= 2 * err_torch + 1e-3
+
+
+def test_decode_attention_position_is_read_on_the_device(dev):
+    # a HIP graph captured once replays with whatever position the device tensor then holds
+    g = torch.Generator().manual_seed(4)
+    B, H, hd, max_len = 2, 4, 128, 64
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v = mk(B, 1, H, hd), mk(B, 1, H, hd), mk(B, 1, H, hd)
+    kc, vc = mk(B, H, max_len, hd), mk(B, H, max_len, hd)
+    cos_t, sin_t = rope_tables(hd, max_len, dev, dtype=torch.bfloat16)
+    pos_t = torch.zeros(1, dtype=torch.int64, device=dev)
+    out = torch.empty(B, 1, H, hd, dtype=torch.bfloat16, device=dev)
+    side = torch.cuda.Stream()
+    kc_g, vc_g = kc.clone(), vc.clone()
+    with torch.cuda.stream(side):
+        kops.decode_attention(q, k, v, cos_t, sin_t, pos_t, kc_g, vc_g)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            out.copy_(kops.decode_attention(q, k, v, cos_t, sin_t, pos_t, kc_g, vc_g))
+    torch.cuda.synchronize()
+    for p in (5, 40, 6, 63):
+        kc_g.copy_(kc)
+        vc_g.copy_(vc)
+        pos_t.fill_(p)
+        graph.replay()
+        torch.cuda.synchronize()
+        kc_e, vc_e = kc.clone(), vc.clone()
+        eager = kops.decode_attention(q, k, v, cos_t, sin_t, pos_t, kc_e, vc_e)
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), p
+        assert torch.equal(kc_g.view(torch.int16), kc_e.view(torch.int16))
+
+
+def test_decode_attention_rejects(dev):
+    hd = 128
+    z = lambda *s, dt=torch.bfloat16: torch.zeros(*s, dtype=dt, device=dev)
+    cos_t, sin_t = rope_tables(hd, 16, dev, dtype=torch.bfloat16)
+    pos = torch.zeros(1, dtype=torch.int64, device=dev)
+    q = z(1, 1, 2, hd)
+    with pytest.raises(ValueError):
+        kops.decode_attention(z(1, 2, 2, hd), z(1, 2, 2, hd), z(1, 2, 2, hd), cos_t, sin_t, pos,
+                              z(1, 2, 16, hd), z(1, 2, 16, hd))
+    with pytest.raises(ValueError):
+        kops.decode_attention(q, q, q, cos_t, sin_t, pos, z(1, 2, 8, hd), z(1, 2, 8, hd))
+    with pytest.raises(ValueError):
+        kops.decode_attention(q, q, q, cos_t, sin_t, pos.to(torch.int32), z(1, 2, 16, hd), z(1, 2, 16, hd))
+    with pytest.raises(TypeError):
+        kops.decode_attention(q.float(), q.float(), q.float(), cos_t, sin_t, pos,
+                              z(1, 2, 16, hd), z(1, 2, 16, hd))
+    assert not kops.decode_attention_supported(z(1, 1, 2, 64), z(1, 2, 16, 64))
