@@ -82,7 +82,7 @@ def main():
                     "step and only these further sections (for profiler runs); default: all")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
-    unknown = only - {"none", "ceiling", "sweep", "einsum", "gemv", "decode", "cpu"}
+    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "decode", "cpu"}
     if unknown:
         sys.exit(f"bench.py: unknown section(s) {sorted(unknown)}")
     want = (lambda name: not only or name in only)
@@ -171,6 +171,17 @@ def main():
     torch.cuda.synchronize()
     quant_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
     quant_bytes = M * K * 2 + M * K + M * 2
+
+    # ------------------------------------------------------------------ counter calibration
+    # only on request (--only ...,calib), for profiler runs: device copies of known size, so that
+    # the same run that counts a kernel's FETCH_SIZE / WRITE_SIZE also counts these
+    if "calib" in only:
+        for mib in (64, 256):
+            src_ = torch.randint(0, 255, (mib << 20,), dtype=torch.uint8, device=dev)
+            for _ in range(5):
+                dst_ = src_.clone()
+            torch.cuda.synchronize()
+            del src_, dst_
 
     # ------------------------------------------------------------------ matrix cores alone
     # What the int8 matrix cores sustain on this board with nothing else running: a loop of
