@@ -413,6 +413,42 @@ int k3q_embedding_lookup(const void* ids, int ids_dtype, int64_t count, const in
                          void* out, int* oob_flag, void* stream);
 
 /*
+ * Decode-sized int8 Dense forward in ONE launch, from a strip-linear copy of the int8 kernel:
+ * the rows of x (1 ... 16, bfloat16) are abs-max quantised inside the kernel exactly as
+ * k3q_absmax_quantize does (same roundings, same int8 values and scales), multiplied exactly
+ * (int32 sums of all of K inside a workgroup: no partial sums in memory, no workspace) and
+ * de-scaled with the bit-exact bfloat16 epilogue of k3q_gemm_i8 (flags bit 0):
+ *     y = bf16(bf16(acc) / bf16(sa * sb)) (+ bias, one more rounding).
+ * Same bits as k3q_absmax_quantize followed by k3q_gemm_i8 with K3Q_GEMM_EXACT_EPILOGUE.
+ * Replaces the chain keras/src/layers/core/dense.py:956-972 (inputs_quantizer, ops.matmul,
+ * cast, divide by the scales, bias add) and einsum_dense.py:1063-1083 for GEMM-shaped
+ * equations, for calls of up to 16 rows.
+ *
+ * shadow (k3q_w8s_pack from the stored [K, N] int8 kernel, once per layer):
+ * [strip = n/16][unit = k/64][lane = 64][16 bytes]; lane i + 16 g holds column 16 strip + i,
+ * bytes k = 64 unit + 16 g + (0 ... 15); the strip count is padded to even with zero strips;
+ * k3q_w8s_shadow_bytes gives its size.  kernel_scale: bfloat16 [N].  bias: bfloat16, N values
+ * (bias_stride 0) or M x N (bias_stride N: a row per row of x), or null.
+ * epsilon, range_lo, range_hi: the quantizer's settings (1e-7, -127, 127 by default).
+ * Needs K % 512 == 0, K >= 1024, N % 16 == 0, N >= 3072 and M x K small enough for LDS
+ * (k3q_dense_i8_w8s_supported says; K3Q_ERR_SHAPE otherwise).
+ *
+ * k3q_gemm_i8_w8s is the same kernel for rows that are already quantised (a: int8 [M, K],
+ * a_scale: bfloat16 [M], as k3q_absmax_quantize writes them): every workgroup re-quantising
+ * all of x costs more than a quantizer launch from about 16 K values of x on, and layers that
+ * share their input quantise it once.  Same shapes, same bits.
+ */
+int64_t k3q_w8s_shadow_bytes(int64_t K, int64_t N);
+int k3q_w8s_pack(const int8_t* w, int64_t K, int64_t N, void* shadow, void* stream);
+int k3q_dense_i8_w8s_supported(int64_t M, int64_t K, int64_t N);
+int k3q_dense_i8_w8s(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* shadow,
+                     const void* kernel_scale, const void* bias, int64_t bias_stride, float epsilon,
+                     float range_lo, float range_hi, void* y, void* stream);
+int k3q_gemm_i8_w8s(const int8_t* a, const void* a_scale, int scale_dtype, int64_t M, int64_t K, int64_t N,
+                    const void* shadow, const void* kernel_scale, const void* bias, int64_t bias_stride,
+                    void* y, void* stream);
+
+/*
  * One new position of causal self-attention against a key / value cache (the decoder
  * harness's step between the quantized projections): rotate-half RoPE of the new query and
  * key with the table rows of *pos, the new key and value rows written into the caches at

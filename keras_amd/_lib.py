@@ -103,6 +103,14 @@ SIGNATURES = {
     ),
     "k3q_gemv_w4s_multi": (_int, [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr]),
     "k3q_w4_kmajor_pack": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "k3q_w8s_shadow_bytes": (_i64, [_i64, _i64]),
+    "k3q_w8s_pack": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "k3q_dense_i8_w8s_supported": (_int, [_i64, _i64, _i64]),
+    "k3q_dense_i8_w8s": (
+        _int,
+        [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _f32, _f32, _f32, _ptr, _ptr],
+    ),
+    "k3q_gemm_i8_w8s": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
     "k3q_decode_attention": (
         _int,
         [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr],

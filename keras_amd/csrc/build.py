@@ -26,6 +26,7 @@ SOURCES = [
     "k3q_gemm_i8_skinny.hip",
     "k3q_embedding.hip",
     "k3q_decode_attn.hip",
+    "k3q_gemv_w8s.hip",
 ]
 
 FLAGS = [

@@ -1,0 +1,453 @@
+// Decode-sized int8 Dense forward in one launch, from a strip-linear copy of the int8 kernel:
+//     q, sa = abs_max_quantize(x, axis=-1)          (x: up to 16 bfloat16 rows)
+//     y[m,n] = bf16( bf16(acc[m,n]) / bf16(sa[m] * sb[n]) ) (+ bias),  acc = sum_k q[m,k] * w[k,n]
+// with every rounding step of the reference's op sequence (the bit-exact epilogue of the tile GEMM).
+//
+// Copy layout ("w8s"): [strip = n / 16][unit = k / 64][lane = 64][16 bytes], 1 KiB per
+// (strip, unit); lane = i + 16 g holds column n = 16 strip + i, bytes k = 64 unit + 16 g + (0..15):
+// the B operand of v_mfma_i32_16x16x64_i8 as it lies, a wave instruction reads 1 KiB contiguous.
+// The strip count is padded to even with zero strips.
+//
+// Workgroup: 8 waves.  A workgroup owns groups of kSW strips and all of K for them: wave q takes
+// a contiguous slice of the units, so no partial sums leave the workgroup.  Every workgroup
+// quantises x itself (x is a few KiB to a few hundred KiB and comes from L2): row maxima through
+// LDS, the int8 rows into LDS, the scales stay there for the epilogue.  The weights go through
+// a register ring of kD units per strip that is refilled right after a unit is consumed and
+// runs on across group boundaries (a workgroup with several groups streams without a gap).
+#include <mutex>
+#include <set>
+
+#include "k3q_common.h"
+
+namespace k3q {
+namespace {
+
+constexpr int kQ = 8;            // waves per workgroup
+constexpr int kT = 64 * kQ;
+constexpr int kMaxRows8 = 16;
+constexpr int kResident8 = 256;  // workgroups the chip holds at once (one per CU)
+
+struct W8sParams {
+    const uint16_t* x;      // [M, K] bfloat16 (quantised in the kernel), or
+    const int8_t* xq;       // [M, K] int8 with
+    const uint16_t* xs;     // [M] bfloat16 scales (already quantised rows)
+    const v4i* w;           // strip-linear copy
+    const uint16_t* scale;  // [N] bfloat16 kernel scale
+    const uint16_t* bias;   // [N] or [M, N] bfloat16, or null
+    uint16_t* y;            // [M, N] bfloat16
+    int64_t bias_stride;    // 0: one row for all, N: a row per row of x
+    int M, K, N;
+    int units;              // K / 64
+    int groups;             // strip groups (kSW strips each)
+    int row_magic;          // ceil(2^32 / (K / 8)): piece -> row
+    float eps, qlo, qhi;    // quantizer settings (eps already rounded to bfloat16)
+};
+
+__device__ __forceinline__ float scale_from_amax_bf16(float amax, float eps, float qhi) {
+    return round_bf16(qhi / round_bf16(amax + eps));
+}
+__device__ __forceinline__ u32 quantize_bf16(float v, float s, float qlo, float qhi) {
+    float p = rintf(round_bf16(v * s));  // round half to even
+    p = fminf(fmaxf(p, qlo), qhi);
+    return (u32)(int)p & 0xffu;
+}
+
+// y = T(T(acc) / T(sa * sb)) (+ bias), T = bfloat16: the reference's sequence, every step rounded
+__device__ __forceinline__ float descale_exact_bf16(int acc, float sa, float sb, float bv, bool has_bias) {
+    const float os = round_bf16(sb * sa);
+    float r = div_round_bf16(round_bf16((float)acc), os);
+    if (has_bias) r = round_bf16(r + bv);
+    return r;
+}
+
+// kNP: 16-byte pieces of x a thread keeps in registers between the row maxima and the
+// quantisation (0: it reads them twice); -1: the rows arrive quantised (p.xq, p.xs).
+template <int kSW, int kD, int kNP>
+__global__ __launch_bounds__(kT) void gemv_w8s(W8sParams p) {
+    extern __shared__ __attribute__((aligned(16))) char w8s_lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int q = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = p.M, K = p.K;
+    const int pitch = K + 16;
+    // LDS: x rows as int8 | row maxima (uint bits) | row scales | reduction buffers
+    char* xs = w8s_lds;
+    u32* rowmax = (u32*)(w8s_lds + ((M * pitch + 255) & ~255));
+    float* sa = (float*)(rowmax + kMaxRows8);
+    const int mq = (M + 3) >> 2;  // accumulator row quads that hold rows of x
+    int* red = (int*)(sa + kMaxRows8);
+    const int red_one = kQ * kSW * mq * 16 * 4;  // ints per buffer
+
+    // ---- this wave's slice of the units: blocks of kD units, the first waves take one more ----
+    const int blocks = p.units / kD;
+    const int per = blocks / kQ, extra = blocks - per * kQ;
+    const int b0 = q * per + (q < extra ? q : extra);
+    const int my_units = (per + (q < extra ? 1 : 0)) * kD;
+    const int u_begin = b0 * kD;
+
+    // ---- the weight stream: the load cursor (group, first unit of a block) runs one block of
+    // kD units ahead of the consumer, across group boundaries ----
+    const int stride = gridDim.x;
+    int lg = blockIdx.x, lu = u_begin;
+    const int last_group = p.groups - 1;
+    const v4i* nb[kSW];  // this lane's pieces of the block at the cursor, unit by unit 64 entries apart
+    auto at_cursor = [&]() {
+        const int g2 = lg < last_group ? lg : last_group;  // past the end: a valid address, never used
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) nb[t] = p.w + ((int64_t)(g2 * kSW + t) * p.units + lu) * 64 + lane;
+    };
+    auto advance = [&]() {
+        lu += kD;
+        if (lu == u_begin + my_units) {
+            lu = u_begin;
+            lg += stride;
+        }
+        at_cursor();
+    };
+    v4i W[kD][kSW];
+    auto refill = [&](int d) {
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) W[d][t] = __builtin_nontemporal_load(nb[t] + d * 64);
+    };
+    at_cursor();
+
+    // ---- stage x ----
+    if constexpr (kNP < 0) {
+        // rows already quantised: copy them (16 int8 per piece) and their scales into LDS
+        const int pieces = M * (K >> 4);
+        constexpr int kCP = 4;  // pieces in flight per thread and round
+#pragma unroll
+        for (int d = 0; d < kD; ++d) refill(d);
+        advance();
+        for (int base = 0; base < pieces; base += kCP * kT) {
+            v4u c[kCP];
+#pragma unroll
+            for (int i = 0; i < kCP; ++i) {
+                const int pi = base + i * kT + tid;
+                c[i] = ((const v4u*)p.xq)[pi < pieces ? pi : pieces - 1];
+            }
+#pragma unroll
+            for (int i = 0; i < kCP; ++i) {
+                const int pi = base + i * kT + tid;
+                if (pi < pieces) {
+                    const int row = (int)__umulhi((u32)pi, (u32)p.row_magic);  // magic of K / 16 here
+                    const int col = (pi - row * (K >> 4)) << 4;
+                    *(v4u*)(xs + row * pitch + col) = c[i];
+                }
+            }
+        }
+        if (tid < M) sa[tid] = bf16_bits_to_f32(p.xs[tid]);
+    } else {
+        // row maxima, scales, int8 rows: abs_max_quantize of the rows inside the workgroup
+        const int pieces = M * (K >> 3);  // 16-byte pieces of x (8 values)
+        if (tid < kMaxRows8) rowmax[tid] = 0u;
+        v4u xr[kNP > 0 ? kNP : 1];
+        if (kNP > 0) {
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                const int pi = tid + i * kT;
+                xr[i] = ((const v4u*)p.x)[pi < pieces ? pi : pieces - 1];
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < kD; ++d) refill(d);
+        advance();
+        __syncthreads();  // rowmax cleared
+        auto piece_amax = [](const v4u& c) {
+            float a = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a = fmaxf(a, fabsf(__uint_as_float(c[e] << 16)));
+                a = fmaxf(a, fabsf(__uint_as_float(c[e] & 0xffff0000u)));
+            }
+            return a;
+        };
+        // a wave's 64 consecutive pieces lie in one row (K % 512 == 0): one LDS atomic per wave and turn
+        auto fold_amax = [&](int pi, float a) {
+            a = wave_max(a);
+            const int row = (int)__umulhi((u32)(pi < pieces ? pi : pieces - 1), (u32)p.row_magic);
+            if (lane == 0 && pi < pieces) atomicMax(rowmax + row, __float_as_uint(a));
+        };
+        if (kNP > 0) {
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                const int pi = tid + i * kT;
+                if (pi - lane < pieces) fold_amax(pi, piece_amax(xr[i]));
+            }
+        } else {
+            for (int base = 0; base < pieces; base += kT) {
+                const int pi = base + tid;
+                const v4u c = ((const v4u*)p.x)[pi < pieces ? pi : pieces - 1];
+                if (pi - lane < pieces) fold_amax(pi, piece_amax(c));
+            }
+        }
+        __syncthreads();
+        if (tid < M) sa[tid] = scale_from_amax_bf16(__uint_as_float(rowmax[tid]), p.eps, p.qhi);
+        __syncthreads();
+        auto quantize_piece = [&](int pi, const v4u& c) {
+            const int row = (int)__umulhi((u32)pi, (u32)p.row_magic);
+            const int col = (pi - row * (K >> 3)) << 3;
+            const float s = sa[row];
+            u32 lo = 0, hi = 0;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                lo |= quantize_bf16(__uint_as_float(c[e] << 16), s, p.qlo, p.qhi) << (16 * e);
+                lo |= quantize_bf16(__uint_as_float(c[e] & 0xffff0000u), s, p.qlo, p.qhi) << (16 * e + 8);
+                hi |= quantize_bf16(__uint_as_float(c[2 + e] << 16), s, p.qlo, p.qhi) << (16 * e);
+                hi |= quantize_bf16(__uint_as_float(c[2 + e] & 0xffff0000u), s, p.qlo, p.qhi) << (16 * e + 8);
+            }
+            const v2u o = {lo, hi};
+            *(v2u*)(xs + row * pitch + col) = o;
+        };
+        if (kNP > 0) {
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                const int pi = tid + i * kT;
+                if (pi < pieces) quantize_piece(pi, xr[i]);
+            }
+        } else {
+            for (int base = 0; base < pieces; base += kT) {
+                const int pi = base + tid;
+                const v4u c = ((const v4u*)p.x)[pi < pieces ? pi : pieces - 1];
+                if (pi < pieces) quantize_piece(pi, c);
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- groups of strips ----
+    const int i16 = lane & 15, g = lane >> 4;
+    const bool row_live = i16 < M;
+    const char* xrow = xs + (row_live ? i16 : 0) * pitch + 16 * g;
+    const bool has_bias = p.bias != nullptr;
+    int turn = 0;
+    for (int grp = blockIdx.x; grp < p.groups; grp += stride, ++turn) {
+        // epilogue operands of this group, asked for before the group's units (loads return in
+        // order: asked for late they would wait for the next group's first units)
+        const int n0 = grp * kSW * 16;
+        u32 sb_raw[kSW], bias_raw[kSW][4];
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) {
+            const int n = n0 + t * 16 + i16;
+            const int nn = n < p.N ? n : p.N - 1;
+            sb_raw[t] = p.scale[nn];
+            const uint16_t* bp = has_bias ? p.bias : p.scale;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = 4 * g + r;
+                bias_raw[t][r] = bp[(has_bias && m < M ? (int64_t)m * p.bias_stride : 0) + nn];
+            }
+        }
+        v4i acc[kSW];
+#pragma unroll
+        for (int t = 0; t < kSW; ++t) acc[t] = v4i{0, 0, 0, 0};
+        v4i a_next = *(const v4i*)(xrow + u_begin * 64);
+        for (int u = u_begin; u < u_begin + my_units; u += kD) {
+#pragma unroll
+            for (int d = 0; d < kD; ++d) {
+                v4i a = a_next;
+                if (!row_live) a = v4i{0, 0, 0, 0};
+                // (the read past this wave's slice stays inside the row's padding or the next row)
+                a_next = *(const v4i*)(xrow + (u + d + 1) * 64);
+#pragma unroll
+                for (int t = 0; t < kSW; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, W[d][t], acc[t], 0, 0, 0);
+                refill(d);
+                __builtin_amdgcn_sched_barrier(0);  // the refill stays here: right behind its unit's last use
+            }
+            advance();
+        }
+        // ---- sum the waves' slices (exact integers), de-scale, store ----
+        int* rbuf = red + (turn & 1) * red_one;
+        if (g < mq) {
+#pragma unroll
+            for (int t = 0; t < kSW; ++t) *(v4i*)(rbuf + (((q * kSW + t) * mq + g) * 16 + i16) * 4) = acc[t];
+        }
+        __syncthreads();
+        if (q < kSW && g < mq) {
+            v4i tot = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int qq = 0; qq < kQ; ++qq) tot += *(const v4i*)(rbuf + (((qq * kSW + q) * mq + g) * 16 + i16) * 4);
+            u32 sbq = sb_raw[0];
+            u32 bq[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) bq[r] = bias_raw[0][r];
+#pragma unroll
+            for (int t = 1; t < kSW; ++t) {
+                if (q == t) {
+                    sbq = sb_raw[t];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) bq[r] = bias_raw[t][r];
+                }
+            }
+            const int n = n0 + q * 16 + i16;
+            if (n < p.N) {
+                const float sb = bf16_bits_to_f32(sbq);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int m = 4 * g + r;
+                    if (m < M) {
+                        const float yv = descale_exact_bf16(tot[r], sa[m], sb, bf16_bits_to_f32(bq[r]), has_bias);
+                        p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_bf16_bits(yv);
+                    }
+                }
+            }
+        }
+        // (the next group's partials go to the other buffer: no second barrier)
+    }
+}
+
+// One thread per 16-byte lane entry of the copy.  w: the stored int8 kernel, row-major [K, N].
+__global__ __launch_bounds__(256) void w8s_pack(const int8_t* __restrict__ w, v4u* __restrict__ out, int64_t K,
+                                               int64_t N, int64_t strips) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t units = K / 64;
+    if (t >= strips * units * 64) return;
+    const int lane = (int)(t & 63);
+    const int64_t u = (t >> 6) % units, s = (t >> 6) / units;
+    const int64_t n = s * 16 + (lane & 15);
+    const int64_t k0 = u * 64 + (lane >> 4) * 16;
+    v4u o = {0, 0, 0, 0};
+    if (n < N) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[e >> 2] |= ((u32)(uint8_t)w[(k0 + e) * N + n]) << (8 * (e & 3));
+    }
+    out[t] = o;
+}
+
+int64_t strips_padded8(int64_t N) { return ((N + 15) / 16 + 1) / 2 * 2; }
+
+struct W8sPlan {
+    bool ok;
+    int sw, d, np;
+    int64_t groups, blocks;
+    size_t lds;
+};
+
+W8sPlan w8s_plan(int64_t M, int64_t K, int64_t N) {
+    W8sPlan pl{};
+    // a wave's 64 pieces of x stay inside a row (K % 512), whole strips (N % 16)
+    if (M < 1 || M > kMaxRows8 || K < 1024 || (K % 512) != 0 || (N % 16) != 0 || N < 16) return pl;
+    const int64_t units = K / 64, strips = N / 16;
+    if (strips < 192) return pl;  // all of K stays inside a workgroup: the strips alone fill the chip
+    pl.d = (units / 4 >= 2 * kQ) ? 4 : 2;
+    if ((units % pl.d) != 0 || units / pl.d < kQ) return pl;
+    pl.sw = strips >= 2 * kResident8 ? 2 : 1;
+    pl.groups = (strips + pl.sw - 1) / pl.sw;
+    const int64_t turns = (pl.groups + kResident8 - 1) / kResident8;
+    pl.blocks = (pl.groups + turns - 1) / turns;
+    const int64_t pieces = M * K / 8;
+    pl.np = pieces <= kT ? 1 : pieces <= 4 * kT ? 4 : pieces <= 16 * kT ? 16 : 0;
+    const size_t red_one = (size_t)kQ * pl.sw * ((M + 3) / 4) * 16 * 4 * 4;
+    pl.lds = (size_t)((M * (K + 16) + 255) & ~255) + 2 * kMaxRows8 * 4 + (turns > 1 ? 2 : 1) * red_one;
+    pl.ok = pl.lds <= 160 * 1024;
+    return pl;
+}
+
+typedef void (*W8sKernel)(W8sParams);
+
+template <int kSW, int kD>
+W8sKernel pick_np8(int np) {
+    switch (np) {
+        case -1: return gemv_w8s<kSW, kD, -1>;
+        case 1: return gemv_w8s<kSW, kD, 1>;
+        case 4: return gemv_w8s<kSW, kD, 4>;
+        case 16: return gemv_w8s<kSW, kD, 16>;
+        default: return gemv_w8s<kSW, kD, 0>;
+    }
+}
+
+W8sKernel pick_kernel8(const W8sPlan& pl) {
+    if (pl.sw == 2) return pl.d == 4 ? pick_np8<2, 4>(pl.np) : pick_np8<2, 2>(pl.np);
+    return pl.d == 4 ? pick_np8<1, 4>(pl.np) : pick_np8<1, 2>(pl.np);
+}
+
+}  // namespace
+}  // namespace k3q
+
+using namespace k3q;
+
+extern "C" int64_t k3q_w8s_shadow_bytes(int64_t K, int64_t N) {
+    if (K <= 0 || N <= 0 || (K % 64) != 0) return 0;
+    return strips_padded8(N) * (K / 64) * 1024;
+}
+
+extern "C" int k3q_w8s_pack(const int8_t* w, int64_t K, int64_t N, void* shadow, void* stream) {
+    if (K <= 0 || N <= 0 || (K % 64) != 0) return K3Q_ERR_SHAPE;
+    if (!w || !shadow) return K3Q_ERR_NULL;
+    if (!aligned_to(shadow, 16)) return K3Q_ERR_ALIGN;
+    const int64_t entries = k3q_w8s_shadow_bytes(K, N) / 16;
+    w8s_pack<<<(unsigned)((entries + 255) / 256), 256, 0, (hipStream_t)stream>>>(w, (v4u*)shadow, K, N,
+                                                                                 strips_padded8(N));
+    return launch_status();
+}
+
+extern "C" int k3q_dense_i8_w8s_supported(int64_t M, int64_t K, int64_t N) { return w8s_plan(M, K, N).ok ? 1 : 0; }
+
+namespace {
+int launch_w8s(const void* x, const int8_t* xq, const void* xs, int64_t M, int64_t K, int64_t N,
+               const void* shadow, const void* kernel_scale, const void* bias, int64_t bias_stride,
+               float epsilon, float range_lo, float range_hi, void* y, hipStream_t stream) {
+    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    if (bias_stride != 0 && bias_stride != N) return K3Q_ERR_SHAPE;
+    W8sPlan pl = w8s_plan(M, K, N);
+    if (!pl.ok) return K3Q_ERR_SHAPE;
+    const bool quantised = xq != nullptr;
+    if (!(quantised ? (const void*)xs : x) || !shadow || !kernel_scale || !y) return K3Q_ERR_NULL;
+    if (!aligned_to(quantised ? (const void*)xq : x, 16) || !aligned_to(shadow, 16) || !aligned_to(y, 2) ||
+        !aligned_to(kernel_scale, 2) || (bias && !aligned_to(bias, 2)) || (xs && !aligned_to(xs, 2)))
+        return K3Q_ERR_ALIGN;
+    W8sParams p;
+    p.x = (const uint16_t*)x;
+    p.xq = xq;
+    p.xs = (const uint16_t*)xs;
+    p.w = (const v4i*)shadow;
+    p.scale = (const uint16_t*)kernel_scale;
+    p.bias = (const uint16_t*)bias;
+    p.y = (uint16_t*)y;
+    p.bias_stride = bias ? bias_stride : 0;
+    p.M = (int)M;
+    p.K = (int)K;
+    p.N = (int)N;
+    p.units = (int)(K / 64);
+    p.groups = (int)pl.groups;
+    const uint64_t per_row = (uint64_t)K / (quantised ? 16 : 8);
+    p.row_magic = (int)(uint32_t)((((uint64_t)1 << 32) + per_row - 1) / per_row);
+    p.eps = host_round_bf16(epsilon);  // torch rounds the epsilon operand to the tensor dtype before the add
+    p.qlo = range_lo;
+    p.qhi = range_hi;
+    if (quantised) pl.np = -1;
+    const W8sKernel kernel = pick_kernel8(pl);
+    {
+        static std::mutex mu;
+        static std::set<const void*> raised;
+        std::lock_guard<std::mutex> lock(mu);
+        if (!raised.count((const void*)kernel)) {
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
+                hipSuccess)
+                return K3Q_ERR_LAUNCH;
+            raised.insert((const void*)kernel);
+        }
+    }
+    kernel<<<(unsigned)pl.blocks, kT, pl.lds, stream>>>(p);
+    return launch_status();
+}
+}  // namespace
+
+extern "C" int k3q_dense_i8_w8s(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N, const void* shadow,
+                                const void* kernel_scale, const void* bias, int64_t bias_stride, float epsilon,
+                                float range_lo, float range_hi, void* y, void* stream) {
+    if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (!(range_lo >= -128.f && range_hi <= 127.f && range_lo < range_hi)) return K3Q_ERR_SHAPE;
+    return launch_w8s(x, nullptr, nullptr, M, K, N, shadow, kernel_scale, bias, bias_stride, epsilon, range_lo,
+                      range_hi, y, (hipStream_t)stream);
+}
+
+extern "C" int k3q_gemm_i8_w8s(const int8_t* a, const void* a_scale, int scale_dtype, int64_t M, int64_t K,
+                               int64_t N, const void* shadow, const void* kernel_scale, const void* bias,
+                               int64_t bias_stride, void* y, void* stream) {
+    if (scale_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (M > 0 && !a) return K3Q_ERR_NULL;
+    return launch_w8s(nullptr, a, a_scale, M, K, N, shadow, kernel_scale, bias, bias_stride, 0.f, -127.f, 127.f,
+                      y, (hipStream_t)stream);
+}

@@ -81,6 +81,15 @@ def kmajor_rows(rows, units, input_dim=0):
     return low <= rows <= KMAJOR_MAX_ROWS
 
 
+def int8_strip_route(quantizer, x2, units):
+    """Whether an int8 call of these rows goes to `ops.int8_dense_strip`: bfloat16 rows on the
+    device, few enough, a plain abs-max quantizer (whatever its range and epsilon), a shape the
+    kernel takes."""
+    return (type(quantizer) is quantizers.AbsMaxQuantizer and quantizer.output_dtype == "int8"
+            and x2.is_cuda and x2.dtype == torch.bfloat16 and 0 < x2.shape[0] <= kops.INT8_STRIP_MAX_ROWS
+            and kops.int8_strip_supported(x2.shape[0], x2.shape[1], units))
+
+
 class Dense(Layer):
     def __init__(self, units, activation=None, use_bias=True, kernel_initializer=None,
                  bias_initializer="zeros", dtype=None, name=None, device=None,
@@ -288,11 +297,22 @@ class Dense(Layer):
             return y
         lead = inputs.shape[:-1]
         x2 = inputs.reshape(-1, inputs.shape[-1])
-        q, scale = quantize_rows(self.inputs_quantizer, x2)
         M, N = x2.shape[0], self.units
         exact = self.exact_epilogue
         if exact is None:
             exact = True
+        if exact and int8_strip_route(self.inputs_quantizer, x2, N):
+            # decode sizes: quantizer, matmul and de-scale in one launch, from the strip-linear copy
+            y = kops.int8_dense_strip(
+                x2, self._cached("w8s", self._kernel, kops.int8_strip_copy), N,
+                self._read_cached("kernel_scale", self.kernel_scale), bias=self._call_bias(),
+                epsilon=self.inputs_quantizer.epsilon, value_range=self.inputs_quantizer.value_range,
+                quantize=lambda rows: quantize_rows(self.inputs_quantizer, rows))
+            y = y.reshape(*lead, N)
+            if self.activation is not None:
+                y = self.activation(y)
+            return y
+        q, scale = quantize_rows(self.inputs_quantizer, x2)
         y = kops.int8_matmul(
             q, as_tensor(self._kernel), a_scale=scale,
             kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),

@@ -18,7 +18,7 @@ import string
 import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
-from keras_amd.layers.dense import (_ACTIVATIONS, activation_name, glorot_uniform,
+from keras_amd.layers.dense import (_ACTIVATIONS, activation_name, glorot_uniform, int8_strip_route,
                                     serialize_quantization_config)
 from keras_amd.layers.layer import Layer, as_tensor, require_default_g_idx, to_torch_dtype
 from keras_amd.layers.together import quantize_rows
@@ -519,10 +519,19 @@ class EinsumDense(Layer):
                              lambda t: t.to(cd).reshape(-1).contiguous()),
                 bias=bias, prepacked=pre)
             return self._finish(y2, free_shape, gv, fused)
-        q, scale = quantize_rows(self.inputs_quantizer, x2)
         exact = self.exact_epilogue
         if exact is None:
             exact = True
+        if exact and int8_strip_route(self.inputs_quantizer, x2, n):
+            # decode sizes, as Dense: one launch from the strip-linear copy of the [K, N] matrix
+            y2 = kops.int8_dense_strip(
+                x2, self._cached("w8s", self._kernel, lambda t: kops.int8_strip_copy(kernel_matrix(t))), n,
+                self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).reshape(-1).contiguous()),
+                bias=bias, epsilon=self.inputs_quantizer.epsilon,
+                value_range=self.inputs_quantizer.value_range,
+                quantize=lambda rows: quantize_rows(self.inputs_quantizer, rows))
+            return self._finish(y2, free_shape, gv, fused)
+        q, scale = quantize_rows(self.inputs_quantizer, x2)
         y2 = kops.int8_matmul(
             q, k2, a_scale=scale,
             kernel_scale=self._cached("kernel_scale", self.kernel_scale,

@@ -683,6 +683,86 @@ def float_matmul_nk(x, wt, parts=1, bias=None):
 
 
 
+INT8_STRIP_MAX_ROWS = 16
+
+
+def int8_strip_supported(M, K, N):
+    """Whether `int8_dense_strip` takes M rows against a [K, N] int8 kernel."""
+    return bool(_lib.load().k3q_dense_i8_w8s_supported(int(M), int(K), int(N)))
+
+
+def int8_strip_copy(kernel):
+    """The strip-linear copy of a stored int8 kernel `[K, N]` that `int8_dense_strip` reads
+    (include/k3q.h, k3q_w8s_pack): uint8 bytes, made once per layer."""
+    _lib.require_device(kernel)
+    if kernel.dtype != torch.int8 or kernel.dim() != 2:
+        raise ValueError(f"expected the stored int8 kernel [K, N], got {kernel.dtype} {tuple(kernel.shape)}")
+    lib = _lib.load()
+    K, N = (int(d) for d in kernel.shape)
+    nbytes = lib.k3q_w8s_shadow_bytes(K, N)
+    if nbytes <= 0:
+        raise ValueError(f"no strip-linear copy for a [{K}, {N}] kernel (K % 64 != 0)")
+    src = kernel if kernel.is_contiguous() else kernel.contiguous()
+    out = torch.empty(nbytes, dtype=torch.uint8, device=src.device)
+    _lib.check(lib.k3q_w8s_pack(_lib.ptr(src), K, N, _lib.ptr(out), _lib.stream_ptr(src.device)), "k3q_w8s_pack")
+    return out
+
+
+# values of x up to which every workgroup of `int8_dense_strip` quantises the rows itself; beyond,
+# one quantizer launch and the kernel's pre-quantised form are faster (measured: 8 rows of 4096
+# cost 6 us more than one row when quantised in every workgroup, a quantizer launch 3 us)
+INT8_STRIP_FUSED_QUANTIZER_MAX = 16384
+
+
+def int8_dense_strip(x, shadow, units, kernel_scale, bias=None, epsilon=1e-7, value_range=(-127, 127),
+                     quantize=None):
+    """The int8 Dense forward for up to 16 bfloat16 rows: abs-max quantisation of the rows, exact
+    int8 matmul against `int8_strip_copy(kernel)`, bit-exact bfloat16 de-scale, bias (N values)
+    or addend (a row per row of x).  One launch for small x; for larger x the rows are
+    quantised by `quantize(x2)` (default: `quantizers.abs_max_quantize` with these settings)
+    first.  Same bits as `abs_max_quantize` + `int8_matmul(..., exact_epilogue=True)`.
+    Reference: keras/src/layers/core/dense.py:956-972."""
+    _lib.require_device(x, shadow, kernel_scale, bias)
+    lib = _lib.load()
+    if x.dtype != torch.bfloat16 or kernel_scale.dtype != torch.bfloat16:
+        raise TypeError("the strip route computes in bfloat16")
+    K, N = int(x.shape[-1]), int(units)
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    if not lib.k3q_dense_i8_w8s_supported(M, K, N):
+        raise ValueError(f"int8_dense_strip does not take M={M}, K={K}, N={N}")
+    if shadow.dtype != torch.uint8 or shadow.numel() != lib.k3q_w8s_shadow_bytes(K, N):
+        raise ValueError("shadow is not int8_strip_copy(kernel) of this [K, N]")
+    if kernel_scale.numel() != N:
+        raise ValueError(f"kernel_scale holds {kernel_scale.numel()} values, expected {N}")
+    _check_bias_size(bias, M, N)
+    if bias is not None and bias.dtype != torch.bfloat16:
+        raise TypeError("bias must be bfloat16")
+    stride = N if (bias is not None and M > 1 and bias.numel() == M * N) else 0
+    ks = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    if M * K > INT8_STRIP_FUSED_QUANTIZER_MAX:
+        if quantize is None:
+            from keras_amd import quantizers
+
+            q, s = quantizers.abs_max_quantize(x2, axis=-1, value_range=value_range, epsilon=epsilon)
+        else:
+            q, s = quantize(x2)
+        rc = lib.k3q_gemm_i8_w8s(_lib.ptr(q), _lib.ptr(s), _lib.dtype_code(s.dtype), M, K, N, _lib.ptr(shadow),
+                                 _lib.ptr(ks), _lib.ptr(bias) if bias is not None else None, stride,
+                                 _lib.ptr(y), _lib.stream_ptr(x.device))
+        _lib.check(rc, "k3q_gemm_i8_w8s")
+        return y.reshape(*lead, N)
+    rc = lib.k3q_dense_i8_w8s(_lib.ptr(x2), _lib.dtype_code(x.dtype), M, K, N, _lib.ptr(shadow), _lib.ptr(ks),
+                              _lib.ptr(bias) if bias is not None else None, stride, float(epsilon),
+                              float(value_range[0]), float(value_range[1]), _lib.ptr(y),
+                              _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_dense_i8_w8s")
+    return y.reshape(*lead, N)
+
+
 def decode_attention_supported(q, cache_k):
     """bfloat16, head width 128, one new position."""
     return (q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 4 and q.shape[1] == 1
