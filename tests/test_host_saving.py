@@ -166,6 +166,66 @@ def test_number_types_round_trip(dtype):
     assert back["empty"].value.shape == (0, 4)
 
 
+def test_int8_and_bfloat16_dataset_encodings_follow_the_format_specification():
+    # No file in the reference tree holds an int8 or a bfloat16 dataset, so these two encodings
+    # are pinned by what the HDF5 File Format Specification (version 3, IV.A.2.d "The Datatype
+    # Message") fixes, field by field:
+    #   byte 0      version (high nibble) = 1, class (low nibble): 0 fixed-point, 5 opaque
+    #   bytes 1-3   class bit field
+    #   bytes 4-7   element size
+    #   then the class's properties
+    # int8 = what `group[key] = int8 ndarray` makes h5py emit (H5T_STD_I8LE): class 0; bit 0 = 0
+    # little-endian, bits 1-2 = 0 zero padding, bit 3 = 1 two's-complement signed; size 1;
+    # properties: bit offset 0 (uint16), bit precision 8 (uint16).
+    int8_message = bytes([0x10, 0x08, 0x00, 0x00, 0x01, 0x00, 0x00, 0x00, 0x00, 0x00, 0x08, 0x00])
+    # bfloat16 = what `create_dataset(key, data=<ml_dtypes.bfloat16 array>)` asks for
+    # (keras/src/saving/saving_lib.py:1469-1473): numpy sees a 2-byte void-kind dtype, which
+    # h5py maps to H5T_OPAQUE of that size with no tag: class 5; bits 0-7 = length of the ASCII
+    # tag = 0; size 2; no properties.  The value's meaning travels in the attribute
+    # dtype = "bfloat16" (saving_lib.py:1455-1459 reads it back through that attribute).
+    opaque2_message = bytes([0x15, 0x00, 0x00, 0x00, 0x02, 0x00, 0x00, 0x00])
+    assert h5min._datatype_message(np.int8) == int8_message
+    assert h5min._datatype_message(np.dtype("V2")) == opaque2_message
+    # unsigned differs in the sign bit only
+    assert h5min._datatype_message(np.uint8) == bytes([0x10, 0x00, 0, 0, 1, 0, 0, 0, 0, 0, 8, 0])
+
+    rng = np.random.default_rng(3)
+    q = rng.integers(-128, 128, size=(6, 10), dtype=np.int8)
+    bf16_bits = rng.integers(0, 1 << 16, size=(4, 3), dtype=np.uint16)
+    root = h5min.Group({"vars": h5min.Group({
+        "0": h5min.Dataset(q),
+        "1": h5min.Dataset(bf16_bits.view("V2"), attrs={"dtype": "bfloat16"})})})
+    data = h5min.dump(root)
+    # the messages sit in the datasets' (version 1) object headers: type 0x0003, their length
+    # padded to 8, flags 1 (constant), three reserved bytes, then the body
+    for body in (int8_message, opaque2_message):
+        padded = body + b"\0" * (-len(body) % 8)
+        assert struct.pack("<HHB3x", 0x0003, len(padded), 1) + padded in data
+    # the int8 values lie in the file as they lie in memory (contiguous layout, row-major)
+    assert q.tobytes() in data and bf16_bits.tobytes() in data
+    # and the reader -- the code path the reference-written fixture pins for float32 datasets,
+    # attributes and groups -- decodes both
+    back = h5min.load(data)["vars"]
+    assert back["0"].value.dtype == np.int8 and np.array_equal(back["0"].value, q)
+    assert back["1"].value.dtype == np.dtype("V2")
+    assert np.array_equal(back["1"].value.view(np.uint16), bf16_bits)
+    assert back["1"].attrs["dtype"] == "bfloat16"
+    # through the store: a bfloat16 tensor comes back as the same bits, an int8 tensor as int8
+    t = torch.randn(5, 4).to(torch.bfloat16)
+    buf = io.BytesIO()
+    store = saving.H5Store(buf, mode="w")
+    entry = store.make("layers/dense")
+    entry["0"] = torch.from_numpy(q)
+    entry["1"] = t
+    store.close()
+    for body in (int8_message, opaque2_message):
+        padded = body + b"\0" * (-len(body) % 8)
+        assert struct.pack("<HHB3x", 0x0003, len(padded), 1) + padded in buf.getvalue()
+    rd = saving.H5Store(io.BytesIO(buf.getvalue()), mode="r").get("layers/dense")
+    assert np.array_equal(np.asarray(rd["0"]), q) and np.asarray(rd["0"]).dtype == np.int8
+    assert rd["1"].dtype == torch.bfloat16 and torch.equal(rd["1"].view(torch.int16), t.view(torch.int16))
+
+
 # ---------------------------------------------------------------------------- the model walk
 
 
