@@ -60,6 +60,29 @@ def glorot_uniform(shape, dtype, generator=None):
     return ((torch.rand(shape, generator=generator) * 2.0 - 1.0) * limit).to(dtype)
 
 
+def he_uniform(shape, dtype, generator=None):
+    """U(-L, L), L = sqrt(6 / fan_in) (keras/src/initializers/random_initializers.py, `HeUniform`)."""
+    fan_in = shape[0]
+    if len(shape) > 2:
+        receptive = 1
+        for d in shape[:-2]:
+            receptive *= d
+        fan_in = shape[-2] * receptive
+    limit = math.sqrt(6.0 / max(fan_in, 1))
+    return ((torch.rand(shape, generator=generator) * 2.0 - 1.0) * limit).to(dtype)
+
+
+LORA_INITIALIZERS = {"he_uniform": he_uniform, "zeros": "zeros", "ones": "ones"}
+
+
+def lora_initializer(spec):
+    if callable(spec):
+        return spec
+    if spec not in LORA_INITIALIZERS:
+        raise ValueError(f"Unknown initializer: {spec}")
+    return LORA_INITIALIZERS[spec]
+
+
 # rows for which the int4 forward reads the K-contiguous copy of the kernel (measured against
 # the 32-row passes below it and the de-quantise + GEMM route above it, groups of 128, us:
 # K=4096, N=14336: 17 rows 22 against 27, 32 rows 23 against 31, 64 rows 26 against 60, 128 rows
@@ -93,9 +116,11 @@ def int8_strip_route(quantizer, x2, units):
 class Dense(Layer):
     def __init__(self, units, activation=None, use_bias=True, kernel_initializer=None,
                  bias_initializer="zeros", dtype=None, name=None, device=None,
-                 quantization_config=None):
+                 quantization_config=None, lora_rank=None, lora_alpha=None):
         super().__init__(dtype=dtype, name=name, device=device)
         self.quantization_config = quantization_config  # dense.py:98-130
+        self.lora_rank = lora_rank
+        self.lora_alpha = lora_alpha if lora_alpha is not None else lora_rank
         if not isinstance(units, int) or units <= 0:
             raise ValueError(
                 f"Received an invalid value for `units`, expected a positive integer. Received: units={units}"
@@ -127,19 +152,74 @@ class Dense(Layer):
         else:
             self.bias = None
         self.built = True
+        if self.lora_rank:
+            self.enable_lora(self.lora_rank)  # (dense.py:160-161: the alpha is not passed on)
 
     @property
     def kernel(self):
         """The kernel as a consumer sees it: the int4 kernel comes back unpacked to
-        `[input_dim, units]` int8 (keras/src/layers/core/dense.py:163-236)."""
+        `[input_dim, units]` int8; with LoRA enabled the low-rank update is added and the sum
+        cast to the compute dtype (keras/src/layers/core/dense.py:163-236)."""
         if not self.built:
             raise AttributeError("You must build the layer before accessing `kernel`.")
         kernel = as_tensor(self._kernel)
         if self.quantization_mode == "int4":
             kernel = quantizers.unpack_int4(kernel, self._orig_output_dim, axis=-1)
+        if self.lora_enabled:
+            delta = (self.lora_alpha / self.lora_rank) * torch.matmul(
+                as_tensor(self.lora_kernel_a), as_tensor(self.lora_kernel_b))
+            kernel = torch.add(kernel, delta).to(to_torch_dtype(self.compute_dtype))
         return kernel
 
+    def enable_lora(self, rank, lora_alpha=None, a_initializer="he_uniform", b_initializer="zeros"):
+        """keras/src/layers/core/dense.py:251-312: float32 `lora_kernel_a` [input_dim, rank] and
+        `lora_kernel_b` [rank, units]; the forward adds (alpha / rank) * (x . a) . b."""
+        if not self.built:
+            raise ValueError("Cannot enable lora on a layer that isn't yet built.")
+        if self.lora_enabled:
+            raise ValueError("lora is already enabled. This can only be done once per layer.")
+        if self.quantization_mode == "int4" and hasattr(self, "_orig_input_dim"):
+            input_dim = self._orig_input_dim
+        else:
+            input_dim = self._kernel.shape[0]
+        self.lora_kernel_a = self.add_weight(name="lora_kernel_a", shape=(input_dim, rank), dtype="float32",
+                                             initializer=lora_initializer(a_initializer), trainable=True)
+        self.lora_kernel_b = self.add_weight(name="lora_kernel_b", shape=(rank, self.units), dtype="float32",
+                                             initializer=lora_initializer(b_initializer), trainable=True)
+        self.lora_enabled = True
+        self.lora_rank = rank
+        self.lora_alpha = lora_alpha if lora_alpha is not None else rank
+
+    def _quantized_call_with_lora(self, quantized_call, inputs):
+        """The reference's order with LoRA enabled (dense.py:972-986, :1085-1095): the de-scaled
+        quantized product first, then the low-rank term, the cast, the bias, the activation --
+        so the kernels run without their fused bias here."""
+        bias, activation = self.bias, self.activation
+        self.bias, self.activation, self.lora_enabled = None, None, False
+        try:
+            x = quantized_call(inputs)
+        finally:
+            self.bias, self.activation, self.lora_enabled = bias, activation, True
+        x = torch.add(x, self._lora_term(inputs)).to(to_torch_dtype(self.compute_dtype))
+        if bias is not None:
+            x = torch.add(x, self.read(bias))
+        if activation is not None:
+            x = activation(x)
+        return x
+
+    def _lora_term(self, inputs):
+        """(alpha / rank) * (inputs . a) . b as the quantized calls add it (dense.py:977-980,
+        :1086-1089): two small float matmuls in the compute dtype."""
+        lora_x = torch.matmul(inputs, self.read(self.lora_kernel_a))
+        lora_x = torch.matmul(lora_x, self.read(self.lora_kernel_b))
+        return (self.lora_alpha / self.lora_rank) * lora_x
+
     def call(self, inputs, training=None):
+        if self.lora_enabled:
+            x = torch.matmul(inputs, self.kernel)
+            if self.bias is not None:
+                x = torch.add(x, self.read(self.bias))
+            return self.activation(x) if self.activation is not None else x
         x = torch.matmul(inputs, self.read(self._kernel))
         if self.bias is not None:
             x = torch.add(x, self.read(self.bias))
@@ -283,7 +363,7 @@ class Dense(Layer):
     def _int8_call(self, inputs, training=None):
         """keras/src/layers/core/dense.py:938-986: quantise rows, int8 GEMM, de-scale, bias."""
         if self.lora_enabled:
-            raise NotImplementedError("LoRA on a quantized Dense is outside this inference path.")
+            return self._quantized_call_with_lora(self._int8_call, inputs)
         if not self.inputs_quantizer:
             # weight-only: float activations against the int8 kernel, then the de-scale
             y = kops.int8_weight_only_matmul(
@@ -330,7 +410,7 @@ class Dense(Layer):
         """keras/src/layers/core/dense.py:988-1095, weight-only: the packed kernel is
         consumed in place (no unpack, no de-quantised copy)."""
         if self.lora_enabled:
-            raise NotImplementedError("LoRA on a quantized Dense is outside this inference path.")
+            return self._quantized_call_with_lora(self._int4_call, inputs)
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
         if self.inputs_quantizer:
@@ -450,21 +530,77 @@ class Dense(Layer):
             "int4": ["kernel", "bias", "kernel_scale", "kernel_zero", "g_idx"],
         }
 
+    def _get_kernel_with_merged_lora(self):
+        """`(kernel, kernel_scale, kernel_zero)` as they are saved
+        (keras/src/layers/core/dense.py:1301-1427): without LoRA the variables themselves; with
+        it the kernel is de-quantised (int8: `cast(q, compute) / scale`; int4: unpack, then
+        divide or `dequantize_with_sz_map`), `(alpha / rank) * a . b` is added in float, and the sum
+        is quantised again the way `quantize()` does it (host numpy path), giving new scales
+        (and zero points)."""
+        mode = self.quantization_mode
+        if mode is None:
+            return self.kernel, None, None
+        kernel_value = as_tensor(self._kernel)
+        kernel_scale = as_tensor(self.kernel_scale)
+        kernel_zero = as_tensor(self.kernel_zero) if hasattr(self, "kernel_zero") else None
+        if not self.lora_enabled:
+            return kernel_value, kernel_scale, kernel_zero
+        cd = to_torch_dtype(self.compute_dtype)
+        block_size = getattr(self, "_int4_block_size", None)
+        grouped = block_size is not None and block_size != -1
+        if mode == "int4":
+            unpacked = quantizers.unpack_int4(kernel_value, self._orig_output_dim, axis=-1)
+            if grouped:
+                float_kernel = quantizers.dequantize_with_sz_map(
+                    unpacked, kernel_scale, kernel_zero, as_tensor(self.g_idx), group_axis=0).to(cd)
+            else:
+                float_kernel = torch.divide(unpacked.to(cd), kernel_scale)
+            quant_range = (-8, 7)
+        elif mode == "int8":
+            float_kernel = torch.divide(kernel_value.to(cd), kernel_scale)
+            quant_range = (-127, 127)
+        else:
+            raise self._quantization_mode_error(mode)
+        delta = (self.lora_alpha / self.lora_rank) * torch.matmul(
+            as_tensor(self.lora_kernel_a), as_tensor(self.lora_kernel_b))
+        merged = torch.add(float_kernel, delta)
+        if mode == "int4" and grouped:
+            requantized, kernel_scale, kernel_zero = quantizers.abs_max_quantize_grouped_with_zero_point(
+                merged, block_size=block_size, to_numpy=True)
+        else:
+            requantized, kernel_scale = quantizers.abs_max_quantize(
+                merged, axis=0, value_range=quant_range, dtype="int8", to_numpy=True)
+            kernel_scale = torch.squeeze(kernel_scale, dim=0)
+            kernel_zero = None
+        if mode == "int4":
+            kernel_value, _, _ = quantizers.pack_int4(requantized.to(self.device), axis=-1)
+        else:
+            kernel_value = requantized
+        return kernel_value, kernel_scale, kernel_zero
+
     def save_own_variables(self, store):
-        """Write variables under "0", "1", ... in spec order, skipping absent ones."""
+        """Write variables under "0", "1", ... in spec order, skipping absent ones; a LoRA update
+        is merged into what is written (dense.py:314-378)."""
         if not self.built:
             return
         mode = self.quantization_mode
         if mode not in self.variable_serialization_spec:
             raise self._quantization_mode_error(mode)
+        kernel_value, merged_scale, merged_zero = self._get_kernel_with_merged_lora()
         idx = 0
         for name in self.variable_serialization_spec[mode]:
             if name == "kernel":
-                value = self._kernel
+                value = kernel_value
             elif name == "bias" and self.bias is None:
                 continue
-            elif name in ("kernel_zero", "g_idx") and not hasattr(self, name):
+            elif name == "kernel_zero" and mode == "int4":
+                if merged_zero is None:
+                    continue
+                value = merged_zero
+            elif name == "g_idx" and not hasattr(self, name):
                 continue
+            elif name == "kernel_scale" and mode in ("int4", "int8"):
+                value = merged_scale
             else:
                 value = getattr(self, name)
             store[str(idx)] = as_tensor(value)
@@ -488,10 +624,14 @@ class Dense(Layer):
                 target = getattr(self, name)
             target.assign(store[str(idx)])
             idx += 1
+        if self.lora_enabled:
+            # what was saved has the update merged in (dense.py:428-430)
+            self.lora_kernel_a.assign(torch.zeros_like(as_tensor(self.lora_kernel_a)))
+            self.lora_kernel_b.assign(torch.zeros_like(as_tensor(self.lora_kernel_b)))
         self._cache.clear()
 
     def get_config(self):
-        return {
+        config = {
             "name": self.name,
             "units": self.units,
             "activation": activation_name(self.activation),
@@ -499,3 +639,7 @@ class Dense(Layer):
             "dtype": self.dtype_policy.name,
             "quantization_config": serialize_quantization_config(self.quantization_config),
         }
+        if self.lora_rank:
+            config["lora_rank"] = self.lora_rank
+            config["lora_alpha"] = self.lora_alpha
+        return config

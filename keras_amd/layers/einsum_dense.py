@@ -19,6 +19,7 @@ import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
 from keras_amd.layers.dense import (_ACTIVATIONS, activation_name, glorot_uniform, int8_strip_route,
+                                    lora_initializer,
                                     serialize_quantization_config)
 from keras_amd.layers.layer import Layer, as_tensor, require_default_g_idx, to_torch_dtype
 from keras_amd.layers.together import quantize_rows
@@ -222,8 +223,10 @@ class _BatchedView:
 class EinsumDense(Layer):
     def __init__(self, equation, output_shape, activation=None, bias_axes=None,
                  kernel_initializer=None, bias_initializer="zeros", dtype=None, name=None,
-                 device=None, quantization_config=None):
+                 device=None, quantization_config=None, lora_rank=None, lora_alpha=None):
         super().__init__(dtype=dtype, name=name, device=device)
+        self.lora_rank = lora_rank
+        self.lora_alpha = lora_alpha if lora_alpha is not None else lora_rank
         self.quantization_config = quantization_config  # einsum_dense.py __init__ / build
         self.equation = equation
         self.partial_output_shape = (output_shape,) if isinstance(output_shape, int) else tuple(output_shape)
@@ -258,6 +261,8 @@ class EinsumDense(Layer):
         else:
             self.bias = None
         self.built = True
+        if self.lora_rank:
+            self.enable_lora(self.lora_rank, lora_alpha=self.lora_alpha)  # einsum_dense.py:234-235
 
     @property
     def kernel(self):
@@ -267,9 +272,112 @@ class EinsumDense(Layer):
         if self.quantization_mode == "int4":
             kernel = quantizers.unpack_int4(kernel, self._int4_unpacked_column_size, axis=-1)
             kernel = kernel.reshape(self.original_kernel_shape)
+        if self.lora_enabled:  # einsum_dense.py:298-306
+            delta = (self.lora_alpha / self.lora_rank) * torch.matmul(
+                as_tensor(self.lora_kernel_a), as_tensor(self.lora_kernel_b))
+            kernel = torch.add(kernel, delta).to(to_torch_dtype(self.compute_dtype))
         return kernel
 
+    def enable_lora(self, rank, lora_alpha=None, a_initializer="he_uniform", b_initializer="zeros"):
+        """keras/src/layers/core/einsum_dense.py:327-385: float32 `lora_kernel_a` of the kernel's
+        shape with its last axis replaced by `rank`, `lora_kernel_b` [rank, last axis]."""
+        if not self.built:
+            raise ValueError("Cannot enable lora on a layer that isn't yet built.")
+        if self.lora_enabled:
+            raise ValueError("lora is already enabled. This can only be done once per layer.")
+        if self.quantization_mode == "int4":
+            shape = tuple(self.original_kernel_shape)
+        else:
+            shape = tuple(self._kernel.shape)
+        self.lora_kernel_a = self.add_weight(name="lora_kernel_a", shape=shape[:-1] + (rank,), dtype="float32",
+                                             initializer=lora_initializer(a_initializer), trainable=True)
+        self.lora_kernel_b = self.add_weight(name="lora_kernel_b", shape=(rank, shape[-1]), dtype="float32",
+                                             initializer=lora_initializer(b_initializer), trainable=True)
+        self.lora_enabled = True
+        self.lora_rank = rank
+        self.lora_alpha = lora_alpha if lora_alpha is not None else rank
+
+    def _quantized_call_with_lora(self, quantized_call, inputs):
+        """einsum_dense.py:1109-1118, :1251-1261: de-scaled quantized product, + low-rank term, cast,
+        + bias, activation (the kernels run without their fused bias here)."""
+        bias, activation = self.bias, self.activation
+        self.bias, self.activation, self.lora_enabled = None, None, False
+        try:
+            x = quantized_call(inputs)
+        finally:
+            self.bias, self.activation, self.lora_enabled = bias, activation, True
+        lora_x = torch.einsum(self.equation, inputs, self.read(self.lora_kernel_a))
+        lora_x = torch.matmul(lora_x, self.read(self.lora_kernel_b))
+        x = torch.add(x, (self.lora_alpha / self.lora_rank) * lora_x).to(to_torch_dtype(self.compute_dtype))
+        if bias is not None:
+            x = torch.add(x, self.read(bias))
+        if activation is not None:
+            x = activation(x)
+        return x
+
+    def _get_kernel_with_merged_lora(self):
+        """`(kernel, kernel_scale, kernel_zero)` as saved
+        (keras/src/layers/core/einsum_dense.py:1493-1623): with LoRA enabled, de-quantise (int8: the
+        kernel over its scale taken back through the expand / squeeze / transpose bookkeeping;
+        int4: as Dense on the flat matrix, reshaped), add `(alpha / rank) * a . b`, quantise again as
+        `quantize()` does."""
+        mode = self.quantization_mode
+        if mode is None:
+            return self.kernel, None, None
+        kernel_zero = as_tensor(self.kernel_zero) if hasattr(self, "kernel_zero") else None
+        if not self.lora_enabled:
+            return as_tensor(self._kernel), as_tensor(self.kernel_scale), kernel_zero
+        cd = to_torch_dtype(self.compute_dtype)
+        if mode == "int4":
+            unpacked = quantizers.unpack_int4(as_tensor(self._kernel), self._int4_unpacked_column_size, axis=-1)
+            block_size = self._int4_block_size
+            grouped = block_size is not None and block_size != -1
+            if grouped:
+                kernel_fp = quantizers.dequantize_with_sz_map(
+                    unpacked, as_tensor(self.kernel_scale), kernel_zero, as_tensor(self.g_idx), group_axis=0)
+            else:
+                kernel_fp = torch.divide(unpacked.to(cd), as_tensor(self.kernel_scale))
+            kernel_fp = kernel_fp.reshape(self.original_kernel_shape)
+        elif mode == "int8":
+            part = self._quant_info["kernel"]
+            scale = as_tensor(self.kernel_scale)
+            for ax in sorted(part["squeeze"]):
+                scale = scale.unsqueeze(ax)
+            for ax in sorted(part["expand"], reverse=True):
+                scale = scale.squeeze(ax)
+            if part["transpose"]:
+                perm = part["transpose"]
+                scale = scale.permute(sorted(range(len(perm)), key=perm.__getitem__))
+            kernel_fp = torch.divide(as_tensor(self._kernel), scale)
+        else:
+            raise self._quantization_mode_error(mode)
+        update = (self.lora_alpha / self.lora_rank) * torch.matmul(
+            as_tensor(self.lora_kernel_a), as_tensor(self.lora_kernel_b))
+        merged = torch.add(kernel_fp, update)
+        if mode == "int4":
+            flat = merged.reshape(self._int4_rows, self._int4_unpacked_column_size)
+            if grouped:
+                q, new_scale, kernel_zero = quantizers.abs_max_quantize_grouped_with_zero_point(
+                    flat, block_size=block_size, to_numpy=True)
+            else:
+                q, new_scale = quantizers.abs_max_quantize(flat, axis=0, value_range=(-8, 7), dtype="int8",
+                                                           to_numpy=True)
+                new_scale = torch.squeeze(new_scale, dim=0)
+                kernel_zero = None
+            new_kernel, _, _ = quantizers.pack_int4(q.to(self.device), axis=-1)
+        else:
+            new_kernel, new_scale = quantizers.abs_max_quantize(
+                merged, axis=tuple(self._kernel_reduced_axes), to_numpy=True)
+            new_scale = _adjust_scale(new_scale, self._quant_info["kernel"]).contiguous()
+            kernel_zero = None
+        return new_kernel, new_scale, kernel_zero
+
     def call(self, inputs, training=None):
+        if self.lora_enabled:
+            x = torch.einsum(self.equation, inputs, self.kernel)
+            if self.bias is not None:
+                x = torch.add(x, self.read(self.bias))
+            return self.activation(x) if self.activation is not None else x
         x = torch.einsum(self.equation, inputs, self.read(self._kernel))
         if self.bias is not None:
             x = torch.add(x, self.read(self.bias))
@@ -493,7 +601,7 @@ class EinsumDense(Layer):
     def _int8_call(self, inputs, training=None):
         """keras/src/layers/core/einsum_dense.py:1030-1118 as quantise-rows + int8 GEMM."""
         if self.lora_enabled:
-            raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
+            return self._quantized_call_with_lora(self._int8_call, inputs)
         if self._gemm is None and self._batched is not None:
             return self._int8_call_batched(inputs)
         gv = self._gemm_view()
@@ -636,7 +744,7 @@ class EinsumDense(Layer):
     def _int4_call(self, inputs, training=None):
         """keras/src/layers/core/einsum_dense.py:1120-1261, weight-only."""
         if self.lora_enabled:
-            raise NotImplementedError("LoRA on a quantized EinsumDense is outside this inference path.")
+            return self._quantized_call_with_lora(self._int4_call, inputs)
         if self._gemm is None and self._batched is not None:
             return self._int4_call_batched(inputs)
         gv = self._gemm_view()
@@ -789,7 +897,7 @@ class EinsumDense(Layer):
 
     # ---- serialization -------------------------------------------------------------------------
     def get_config(self):
-        return {
+        config = {
             "name": self.name,
             "output_shape": list(self.partial_output_shape),
             "equation": self.equation,
@@ -798,6 +906,10 @@ class EinsumDense(Layer):
             "dtype": self.dtype_policy.name,
             "quantization_config": serialize_quantization_config(self.quantization_config),
         }
+        if self.lora_rank:
+            config["lora_rank"] = self.lora_rank
+            config["lora_alpha"] = self.lora_alpha
+        return config
 
     @property
     def variable_serialization_spec(self):
@@ -811,14 +923,22 @@ class EinsumDense(Layer):
     def save_own_variables(self, store):
         if not self.built:
             return
+        mode = self.quantization_mode
+        kernel_value, merged_scale, merged_zero = self._get_kernel_with_merged_lora()
         idx = 0
-        for name in self.variable_serialization_spec[self.quantization_mode]:
+        for name in self.variable_serialization_spec[mode]:
             if name == "kernel":
-                value = self._kernel
+                value = kernel_value
             elif name == "bias" and self.bias is None:
                 continue
-            elif name in ("kernel_zero", "g_idx") and not hasattr(self, name):
+            elif name == "kernel_zero" and mode == "int4":
+                if merged_zero is None:
+                    continue
+                value = merged_zero
+            elif name == "g_idx" and not hasattr(self, name):
                 continue
+            elif name == "kernel_scale" and mode in ("int4", "int8"):
+                value = merged_scale
             else:
                 value = getattr(self, name)
             store[str(idx)] = as_tensor(value)
@@ -839,4 +959,7 @@ class EinsumDense(Layer):
                 target = getattr(self, name)
             target.assign(store[str(idx)])
             idx += 1
+        if self.lora_enabled:  # einsum_dense.py:497-499: the saved kernel holds the update
+            self.lora_kernel_a.assign(torch.zeros_like(as_tensor(self.lora_kernel_a)))
+            self.lora_kernel_b.assign(torch.zeros_like(as_tensor(self.lora_kernel_b)))
         self._cache.clear()

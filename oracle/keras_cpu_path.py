@@ -417,6 +417,54 @@ def dense_int4_call(inputs, kernel, kernel_scale, orig_output_dim,
 # --------------------------------------------------------------------------
 # a11 / a13: EinsumDense
 # --------------------------------------------------------------------------
+def dense_lora_term(inputs, lora_a, lora_b, alpha, rank, compute_dtype=None):
+    """keras/src/layers/core/dense.py:977-980 / :1086-1089: what a quantized call adds when LoRA
+    is enabled, before the bias (the float32 LoRA variables are read in the compute dtype)."""
+    cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
+    x = torch.matmul(inputs.to(cd), _read_var(lora_a, cd))
+    x = torch.matmul(x, _read_var(lora_b, cd))
+    return (alpha / rank) * x
+
+
+def dense_merged_lora_kernel(mode, kernel, kernel_scale, lora_a, lora_b, alpha, rank,
+                             compute_dtype="float32", kernel_zero=None, g_idx=None, block_size=None,
+                             orig_output_dim=None):
+    """keras/src/layers/core/dense.py:1341-1427: de-quantise, add (alpha / rank) * a . b, quantise
+    again as `quantize()` does.  The variables are read outside a call here, i.e. in their own
+    dtype (float32 scales): `cast(q, compute) / scale` is then float32 whatever the compute
+    dtype.  -> (kernel, kernel_scale, kernel_zero) as saved.
+
+    Pinned by: a zero update returns the quantized kernel it started from (per-channel: every
+    column of an abs-max quantised kernel holds a +-127 / +-8|7 extreme, so the new scale maps
+    the integers onto themselves); a non-zero update de-quantises to within half a step of
+    (old de-quantised kernel + update); tests/test_oracle.py."""
+    cd = _tdtype(compute_dtype)
+    grouped = block_size is not None and block_size != -1
+    if mode == "int4":
+        unpacked = unpack_int4(kernel, orig_output_dim, axis=-1)
+        if grouped:
+            float_kernel = dequantize_with_sz_map(unpacked, kernel_scale, kernel_zero, g_idx, group_axis=0).to(cd)
+        else:
+            float_kernel = torch.divide(unpacked.to(cd), kernel_scale)
+        quant_range = (-8, 7)
+    elif mode == "int8":
+        float_kernel = torch.divide(kernel.to(cd), kernel_scale)
+        quant_range = (-127, 127)
+    else:
+        raise ValueError(f"Unsupported quantization mode: {mode}")
+    delta = (alpha / rank) * torch.matmul(lora_a, lora_b)
+    merged = torch.add(float_kernel, delta)
+    if mode == "int4" and grouped:
+        q, scale, zero = abs_max_quantize_grouped_with_zero_point(merged, block_size=block_size)
+    else:
+        q, scale = abs_max_quantize(merged, axis=0, value_range=quant_range, dtype="int8", to_numpy=True)
+        scale = torch.squeeze(scale, dim=0)
+        zero = None
+    if mode == "int4":
+        q, _, _ = pack_int4(q, axis=-1)
+    return q, scale, zero
+
+
 def _einsum_specs(equation, input_rank):
     """Canonical (input, kernel, output) label strings.
 
@@ -568,6 +616,32 @@ def einsum_dense_int8_call(inputs, kernel, kernel_scale, equation, bias=None,
     if return_intermediates:
         return x, dict(q=q, inputs_scale=s_in, acc=acc)
     return x
+
+
+def einsum_dense_merged_lora_kernel(mode, kernel, kernel_scale, lora_a, lora_b, alpha, rank, equation,
+                                    input_rank, compute_dtype="float32", qk=None, block_size=None):
+    """keras/src/layers/core/einsum_dense.py:1536-1623: de-quantise (int8: kernel over its scale
+    taken back through `_adjust_scale_for_dequant`; int4: `qk` as `einsum_dense_quantize_int4`
+    returns it, as Dense on the flat matrix), add (alpha / rank) * a . b, quantise again as
+    `quantize()` does.  Pinned like `dense_merged_lora_kernel` (zero update = identity)."""
+    cd = _tdtype(compute_dtype)
+    info = einsum_quantization_info(equation, input_rank)
+    update = (alpha / rank) * torch.matmul(lora_a, lora_b)
+    if mode == "int8":
+        kernel_fp = torch.divide(kernel, _adjust_scale_for_dequant(kernel_scale, info["kernel"]))
+        merged = torch.add(kernel_fp, update)
+        q, s = AbsMaxQuantizer(axis=tuple(info["kernel"]["reduced"]))(merged, to_numpy=True)
+        return q, _adjust_scale(s, info["kernel"]).contiguous(), None
+    grouped = block_size is not None and block_size != -1
+    unpacked = unpack_int4(qk["kernel"], qk["cols"], axis=-1)
+    if grouped:
+        kernel_fp = dequantize_with_sz_map(unpacked, qk["kernel_scale"], qk["kernel_zero"], qk["g_idx"],
+                                           group_axis=0)
+    else:
+        kernel_fp = torch.divide(unpacked.to(cd), qk["kernel_scale"])
+    merged = torch.add(kernel_fp.reshape(qk["original_kernel_shape"]), update)
+    out = dense_quantize_int4(merged.reshape(qk["rows"], qk["cols"]), block_size)
+    return out["kernel"], out["kernel_scale"], out["kernel_zero"]
 
 
 def einsum_dense_quantize_int4(kernel, equation, input_rank, block_size=128):

@@ -354,6 +354,132 @@ def test_unsupported_paths_raise(dev):
         cpu_layer(torch.randn(2, 32))  # no CPU fallback
 
 
+@pytest.mark.parametrize("mode,block_size", [("int8", None), ("int4", None), ("int4", 128)])
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_dense_lora_on_quantized_layer_and_merge_on_save(dev, mode, block_size, policy):
+    # keras/src/layers/core/dense.py:251-312 (enable_lora), :972-986 / :1085-1095 (the quantized
+    # calls add the low-rank term before the bias), :1301-1427 (the update is merged into what is
+    # saved: de-quantise, add, quantise again), :428-430 (a load zeroes the update)
+    g = torch.Generator().manual_seed(23)
+    M, K, N, rank, alpha = 6, 256, 192, 4, 8
+    layer = build_dense(dev, K, N, policy, seed=4)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f, bias_f = layer._kernel.value.cpu(), layer.bias.value.cpu()
+    if mode == "int8":
+        layer.quantize("int8")
+    else:
+        layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=block_size))
+    with pytest.raises(ValueError):
+        Dense(4, device=dev).enable_lora(2)          # not built
+    layer.enable_lora(rank, lora_alpha=alpha)
+    with pytest.raises(ValueError):
+        layer.enable_lora(rank)                      # only once
+    assert tuple(layer.lora_kernel_a.shape) == (K, rank) and tuple(layer.lora_kernel_b.shape) == (rank, N)
+    assert layer.lora_kernel_a.dtype == "float32" and layer.lora_kernel_b.dtype == "float32"
+    assert float(layer.lora_kernel_b.value.abs().max()) == 0.0    # b starts at zero
+    a = torch.randn(K, rank, generator=g) * 0.05
+    b = torch.randn(rank, N, generator=g) * 0.05
+    layer.lora_kernel_a.assign(a)
+    layer.lora_kernel_b.assign(b)
+    x = torch.randn(M, K, generator=g)
+    y = layer(x)
+    # forward against the oracle: quantized product, + low-rank term, cast, + bias
+    if mode == "int8":
+        qk, ks = ref.dense_quantize_int8(kernel_f)
+        base = ref.dense_int8_call(x.to(cd), qk, ks, None, compute_dtype=cd)
+        merged = ref.dense_merged_lora_kernel("int8", qk, ks, a, b, alpha, rank, compute_dtype=cd)
+    else:
+        q4 = ref.dense_quantize_int4(kernel_f, block_size)
+        qk, ks = q4["kernel"], q4["kernel_scale"]
+        base = ref.dense_int4_call(x.to(cd), qk, ks, N, kernel_zero=q4["kernel_zero"], g_idx=q4["g_idx"],
+                                   block_size=block_size, bias=None, compute_dtype=cd)
+        merged = ref.dense_merged_lora_kernel("int4", qk, ks, a, b, alpha, rank, compute_dtype=cd,
+                                              kernel_zero=q4["kernel_zero"], g_idx=q4["g_idx"],
+                                              block_size=block_size, orig_output_dim=N)
+    want = (base + ref.dense_lora_term(x, a, b, alpha, rank, compute_dtype=cd)).to(cd) + bias_f.to(cd)
+    assert y.dtype == cd and max_rel_err(y, want) <= RTOL[cd]
+    if mode == "int8" and cd == torch.float32:
+        # the base product is bit-exact; only the two small float matmuls differ in their sums
+        assert max_rel_err(y, want) <= 1e-5
+    # what is saved: the merged kernel, its new scales (and zero points), bit for bit the oracle's
+    store = {}
+    layer.save_own_variables(store)
+    names = [n for n in layer.variable_serialization_spec[mode]
+             if not (n in ("kernel_zero", "g_idx") and (mode == "int8" or not block_size))]
+    got = dict(zip(names, (store[str(i)] for i in range(len(names)))))
+    assert len(store) == len(names)
+    assert torch.equal(got["kernel"].cpu(), merged[0])
+    assert torch.equal(got["kernel_scale"].cpu(), merged[1])
+    if block_size:
+        assert torch.equal(got["kernel_zero"].cpu(), merged[2])
+    assert not torch.equal(got["kernel"].cpu(), qk)
+    # a fresh quantized layer without LoRA that loads the store answers like the LoRA layer,
+    # to within the quantisation of the merged kernel
+    cfg = layer.get_config()
+    assert cfg["lora_rank"] == rank and cfg["lora_alpha"] == alpha
+    plain = Dense(N, dtype=layer.dtype_policy.name, device=dev)
+    plain.build((None, K))
+    plain.load_own_variables(store)
+    y2 = plain(x)
+    assert max_rel_err(y2, y) <= (3e-2 if mode == "int8" else 0.25)
+    # loading into the LoRA layer itself zeroes the update (it is in the kernel now)
+    layer.load_own_variables(store)
+    assert float(layer.lora_kernel_a.value.abs().max()) == 0.0
+    assert float(layer.lora_kernel_b.value.abs().max()) == 0.0
+    assert torch.equal(bits(layer(x).cpu().contiguous()), bits(y2.cpu().contiguous()))
+
+
+@pytest.mark.parametrize("mode,block_size", [("int8", None), ("int4", None), ("int4", 64)])
+@pytest.mark.parametrize("equation,output_shape,input_shape", [
+    ("btd,dnh->btnh", (None, 4, 32), (3, 5, 256)), ("btnh,nhd->btd", (None, 256), (3, 5, 4, 64))])
+def test_einsum_dense_lora_on_quantized_layer_and_merge_on_save(dev, mode, block_size, equation, output_shape,
+                                                                input_shape):
+    # keras/src/layers/core/einsum_dense.py:327-385, :1109-1118 / :1251-1261, :1493-1623, :497-499
+    g = torch.Generator().manual_seed(29)
+    rank, alpha = 4, 2
+    layer = EinsumDense(equation, output_shape, bias_axes=None, dtype="float32", device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d))
+    layer.build(input_shape)
+    kernel_f = layer._kernel.value.cpu()
+    kshape = tuple(kernel_f.shape)
+    if mode == "int8":
+        layer.quantize("int8")
+        qk, ks, _ = ref.einsum_dense_quantize_int8(kernel_f, equation, len(input_shape))
+    else:
+        layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=block_size))
+        q4 = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), block_size)
+    layer.enable_lora(rank, lora_alpha=alpha)
+    assert tuple(layer.lora_kernel_a.shape) == kshape[:-1] + (rank,)
+    assert tuple(layer.lora_kernel_b.shape) == (rank, kshape[-1])
+    a = torch.randn(kshape[:-1] + (rank,), generator=g) * 0.05
+    b = torch.randn(rank, kshape[-1], generator=g) * 0.05
+    layer.lora_kernel_a.assign(a)
+    layer.lora_kernel_b.assign(b)
+    x = torch.rand(input_shape, generator=g) - 0.4
+    y = layer(x)
+    lora = (alpha / rank) * torch.matmul(torch.einsum(equation, x, a), b)
+    if mode == "int8":
+        want = ref.einsum_dense_int8_call(x, qk, ks, equation) + lora
+        merged = ref.einsum_dense_merged_lora_kernel("int8", qk, ks, a, b, alpha, rank, equation, len(input_shape))
+    else:
+        want = ref.einsum_dense_int4_call(x, q4, equation, block_size=block_size) + lora
+        merged = ref.einsum_dense_merged_lora_kernel("int4", None, None, a, b, alpha, rank, equation,
+                                                     len(input_shape), qk=q4, block_size=block_size)
+    assert max_rel_err(y, want) <= 1e-3
+    store = {}
+    layer.save_own_variables(store)
+    assert torch.equal(store["0"].cpu(), merged[0])
+    assert tuple(store["1"].shape) == tuple(merged[1].shape) and torch.equal(store["1"].cpu(), merged[1])
+    if block_size:
+        assert torch.equal(store["2"].cpu(), merged[2])
+    plain = EinsumDense(equation, output_shape, dtype=layer.dtype_policy.name, device=dev)
+    plain.build(input_shape)
+    plain.load_own_variables(store)
+    assert max_rel_err(plain(x), y) <= (3e-2 if mode == "int8" else 0.25)
+    layer.load_own_variables(store)
+    assert float(layer.lora_kernel_a.value.abs().max()) == 0.0 and float(layer.lora_kernel_b.value.abs().max()) == 0.0
+
+
 def test_non_default_g_idx_is_rejected(dev):
     # the reference looks the group of row k up in g_idx (quantizers.py:1659-1668); the fused kernels
     # take k // block_size, so a stored map that says anything else has to raise, not compute

@@ -254,6 +254,48 @@ def test_dense_int4_call_against_f64(block_size):
     assert (y - x @ kernel).pow(2).mean().item() < 2e-2
 
 
+# ---------------------------------------------------------------- LoRA merged on save
+@pytest.mark.parametrize("mode,block_size", [("int8", None), ("int4", None), ("int4", 32)])
+def test_merged_lora_kernel_invariants(mode, block_size):
+    g = torch.Generator().manual_seed(17)
+    K, N, rank, alpha = 96, 40, 4, 8.0
+    kernel = ref.glorot_uniform(K, N, generator=g)
+    if mode == "int8":
+        qk, ks = ref.dense_quantize_int8(kernel)
+        kw = dict()
+        dequant = lambda q, s, z: q.float() / s
+    else:
+        q4 = ref.dense_quantize_int4(kernel, block_size)
+        qk, ks = q4["kernel"], q4["kernel_scale"]
+        kw = dict(kernel_zero=q4["kernel_zero"], g_idx=q4["g_idx"], block_size=block_size, orig_output_dim=N)
+        if block_size:
+            dequant = lambda q, s, z: ref.dequantize_with_sz_map(ref.unpack_int4(q, N, axis=-1), s, z, q4["g_idx"], group_axis=0)
+        else:
+            dequant = lambda q, s, z: ref.unpack_int4(q, N, axis=-1).float() / s
+    a = torch.randn(K, rank, generator=g) * 0.05
+    zero_b = torch.zeros(rank, N)
+    # a zero update: quantising the de-quantised kernel again gives the same integers (every
+    # column / group of an abs-max quantised kernel holds an extreme of the range)
+    q0, s0, z0 = ref.dense_merged_lora_kernel(mode, qk, ks, a, zero_b, alpha, rank, **kw)
+    if not block_size:
+        assert torch.equal(q0, qk)
+        assert torch.allclose(s0, ks, rtol=1e-5, atol=0)
+        assert z0 is None
+    else:
+        # (grouped: the asymmetric re-quantisation need not hit the same integers, the values must)
+        assert (dequant(q0, s0, z0) - dequant(qk, ks, kw["kernel_zero"])).abs().max() <= 0.51 / s0.min()
+    # a real update: the saved kernel de-quantises to (old de-quantised kernel + update) within
+    # half a quantisation step of its own scales
+    b = torch.randn(rank, N, generator=g) * 0.05
+    q1, s1, z1 = ref.dense_merged_lora_kernel(mode, qk, ks, a, b, alpha, rank, **kw)
+    target = dequant(qk, ks, kw.get("kernel_zero")) + (alpha / rank) * (a @ b)
+    got = dequant(q1, s1, z1)
+    step = (1.0 / s1) if s1.dim() == 1 else (1.0 / s1).repeat_interleave(block_size, dim=0)[:K]
+    assert ((got - target).abs() <= 0.5001 * step + 1e-6).all()
+    assert q1.dtype == torch.int8 and tuple(q1.shape) == tuple(qk.shape)
+    assert not torch.equal(q1, qk)
+
+
 # ---------------------------------------------------------------- EinsumDense bookkeeping
 def test_einsum_info_hand_derived_rows():
     a = ref.einsum_quantization_info("btd,dnh->btnh", 3)
