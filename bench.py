@@ -78,11 +78,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
-    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,decode,cpu: run the headline "
+    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,decode,cpu: run the headline "
                     "step and only these further sections (for profiler runs); default: all")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
-    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "decode", "cpu"}
+    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "decode", "cpu"}
     if unknown:
         sys.exit(f"bench.py: unknown section(s) {sorted(unknown)}")
     want = (lambda name: not only or name in only)
@@ -351,6 +351,48 @@ def main():
             del graph
         del xg
 
+    # ------------------------------------------------------------------ int8 decode forward
+    # Dense int8 at decode sizes, K = N = 8192: quantizer + exact int8 matmul + bit-exact de-scale,
+    # one launch from the strip-linear copy of the int8 kernel (x above 16 K values: a quantizer
+    # launch first); 6 kernels of 64 MiB in rotation, each call a graph node
+    gemv8 = []
+    if want("gemv8"):
+        n_rot8 = 6
+        w8 = [torch.randint(-127, 128, (Kg, Ng), dtype=torch.int8, device=dev) for _ in range(n_rot8)]
+        s8 = [kops.int8_strip_copy(w) for w in w8]
+        del w8
+        ks8 = (torch.rand(Ng, device=dev) * 50 + 50).to(torch.bfloat16)
+        for M8 in (1, 8, 16):
+            x8 = torch.randn(M8, Kg, device=dev).to(torch.bfloat16)
+            reps = 4 * n_rot8
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                for i in range(n_rot8):
+                    kops.int8_dense_strip(x8, s8[i], Ng, ks8)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(reps):
+                        kops.int8_dense_strip(x8, s8[i % n_rot8], Ng, ks8)
+            torch.cuda.synchronize()
+            spin_up(torch, graph.replay, 0.05)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / (3 * reps) * 1e3
+            nbytes = Kg * Ng + 2 * M8 * Kg + 2 * M8 * Ng + 2 * Ng
+            gbs = nbytes / (us * 1e-6) / 1e9
+            gemv8.append({"M": M8, "K": Kg, "N": Ng, "kernel": "gemv_w8s (strip-linear copy)"
+                          + ("" if M8 * Kg <= kops.INT8_STRIP_FUSED_QUANTIZER_MAX else " + quantize_rows_vec"),
+                          "us_per_call": round(us, 2), "algorithmic_bytes": nbytes,
+                          "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                                       "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}})
+            del graph, x8
+        del s8
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ end-to-end decode
     # Llama-style 32-layer decoder (d_model 4096, 32 heads, SwiGLU 14336, vocab 32000), every
     # weight matrix int4 (grouped, block 128) with synthetic values written on the device;
@@ -450,6 +492,7 @@ def main():
         "int8_gemm_sweep": sweep,
         "einsum_int8": einsum,
         "int4_gemv": gemv,
+        "int8_decode_dense": gemv8,
         "llama_decode_int4": decode,
         "llama_decode_int8": decode_int8,
         "cpu_baseline": cpu,
