@@ -464,6 +464,18 @@ int k3q_decode_attention(const void* q, const void* k, const void* v, int dtype,
                          int64_t head_dim, int64_t max_len, const void* cos_table, const void* sin_table,
                          const int64_t* pos, void* k_cache, void* v_cache, void* out, void* stream);
 
+/*
+ * Two more pieces of the decoder harness's glue (no counterpart in the quantized layers; they
+ * stand for `rms_norm` and `silu(gate) * up` between the Dense calls of a decoder block), bfloat16:
+ * k3q_rmsnorm: y[r, :] = bf16(x[r, :] * rsqrt(mean(x[r, :]^2) + epsilon) * weight[:]), float32
+ * arithmetic and one rounding; dim % 8 == 0, dim <= 8192; row strides in elements (% 8 == 0).
+ * k3q_silu_mul: y = bf16(bf16(g / (1 + exp(-g))) * u) element by element, rows given by strides.
+ */
+int k3q_rmsnorm(const void* x, const void* weight, int dtype, int64_t rows, int64_t dim, int64_t x_row_stride,
+                float epsilon, void* y, int64_t y_row_stride, void* stream);
+int k3q_silu_mul(const void* gate, const void* up, int dtype, int64_t rows, int64_t dim, int64_t gate_row_stride,
+                 int64_t up_row_stride, void* y, int64_t y_row_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

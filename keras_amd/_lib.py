@@ -111,6 +111,8 @@ SIGNATURES = {
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _f32, _f32, _f32, _ptr, _ptr],
     ),
     "k3q_gemm_i8_w8s": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
+    "k3q_rmsnorm": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _f32, _ptr, _i64, _ptr]),
+    "k3q_silu_mul": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "k3q_decode_attention": (
         _int,
         [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr],

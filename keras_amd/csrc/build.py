@@ -27,6 +27,7 @@ SOURCES = [
     "k3q_embedding.hip",
     "k3q_decode_attn.hip",
     "k3q_gemv_w8s.hip",
+    "k3q_glue.hip",
 ]
 
 FLAGS = [

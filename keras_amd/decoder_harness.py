@@ -34,7 +34,16 @@ class RMSNorm(Layer):
         self.built = True
 
     def call(self, x, training=None):
-        return torch.nn.functional.rms_norm(x, (self.dim,), self.read(self.scale), self.epsilon)
+        w = self.read(self.scale)
+        if x.numel() <= (64 << 10) and kops.rmsnorm_supported(x, w):
+            return kops.rmsnorm(x, w, self.epsilon)  # decode sizes: one short launch
+        return torch.nn.functional.rms_norm(x, (self.dim,), w, self.epsilon)
+
+
+def _silu_mul(gate, up):
+    if gate.numel() <= (256 << 10) and kops.silu_mul_supported(gate, up):
+        return kops.silu_mul(gate, up)
+    return torch.nn.functional.silu(gate) * up
 
 
 def rope_tables(head_dim, max_len, device, base=10000.0, dtype=torch.float32):
@@ -95,7 +104,7 @@ class DecoderBlock(Layer):
             x = call_add(self.attn_out, a, x)
             h = self.ffn_norm(x)
             gate, up = call_together((self.gate, self.up), h)
-            return call_add(self.down, torch.nn.functional.silu(gate) * up, x)
+            return call_add(self.down, _silu_mul(gate, up), x)
         # one rotation over the query and key heads together (half the elementwise launches)
         qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
         q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
@@ -108,7 +117,7 @@ class DecoderBlock(Layer):
         x = call_add(self.attn_out, a.transpose(1, 2), x)
         h = self.ffn_norm(x)
         gate, up = call_together((self.gate, self.up), h)
-        return call_add(self.down, torch.nn.functional.silu(gate) * up, x)
+        return call_add(self.down, _silu_mul(gate, up), x)
 
 
 class LlamaStyleDecoder(Model):

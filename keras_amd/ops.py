@@ -803,3 +803,51 @@ def decode_attention(q, k, v, cos_table, sin_table, pos, cache_k, cache_v):
                                   _lib.stream_ptr(q.device))
     _lib.check(rc, "k3q_decode_attention")
     return out
+
+
+def _rows_view(t):
+    """[rows, dim] view of a tensor whose last axis is contiguous and whose leading axes collapse
+    into one stride (else a contiguous copy): (tensor, rows, dim, row stride in elements)."""
+    dim = t.shape[-1]
+    t2 = t.reshape(-1, dim) if t.dim() != 2 else t
+    if t2.stride(-1) != 1 or (t2.shape[0] > 1 and t2.stride(0) % 8):
+        t2 = t2.contiguous()
+    return t2, t2.shape[0], dim, (t2.stride(0) if t2.shape[0] > 1 else dim)
+
+
+def rmsnorm_supported(x, weight):
+    return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and x.shape[-1] % 8 == 0 and x.shape[-1] <= 8192 and weight.numel() == x.shape[-1])
+
+
+def rmsnorm(x, weight, epsilon):
+    """`rms_norm(x, weight, epsilon)` over the last axis, bfloat16, one short launch (the decoder
+    harness's normalisation between the quantized layers)."""
+    _lib.require_device(x, weight)
+    lib = _lib.load()
+    x2, rows, dim, xs = _rows_view(x)
+    w = weight if weight.is_contiguous() else weight.contiguous()
+    y = torch.empty((rows, dim), dtype=x.dtype, device=x.device)
+    rc = lib.k3q_rmsnorm(_lib.ptr(x2), _lib.ptr(w), _lib.dtype_code(x.dtype), rows, dim, xs, float(epsilon),
+                         _lib.ptr(y), dim, _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_rmsnorm")
+    return y.reshape(x.shape)
+
+
+def silu_mul_supported(gate, up):
+    return (gate.is_cuda and gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
+            and gate.shape == up.shape and gate.shape[-1] % 8 == 0)
+
+
+def silu_mul(gate, up):
+    """`silu(gate) * up`, bfloat16, one launch; the operands may be column slices of a wider
+    tensor (rows given by a stride)."""
+    _lib.require_device(gate, up)
+    lib = _lib.load()
+    g2, rows, dim, gs = _rows_view(gate)
+    u2, _, _, us = _rows_view(up)
+    y = torch.empty((rows, dim), dtype=gate.dtype, device=gate.device)
+    rc = lib.k3q_silu_mul(_lib.ptr(g2), _lib.ptr(u2), _lib.dtype_code(gate.dtype), rows, dim, gs, us,
+                          _lib.ptr(y), dim, _lib.stream_ptr(gate.device))
+    _lib.check(rc, "k3q_silu_mul")
+    return y.reshape(gate.shape)

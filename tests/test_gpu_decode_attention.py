@@ -113,3 +113,40 @@ def test_decode_attention_rejects(dev):
         kops.decode_attention(q.float(), q.float(), q.float(), cos_t, sin_t, pos,
                               z(1, 2, 16, hd), z(1, 2, 16, hd))
     assert not kops.decode_attention_supported(z(1, 1, 2, 64), z(1, 2, 16, 64))
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (8, 4096), (3, 128), (2, 8192), (5, 2056)])
+def test_rmsnorm_matches_torch(dev, rows, dim):
+    g = torch.Generator().manual_seed(rows + dim)
+    x = (torch.randn(rows, 1, dim, generator=g) * 3).to(torch.bfloat16).to(dev)
+    w = (torch.rand(dim, generator=g) + 0.5).to(torch.bfloat16).to(dev)
+    assert kops.rmsnorm_supported(x, w)
+    got = kops.rmsnorm(x, w, 1e-6)
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    exact = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()
+    want = torch.nn.functional.rms_norm(x, (dim,), w, 1e-6)
+    # one rounding of the float32 result: within one bfloat16 ulp of the exact value, and as
+    # close to it as torch's own kernel
+    rel = lambda a: ((a.double() - exact).abs() / exact.abs().clamp_min(1e-3)).max().item()
+    assert rel(got) <= 2 ** -8 and rel(got) <= rel(want) + 2 ** -9
+    # rows given by a stride (a column slice of a wider tensor)
+    wide = torch.randn(rows, dim + 64, generator=g).to(torch.bfloat16).to(dev)
+    assert torch.equal(kops.rmsnorm(wide[:, :dim], w, 1e-6).view(torch.int16),
+                       kops.rmsnorm(wide[:, :dim].contiguous(), w, 1e-6).view(torch.int16))
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 14336), (8, 14336), (3, 64), (2, 11008)])
+def test_silu_mul_matches_torch(dev, rows, dim):
+    g = torch.Generator().manual_seed(rows * 7 + dim)
+    both = (torch.randn(rows, 2 * dim, generator=g) * 2).to(torch.bfloat16).to(dev)
+    gate, up = both[:, :dim], both[:, dim:]          # column slices: rows by stride
+    assert kops.silu_mul_supported(gate, up)
+    got = kops.silu_mul(gate, up)
+    want = torch.nn.functional.silu(gate) * up
+    assert got.shape == want.shape and got.dtype == torch.bfloat16
+    # the same two roundings; exp may differ in its last float32 bit, which moves a rounding
+    # of silu(g) by one bfloat16 ulp on a few elements at most
+    diff = (got.float() - want.float()).abs()
+    assert (diff <= want.float().abs() * 2 ** -7 + 1e-30).all()
+    assert (diff > 0).float().mean().item() < 0.01
+    assert torch.equal(kops.silu_mul(gate.contiguous(), up.contiguous()).view(torch.int16), got.view(torch.int16))
