@@ -64,31 +64,49 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
     __syncthreads();  // the new rows are written (and acknowledged) before any wave reads the cache
 
     // ---- scores ----
+    // Blocks of 4 cache rows go to the waves round-robin; a wave asks for kU blocks of keys at once
+    // and -- for its first kU blocks -- for the value rows too, before the softmax, so that the
+    // weighted sum below finds them in registers (the value rows do not depend on the scores).
     const int n = pos + 1;
     const int nblk = (n + 3) >> 2;
     const int sub = lane >> 4, dl = (lane & 15) * 8;
+    constexpr int kU = 8;
     float qv[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) qv[e] = qs[dl + e];
     float mx = -INFINITY;
-#pragma unroll 4
-    for (int kb = wave; kb < nblk; kb += kAW) {
-        const int j = 4 * kb + sub;
-        const int jj = j < n ? j : pos;
-        const v4u kk = *(const v4u*)(p.kc + (row0 + jj) * kHd + dl);
-        float dot = 0.f;
+    v4u vv0[kU];
+    for (int kb0 = wave; kb0 < nblk; kb0 += kAW * kU) {
+        v4u kk[kU];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            dot += qv[2 * e] * __uint_as_float(kk[e] << 16);
-            dot += qv[2 * e + 1] * __uint_as_float(kk[e] & 0xffff0000u);
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (kb0 + u * kAW) + sub;
+            kk[u] = *(const v4u*)(p.kc + (row0 + (j < n ? j : pos)) * kHd + dl);
         }
-        dot += __shfl_xor(dot, 1, kWave);
-        dot += __shfl_xor(dot, 2, kWave);
-        dot += __shfl_xor(dot, 4, kWave);
-        dot += __shfl_xor(dot, 8, kWave);
-        if (j < n) {
-            mx = fmaxf(mx, dot);
-            if ((lane & 15) == 0) sc[j] = dot;
+        if (kb0 == wave) {
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                const int j = 4 * (kb0 + u * kAW) + sub;
+                vv0[u] = *(const v4u*)(p.vc + (row0 + (j < n ? j : pos)) * kHd + dl);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (kb0 + u * kAW) + sub;
+            float dot = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                dot += qv[2 * e] * __uint_as_float(kk[u][e] << 16);
+                dot += qv[2 * e + 1] * __uint_as_float(kk[u][e] & 0xffff0000u);
+            }
+            dot += __shfl_xor(dot, 1, kWave);
+            dot += __shfl_xor(dot, 2, kWave);
+            dot += __shfl_xor(dot, 4, kWave);
+            dot += __shfl_xor(dot, 8, kWave);
+            if (j < n) {
+                mx = fmaxf(mx, dot);
+                if ((lane & 15) == 0) sc[j] = dot;
+            }
         }
     }
 #pragma unroll
@@ -117,16 +135,31 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-#pragma unroll 4
-    for (int kb = wave; kb < nblk; kb += kAW) {
-        const int j = 4 * kb + sub;
-        const int jj = j < n ? j : pos;
-        const v4u vv = *(const v4u*)(p.vc + (row0 + jj) * kHd + dl);
-        const float w = j < n ? sc[j] : 0.f;
+    auto add_row = [&](const v4u& vv, const float w) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             acc[2 * e] += w * __uint_as_float(vv[e] << 16);
             acc[2 * e + 1] += w * __uint_as_float(vv[e] & 0xffff0000u);
+        }
+    };
+    if (wave < nblk) {
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (wave + u * kAW) + sub;
+            add_row(vv0[u], j < n ? sc[j] : 0.f);
+        }
+    }
+    for (int kb0 = wave + kAW * kU; kb0 < nblk; kb0 += kAW * kU) {
+        v4u vv[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (kb0 + u * kAW) + sub;
+            vv[u] = *(const v4u*)(p.vc + (row0 + (j < n ? j : pos)) * kHd + dl);
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (kb0 + u * kAW) + sub;
+            add_row(vv[u], j < n ? sc[j] : 0.f);
         }
     }
 #pragma unroll
