@@ -447,6 +447,23 @@ int k3q_dense_i8_w8s(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N
 int k3q_gemm_i8_w8s(const int8_t* a, const void* a_scale, int scale_dtype, int64_t M, int64_t K, int64_t N,
                     const void* shadow, const void* kernel_scale, const void* bias, int64_t bias_stride,
                     void* y, void* stream);
+/*
+ * Several int8 layers against ONE x in one launch (the query / key / value projections of an
+ * attention block, gate / up of an MLP): each result is what k3q_dense_i8_w8s (a == NULL: the rows
+ * are quantised in the kernel) or k3q_gemm_i8_w8s (a, a_scale: rows already quantised) gives for
+ * that problem alone, bit for bit; problems whose launch plans differ run in launches of their own.
+ * bias: N values or NULL.  No counterpart in the reference (its layers each run their own matmul).
+ */
+typedef struct {
+    int64_t N;
+    const void* shadow;       /* k3q_w8s_pack of the layer's [K, N] kernel */
+    const void* kernel_scale; /* bfloat16 [N] */
+    const void* bias;         /* bfloat16 [N] or NULL */
+    void* y;                  /* bfloat16 [M, N] */
+} k3q_w8s_problem;
+int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* a, const void* a_scale, int64_t M, int64_t K,
+                           int count, const k3q_w8s_problem* problems, float epsilon, float range_lo,
+                           float range_hi, void* stream);
 
 /*
  * One new position of causal self-attention against a key / value cache (the decoder

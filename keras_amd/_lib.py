@@ -111,6 +111,8 @@ SIGNATURES = {
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _f32, _f32, _f32, _ptr, _ptr],
     ),
     "k3q_gemm_i8_w8s": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
+    "k3q_dense_i8_w8s_multi": (
+        _int, [_ptr, _int, _ptr, _ptr, _i64, _i64, _int, _ptr, _f32, _f32, _f32, _ptr]),
     "k3q_rmsnorm": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _f32, _ptr, _i64, _ptr]),
     "k3q_silu_mul": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "k3q_decode_attention": (
@@ -147,6 +149,13 @@ class GemvW4sProblem(ctypes.Structure):
 
     _fields_ = [("N", ctypes.c_int64), ("shadow", ctypes.c_void_p), ("scale", ctypes.c_void_p),
                 ("gparams", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p)]
+
+
+class W8sProblem(ctypes.Structure):
+    """`k3q_w8s_problem` of include/k3q.h."""
+
+    _fields_ = [("N", ctypes.c_int64), ("shadow", ctypes.c_void_p), ("kernel_scale", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p)]
 
 
 _lib = None

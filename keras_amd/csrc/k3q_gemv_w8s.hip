@@ -63,7 +63,7 @@ __device__ __forceinline__ float descale_exact_bf16(int acc, float sa, float sb,
 // kNP: 16-byte pieces of x a thread keeps in registers between the row maxima and the
 // quantisation (0: it reads them twice); -1: the rows arrive quantised (p.xq, p.xs).
 template <int kSW, int kD, int kNP>
-__global__ __launch_bounds__(kT) void gemv_w8s(W8sParams p) {
+__device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int block, const int n_blocks) {
     extern __shared__ __attribute__((aligned(16))) char w8s_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int q = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -86,8 +86,8 @@ __global__ __launch_bounds__(kT) void gemv_w8s(W8sParams p) {
 
     // ---- the weight stream: the load cursor (group, first unit of a block) runs one block of
     // kD units ahead of the consumer, across group boundaries ----
-    const int stride = gridDim.x;
-    int lg = blockIdx.x, lu = u_begin;
+    const int stride = n_blocks;
+    int lg = block, lu = u_begin;
     const int last_group = p.groups - 1;
     const v4i* nb[kSW];  // this lane's pieces of the block at the cursor, unit by unit 64 entries apart
     auto at_cursor = [&]() {
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kT) void gemv_w8s(W8sParams p) {
     const char* xrow = xs + (row_live ? i16 : 0) * pitch + 16 * g;
     const bool has_bias = p.bias != nullptr;
     int turn = 0;
-    for (int grp = blockIdx.x; grp < p.groups; grp += stride, ++turn) {
+    for (int grp = block; grp < p.groups; grp += stride, ++turn) {
         // epilogue operands of this group, asked for before the group's units (loads return in
         // order: asked for late they would wait for the next group's first units)
         const int n0 = grp * kSW * 16;
@@ -296,6 +296,28 @@ __global__ __launch_bounds__(kT) void gemv_w8s(W8sParams p) {
     }
 }
 
+template <int kSW, int kD, int kNP>
+__global__ __launch_bounds__(kT) void gemv_w8s(W8sParams p) {
+    gemv_w8s_body<kSW, kD, kNP>(p, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// Up to kMaxProblems8 kernels against one x in one launch (the query / key / value projections of
+// an attention block, gate / up of an MLP): workgroups [first[i], first[i+1]) work on problem i,
+// every workgroup stages (and, fused, quantises) x as in the single launch.
+constexpr int kMaxProblems8 = 4;
+struct W8sMulti {
+    W8sParams p[kMaxProblems8];
+    int first[kMaxProblems8 + 1];
+    int count;
+};
+template <int kSW, int kD, int kNP>
+__global__ __launch_bounds__(kT) void gemv_w8s_multi(W8sMulti mp) {
+    const int bx = blockIdx.x;
+    int i = 0;
+    while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
+    gemv_w8s_body<kSW, kD, kNP>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
+}
+
 // One thread per 16-byte lane entry of the copy.  w: the stored int8 kernel, row-major [K, N].
 __global__ __launch_bounds__(256) void w8s_pack(const int8_t* __restrict__ w, v4u* __restrict__ out, int64_t K,
                                                int64_t N, int64_t strips) {
@@ -344,6 +366,7 @@ W8sPlan w8s_plan(int64_t M, int64_t K, int64_t N) {
 }
 
 typedef void (*W8sKernel)(W8sParams);
+typedef void (*W8sMultiKernel)(W8sMulti);
 
 template <int kSW, int kD>
 W8sKernel pick_np8(int np) {
@@ -354,6 +377,22 @@ W8sKernel pick_np8(int np) {
         case 16: return gemv_w8s<kSW, kD, 16>;
         default: return gemv_w8s<kSW, kD, 0>;
     }
+}
+
+template <int kSW, int kD>
+W8sMultiKernel pick_np8_multi(int np) {
+    switch (np) {
+        case -1: return gemv_w8s_multi<kSW, kD, -1>;
+        case 1: return gemv_w8s_multi<kSW, kD, 1>;
+        case 4: return gemv_w8s_multi<kSW, kD, 4>;
+        case 16: return gemv_w8s_multi<kSW, kD, 16>;
+        default: return gemv_w8s_multi<kSW, kD, 0>;
+    }
+}
+
+W8sMultiKernel pick_kernel8_multi(const W8sPlan& pl) {
+    if (pl.sw == 2) return pl.d == 4 ? pick_np8_multi<2, 4>(pl.np) : pick_np8_multi<2, 2>(pl.np);
+    return pl.d == 4 ? pick_np8_multi<1, 4>(pl.np) : pick_np8_multi<1, 2>(pl.np);
 }
 
 W8sKernel pick_kernel8(const W8sPlan& pl) {
@@ -384,20 +423,16 @@ extern "C" int k3q_w8s_pack(const int8_t* w, int64_t K, int64_t N, void* shadow,
 extern "C" int k3q_dense_i8_w8s_supported(int64_t M, int64_t K, int64_t N) { return w8s_plan(M, K, N).ok ? 1 : 0; }
 
 namespace {
-int launch_w8s(const void* x, const int8_t* xq, const void* xs, int64_t M, int64_t K, int64_t N,
-               const void* shadow, const void* kernel_scale, const void* bias, int64_t bias_stride,
-               float epsilon, float range_lo, float range_hi, void* y, hipStream_t stream) {
-    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
-    if (M == 0) return K3Q_OK;
+// checks the operands of one problem and fills its kernel parameters
+int fill_params8(W8sParams& p, const W8sPlan& pl, const void* x, const int8_t* xq, const void* xs, int64_t M,
+                 int64_t K, int64_t N, const void* shadow, const void* kernel_scale, const void* bias,
+                 int64_t bias_stride, float epsilon, float range_lo, float range_hi, void* y) {
     if (bias_stride != 0 && bias_stride != N) return K3Q_ERR_SHAPE;
-    W8sPlan pl = w8s_plan(M, K, N);
-    if (!pl.ok) return K3Q_ERR_SHAPE;
     const bool quantised = xq != nullptr;
     if (!(quantised ? (const void*)xs : x) || !shadow || !kernel_scale || !y) return K3Q_ERR_NULL;
     if (!aligned_to(quantised ? (const void*)xq : x, 16) || !aligned_to(shadow, 16) || !aligned_to(y, 2) ||
         !aligned_to(kernel_scale, 2) || (bias && !aligned_to(bias, 2)) || (xs && !aligned_to(xs, 2)))
         return K3Q_ERR_ALIGN;
-    W8sParams p;
     p.x = (const uint16_t*)x;
     p.xq = xq;
     p.xs = (const uint16_t*)xs;
@@ -416,19 +451,36 @@ int launch_w8s(const void* x, const int8_t* xq, const void* xs, int64_t M, int64
     p.eps = host_round_bf16(epsilon);  // torch rounds the epsilon operand to the tensor dtype before the add
     p.qlo = range_lo;
     p.qhi = range_hi;
-    if (quantised) pl.np = -1;
-    const W8sKernel kernel = pick_kernel8(pl);
-    {
-        static std::mutex mu;
-        static std::set<const void*> raised;
-        std::lock_guard<std::mutex> lock(mu);
-        if (!raised.count((const void*)kernel)) {
-            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
-                hipSuccess)
-                return K3Q_ERR_LAUNCH;
-            raised.insert((const void*)kernel);
-        }
+    return K3Q_OK;
+}
+
+// more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+int raise_lds(const void* kernel) {
+    static std::mutex mu;
+    static std::set<const void*> raised;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!raised.count(kernel)) {
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return K3Q_ERR_LAUNCH;
+        raised.insert(kernel);
     }
+    return K3Q_OK;
+}
+
+int launch_w8s(const void* x, const int8_t* xq, const void* xs, int64_t M, int64_t K, int64_t N,
+               const void* shadow, const void* kernel_scale, const void* bias, int64_t bias_stride,
+               float epsilon, float range_lo, float range_hi, void* y, hipStream_t stream) {
+    if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
+    if (M == 0) return K3Q_OK;
+    W8sPlan pl = w8s_plan(M, K, N);
+    if (!pl.ok) return K3Q_ERR_SHAPE;
+    W8sParams p;
+    int rc = fill_params8(p, pl, x, xq, xs, M, K, N, shadow, kernel_scale, bias, bias_stride, epsilon, range_lo,
+                          range_hi, y);
+    if (rc != K3Q_OK) return rc;
+    if (xq) pl.np = -1;
+    const W8sKernel kernel = pick_kernel8(pl);
+    if ((rc = raise_lds((const void*)kernel)) != K3Q_OK) return rc;
     kernel<<<(unsigned)pl.blocks, kT, pl.lds, stream>>>(p);
     return launch_status();
 }
@@ -450,4 +502,73 @@ extern "C" int k3q_gemm_i8_w8s(const int8_t* a, const void* a_scale, int scale_d
     if (M > 0 && !a) return K3Q_ERR_NULL;
     return launch_w8s(nullptr, a, a_scale, M, K, N, shadow, kernel_scale, bias, bias_stride, 0.f, -127.f, 127.f,
                       y, (hipStream_t)stream);
+}
+
+extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* a, const void* a_scale, int64_t M,
+                                      int64_t K, int count, const k3q_w8s_problem* problems, float epsilon,
+                                      float range_lo, float range_hi, void* stream) {
+    if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
+    if (count < 0 || M < 0 || K <= 0) return K3Q_ERR_SHAPE;
+    if (!(range_lo >= -128.f && range_hi <= 127.f && range_lo < range_hi)) return K3Q_ERR_SHAPE;
+    if (count == 0 || M == 0) return K3Q_OK;
+    if (!problems) return K3Q_ERR_NULL;
+    int at = 0;
+    while (at < count) {
+        // problems whose plans agree share a launch, up to kMaxProblems8 at a time
+        W8sMulti mp{};
+        W8sPlan pl0{};
+        int64_t groups[kMaxProblems8], total = 0;
+        size_t lds_two = 0, lds_red_one = 0;
+        int n = 0;
+        for (; at + n < count && n < kMaxProblems8; ++n) {
+            const k3q_w8s_problem& q = problems[at + n];
+            if (q.N <= 0) return K3Q_ERR_SHAPE;
+            const W8sPlan pl = w8s_plan(M, K, q.N);
+            if (!pl.ok) return K3Q_ERR_SHAPE;
+            if (n == 0) {
+                pl0 = pl;
+                // workgroups of a shared launch may take turns even where a problem alone would not
+                lds_red_one = (size_t)kQ * pl.sw * ((M + 3) / 4) * 16 * 4 * 4;
+                lds_two = (size_t)((M * (K + 16) + 255) & ~255) + 2 * kMaxRows8 * 4 + 2 * lds_red_one;
+            } else if (pl.sw != pl0.sw || pl.d != pl0.d) {
+                break;
+            }
+            const int rc = fill_params8(mp.p[n], pl, x, a, a_scale, M, K, q.N, q.shadow, q.kernel_scale, q.bias, 0,
+                                        epsilon, range_lo, range_hi, q.y);
+            if (rc != K3Q_OK) return rc;
+            groups[n] = pl.groups;
+            total += pl.groups;
+        }
+        // the launch as a whole is cut for the chip: about kResident8 workgroups, each problem its share;
+        // workgroups that take turns need both reduction buffers, and where those do not fit beside x
+        // the first problem goes alone, with its own plan
+        int64_t turns = (total + kResident8 - 1) / kResident8;
+        size_t lds = turns > 1 ? lds_two : lds_two - lds_red_one;
+        if (lds > (size_t)160 * 1024) {
+            n = 1;
+            turns = (groups[0] + kResident8 - 1) / kResident8;
+            lds = pl0.lds;
+        }
+        int next_block = 0;
+        for (int i = 0; i < n; ++i) {
+            mp.first[i] = next_block;
+            next_block += (int)((groups[i] + turns - 1) / turns);
+        }
+        mp.first[n] = next_block;
+        mp.count = n;
+        if (a) pl0.np = -1;
+        int rc;
+        if (n == 1) {
+            const W8sKernel kernel = pick_kernel8(pl0);
+            if ((rc = raise_lds((const void*)kernel)) != K3Q_OK) return rc;
+            kernel<<<(unsigned)next_block, kT, lds, (hipStream_t)stream>>>(mp.p[0]);
+        } else {
+            const W8sMultiKernel kernel = pick_kernel8_multi(pl0);
+            if ((rc = raise_lds((const void*)kernel)) != K3Q_OK) return rc;
+            kernel<<<(unsigned)next_block, kT, lds, (hipStream_t)stream>>>(mp);
+        }
+        if ((rc = launch_status()) != K3Q_OK) return rc;
+        at += n;
+    }
+    return K3Q_OK;
 }

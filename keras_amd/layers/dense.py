@@ -488,6 +488,32 @@ class Dense(Layer):
     def _rows_of(self, inputs):
         return inputs.numel() // inputs.shape[-1]
 
+    def _int8_together_spec(self, inputs):
+        """What `call_together` needs to run this layer's int8 forward in a launch shared with other
+        layers (decode sizes, the strip-linear copy): rows, quantizer settings, operands, and the
+        step from the [M, N] result to the layer's output.  None when the layer's forward is
+        anything else."""
+        if (not self.built or self.quantization_mode != "int8" or self.lora_enabled
+                or self.exact_epilogue is False):
+            return None
+        x2 = inputs.reshape(-1, inputs.shape[-1])
+        if not int8_strip_route(self.inputs_quantizer, x2, self.units):
+            return None
+        bias = self._call_bias()
+        if bias is not None and bias.numel() != self.units:
+            return None
+        lead = inputs.shape[:-1]
+
+        def finish(y2):
+            y = y2.reshape(*lead, self.units)
+            return self.activation(y) if self.activation is not None else y
+
+        q = self.inputs_quantizer
+        return dict(x2=x2, settings=(float(q.epsilon), tuple(float(v) for v in q.value_range)), quantizer=q,
+                    kernel=dict(shadow=self._cached("w8s", self._kernel, kops.int8_strip_copy), units=self.units,
+                                kernel_scale=self._read_cached("kernel_scale", self.kernel_scale), bias=bias),
+                    finish=finish)
+
     def _int4_together_spec(self, inputs):
         """What `call_together` needs to run this layer's weight-only int4 forward in a launch
         shared with other layers: the [M, K] rows, the kernel's operands and the step that

@@ -810,6 +810,36 @@ class EinsumDense(Layer):
         )
         return self._finish(y2, free_shape, gv, fused)
 
+    def _int8_together_spec(self, inputs):
+        """As Dense._int8_together_spec, for GEMM-shaped equations."""
+        if (not self.built or self.quantization_mode != "int8" or self.lora_enabled
+                or self.exact_epilogue is False or getattr(self, "_gemm", None) is None):
+            return None
+        gv = self._gemm_view()
+        x2, free_shape = self._input_rows(inputs, gv)
+        cd = to_torch_dtype(self.compute_dtype)
+
+        def kernel_matrix(t):
+            k2 = t if gv.k_is_view else t.permute(gv.k_perm)
+            return k2.reshape(x2.shape[1], -1).contiguous()
+
+        n = 1
+        for c in gv.kept:
+            n *= self.full_output_shape_of(c)
+        if not int8_strip_route(self.inputs_quantizer, x2, n):
+            return None
+        bias, fused = self._fusable_bias(gv, n)
+        if bias is not None and bias.numel() != n:
+            return None
+        q = self.inputs_quantizer
+        return dict(x2=x2, settings=(float(q.epsilon), tuple(float(v) for v in q.value_range)), quantizer=q,
+                    kernel=dict(shadow=self._cached("w8s", self._kernel,
+                                                    lambda t: kops.int8_strip_copy(kernel_matrix(t))),
+                                units=n, bias=bias,
+                                kernel_scale=self._cached("kernel_scale", self.kernel_scale,
+                                                          lambda t: t.to(cd).reshape(-1).contiguous())),
+                    finish=lambda y2: self._finish(y2, free_shape, gv, fused))
+
     def _int4_together_spec(self, inputs):
         """As Dense._int4_together_spec, for equations whose input rows and stored kernel are
         the GEMM's operands as they lie (e.g. "btd,dnh->btnh")."""

@@ -82,6 +82,23 @@ def _call_together(layers, inputs):
     x = x.contiguous()
     # (from here on the layers are handed x: moved and cast once, and the same tensor for all,
     # which is what lets them share its quantised rows)
+    # int8 layers at decode sizes that quantise their input alike: one launch from their strip copies
+    specs8 = []
+    for layer in layers:
+        make = getattr(layer, "_int8_together_spec", None)
+        spec = make(x) if make is not None else None
+        if spec is None:
+            break
+        specs8.append(spec)
+    if (len(specs8) == len(layers)
+            and all(s["x2"].shape == specs8[0]["x2"].shape and s["x2"].data_ptr() == specs8[0]["x2"].data_ptr()
+                    and s["x2"].stride() == specs8[0]["x2"].stride() and s["settings"] == specs8[0]["settings"]
+                    for s in specs8)):
+        eps, rng = specs8[0]["settings"]
+        quantizer = specs8[0]["quantizer"]
+        outs = kops.int8_dense_strip_multi(specs8[0]["x2"], [s["kernel"] for s in specs8], epsilon=eps,
+                                           value_range=rng, quantize=lambda rows: quantize_rows(quantizer, rows))
+        return [s["finish"](y) for s, y in zip(specs8, outs)]
     specs = []
     for layer in layers:
         make = getattr(layer, "_int4_together_spec", None)

@@ -763,6 +763,56 @@ def int8_dense_strip(x, shadow, units, kernel_scale, bias=None, epsilon=1e-7, va
     return y.reshape(*lead, N)
 
 
+def int8_dense_strip_multi(x, kernels, epsilon=1e-7, value_range=(-127, 127), quantize=None):
+    """`[int8_dense_strip(x, k) for k in kernels]` for layers that share `x[..., K]` (up to 16
+    bfloat16 rows) and quantise it alike: one launch for those whose launch plans agree, the same
+    bits as the separate calls.  kernels: dicts with `shadow`, `units`, `kernel_scale` and
+    optionally `bias` [N]."""
+    lib = _lib.load()
+    K = int(x.shape[-1])
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    if x.dtype != torch.bfloat16:
+        raise TypeError("the strip route computes in bfloat16")
+    problems = (_lib.W8sProblem * len(kernels))()
+    outs, keep = [], []
+    for i, k in enumerate(kernels):
+        N = int(k["units"])
+        bias, ks = k.get("bias"), k["kernel_scale"]
+        _lib.require_device(x, k["shadow"], ks, bias)
+        if not lib.k3q_dense_i8_w8s_supported(M, K, N):
+            raise ValueError(f"int8_dense_strip_multi does not take M={M}, K={K}, N={N}")
+        if k["shadow"].dtype != torch.uint8 or k["shadow"].numel() != lib.k3q_w8s_shadow_bytes(K, N):
+            raise ValueError("shadow is not int8_strip_copy(kernel) of this [K, N]")
+        if ks.dtype != torch.bfloat16 or ks.numel() != N:
+            raise ValueError(f"kernel_scale must hold {N} bfloat16 values")
+        if bias is not None and (bias.numel() != N or bias.dtype != torch.bfloat16):
+            raise ValueError(f"bias must hold {N} bfloat16 values")
+        ks = ks if ks.is_contiguous() else ks.contiguous()
+        keep.append(ks)
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        outs.append(y)
+        problems[i] = _lib.W8sProblem(N, k["shadow"].data_ptr(), ks.data_ptr(),
+                                      bias.data_ptr() if bias is not None else None, y.data_ptr())
+    q = s = None
+    if M * K > INT8_STRIP_FUSED_QUANTIZER_MAX:
+        if quantize is None:
+            from keras_amd import quantizers
+
+            q, s = quantizers.abs_max_quantize(x2, axis=-1, value_range=value_range, epsilon=epsilon)
+        else:
+            q, s = quantize(x2)
+        if s.dtype != torch.bfloat16:
+            raise TypeError("the rows' scales must be bfloat16")
+    rc = lib.k3q_dense_i8_w8s_multi(_lib.ptr(x2), _lib.K3Q_BF16, _lib.ptr(q), _lib.ptr(s), M, K, len(kernels),
+                                    ctypes.byref(problems), float(epsilon), float(value_range[0]),
+                                    float(value_range[1]), _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_dense_i8_w8s_multi")
+    return [y.reshape(*lead, y.shape[1]) for y in outs]
+
+
 def decode_attention_supported(q, cache_k):
     """bfloat16, head width 128, one new position."""
     return (q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 4 and q.shape[1] == 1

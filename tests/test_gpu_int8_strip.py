@@ -110,6 +110,62 @@ def test_dense_int8_strip_repeatable_and_graph(dev):
         assert torch.equal(bits(out), bits(first))
 
 
+@pytest.mark.parametrize("M", [1, 8])
+@pytest.mark.parametrize("fused", [True, False])
+def test_dense_int8_strip_multi_matches_single_calls(dev, M, fused, monkeypatch):
+    # several kernels against one x in one launch: every workgroup computes what it computes in a
+    # single call (integer sums), so the bits are the single calls' bits -- also where the shared
+    # launch makes workgroups take turns that a problem alone would not need
+    monkeypatch.setattr(kops, "INT8_STRIP_FUSED_QUANTIZER_MAX", 1 << 30 if fused else 0)
+    K = 4096
+    widths = [4096, 4096, 4096, 14336, 3072]
+    g = torch.Generator().manual_seed(40 + M)
+    x = (torch.randn(M, K, generator=g) * 2).to(torch.bfloat16).to(dev)
+    kernels, singles = [], []
+    for i, N in enumerate(widths):
+        w = torch.randint(-127, 128, (K, N), generator=g, dtype=torch.int8).to(dev)
+        ks = (torch.rand(N, generator=g) * 50 + 50).to(torch.bfloat16).to(dev)
+        bias = (torch.randn(N, generator=g) * 0.1).to(torch.bfloat16).to(dev) if i % 2 == 0 else None
+        spec = dict(shadow=kops.int8_strip_copy(w), units=N, kernel_scale=ks, bias=bias)
+        kernels.append(spec)
+        singles.append(kops.int8_dense_strip(x, spec["shadow"], N, ks, bias=bias))
+    for base, end in ((0, 3), (0, 5), (3, 5)):
+        got = kops.int8_dense_strip_multi(x, kernels[base:end])
+        for j, y in enumerate(got):
+            assert torch.equal(bits(y), bits(singles[base + j])), (base, j)
+
+
+@pytest.mark.parametrize("rows", [1, 8])
+def test_call_together_int8_layers_at_decode_widths(dev, rows):
+    # Dense and EinsumDense int8 layers on one input go through one launch and give the bits of
+    # the separate calls (which are the oracle's, tested above)
+    import keras_amd as ka
+    from keras_amd.layers import Dense, EinsumDense
+
+    g = torch.Generator().manual_seed(77)
+    init = lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d)
+    proj = [EinsumDense("btd,dnh->btnh", (None, 32, 128), dtype="bfloat16", device=dev, kernel_initializer=init)
+            for _ in range(3)]
+    x = torch.randn((rows, 1, 4096), generator=g).to(torch.bfloat16).to(dev)
+    for layer in proj:
+        layer.build((None, 1, 4096))
+        layer.quantize("int8")
+    want = [layer(x) for layer in proj]
+    got = ka.layers.call_together(proj, x)
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and torch.equal(bits(a), bits(b))
+    mlp = [Dense(14336, use_bias=False, dtype="bfloat16", device=dev, kernel_initializer=init),
+           Dense(14336, use_bias=True, activation="relu", dtype="bfloat16", device=dev, kernel_initializer=init)]
+    x2 = x.reshape(rows, 4096)
+    for layer in mlp:
+        layer.build((None, 4096))
+        layer.quantize("int8")
+    want = [layer(x2) for layer in mlp]
+    got = ka.layers.call_together(mlp, x2)
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and torch.equal(bits(a), bits(b))
+
+
 def test_dense_int8_strip_rejects(dev):
     for M, K, N in [(17, 4096, 4096), (1, 4096, 1024), (1, 4000, 4096), (1, 4096, 4100), (16, 14336, 4096),
                     (1, 512, 4096)]:
