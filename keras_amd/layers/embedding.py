@@ -39,7 +39,8 @@ def _promote(a, b):
 
 class Embedding(Layer):
     def __init__(self, input_dim, output_dim, embeddings_initializer=None, mask_zero=False,
-                 dtype=None, name=None, device=None, quantization_config=None):
+                 dtype=None, name=None, device=None, quantization_config=None, lora_rank=None,
+                 lora_alpha=None):
         if not isinstance(input_dim, int) or isinstance(input_dim, bool) or input_dim <= 0:
             raise ValueError(
                 "`input_dim` must be a positive integer. "
@@ -57,6 +58,8 @@ class Embedding(Layer):
         self.mask_zero = mask_zero
         self.autocast = False
         self.lora_enabled = False
+        self.lora_rank = lora_rank
+        self.lora_alpha = lora_alpha if lora_alpha is not None else lora_rank
         self.quantization_config = quantization_config
         # raise IndexError for ids outside the table as the reference does; costs one
         # device -> host read per call, switch off in a serving loop
@@ -76,17 +79,102 @@ class Embedding(Layer):
                 initializer=self.embeddings_initializer, trainable=True,
             )
         self.built = True
+        if self.lora_rank:
+            self.enable_lora(self.lora_rank)  # embedding.py:166-167
 
     @property
     def embeddings(self):
         """The table as a consumer sees it: int4 comes back unpacked to int8
-        `[vocab, dim]` (embedding.py:169-191)."""
+        `[vocab, dim]`; with LoRA enabled the low-rank update is added (embedding.py:169-191)."""
         if not self.built:
             raise AttributeError("You must build the layer before accessing `embeddings`.")
         embeddings = as_tensor(self._embeddings)
         if self.quantization_mode == "int4":
             embeddings = quantizers.unpack_int4(embeddings, self._orig_output_dim, axis=-1)
+        if self.lora_enabled:
+            embeddings = torch.add(embeddings, self._lora_delta())
         return embeddings
+
+    def enable_lora(self, rank, lora_alpha=None, a_initializer="he_uniform", b_initializer="zeros"):
+        """embedding.py:214-261: float32 `lora_embeddings_a` [input_dim, rank] and
+        `lora_embeddings_b` [rank, output_dim]; a lookup adds (alpha / rank) * a[ids] . b."""
+        from keras_amd.layers.dense import lora_initializer
+
+        if not self.built:
+            raise ValueError("Cannot enable lora on a layer that isn't yet built.")
+        if self.lora_enabled:
+            raise ValueError("lora is already enabled. This can only be done once per layer.")
+        self.lora_embeddings_a = self.add_weight(name="lora_embeddings_a", shape=(self.input_dim, rank),
+                                                 dtype="float32", initializer=lora_initializer(a_initializer),
+                                                 trainable=True)
+        self.lora_embeddings_b = self.add_weight(name="lora_embeddings_b", shape=(rank, self.output_dim),
+                                                 dtype="float32", initializer=lora_initializer(b_initializer),
+                                                 trainable=True)
+        self.lora_enabled = True
+        self.lora_rank = rank
+        self.lora_alpha = lora_alpha if lora_alpha is not None else rank
+
+    def _lora_delta(self):
+        return (self.lora_alpha / self.lora_rank) * torch.matmul(
+            as_tensor(self.lora_embeddings_a), as_tensor(self.lora_embeddings_b))
+
+    def _add_lora_rows(self, outputs, inputs):
+        """embedding.py:533-540 / :575-582: the rows of `a` at the ids times `b`, scaled, added to the
+        de-quantised rows, the sum cast to the compute dtype (the layer does not autocast, so
+        the update is float32)."""
+        idx = inputs.long()
+        idx = torch.where(idx < 0, idx + self.input_dim, idx)
+        lora = torch.matmul(torch.nn.functional.embedding(idx, as_tensor(self.lora_embeddings_a)),
+                            as_tensor(self.lora_embeddings_b))
+        out = torch.add(outputs, (self.lora_alpha / self.lora_rank) * lora)
+        return out.to(to_torch_dtype(self.compute_dtype))
+
+    def _get_embeddings_with_merged_lora(self):
+        """`(embeddings, embeddings_scale, embeddings_zero)` as saved (embedding.py:683-818): with LoRA
+        enabled the table is de-quantised, `(alpha / rank) * a . b` added, and the sum quantised again
+        the way `quantize()` does it."""
+        mode = self.quantization_mode
+        if mode is None:
+            return self.embeddings, None, None
+        value = as_tensor(self._embeddings)
+        scale = as_tensor(self.embeddings_scale)
+        zero = as_tensor(self.embeddings_zero) if hasattr(self, "embeddings_zero") else None
+        if not self.lora_enabled:
+            return value, scale, zero
+        cd = to_torch_dtype(self.compute_dtype)
+        block_size = getattr(self, "_int4_block_size", None)
+        grouped = block_size is not None and block_size != -1
+        if mode == "int4":
+            unpacked = quantizers.unpack_int4(value, self._orig_output_dim, axis=-1)
+            if grouped:
+                table = quantizers.dequantize_with_sz_map(unpacked.to(cd), scale, zero, as_tensor(self.g_idx),
+                                                          group_axis=-1)
+            else:
+                table = torch.divide(unpacked.to(cd), torch.unsqueeze(scale, -1))
+            quant_range = (-8, 7)
+        elif mode == "int8":
+            table = torch.divide(value.to(cd), torch.unsqueeze(scale, -1))
+            quant_range = (-127, 127)
+        else:
+            raise self._quantization_mode_error(mode)
+        merged = torch.add(table, self._lora_delta())
+        if mode == "int4" and grouped:
+            value_t, scale_t, zero_t = quantizers.abs_max_quantize_grouped_with_zero_point(
+                torch.transpose(merged, 0, 1), block_size=block_size, value_range=quant_range, dtype="int8",
+                to_numpy=True)
+            requantized = torch.transpose(value_t, 0, 1).contiguous()
+            scale = torch.transpose(scale_t, 0, 1).contiguous()
+            zero = torch.transpose(zero_t, 0, 1).contiguous()
+        else:
+            requantized, scale = quantizers.abs_max_quantize(merged, axis=-1, value_range=quant_range,
+                                                            dtype="int8", to_numpy=True)
+            scale = torch.squeeze(scale, dim=-1)
+            zero = None
+        if mode == "int4":
+            value, _, _ = quantizers.pack_int4(requantized.to(self.device), axis=-1)
+        else:
+            value = requantized
+        return value, scale, zero
 
     def __call__(self, inputs, training=None, **kwargs):
         # ids are not cast to the compute dtype (layer.py:883-901 only touches floats)
@@ -105,7 +193,7 @@ class Embedding(Layer):
             inputs = inputs.to(torch.int32)
         idx = inputs.long()
         idx = torch.where(idx < 0, idx + self.input_dim, idx)
-        out = torch.nn.functional.embedding(idx, as_tensor(self._embeddings))
+        out = torch.nn.functional.embedding(idx, self.embeddings if self.lora_enabled else as_tensor(self._embeddings))
         return out.to(to_torch_dtype(self.compute_dtype))
 
     def compute_mask(self, inputs, mask=None):
@@ -175,29 +263,27 @@ class Embedding(Layer):
 
     def _int8_call(self, inputs, training=None):
         """embedding.py:521-541: gather rows and scales, cast, divide -- one kernel."""
-        if self.lora_enabled:
-            raise NotImplementedError("LoRA on a quantized Embedding is outside this inference path.")
-        return kops.embedding_lookup(
+        out = kops.embedding_lookup(
             inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
             self.output_dim, bits=8, out_dtype=self._lookup_dtype(), check_ids=self.check_ids,
         )
+        return self._add_lora_rows(out, inputs) if self.lora_enabled else out
 
     def _int4_call(self, inputs, training=None):
         """embedding.py:542-582: the packed rows are gathered and de-quantised in one kernel;
         the table is never unpacked in memory."""
-        if self.lora_enabled:
-            raise NotImplementedError("LoRA on a quantized Embedding is outside this inference path.")
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
         if grouped:
             require_default_g_idx(self, block_size)
-        return kops.embedding_lookup(
+        out = kops.embedding_lookup(
             inputs, as_tensor(self._embeddings), as_tensor(self.embeddings_scale),
             self._orig_output_dim, bits=4,
             zero=as_tensor(self.embeddings_zero) if grouped else None,
             block_size=block_size if grouped else None,
             out_dtype=self._lookup_dtype(), check_ids=self.check_ids,
         )
+        return self._add_lora_rows(out, inputs) if self.lora_enabled else out
 
     # ---- quantize (one-time, host side) ---------------------------------------------
     def _drop(self, attr):
@@ -280,10 +366,17 @@ class Embedding(Layer):
         return out
 
     def save_own_variables(self, store):
+        """Store order of `_spec_entries`; a LoRA update is merged into the table, the scales and
+        the zero points that are written (embedding.py:263-309)."""
         if not self.built:
             return
-        for idx, (_, var) in enumerate(self._spec_entries()):
-            store[str(idx)] = as_tensor(var)
+        merged = {}
+        if self.lora_enabled:
+            value, scale, zero = self._get_embeddings_with_merged_lora()
+            merged = {"embeddings": value, "embeddings_scale": scale, "embeddings_zero": zero}
+        for idx, (name, var) in enumerate(self._spec_entries()):
+            value = merged.get(name)
+            store[str(idx)] = as_tensor(var) if value is None else value
 
     def load_own_variables(self, store):
         if not self.built:
@@ -293,9 +386,12 @@ class Embedding(Layer):
             if name == "g_idx" and isinstance(value, torch.Tensor):
                 value = value.to(as_tensor(var).dtype)
             var.assign(value)
+        if self.lora_enabled:  # embedding.py:355-361: what was saved holds the update
+            self.lora_embeddings_a.assign(torch.zeros_like(as_tensor(self.lora_embeddings_a)))
+            self.lora_embeddings_b.assign(torch.zeros_like(as_tensor(self.lora_embeddings_b)))
 
     def get_config(self):
-        return {
+        config = {
             "name": self.name,
             "input_dim": self.input_dim,
             "output_dim": self.output_dim,
@@ -308,6 +404,10 @@ class Embedding(Layer):
                 }
             ),
         }
+        if self.lora_rank:
+            config["lora_rank"] = self.lora_rank
+            config["lora_alpha"] = self.lora_alpha
+        return config
 
 
 class ReversibleEmbedding(Embedding):

@@ -756,6 +756,43 @@ def embedding_int4_call(ids, embeddings, embeddings_scale, orig_output_dim,
     return dequantize_with_sz_map(outputs.to(cd), scale, zero, g_idx, group_axis=-1)
 
 
+def embedding_merged_lora_table(mode, embeddings, embeddings_scale, lora_a, lora_b, alpha, rank,
+                                compute_dtype="float32", embeddings_zero=None, g_idx=None, block_size=None,
+                                orig_output_dim=None):
+    """keras/src/layers/core/embedding.py:721-818: de-quantise the table (rows over their scales, or
+    `dequantize_with_sz_map` along the output axis), add (alpha / rank) * a . b, quantise again per
+    row (grouped: through the transpose, as `quantize()` does).  -> (table, scale, zero) as saved.
+    Pinned like `dense_merged_lora_kernel`: a zero update is the identity on the integers."""
+    cd = _tdtype(compute_dtype)
+    grouped = block_size is not None and block_size != -1
+    if mode == "int4":
+        unpacked = unpack_int4(embeddings, orig_output_dim, axis=-1)
+        if grouped:
+            table = dequantize_with_sz_map(unpacked.to(cd), embeddings_scale, embeddings_zero, g_idx, group_axis=-1)
+        else:
+            table = torch.divide(unpacked.to(cd), torch.unsqueeze(embeddings_scale, -1))
+        quant_range = (-8, 7)
+    elif mode == "int8":
+        table = torch.divide(embeddings.to(cd), torch.unsqueeze(embeddings_scale, -1))
+        quant_range = (-127, 127)
+    else:
+        raise ValueError(f"Unsupported quantization mode: {mode}")
+    merged = torch.add(table, (alpha / rank) * torch.matmul(lora_a, lora_b))
+    if mode == "int4" and grouped:
+        q_t, s_t, z_t = abs_max_quantize_grouped_with_zero_point(
+            torch.transpose(merged, 0, 1), block_size=block_size, value_range=quant_range, dtype="int8")
+        q = torch.transpose(q_t, 0, 1).contiguous()
+        scale = torch.transpose(s_t, 0, 1).contiguous()
+        zero = torch.transpose(z_t, 0, 1).contiguous()
+    else:
+        q, scale = abs_max_quantize(merged, axis=-1, value_range=quant_range, dtype="int8", to_numpy=True)
+        scale = torch.squeeze(scale, dim=-1)
+        zero = None
+    if mode == "int4":
+        q, _, _ = pack_int4(q, axis=-1)
+    return q, scale, zero
+
+
 def reversible_embedding_int8_reverse(inputs, embeddings, embeddings_scale,
                                       compute_dtype=None, logit_soft_cap=None,
                                       return_intermediates=False):

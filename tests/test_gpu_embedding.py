@@ -159,6 +159,61 @@ def test_embedding_int8_layer(dev, policy, V, D):
     assert torch.equal(bits(clone(ids).cpu()), bits(want))
 
 
+@pytest.mark.parametrize("mode,block_size", [("int8", None), ("int4", None), ("int4", 64)])
+@pytest.mark.parametrize("policy", ["float32", "bfloat16"])
+def test_embedding_lora_on_quantized_layer_and_merge_on_save(dev, mode, block_size, policy):
+    # keras/src/layers/core/embedding.py:214-261 (enable_lora), :533-540 / :575-582 (a lookup adds the
+    # rows of the update), :683-818 (the update is merged into what is saved), :355-361 (zeroed on load)
+    g = torch.Generator().manual_seed(31)
+    V, D, rank, alpha = 200, 256, 4, 8
+    layer = build_embedding(Embedding, dev, V, D, policy, seed=6)
+    t = layer._embeddings.value.cpu()
+    if mode == "int8":
+        layer.quantize("int8")
+        q, s = ref.embedding_quantize_int8(t)
+        zero = g_idx = None
+    else:
+        layer.quantize("int4", config=Int4QuantizationConfig(block_size=block_size))
+        qd = ref.embedding_quantize_int4(t, block_size=block_size)
+        q, s, zero, g_idx = qd["embeddings"], qd["embeddings_scale"], qd["embeddings_zero"], qd["g_idx"]
+    layer.enable_lora(rank, lora_alpha=alpha)
+    with pytest.raises(ValueError):
+        layer.enable_lora(rank)
+    assert tuple(layer.lora_embeddings_a.shape) == (V, rank) and tuple(layer.lora_embeddings_b.shape) == (rank, D)
+    a = torch.randn(V, rank, generator=g) * 0.02
+    b = torch.randn(rank, D, generator=g) * 0.02
+    layer.lora_embeddings_a.assign(a)
+    layer.lora_embeddings_b.assign(b)
+    ids = torch.randint(0, V, (5, 7), generator=g)
+    y = layer(ids)
+    cd = layer.compute_dtype
+    if mode == "int8":
+        base = ref.embedding_int8_call(ids, q, s, compute_dtype=cd)
+    else:
+        base = ref.embedding_int4_call(ids, q, s, D, embeddings_zero=zero, g_idx=g_idx, block_size=block_size,
+                                       compute_dtype=cd)
+    want = (base + (alpha / rank) * (a[ids] @ b)).to(y.dtype)
+    assert y.dtype == want.dtype and (y.float().cpu() - want.float()).abs().max().item() <= 1e-2 * want.abs().max().item()
+    merged = ref.embedding_merged_lora_table(mode, q, s, a, b, alpha, rank, compute_dtype=cd, embeddings_zero=zero,
+                                             g_idx=g_idx, block_size=block_size, orig_output_dim=D)
+    store = {}
+    layer.save_own_variables(store)
+    assert torch.equal(store["0"].cpu(), merged[0])
+    assert torch.equal(bits(store["1"].cpu()), bits(merged[1]))
+    if block_size:
+        assert torch.equal(store["2"].cpu(), merged[2])
+    assert not torch.equal(store["0"].cpu(), q)
+    plain = Embedding(V, D, dtype=layer.dtype_policy.name, device=dev)
+    plain.build()
+    plain.load_own_variables(store)
+    y2 = plain(ids)
+    assert (y2.float().cpu() - y.float().cpu()).abs().max().item() <= (0.02 if mode == "int8" else 0.2) * y.float().abs().max().item()
+    layer.load_own_variables(store)
+    assert float(layer.lora_embeddings_a.value.abs().max()) == 0.0
+    assert torch.equal(bits(layer(ids).cpu()), bits(y2.cpu()))
+    assert layer.get_config()["lora_rank"] == rank
+
+
 @pytest.mark.parametrize("policy", ["float32", "bfloat16"])
 @pytest.mark.parametrize("block_size", [128, 64, 8, None, -1])
 @pytest.mark.parametrize("V,D", [(10, 16), (100, 256), (300, 4096)])
