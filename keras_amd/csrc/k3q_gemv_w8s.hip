@@ -109,22 +109,29 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
         for (int t = 0; t < kSW; ++t) W[d][t] = __builtin_nontemporal_load(nb[t] + d * 64);
     };
     at_cursor();
+    // Every wave's first x requests go out before any wave's weight requests: a compute unit's
+    // memory pipeline serves requests in the order they were issued, and x behind 64 KiB of another
+    // wave's weights reaches LDS that much later.  (A bare barrier: nothing is waited for.)
+    auto x_before_weights = []() {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
 
     // ---- stage x ----
     if constexpr (kNP < 0) {
         // rows already quantised: copy them (16 int8 per piece) and their scales into LDS
         const int pieces = M * (K >> 4);
         constexpr int kCP = 4;  // pieces in flight per thread and round
-#pragma unroll
-        for (int d = 0; d < kD; ++d) refill(d);
-        advance();
-        for (int base = 0; base < pieces; base += kCP * kT) {
-            v4u c[kCP];
+        v4u c[kCP];
+        auto copy_load = [&](int base) {
 #pragma unroll
             for (int i = 0; i < kCP; ++i) {
                 const int pi = base + i * kT + tid;
                 c[i] = ((const v4u*)p.xq)[pi < pieces ? pi : pieces - 1];
             }
+        };
+        auto copy_store = [&](int base) {
 #pragma unroll
             for (int i = 0; i < kCP; ++i) {
                 const int pi = base + i * kT + tid;
@@ -134,6 +141,16 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
                     *(v4u*)(xs + row * pitch + col) = c[i];
                 }
             }
+        };
+        copy_load(0);
+        x_before_weights();
+#pragma unroll
+        for (int d = 0; d < kD; ++d) refill(d);
+        advance();
+        copy_store(0);
+        for (int base = kCP * kT; base < pieces; base += kCP * kT) {
+            copy_load(base);
+            copy_store(base);
         }
         if (tid < M) sa[tid] = bf16_bits_to_f32(p.xs[tid]);
     } else {
@@ -147,6 +164,7 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
                 const int pi = tid + i * kT;
                 xr[i] = ((const v4u*)p.x)[pi < pieces ? pi : pieces - 1];
             }
+            x_before_weights();
         }
 #pragma unroll
         for (int d = 0; d < kD; ++d) refill(d);
