@@ -351,11 +351,83 @@ def main():
             del graph
         del xg
 
+    # ------------------------------------------------------------------ what reading costs
+    # The same graph-node timing for a launch that only READS a kernel's bytes (libk3q_probe.so:
+    # the decode kernels' access pattern without their arithmetic, best of a few grid sizes and
+    # queue depths) and for a launch that does nothing: the decode kernels are compared with these.
+    def graph_node_us(call, count, reps):
+        side_ = torch.cuda.Stream()
+        with torch.cuda.stream(side_):
+            for i in range(count):
+                call(i)
+            graph_ = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph_, stream=side_):
+                for i in range(reps):
+                    call(i)
+        torch.cuda.synchronize()
+        spin_up(torch, graph_.replay, 0.05)
+        e0_, e1_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0_.record()
+        for _ in range(3):
+            graph_.replay()
+        e1_.record()
+        torch.cuda.synchronize()
+        return e0_.elapsed_time(e1_) / (3 * reps) * 1e3
+
+    def load_stream_probe():
+        import ctypes
+
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "keras_amd", "libk3q_probe.so")
+        if not os.path.exists(path):
+            return None
+        lib_ = ctypes.CDLL(path)
+        lib_.k3q_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                               ctypes.c_void_p, ctypes.c_void_p]
+        lib_.k3q_probe_empty.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        return lib_
+
+    def read_reference(buffers, nbytes):
+        """Best time per graph node of a pure read of `nbytes` from each of `buffers` in turn."""
+        import ctypes
+
+        lib_ = load_stream_probe()
+        if lib_ is None:
+            return None
+        sink = torch.zeros(4096, dtype=torch.int32, device=dev)
+        best = None
+        for wgs, depth in ((256, 8), (256, 16), (512, 4), (512, 8), (1024, 4), (1024, 8)):
+            if nbytes % (wgs * 8 * depth * 1024) or nbytes // (wgs * 8) < 2048 * depth:
+                continue  # (the probe wants at least two rounds of whole KiB pieces per wave)
+            def call(i):
+                rc = lib_.k3q_probe_stream_read(ctypes.c_void_p(buffers[i % len(buffers)].data_ptr()), nbytes, wgs, depth,
+                                                ctypes.c_void_p(sink.data_ptr()),
+                                                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+                if rc != 0:
+                    sys.exit("bench.py: the read-only probe did not launch")
+            us_ = graph_node_us(call, len(buffers), 4 * len(buffers))
+            if best is None or us_ < best["us_per_launch"]:
+                best = {"bytes": nbytes, "us_per_launch": round(us_, 2), "workgroups": wgs, "loads_in_flight_per_wave": depth,
+                        "gbs": round(nbytes / us_ / 1e3, 1)}
+
+        def nothing(i):
+            lib_.k3q_probe_empty(ctypes.c_void_p(sink.data_ptr()),
+                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        best["empty_launch_us"] = round(graph_node_us(nothing, 4, 400), 2)
+        return best
+
+    read_ref4 = None
+    if want("gemv"):
+        read_ref4 = read_reference(strips, Kg * Ng // 2)
+        if read_ref4:
+            for row in gemv:
+                row["frac_of_read_only_launch"] = round(read_ref4["us_per_launch"] / row["us_per_call"], 3)
+
     # ------------------------------------------------------------------ int8 decode forward
     # Dense int8 at decode sizes, K = N = 8192: quantizer + exact int8 matmul + bit-exact de-scale,
     # one launch from the strip-linear copy of the int8 kernel (x above 16 K values: a quantizer
     # launch first); 6 kernels of 64 MiB in rotation, each call a graph node
     gemv8 = []
+    read_ref8 = None
     if want("gemv8"):
         n_rot8 = 6
         w8 = [torch.randint(-127, 128, (Kg, Ng), dtype=torch.int8, device=dev) for _ in range(n_rot8)]
@@ -390,6 +462,10 @@ def main():
                           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                                        "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}})
             del graph, x8
+        read_ref8 = read_reference(s8, Kg * Ng)
+        if read_ref8:
+            for row in gemv8:
+                row["frac_of_read_only_launch"] = round(read_ref8["us_per_launch"] / row["us_per_call"], 3)
         del s8
         torch.cuda.empty_cache()
 
@@ -492,7 +568,9 @@ def main():
         "int8_gemm_sweep": sweep,
         "einsum_int8": einsum,
         "int4_gemv": gemv,
+        "read_only_launch_32MiB": read_ref4,
         "int8_decode_dense": gemv8,
+        "read_only_launch_64MiB": read_ref8,
         "llama_decode_int4": decode,
         "llama_decode_int8": decode_int8,
         "cpu_baseline": cpu,

@@ -71,13 +71,14 @@ def build(verbose=True, jobs=8):
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
     # the measurement aid bench.py uses: a library of its own, never loaded by the package
-    cmd = [hipcc(), *FLAGS, "-shared", "-o", PROBE_LIB, os.path.join(HERE, "k3q_probe_mfma.hip")]
+    cmd = [hipcc(), *FLAGS, "-shared", "-o", PROBE_LIB, os.path.join(HERE, "k3q_probe_mfma.hip"),
+           os.path.join(HERE, "k3q_probe_stream.hip")]
     if verbose:
         print(" ".join(cmd), flush=True)
     out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
     if out.returncode != 0:
         sys.stderr.write(out.stdout.decode())
-        raise RuntimeError("hipcc failed on k3q_probe_mfma.hip")
+        raise RuntimeError("hipcc failed on the probe library")
     return LIB
 
 

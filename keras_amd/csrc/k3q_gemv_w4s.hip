@@ -56,6 +56,8 @@ struct W4sParams {
     int M, K, N, units;      // units = K / 128
     int row_magic;           // ceil(2^32 / pieces per staged row): piece -> row without a division
     int slice_magic;         // (x staged in halves) ceil(2^32 / pieces per half slice)
+    int own_magic[2];        // (waves stage their own slices) ceil(2^32 / pieces per row of a slice): short, long slice
+    int own;                 // 1: every wave stages its own slice of x; 0: the workgroup's threads share all of x
 };
 
 struct W4sMulti {
@@ -98,34 +100,42 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     float* red = (float*)(w4s_lds + ((M * pitch + 255) & ~255));
 
     // ---- x into registers first (every load unconditional: pieces past the end re-read piece 0) ----
-    // whole rows, or (kHalves) half h of every wave's slice: row m = [slice 0 | slice 1 | ...]
-    const int per_row = kHalves ? K >> 4 : K >> 3;
+    // Whole rows (kHalves: half h of every wave's slice, row m = [slice 0 | slice 1 | ...]), spread over
+    // the workgroup's threads -- or, for a small x (p.own), every wave loads and stores ITS OWN slice of
+    // every row, the only part of x it reads back: nothing is exchanged between waves then, and no
+    // barrier stands between a wave's x (the oldest requests in its queue) and its first weights.
+    // (Measured: worth 0.3 us up to 32 KiB of x, a loss beyond.)
+    const bool own = !kHalves && p.own;
+    const int per_row = kHalves ? K >> 4 : own ? U * 16 : K >> 3;
     const int pieces = M * per_row;
+    const u32 row_magic = own ? (u32)p.own_magic[q < extra ? 1 : 0] : (u32)p.row_magic;
+    const int own_col = own ? u0 * 16 : 0;  // first piece of the wave's slice within a row
+    const int row_pieces = K >> 3;
     v4u xst[kNP];
     auto stage_load = [&](const int h) {
 #pragma unroll
         for (int i = 0; i < kNP; ++i) {
-            int pi = i * kT + tid;
+            int pi = own ? i * 64 + lane : i * kT + tid;
             pi = pi < pieces ? pi : 0;
+            const int m = (int)__umulhi((unsigned)pi, row_magic);
+            const int c = pi - m * per_row;
             if (kHalves) {
-                const int m = (int)__umulhi((unsigned)pi, (unsigned)p.row_magic);
-                const int c = pi - m * per_row;
                 const int qq = (int)__umulhi((unsigned)c, (unsigned)p.slice_magic);  // c / (Uh * 16)
                 const int cc = c - qq * (Uh * 16);
                 xst[i] = *(const v4u*)(p.x + (int64_t)m * K + (int64_t)(qq * U + h * Uh) * 128 + cc * 8);
             } else {
-                xst[i] = *(const v4u*)(p.x + (int64_t)pi * 8);
+                xst[i] = *(const v4u*)(p.x + ((int64_t)m * row_pieces + own_col + c) * 8);
             }
         }
     };
     auto stage_store = [&]() {
 #pragma unroll
         for (int i = 0; i < kNP; ++i) {
-            const int pi = i * kT + tid;
+            const int pi = own ? i * 64 + lane : i * kT + tid;
             if (pi < pieces) {
-                const int m = (int)__umulhi((unsigned)pi, (unsigned)p.row_magic);
+                const int m = (int)__umulhi((unsigned)pi, row_magic);
                 const int c = pi - m * per_row;
-                *(v4u*)(w4s_lds + m * pitch + c * 16) = xst[i];
+                *(v4u*)(w4s_lds + m * pitch + (own_col + c) * 16) = xst[i];
             }
         }
     };
@@ -179,7 +189,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     __builtin_amdgcn_sched_barrier(0);
     // ---- x into LDS: the stores wait for the x loads only (they are the older ones) ----
     stage_store();
-    __syncthreads();
+    if (!own) __syncthreads();  // (own slices: a wave reads back only what it wrote itself)
 
     const char* xrow = w4s_lds + jj * pitch + (kHalves ? q * Uh : u0) * 256 + g * 16;
     const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
@@ -496,6 +506,7 @@ inline int64_t strips_padded(int64_t N) { return ((N + 15) / 16 + 1) / 2 * 2; }
 struct W4sPlan {
     bool ok;
     bool halves;  // x staged in two halves (9 ... 16 rows of a long K)
+    bool own;     // every wave stages its own slice of x (a small x)
     int sw, d, np;
     int64_t groups;  // strip groups (kSW strips each)
     int64_t blocks;  // workgroups: each takes groups block, block + blocks, ...
@@ -530,8 +541,14 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
     pl.lds = (size_t)((M * (K * 2 + 16) + 255) & ~255) + red;
     pl.lds_two = pl.lds - red + 2 * red_one;
     if (M * K <= stage_max && pl.lds <= lds_limit) {
+        // a small x: every wave stages its own slice of every row (16 pieces per unit and row, over 64 lanes)
+        const int64_t ring_blocks = units / pl.d;
+        const int64_t longest = (ring_blocks / kQ + (ring_blocks % kQ ? 1 : 0)) * pl.d;  // units of the longest slice
+        const int64_t per_lane = (M * longest * 16 + 63) / 64;
         const int64_t pieces = M * K / 8;
-        pl.np = pieces <= 2 * kT ? 2 : pieces <= 4 * kT ? 4 : pieces <= 8 * kT ? 8 : 16;
+        pl.own = M * K * 2 <= 32 * 1024 && per_lane <= 4;
+        if (pl.own) pl.np = per_lane <= 2 ? 2 : 4;
+        else pl.np = pieces <= 2 * kT ? 2 : pieces <= 4 * kT ? 4 : pieces <= 8 * kT ? 8 : 16;
         pl.ok = true;
         return pl;
     }
@@ -594,6 +611,14 @@ int fill_params(W4sParams& p, const W4sPlan& pl, const void* x, int64_t M, int64
     p.units = (int)(K / 128);
     const uint64_t per_row = (uint64_t)K / (pl.halves ? 16 : 8);
     p.row_magic = (int)(uint32_t)((((uint64_t)1 << 32) + per_row - 1) / per_row);
+    {
+        const uint64_t ring_blocks = (uint64_t)(K / 128) / pl.d, base = ring_blocks / kQ;
+        for (int e = 0; e < 2; ++e) {
+            const uint64_t own = (base + e) * pl.d * 16;  // pieces per row of a slice of base (+ 1) ring blocks
+            p.own_magic[e] = own ? (int)(uint32_t)((((uint64_t)1 << 32) + own - 1) / own) : 0;
+        }
+    }
+    p.own = pl.own ? 1 : 0;
     const uint64_t per_half_slice = (uint64_t)(K / 128 / kQ / 2) * 16;
     p.slice_magic = pl.halves ? (int)(uint32_t)((((uint64_t)1 << 32) + per_half_slice - 1) / per_half_slice) : 0;
     return K3Q_OK;
@@ -707,7 +732,7 @@ extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t
             const W4sPlan pl = w4s_plan(M, K, q.N, block_size);
             if (!pl.ok) return K3Q_ERR_SHAPE;
             if (n == 0) pl0 = pl;
-            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np || pl.halves || pl0.halves) break;
+            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np || pl.own != pl0.own || pl.halves || pl0.halves) break;
             const int rc = fill_params(mp.p[n], pl, x, M, K, q.N, q.shadow, q.scale, q.gparams, block_size,
                                        q.bias, 0, q.y);
             if (rc != K3Q_OK) return rc;
