@@ -64,10 +64,24 @@ __device__ __forceinline__ float div_round_bf16(float a, float b) {
     return round_bf16(a / b);
 }
 
+// Maximum over the 64 lanes of a wave, in every lane.  Data-parallel-primitive moves instead of
+// shuffles through the LDS crossbar: six dependent steps at register speed (a shuffle step costs an
+// LDS round trip, which a kernel that reduces per 16-byte piece pays many times over).  A lane whose
+// source lane is outside its row, or masked, keeps its own value: fmaxf(v, v).  All 64 lanes must be
+// active.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_move(float v) {
+    const int i = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_update_dpp(i, i, kCtrl, kRowMask, 0xf, false));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1, 0xf>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E, 0xf>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_move<0x141, 0xf>(v));  // row_half_mirror: the other quad of each half row
+    v = fmaxf(v, dpp_move<0x140, 0xf>(v));  // row_mirror: the other half of each row of 16
+    v = fmaxf(v, dpp_move<0x142, 0xa>(v));  // row_bcast15: rows 1 and 3 take in rows 0 and 2
+    v = fmaxf(v, dpp_move<0x143, 0xc>(v));  // row_bcast31: rows 2 and 3 take in row 1 (= rows 0, 1)
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // byte select: result byte i = byte sel[i] of the 8-byte pool {lo: bytes 0-3, hi: bytes 4-7}
