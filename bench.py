@@ -457,7 +457,7 @@ def main():
             nbytes = Kg * Ng + 2 * M8 * Kg + 2 * M8 * Ng + 2 * Ng
             gbs = nbytes / (us * 1e-6) / 1e9
             gemv8.append({"M": M8, "K": Kg, "N": Ng, "kernel": "gemv_w8s (strip-linear copy)"
-                          + ("" if M8 * Kg <= kops.INT8_STRIP_FUSED_QUANTIZER_MAX else " + quantize_rows_vec"),
+                          + ("" if kops.int8_strip_quantises_inside(M8, Kg, (-127, 127)) else " + quantize_rows_vec"),
                           "us_per_call": round(us, 2), "algorithmic_bytes": nbytes,
                           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                                        "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}})

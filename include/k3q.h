@@ -429,7 +429,10 @@ int k3q_embedding_lookup(const void* ids, int ids_dtype, int64_t count, const in
  * bytes k = 64 unit + 16 g + (0 ... 15); the strip count is padded to even with zero strips;
  * k3q_w8s_shadow_bytes gives its size.  kernel_scale: bfloat16 [N].  bias: bfloat16, N values
  * (bias_stride 0) or M x N (bias_stride N: a row per row of x), or null.
- * epsilon, range_lo, range_hi: the quantizer's settings (1e-7, -127, 127 by default).
+ * epsilon, range_lo, range_hi: the quantizer's settings (1e-7, -127, 127 by default); the range
+ * inside [-128, 127] (K3Q_ERR_SHAPE) with integer ends (K3Q_ERR_RANGE: the kernel clips before it
+ * rounds, which equals the reference's round-then-clip only between integers; other ranges go
+ * through k3q_absmax_quantize + k3q_gemm_i8_w8s).
  * Needs K % 512 == 0, K >= 1024, N % 16 == 0, N >= 3072 and M x K small enough for LDS
  * (k3q_dense_i8_w8s_supported says; K3Q_ERR_SHAPE otherwise).
  *

@@ -46,12 +46,6 @@ struct W8sParams {
 __device__ __forceinline__ float scale_from_amax_bf16(float amax, float eps, float qhi) {
     return round_bf16(qhi / round_bf16(amax + eps));
 }
-__device__ __forceinline__ u32 quantize_bf16(float v, float s, float qlo, float qhi) {
-    float p = rintf(round_bf16(v * s));  // round half to even
-    p = fminf(fmaxf(p, qlo), qhi);
-    return (u32)(int)p & 0xffu;
-}
-
 // y = T(T(acc) / T(sa * sb)) (+ bias), T = bfloat16: the reference's sequence, every step rounded
 __device__ __forceinline__ float descale_exact_bf16(int acc, float sa, float sb, float bv, bool has_bias) {
     const float os = round_bf16(sb * sa);
@@ -201,19 +195,26 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
         __syncthreads();
         if (tid < M) sa[tid] = scale_from_amax_bf16(__uint_as_float(rowmax[tid]), p.eps, p.qhi);
         __syncthreads();
+        // Eight values of a piece -> eight int8: product, its bfloat16 rounding (one conversion per
+        // pair), clip, and rint + int conversion in one addition (1.5 * 2^23 + v leaves rint(v), half to
+        // even, in the low mantissa bits: the byte is its two's complement).  The clip comes first:
+        // the range's ends are integers (the entry point sees to it), so it commutes with rint.
         auto quantize_piece = [&](int pi, const v4u& c) {
             const int row = (int)__umulhi((u32)pi, (u32)p.row_magic);
             const int col = (pi - row * (K >> 3)) << 3;
             const float s = sa[row];
-            u32 lo = 0, hi = 0;
+            u32 t[8];
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                lo |= quantize_bf16(__uint_as_float(c[e] << 16), s, p.qlo, p.qhi) << (16 * e);
-                lo |= quantize_bf16(__uint_as_float(c[e] & 0xffff0000u), s, p.qlo, p.qhi) << (16 * e + 8);
-                hi |= quantize_bf16(__uint_as_float(c[2 + e] << 16), s, p.qlo, p.qhi) << (16 * e);
-                hi |= quantize_bf16(__uint_as_float(c[2 + e] & 0xffff0000u), s, p.qlo, p.qhi) << (16 * e + 8);
+            for (int e = 0; e < 4; ++e) {
+                const u32 pk = pack_bf16x2(__uint_as_float(c[e] << 16) * s, __uint_as_float(c[e] & 0xffff0000u) * s);
+                const float v0 = fminf(fmaxf(__uint_as_float(pk << 16), p.qlo), p.qhi);
+                const float v1 = fminf(fmaxf(__uint_as_float(pk & 0xffff0000u), p.qlo), p.qhi);
+                t[2 * e] = __float_as_uint(v0 + 12582912.0f);
+                t[2 * e + 1] = __float_as_uint(v1 + 12582912.0f);
             }
-            const v2u o = {lo, hi};
+            const u32 a0 = byte_perm(t[1], t[0], 0x0c0c0400u), a1 = byte_perm(t[3], t[2], 0x0c0c0400u);
+            const u32 b0 = byte_perm(t[5], t[4], 0x0c0c0400u), b1 = byte_perm(t[7], t[6], 0x0c0c0400u);
+            const v2u o = {a0 | (a1 << 16), b0 | (b1 << 16)};
             *(v2u*)(xs + row * pitch + col) = o;
         };
         if (kNP > 0) {
@@ -509,6 +510,8 @@ extern "C" int k3q_dense_i8_w8s(const void* x, int x_dtype, int64_t M, int64_t K
                                 float range_lo, float range_hi, void* y, void* stream) {
     if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (!(range_lo >= -128.f && range_hi <= 127.f && range_lo < range_hi)) return K3Q_ERR_SHAPE;
+    // (the in-kernel quantizer clips before it rounds: exact only between integer ends)
+    if (range_lo != rintf(range_lo) || range_hi != rintf(range_hi)) return K3Q_ERR_RANGE;
     return launch_w8s(x, nullptr, nullptr, M, K, N, shadow, kernel_scale, bias, bias_stride, epsilon, range_lo,
                       range_hi, y, (hipStream_t)stream);
 }
@@ -528,6 +531,8 @@ extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* 
     if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (count < 0 || M < 0 || K <= 0) return K3Q_ERR_SHAPE;
     if (!(range_lo >= -128.f && range_hi <= 127.f && range_lo < range_hi)) return K3Q_ERR_SHAPE;
+    // (the in-kernel quantizer clips before it rounds: exact only between integer ends)
+    if (range_lo != rintf(range_lo) || range_hi != rintf(range_hi)) return K3Q_ERR_RANGE;
     if (count == 0 || M == 0) return K3Q_OK;
     if (!problems) return K3Q_ERR_NULL;
     int at = 0;

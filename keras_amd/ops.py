@@ -708,10 +708,19 @@ def int8_strip_copy(kernel):
     return out
 
 
-# values of x up to which every workgroup of `int8_dense_strip` quantises the rows itself; beyond,
-# one quantizer launch and the kernel's pre-quantised form are faster (measured: 8 rows of 4096
-# cost 6 us more than one row when quantised in every workgroup, a quantizer launch 3 us)
-INT8_STRIP_FUSED_QUANTIZER_MAX = 16384
+# rows and values of x up to which every workgroup of `int8_dense_strip` quantises the rows itself;
+# beyond, one quantizer launch and the kernel's pre-quantised form are faster (measured at
+# K = N = 8192: 4 rows 17.5 us against 18.9, 8 rows 19.9 against 19.5; 8 rows of 4096: 9.7 against 9.3)
+INT8_STRIP_FUSED_MAX_ROWS = 4
+INT8_STRIP_FUSED_QUANTIZER_MAX = 32768
+
+
+def int8_strip_quantises_inside(M, K, value_range):
+    """Whether the strip kernel quantises these rows itself (otherwise a quantizer launch comes first).
+    Its quantizer clips before it rounds, which is exact only between integer ends of the range."""
+    lo, hi = float(value_range[0]), float(value_range[1])
+    return (M <= INT8_STRIP_FUSED_MAX_ROWS and M * K <= INT8_STRIP_FUSED_QUANTIZER_MAX and lo == round(lo) and hi == round(hi)
+            and -128 <= lo < hi <= 127)
 
 
 def int8_dense_strip(x, shadow, units, kernel_scale, bias=None, epsilon=1e-7, value_range=(-127, 127),
@@ -743,7 +752,7 @@ def int8_dense_strip(x, shadow, units, kernel_scale, bias=None, epsilon=1e-7, va
     stride = N if (bias is not None and M > 1 and bias.numel() == M * N) else 0
     ks = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    if M * K > INT8_STRIP_FUSED_QUANTIZER_MAX:
+    if not int8_strip_quantises_inside(M, K, value_range):
         if quantize is None:
             from keras_amd import quantizers
 
@@ -797,7 +806,7 @@ def int8_dense_strip_multi(x, kernels, epsilon=1e-7, value_range=(-127, 127), qu
         problems[i] = _lib.W8sProblem(N, k["shadow"].data_ptr(), ks.data_ptr(),
                                       bias.data_ptr() if bias is not None else None, y.data_ptr())
     q = s = None
-    if M * K > INT8_STRIP_FUSED_QUANTIZER_MAX:
+    if not int8_strip_quantises_inside(M, K, value_range):
         if quantize is None:
             from keras_amd import quantizers
 

@@ -73,6 +73,7 @@ def test_dense_int8_strip_bit_exact(dev, M, K, N, fused, monkeypatch):
     # both forms of the kernel at every shape: the rows quantised inside every workgroup, and
     # quantised by the quantizer kernel first
     monkeypatch.setattr(kops, "INT8_STRIP_FUSED_QUANTIZER_MAX", 1 << 30 if fused else 0)
+    monkeypatch.setattr(kops, "INT8_STRIP_FUSED_MAX_ROWS", 16)
     if not kops.int8_strip_supported(M, K, N):
         # too many rows of this width for LDS: the two-launch route keeps those
         assert M * K > 114688
@@ -117,6 +118,7 @@ def test_dense_int8_strip_multi_matches_single_calls(dev, M, fused, monkeypatch)
     # single call (integer sums), so the bits are the single calls' bits -- also where the shared
     # launch makes workgroups take turns that a problem alone would not need
     monkeypatch.setattr(kops, "INT8_STRIP_FUSED_QUANTIZER_MAX", 1 << 30 if fused else 0)
+    monkeypatch.setattr(kops, "INT8_STRIP_FUSED_MAX_ROWS", 16)
     K = 4096
     widths = [4096, 4096, 4096, 14336, 3072]
     g = torch.Generator().manual_seed(40 + M)
@@ -182,3 +184,23 @@ def test_dense_int8_strip_rejects(dev):
         kops.int8_dense_strip(x.float(), shadow, 4096, ks)
     with pytest.raises(ValueError):
         kops.int8_dense_strip(torch.zeros(17, 4096, dtype=torch.bfloat16, device=dev), shadow, 4096, ks)
+
+
+def test_dense_int8_strip_fractional_range(dev):
+    """Between non-integer ends clip-then-round is not round-then-clip: the in-kernel quantizer refuses
+    such a range, and the op quantises the rows with the quantizer kernel first (same bits as the
+    oracle either way)."""
+    import ctypes
+
+    from keras_amd import _lib
+
+    run_case(dev, 2, 4096, 4096, with_bias=True, value_range=(-100.5, 90.25), seed=9)
+    lib = _lib.load()
+    x = torch.zeros(1, 4096, dtype=torch.bfloat16, device=dev)
+    ks = torch.ones(4096, dtype=torch.bfloat16, device=dev)
+    shadow = kops.int8_strip_copy(torch.zeros(4096, 4096, dtype=torch.int8, device=dev))
+    y = torch.empty(1, 4096, dtype=torch.bfloat16, device=dev)
+    rc = lib.k3q_dense_i8_w8s(_lib.ptr(x), _lib.K3Q_BF16, 1, 4096, 4096, _lib.ptr(shadow), _lib.ptr(ks), None, 0,
+                              1e-7, -100.5, 90.25, _lib.ptr(y), _lib.stream_ptr(dev))
+    assert rc == -7
+    torch.cuda.synchronize()
