@@ -314,6 +314,34 @@ int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int cou
                        const k3q_gemv_w4s_problem* problems, int64_t block_size, void* stream);
 
 /*
+ * The decode matmuls with an operation on their input folded in: the rows of x are transformed on
+ * their way into the workgroup's LDS, which saves the launch and the round trip through memory of a
+ * separate elementwise kernel between two layers of a decoder block.
+ *   K3Q_INPUT_RMS_NORM:  x' = T(x * rsqrt(mean(x^2) + epsilon) * operand), operand = the gain,
+ *                        bfloat16 [K]; the bits k3q_rmsnorm writes.  K % 512 == 0, K <= 65536.
+ *   K3Q_INPUT_SILU_GATE: x' = T(T(silu(operand)) * x), operand = the gate, bfloat16 [M, K], dense;
+ *                        the bits k3q_silu_mul(gate = operand, up = x) writes.
+ * Every workgroup repeats the transform on all of x: worth it for the few rows of a decode step.
+ * k3q_gemv_w4s_pre: as k3q_gemv_w4s_multi (count >= 1 kernels against one x); bias_rows != 0: every
+ * problem's bias is an [M, N] addend (a row per row of x) instead of [N].  x whole in LDS only (no
+ * staging in halves): K3Q_ERR_SHAPE otherwise.
+ * k3q_dense_i8_w8s_pre: as k3q_dense_i8_w8s_multi with x given in bfloat16 (the rows are transformed,
+ * then quantised, inside the kernel); same bias_rows.
+ * No counterpart in the reference, whose layers each run their own ops
+ * (keras/src/layers/core/dense.py:961-986, 988-1095 see the normalised / gated tensor as input).
+ */
+#define K3Q_INPUT_NONE 0
+#define K3Q_INPUT_RMS_NORM 1
+#define K3Q_INPUT_SILU_GATE 2
+typedef struct {
+    int kind;
+    float epsilon;
+    const void* operand;
+} k3q_input_op;
+int k3q_gemv_w4s_pre(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_input_op* pre, int count,
+                     const k3q_gemv_w4s_problem* problems, int64_t block_size, int bias_rows, void* stream);
+
+/*
  * Weight-only int4 matmul for 17 ... 512 bfloat16 rows from a K-contiguous copy of the kernel:
  * the same result as k3q_gemv_w4 to the order of the fp32 sums, with the kernel read once as
  * int4 (k3q_gemv_w4's route for these sizes writes it out as bfloat16 first: nine times the
@@ -467,6 +495,10 @@ typedef struct {
 int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* a, const void* a_scale, int64_t M, int64_t K,
                            int count, const k3q_w8s_problem* problems, float epsilon, float range_lo,
                            float range_hi, void* stream);
+/* with an operation on x before it is quantised: see k3q_gemv_w4s_pre */
+int k3q_dense_i8_w8s_pre(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_input_op* pre, int count,
+                         const k3q_w8s_problem* problems, float epsilon, float range_lo, float range_hi,
+                         int bias_rows, void* stream);
 
 /*
  * One new position of causal self-attention against a key / value cache (the decoder
@@ -488,7 +520,7 @@ int k3q_decode_attention(const void* q, const void* k, const void* v, int dtype,
  * Two more pieces of the decoder harness's glue (no counterpart in the quantized layers; they
  * stand for `rms_norm` and `silu(gate) * up` between the Dense calls of a decoder block), bfloat16:
  * k3q_rmsnorm: y[r, :] = bf16(x[r, :] * rsqrt(mean(x[r, :]^2) + epsilon) * weight[:]), float32
- * arithmetic and one rounding; dim % 8 == 0, dim <= 8192; row strides in elements (% 8 == 0).
+ * arithmetic and one rounding; dim % 8 == 0, dim <= 16384; row strides in elements (% 8 == 0).
  * k3q_silu_mul: y = bf16(bf16(g / (1 + exp(-g))) * u) element by element, rows given by strides.
  */
 int k3q_rmsnorm(const void* x, const void* weight, int dtype, int64_t rows, int64_t dim, int64_t x_row_stride,

@@ -102,6 +102,7 @@ SIGNATURES = {
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr],
     ),
     "k3q_gemv_w4s_multi": (_int, [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr]),
+    "k3q_gemv_w4s_pre": (_int, [_ptr, _int, _i64, _i64, _ptr, _int, _ptr, _i64, _int, _ptr]),
     "k3q_w4_kmajor_pack": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
     "k3q_w8s_shadow_bytes": (_i64, [_i64, _i64]),
     "k3q_w8s_pack": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
@@ -113,6 +114,8 @@ SIGNATURES = {
     "k3q_gemm_i8_w8s": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
     "k3q_dense_i8_w8s_multi": (
         _int, [_ptr, _int, _ptr, _ptr, _i64, _i64, _int, _ptr, _f32, _f32, _f32, _ptr]),
+    "k3q_dense_i8_w8s_pre": (
+        _int, [_ptr, _int, _i64, _i64, _ptr, _int, _ptr, _f32, _f32, _f32, _int, _ptr]),
     "k3q_rmsnorm": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _f32, _ptr, _i64, _ptr]),
     "k3q_silu_mul": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "k3q_decode_attention": (
@@ -149,6 +152,16 @@ class GemvW4sProblem(ctypes.Structure):
 
     _fields_ = [("N", ctypes.c_int64), ("shadow", ctypes.c_void_p), ("scale", ctypes.c_void_p),
                 ("gparams", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p)]
+
+
+class InputOp(ctypes.Structure):
+    """`k3q_input_op` of include/k3q.h."""
+
+    _fields_ = [("kind", ctypes.c_int), ("epsilon", ctypes.c_float), ("operand", ctypes.c_void_p)]
+
+
+K3Q_INPUT_RMS_NORM = 1
+K3Q_INPUT_SILU_GATE = 2
 
 
 class W8sProblem(ctypes.Structure):

@@ -84,6 +84,66 @@ __device__ __forceinline__ float wave_max(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Sum over the 64 lanes of a wave, in every lane, by the same moves (lanes a move does not write
+// add zero).  The tree is fixed: pairs, quads, halves of a row, rows of 16, then
+// (row 3 + row 2) + (row 1 + row 0) -- kernels that must agree bit for bit on a float sum (a
+// normalisation computed alone or inside a matmul kernel) both reduce with this.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_move_or_zero(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_move_or_zero<0xB1, 0xf>(v);
+    v += dpp_move_or_zero<0x4E, 0xf>(v);
+    v += dpp_move_or_zero<0x141, 0xf>(v);
+    v += dpp_move_or_zero<0x140, 0xf>(v);
+    v += dpp_move_or_zero<0x142, 0xa>(v);
+    v += dpp_move_or_zero<0x143, 0xc>(v);
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// Sum of squares of the eight bfloat16 values of a 16-byte piece, float32, fixed order.
+__device__ __forceinline__ float piece_sum_squares(const v4u& c) {
+    float q[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(c[e] << 16), hi = __uint_as_float(c[e] & 0xffff0000u);
+        q[e] = lo * lo + hi * hi;
+    }
+    return (q[0] + q[1]) + (q[2] + q[3]);
+}
+
+// RMS normalisation of a piece: bf16(x * rstd * w), one rounding of the float32 product.
+__device__ __forceinline__ v4u piece_rms_scale(const v4u& x, const v4u& w, float rstd) {
+    v4u o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(x[e] << 16) * rstd * __uint_as_float(w[e] << 16);
+        const float hi = __uint_as_float(x[e] & 0xffff0000u) * rstd * __uint_as_float(w[e] & 0xffff0000u);
+        o[e] = pack_bf16x2(lo, hi);
+    }
+    return o;
+}
+
+// SwiGLU gate of a piece: bf16(bf16(silu(g)) * u), silu(g) = g / (1 + 2^(-g log2 e)) with the
+// hardware's exp2 and reciprocal (each within an ulp or two of float32: the bfloat16 result differs
+// from an exactly rounded one on a fraction of a percent of the elements, by one ulp).
+__device__ __forceinline__ v4u piece_silu_mul(const v4u& g, const v4u& u) {
+    v4u o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float a[2] = {__uint_as_float(g[e] << 16), __uint_as_float(g[e] & 0xffff0000u)};
+        const float b[2] = {__uint_as_float(u[e] << 16), __uint_as_float(u[e] & 0xffff0000u)};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float s = a[h] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a[h] * -1.44269504f));
+            a[h] = round_bf16(s) * b[h];
+        }
+        o[e] = pack_bf16x2(a[0], a[1]);
+    }
+    return o;
+}
+
 // byte select: result byte i = byte sel[i] of the 8-byte pool {lo: bytes 0-3, hi: bytes 4-7}
 __device__ __forceinline__ u32 byte_perm(u32 hi, u32 lo, u32 sel) {
     return __builtin_amdgcn_perm(hi, lo, sel);

@@ -58,6 +58,10 @@ struct W4sParams {
     int slice_magic;         // (x staged in halves) ceil(2^32 / pieces per half slice)
     int own_magic[2];        // (waves stage their own slices) ceil(2^32 / pieces per row of a slice): short, long slice
     int own;                 // 1: every wave stages its own slice of x; 0: the workgroup's threads share all of x
+    // an operation on x on its way into LDS (kernels built with kPre only):
+    int pre_kind;             // 1: rms_norm(x) * pre_op (bf16 [K]); 2: silu(pre_op) * x (pre_op bf16 [M, K])
+    float pre_eps;            // rms_norm's epsilon
+    const uint16_t* pre_op;
 };
 
 struct W4sMulti {
@@ -78,7 +82,11 @@ __device__ __forceinline__ float bf_hi(u32 d) { return __uint_as_float(d & 0xfff
 // kHalves: x does not fit LDS as a whole (9 ... 16 rows of a long K): every wave's slice is cut in two,
 // LDS holds the first halves, then -- once every wave is through with them -- the second halves
 // (one turn per workgroup only: the launch plan sees to it).
-template <int kSW, int kD, int kNP, bool kGrouped, bool kHalves>
+// kPre: x is transformed on its way into LDS (p.pre_kind): the rows are normalised (rms_norm with a
+// gain, as k3q_rmsnorm does, same bits) or multiplied by silu of a second input (as k3q_silu_mul).
+// Every workgroup repeats the transform on all of x -- a few hundred float operations per thread,
+// against a launch and a round trip through memory for the separate kernel.
+template <int kSW, int kD, int kNP, bool kGrouped, bool kHalves, bool kPre = false>
 __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int block, const int stride) {
     extern __shared__ __attribute__((aligned(16))) char w4s_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -105,13 +113,15 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // every row, the only part of x it reads back: nothing is exchanged between waves then, and no
     // barrier stands between a wave's x (the oldest requests in its queue) and its first weights.
     // (Measured: worth 0.3 us up to 32 KiB of x, a loss beyond.)
-    const bool own = !kHalves && p.own;
+    static_assert(!(kPre && kHalves), "no transform of x staged in halves");
+    const bool own = !kHalves && !kPre && p.own;
     const int per_row = kHalves ? K >> 4 : own ? U * 16 : K >> 3;
     const int pieces = M * per_row;
     const u32 row_magic = own ? (u32)p.own_magic[q < extra ? 1 : 0] : (u32)p.row_magic;
     const int own_col = own ? u0 * 16 : 0;  // first piece of the wave's slice within a row
     const int row_pieces = K >> 3;
     v4u xst[kNP];
+    v4u xop[kPre ? kNP : 1];
     auto stage_load = [&](const int h) {
 #pragma unroll
         for (int i = 0; i < kNP; ++i) {
@@ -125,6 +135,8 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
                 xst[i] = *(const v4u*)(p.x + (int64_t)m * K + (int64_t)(qq * U + h * Uh) * 128 + cc * 8);
             } else {
                 xst[i] = *(const v4u*)(p.x + ((int64_t)m * row_pieces + own_col + c) * 8);
+                if constexpr (kPre)  // the gain's piece of this column, or the second input's piece
+                    xop[i] = *(const v4u*)(p.pre_op + (p.pre_kind == 1 ? (int64_t)c : (int64_t)m * row_pieces + c) * 8);
             }
         }
     };
@@ -187,6 +199,39 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
 #pragma unroll
     for (int d = 0; d < kD; ++d) fetch(d, d);
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kPre) {
+        if (p.pre_kind == 1) {
+            // sums of squares: per piece, per block of 64 pieces (a wave's pieces of one turn: K % 512 == 0),
+            // blocks in ascending order -- the order of k3q_rmsnorm
+            float* blk = red;  // [M][blocks per row], then [M] reciprocal root mean squares
+            const int nblk = per_row >> 6;
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                const int first = i * kT + tid - lane;
+                if (first < pieces) {
+                    const float ss = wave_sum(piece_sum_squares(xst[i]));
+                    const int m = (int)__umulhi((unsigned)first, row_magic);
+                    if (lane == 0) blk[m * nblk + ((first - m * per_row) >> 6)] = ss;
+                }
+            }
+            __syncthreads();
+            float* rstd = blk + M * nblk;
+            if (tid < M) {
+                float total = 0.f;
+                for (int b = 0; b < nblk; ++b) total += blk[tid * nblk + b];
+                rstd[tid] = 1.0f / sqrtf(total / (float)K + p.pre_eps);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                const int pi = i * kT + tid;
+                if (pi < pieces) xst[i] = piece_rms_scale(xst[i], xop[i], rstd[(int)__umulhi((unsigned)pi, row_magic)]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) xst[i] = piece_silu_mul(xop[i], xst[i]);
+        }
+    }
     // ---- x into LDS: the stores wait for the x loads only (they are the older ones) ----
     stage_store();
     if (!own) __syncthreads();  // (own slices: a wave reads back only what it wrote itself)
@@ -432,6 +477,14 @@ __global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
     gemv_w4s_body<kSW, kD, kNP, kGrouped, false>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
 }
 
+template <int kSW, int kD, int kNP, bool kGrouped>
+__global__ __launch_bounds__(kT) void gemv_w4s_pre(W4sMulti mp) {
+    const int bx = blockIdx.x;
+    int i = 0;
+    while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
+    gemv_w4s_body<kSW, kD, kNP, kGrouped, false, true>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
+}
+
 // One problem per launch: its parameters ARE the kernel arguments, fetched in one scalar round trip
 // (the several-problem kernel first finds its problem, then fetches that problem's parameters: two
 // dependent round trips more before the first vector load can be issued).
@@ -516,7 +569,7 @@ struct W4sPlan {
 
 constexpr int kResident = 256;  // workgroups the chip holds at once: one per CU (registers)
 
-W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
+W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size, bool pre = false) {
     W4sPlan pl{};
     const bool grouped = block_size > 0;
     if (M < 1 || M > kMaxRows || (K % 128) != 0 || (N % 16) != 0) return pl;
@@ -546,7 +599,7 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
         const int64_t longest = (ring_blocks / kQ + (ring_blocks % kQ ? 1 : 0)) * pl.d;  // units of the longest slice
         const int64_t per_lane = (M * longest * 16 + 63) / 64;
         const int64_t pieces = M * K / 8;
-        pl.own = M * K * 2 <= 32 * 1024 && per_lane <= 4;
+        pl.own = !pre && M * K * 2 <= 32 * 1024 && per_lane <= 4;
         if (pl.own) pl.np = per_lane <= 2 ? 2 : 4;
         else pl.np = pieces <= 2 * kT ? 2 : pieces <= 4 * kT ? 4 : pieces <= 8 * kT ? 8 : 16;
         pl.ok = true;
@@ -556,7 +609,7 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
     pl.lds = (size_t)((M * (K + 16) + 255) & ~255) + red;
     // (grouped kernels with two strips per wave do not fit the register file next to the staged
     // half of x: those calls stay with k3q_gemv_w4)
-    if (M * K / 2 <= stage_max && pl.lds <= lds_limit && turns == 1 && (units % (4 * kQ)) == 0 &&
+    if (!pre && M * K / 2 <= stage_max && pl.lds <= lds_limit && turns == 1 && (units % (4 * kQ)) == 0 &&
         !(grouped && pl.sw == 2)) {
         pl.halves = true;
         pl.d = 2;
@@ -569,15 +622,20 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size) {
 struct W4sKernels {
     void (*multi)(W4sMulti);
     void (*one)(W4sParams);
+    void (*pre)(W4sMulti);  // with a transform of x on its way into LDS
 };
 
 template <int kSW, int kD, bool kGrouped>
 W4sKernels pick_np(int np) {
     switch (np) {
-        case 2: return {gemv_w4s<kSW, kD, 2, kGrouped>, gemv_w4s_one<kSW, kD, 2, kGrouped>};
-        case 4: return {gemv_w4s<kSW, kD, 4, kGrouped>, gemv_w4s_one<kSW, kD, 4, kGrouped>};
-        case 8: return {gemv_w4s<kSW, kD, 8, kGrouped>, gemv_w4s_one<kSW, kD, 8, kGrouped>};
-        default: return {gemv_w4s<kSW, kD, 16, kGrouped>, gemv_w4s_one<kSW, kD, 16, kGrouped>};
+        case 2: return {gemv_w4s<kSW, kD, 2, kGrouped>, gemv_w4s_one<kSW, kD, 2, kGrouped>,
+                        gemv_w4s_pre<kSW, kD, 2, kGrouped>};
+        case 4: return {gemv_w4s<kSW, kD, 4, kGrouped>, gemv_w4s_one<kSW, kD, 4, kGrouped>,
+                        gemv_w4s_pre<kSW, kD, 4, kGrouped>};
+        case 8: return {gemv_w4s<kSW, kD, 8, kGrouped>, gemv_w4s_one<kSW, kD, 8, kGrouped>,
+                        gemv_w4s_pre<kSW, kD, 8, kGrouped>};
+        default: return {gemv_w4s<kSW, kD, 16, kGrouped>, gemv_w4s_one<kSW, kD, 16, kGrouped>,
+                         gemv_w4s_pre<kSW, kD, 16, kGrouped>};
     }
 }
 
@@ -624,14 +682,16 @@ int fill_params(W4sParams& p, const W4sPlan& pl, const void* x, int64_t M, int64
     return K3Q_OK;
 }
 
-int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_blocks, size_t lds, hipStream_t s) {
+int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_blocks, size_t lds, hipStream_t s,
+               bool pre = false) {
     W4sKernels ks = pick_kernel(pl, grouped);
+    if (pre && pl.halves) return K3Q_ERR_SHAPE;
     if (pl.halves) {
         if (mp.count != 1) return K3Q_ERR_SHAPE;
         ks.one = pl.sw == 2 ? (grouped ? gemv_w4s_halves<2, true> : gemv_w4s_halves<2, false>)
                             : (grouped ? gemv_w4s_halves<1, true> : gemv_w4s_halves<1, false>);
     }
-    const void* kernel = mp.count == 1 ? (const void*)ks.one : (const void*)ks.multi;
+    const void* kernel = pre ? (const void*)ks.pre : mp.count == 1 ? (const void*)ks.one : (const void*)ks.multi;
     // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
     {
         static std::mutex mu;
@@ -643,7 +703,8 @@ int launch_w4s(const W4sPlan& pl, bool grouped, const W4sMulti& mp, int total_bl
             raised.insert(kernel);
         }
     }
-    if (mp.count == 1) ks.one<<<(unsigned)total_blocks, kT, lds, s>>>(mp.p[0]);
+    if (pre) ks.pre<<<(unsigned)total_blocks, kT, lds, s>>>(mp);
+    else if (mp.count == 1) ks.one<<<(unsigned)total_blocks, kT, lds, s>>>(mp.p[0]);
     else ks.multi<<<(unsigned)total_blocks, kT, lds, s>>>(mp);
     return launch_status();
 }
@@ -712,16 +773,27 @@ extern "C" int k3q_gemv_w4s(const void* x, int x_dtype, int64_t M, int64_t K, in
     return launch_w4s(pl, block_size > 0, mp, (int)pl.blocks, pl.lds, (hipStream_t)stream);
 }
 
-extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
-                                  const k3q_gemv_w4s_problem* problems, int64_t block_size, void* stream) {
+namespace {
+
+// Problems that share x: launches of up to kMaxProblems problems whose plans agree.  pre: the
+// transform of x (null: none); bias_rows: every bias is [M, N] (a row per row of x) instead of [N].
+int w4s_run_shared(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_input_op* pre, int count,
+                   const k3q_gemv_w4s_problem* problems, int64_t block_size, bool bias_rows, void* stream) {
     if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (count < 0 || M < 0 || K <= 0) return K3Q_ERR_SHAPE;
     if (count == 0 || M == 0) return K3Q_OK;
     if (!problems) return K3Q_ERR_NULL;
+    const bool has_pre = pre != nullptr && pre->kind != K3Q_INPUT_NONE;
+    if (has_pre) {
+        if (pre->kind != K3Q_INPUT_RMS_NORM && pre->kind != K3Q_INPUT_SILU_GATE) return K3Q_ERR_SHAPE;
+        if (!pre->operand) return K3Q_ERR_NULL;
+        if (!aligned_to(pre->operand, 16)) return K3Q_ERR_ALIGN;
+        // (the row sums are taken per block of 64 pieces and kept beside the reduction buffers)
+        if (pre->kind == K3Q_INPUT_RMS_NORM && ((K % 512) != 0 || K > 65536)) return K3Q_ERR_SHAPE;
+    }
     hipStream_t s = (hipStream_t)stream;
     int at = 0;
     while (at < count) {
-        // problems whose plans agree share a launch, up to kMaxProblems at a time
         W4sMulti mp{};
         W4sPlan pl0{};
         int64_t groups[kMaxProblems], total = 0;
@@ -729,13 +801,18 @@ extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t
         for (; at + n < count && n < kMaxProblems; ++n) {
             const k3q_gemv_w4s_problem& q = problems[at + n];
             if (q.N <= 0) return K3Q_ERR_SHAPE;
-            const W4sPlan pl = w4s_plan(M, K, q.N, block_size);
-            if (!pl.ok) return K3Q_ERR_SHAPE;
+            const W4sPlan pl = w4s_plan(M, K, q.N, block_size, has_pre);
+            if (!pl.ok || (has_pre && pl.halves)) return K3Q_ERR_SHAPE;
             if (n == 0) pl0 = pl;
             else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np || pl.own != pl0.own || pl.halves || pl0.halves) break;
             const int rc = fill_params(mp.p[n], pl, x, M, K, q.N, q.shadow, q.scale, q.gparams, block_size,
-                                       q.bias, 0, q.y);
+                                       q.bias, bias_rows ? q.N : 0, q.y);
             if (rc != K3Q_OK) return rc;
+            if (has_pre) {
+                mp.p[n].pre_kind = pre->kind;
+                mp.p[n].pre_eps = pre->epsilon;
+                mp.p[n].pre_op = (const uint16_t*)pre->operand;
+            }
             groups[n] = pl.groups;
             total += pl.groups;
         }
@@ -749,6 +826,7 @@ extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t
             turns = (groups[0] + kResident - 1) / kResident;
             lds = pl0.lds;
         }
+        if (pl0.halves && n != 1) return K3Q_ERR_SHAPE;
         int next_block = 0;
         for (int i = 0; i < n; ++i) {
             mp.first[i] = next_block;
@@ -756,9 +834,22 @@ extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t
         }
         mp.first[n] = next_block;
         mp.count = n;
-        const int rc = launch_w4s(pl0, block_size > 0, mp, next_block, lds, s);
+        const int rc = launch_w4s(pl0, block_size > 0, mp, next_block, lds, s, has_pre);
         if (rc != K3Q_OK) return rc;
         at += n;
     }
     return K3Q_OK;
+}
+
+}  // namespace
+
+extern "C" int k3q_gemv_w4s_multi(const void* x, int x_dtype, int64_t M, int64_t K, int count,
+                                  const k3q_gemv_w4s_problem* problems, int64_t block_size, void* stream) {
+    return w4s_run_shared(x, x_dtype, M, K, nullptr, count, problems, block_size, false, stream);
+}
+
+extern "C" int k3q_gemv_w4s_pre(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_input_op* pre, int count,
+                                const k3q_gemv_w4s_problem* problems, int64_t block_size, int bias_rows,
+                                void* stream) {
+    return w4s_run_shared(x, x_dtype, M, K, pre, count, problems, block_size, bias_rows != 0, stream);
 }

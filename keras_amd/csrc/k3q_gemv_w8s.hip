@@ -41,6 +41,10 @@ struct W8sParams {
     int groups;             // strip groups (kSW strips each)
     int row_magic;          // ceil(2^32 / (K / 8)): piece -> row
     float eps, qlo, qhi;    // quantizer settings (eps already rounded to bfloat16)
+    // an operation on x before it is quantised (kernels built with kPre only):
+    int pre_kind;            // 1: rms_norm(x) * pre_op (bf16 [K]); 2: silu(pre_op) * x (pre_op bf16 [M, K])
+    float pre_eps;           // rms_norm's epsilon
+    const uint16_t* pre_op;
 };
 
 __device__ __forceinline__ float scale_from_amax_bf16(float amax, float eps, float qhi) {
@@ -56,7 +60,9 @@ __device__ __forceinline__ float descale_exact_bf16(int acc, float sa, float sb,
 
 // kNP: 16-byte pieces of x a thread keeps in registers between the row maxima and the
 // quantisation (0: it reads them twice); -1: the rows arrive quantised (p.xq, p.xs).
-template <int kSW, int kD, int kNP>
+// kPre (kNP > 0 only): the rows are transformed before they are quantised (p.pre_kind): rms_norm with
+// a gain, the bits of k3q_rmsnorm, or multiplied by silu of a second input, the bits of k3q_silu_mul.
+template <int kSW, int kD, int kNP, bool kPre = false>
 __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int block, const int n_blocks) {
     extern __shared__ __attribute__((aligned(16))) char w8s_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -151,12 +157,19 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
         // row maxima, scales, int8 rows: abs_max_quantize of the rows inside the workgroup
         const int pieces = M * (K >> 3);  // 16-byte pieces of x (8 values)
         if (tid < kMaxRows8) rowmax[tid] = 0u;
+        static_assert(!kPre || kNP > 0, "the transform works on the pieces kept in registers");
         v4u xr[kNP > 0 ? kNP : 1];
+        v4u xop[kPre ? kNP : 1];
         if (kNP > 0) {
 #pragma unroll
             for (int i = 0; i < kNP; ++i) {
                 const int pi = tid + i * kT;
-                xr[i] = ((const v4u*)p.x)[pi < pieces ? pi : pieces - 1];
+                const int pc = pi < pieces ? pi : pieces - 1;
+                xr[i] = ((const v4u*)p.x)[pc];
+                if constexpr (kPre) {  // the gain's piece of this column, or the second input's piece
+                    const int row = (int)__umulhi((u32)pc, (u32)p.row_magic);
+                    xop[i] = ((const v4u*)p.pre_op)[p.pre_kind == 1 ? pc - row * (K >> 3) : pc];
+                }
             }
             x_before_weights();
         }
@@ -164,6 +177,41 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
         for (int d = 0; d < kD; ++d) refill(d);
         advance();
         __syncthreads();  // rowmax cleared
+        if constexpr (kPre) {
+            if (p.pre_kind == 1) {
+                // sums of squares per piece, per block of 64 pieces (a wave's pieces of one turn), blocks
+                // in ascending order: the order of k3q_rmsnorm.  The reduction buffers are free until
+                // the first group ends.
+                float* blk = (float*)red;  // [M][blocks per row], then [M] reciprocal root mean squares
+                const int per_row = K >> 3, nblk = per_row >> 6;
+#pragma unroll
+                for (int i = 0; i < kNP; ++i) {
+                    const int first = tid + i * kT - lane;
+                    if (first < pieces) {
+                        const float ss = wave_sum(piece_sum_squares(xr[i]));
+                        const int m = (int)__umulhi((u32)first, (u32)p.row_magic);
+                        if (lane == 0) blk[m * nblk + ((first - m * per_row) >> 6)] = ss;
+                    }
+                }
+                __syncthreads();
+                float* rstd = blk + M * nblk;
+                if (tid < M) {
+                    float total = 0.f;
+                    for (int b = 0; b < nblk; ++b) total += blk[tid * nblk + b];
+                    rstd[tid] = 1.0f / sqrtf(total / (float)K + p.pre_eps);
+                }
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < kNP; ++i) {
+                    const int pi = tid + i * kT;
+                    if (pi < pieces)
+                        xr[i] = piece_rms_scale(xr[i], xop[i], rstd[(int)__umulhi((u32)pi, (u32)p.row_magic)]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < kNP; ++i) xr[i] = piece_silu_mul(xop[i], xr[i]);
+            }
+        }
         auto piece_amax = [](const v4u& c) {
             float a = 0.f;
 #pragma unroll
@@ -337,6 +385,14 @@ __global__ __launch_bounds__(kT) void gemv_w8s_multi(W8sMulti mp) {
     gemv_w8s_body<kSW, kD, kNP>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
 }
 
+template <int kSW, int kD, int kNP>
+__global__ __launch_bounds__(kT) void gemv_w8s_pre(W8sMulti mp) {
+    const int bx = blockIdx.x;
+    int i = 0;
+    while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
+    gemv_w8s_body<kSW, kD, kNP, true>(mp.p[i], bx - mp.first[i], mp.first[i + 1] - mp.first[i]);
+}
+
 // One thread per 16-byte lane entry of the copy.  w: the stored int8 kernel, row-major [K, N].
 __global__ __launch_bounds__(256) void w8s_pack(const int8_t* __restrict__ w, v4u* __restrict__ out, int64_t K,
                                                int64_t N, int64_t strips) {
@@ -407,6 +463,21 @@ W8sMultiKernel pick_np8_multi(int np) {
         case 16: return gemv_w8s_multi<kSW, kD, 16>;
         default: return gemv_w8s_multi<kSW, kD, 0>;
     }
+}
+
+template <int kSW, int kD>
+W8sMultiKernel pick_np8_pre(int np) {
+    switch (np) {
+        case 1: return gemv_w8s_pre<kSW, kD, 1>;
+        case 4: return gemv_w8s_pre<kSW, kD, 4>;
+        case 16: return gemv_w8s_pre<kSW, kD, 16>;
+        default: return nullptr;
+    }
+}
+
+W8sMultiKernel pick_kernel8_pre(const W8sPlan& pl) {
+    if (pl.sw == 2) return pl.d == 4 ? pick_np8_pre<2, 4>(pl.np) : pick_np8_pre<2, 2>(pl.np);
+    return pl.d == 4 ? pick_np8_pre<1, 4>(pl.np) : pick_np8_pre<1, 2>(pl.np);
 }
 
 W8sMultiKernel pick_kernel8_multi(const W8sPlan& pl) {
@@ -525,9 +596,10 @@ extern "C" int k3q_gemm_i8_w8s(const int8_t* a, const void* a_scale, int scale_d
                       y, (hipStream_t)stream);
 }
 
-extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* a, const void* a_scale, int64_t M,
-                                      int64_t K, int count, const k3q_w8s_problem* problems, float epsilon,
-                                      float range_lo, float range_hi, void* stream) {
+namespace {
+int w8s_run_shared(const void* x, int x_dtype, const int8_t* a, const void* a_scale, int64_t M, int64_t K,
+                   const k3q_input_op* pre, int count, const k3q_w8s_problem* problems, float epsilon,
+                   float range_lo, float range_hi, bool bias_rows, void* stream) {
     if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (count < 0 || M < 0 || K <= 0) return K3Q_ERR_SHAPE;
     if (!(range_lo >= -128.f && range_hi <= 127.f && range_lo < range_hi)) return K3Q_ERR_SHAPE;
@@ -535,6 +607,13 @@ extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* 
     if (range_lo != rintf(range_lo) || range_hi != rintf(range_hi)) return K3Q_ERR_RANGE;
     if (count == 0 || M == 0) return K3Q_OK;
     if (!problems) return K3Q_ERR_NULL;
+    const bool has_pre = pre != nullptr && pre->kind != K3Q_INPUT_NONE;
+    if (has_pre) {
+        if (a || !x) return K3Q_ERR_NULL;  // the transform works on bfloat16 rows
+        if (pre->kind != K3Q_INPUT_RMS_NORM && pre->kind != K3Q_INPUT_SILU_GATE) return K3Q_ERR_SHAPE;
+        if (!pre->operand) return K3Q_ERR_NULL;
+        if (!aligned_to(pre->operand, 16)) return K3Q_ERR_ALIGN;
+    }
     int at = 0;
     while (at < count) {
         // problems whose plans agree share a launch, up to kMaxProblems8 at a time
@@ -556,9 +635,16 @@ extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* 
             } else if (pl.sw != pl0.sw || pl.d != pl0.d) {
                 break;
             }
-            const int rc = fill_params8(mp.p[n], pl, x, a, a_scale, M, K, q.N, q.shadow, q.kernel_scale, q.bias, 0,
-                                        epsilon, range_lo, range_hi, q.y);
+            const int rc = fill_params8(mp.p[n], pl, x, a, a_scale, M, K, q.N, q.shadow, q.kernel_scale, q.bias,
+                                        bias_rows ? q.N : 0, epsilon, range_lo, range_hi, q.y);
             if (rc != K3Q_OK) return rc;
+            if (has_pre) {
+                // the pieces stay in registers, and the block sums fit the first reduction buffer
+                if (pl.np <= 0 || M * (K / 512 + 1) > 512 * ((M + 3) / 4) * pl.sw) return K3Q_ERR_SHAPE;
+                mp.p[n].pre_kind = pre->kind;
+                mp.p[n].pre_eps = pre->epsilon;
+                mp.p[n].pre_op = (const uint16_t*)pre->operand;
+            }
             groups[n] = pl.groups;
             total += pl.groups;
         }
@@ -581,7 +667,12 @@ extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* 
         mp.count = n;
         if (a) pl0.np = -1;
         int rc;
-        if (n == 1) {
+        if (has_pre) {
+            const W8sMultiKernel kernel = pick_kernel8_pre(pl0);
+            if (!kernel) return K3Q_ERR_SHAPE;
+            if ((rc = raise_lds((const void*)kernel)) != K3Q_OK) return rc;
+            kernel<<<(unsigned)next_block, kT, lds, (hipStream_t)stream>>>(mp);
+        } else if (n == 1) {
             const W8sKernel kernel = pick_kernel8(pl0);
             if ((rc = raise_lds((const void*)kernel)) != K3Q_OK) return rc;
             kernel<<<(unsigned)next_block, kT, lds, (hipStream_t)stream>>>(mp.p[0]);
@@ -594,4 +685,19 @@ extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* 
         at += n;
     }
     return K3Q_OK;
+}
+}  // namespace
+
+extern "C" int k3q_dense_i8_w8s_multi(const void* x, int x_dtype, const int8_t* a, const void* a_scale, int64_t M,
+                                      int64_t K, int count, const k3q_w8s_problem* problems, float epsilon,
+                                      float range_lo, float range_hi, void* stream) {
+    return w8s_run_shared(x, x_dtype, a, a_scale, M, K, nullptr, count, problems, epsilon, range_lo, range_hi, false,
+                          stream);
+}
+
+extern "C" int k3q_dense_i8_w8s_pre(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_input_op* pre,
+                                    int count, const k3q_w8s_problem* problems, float epsilon, float range_lo,
+                                    float range_hi, int bias_rows, void* stream) {
+    return w8s_run_shared(x, x_dtype, nullptr, nullptr, M, K, pre, count, problems, epsilon, range_lo, range_hi,
+                          bias_rows != 0, stream);
 }

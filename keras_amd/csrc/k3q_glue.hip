@@ -8,11 +8,13 @@ namespace {
 
 // y[r, :] = bf16( x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * w[:] ), float32 arithmetic, one rounding.
 // One workgroup of 256 threads per row; D % 8 == 0; a thread keeps up to kMaxChunks 16-byte chunks.
-constexpr int kMaxChunks = 4;  // D <= 8192
+// The sum of squares has a fixed order -- per 16-byte piece, per block of 64 pieces (wave_sum), blocks
+// in ascending order -- which the matmul kernels that normalise their input themselves follow too.
+constexpr int kMaxChunks = 8;  // D <= 16384
 __global__ __launch_bounds__(256) void rmsnorm_rows(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                    uint16_t* __restrict__ y, int D, int64_t x_stride,
                                                    int64_t y_stride, float eps) {
-    __shared__ float part[4];
+    __shared__ float part[4 * kMaxChunks];
     const int tid = threadIdx.x;
     const int chunks = D >> 3;
     const v4u* xr = (const v4u*)(x + (int64_t)blockIdx.x * x_stride);
@@ -24,41 +26,26 @@ __global__ __launch_bounds__(256) void rmsnorm_rows(const uint16_t* __restrict__
         c[i] = xr[cc];
         g[i] = ((const v4u*)w)[cc];
     }
-    float ss = 0.f;
+    // block 4 i + wave holds pieces [64 (4 i + wave), + 64); pieces past the row count zero
 #pragma unroll
     for (int i = 0; i < kMaxChunks; ++i) {
-        if (tid + i * 256 < chunks) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float lo = __uint_as_float(c[i][e] << 16), hi = __uint_as_float(c[i][e] & 0xffff0000u);
-                ss += lo * lo + hi * hi;
-            }
-        }
+        const float ss = wave_sum(tid + i * 256 < chunks ? piece_sum_squares(c[i]) : 0.f);
+        if ((tid & 63) == 0) part[4 * i + (tid >> 6)] = ss;
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
-    if ((tid & 63) == 0) part[tid >> 6] = ss;
     __syncthreads();
-    const float total = (part[0] + part[1]) + (part[2] + part[3]);
+    const int blocks = (chunks + 63) >> 6;
+    float total = 0.f;
+    for (int b = 0; b < blocks; ++b) total += part[b];
     const float rstd = 1.0f / sqrtf(total / (float)D + eps);
     v4u* yr = (v4u*)(y + (int64_t)blockIdx.x * y_stride);
 #pragma unroll
     for (int i = 0; i < kMaxChunks; ++i) {
         const int ci = tid + i * 256;
-        if (ci < chunks) {
-            v4u o;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float lo = __uint_as_float(c[i][e] << 16) * rstd * __uint_as_float(g[i][e] << 16);
-                const float hi = __uint_as_float(c[i][e] & 0xffff0000u) * rstd * __uint_as_float(g[i][e] & 0xffff0000u);
-                o[e] = pack_bf16x2(lo, hi);
-            }
-            yr[ci] = o;
-        }
+        if (ci < chunks) yr[ci] = piece_rms_scale(c[i], g[i], rstd);
     }
 }
 
-// y = bf16( bf16(g / (1 + exp(-g))) * u ): the two roundings of silu(g) followed by the multiply
+// y = bf16( bf16(silu(g)) * u ): the two roundings of silu(g) followed by the multiply (piece_silu_mul)
 __global__ __launch_bounds__(256) void silu_mul_rows(const uint16_t* __restrict__ g, const uint16_t* __restrict__ u,
                                                     uint16_t* __restrict__ y, int chunks_per_row, int64_t g_stride,
                                                     int64_t u_stride, int64_t y_stride, int64_t total_chunks) {
@@ -68,15 +55,7 @@ __global__ __launch_bounds__(256) void silu_mul_rows(const uint16_t* __restrict_
     const int c = (int)(t - r * chunks_per_row);
     const v4u gv = ((const v4u*)(g + r * g_stride))[c];
     const v4u uv = ((const v4u*)(u + r * u_stride))[c];
-    v4u o;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        float a[2] = {__uint_as_float(gv[e] << 16), __uint_as_float(gv[e] & 0xffff0000u)};
-        const float b[2] = {__uint_as_float(uv[e] << 16), __uint_as_float(uv[e] & 0xffff0000u)};
-#pragma unroll
-        for (int h = 0; h < 2; ++h) a[h] = round_bf16(round_bf16(a[h] / (1.0f + expf(-a[h]))) * b[h]);
-        o[e] = pack_bf16x2(a[0], a[1]);
-    }
+    const v4u o = piece_silu_mul(gv, uv);
     ((v4u*)(y + r * y_stride))[c] = o;
 }
 

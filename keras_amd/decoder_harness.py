@@ -33,6 +33,10 @@ class RMSNorm(Layer):
         self.scale = self.add_weight(name="scale", shape=(self.dim,), initializer="ones", trainable=True)
         self.built = True
 
+    def as_input_op(self):
+        """This layer as the `input_op` of `call_together` / `call_add`."""
+        return ("rms_norm", self.read(self.scale), self.epsilon)
+
     def call(self, x, training=None):
         w = self.read(self.scale)
         if x.numel() <= (64 << 10) and kops.rmsnorm_supported(x, w):
@@ -95,16 +99,20 @@ class DecoderBlock(Layer):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
         (an int64 device tensor [T]); mask [T, maxT]: 0 where a key may be attended to, -inf
         elsewhere; tables: the whole (cos, sin) tables, for the one-position kernel."""
-        h = self.attn_norm(x)
-        # the three projections of h in one launch at decode sizes
-        q, k, v = call_together((self.query, self.key, self.value), h)
-        if tables is not None and q.shape[1] == 1 and kops.decode_attention_supported(q, cache[0]):
-            # one position: rotation, cache update and attention in one launch
-            a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
-            x = call_add(self.attn_out, a, x)
-            h = self.ffn_norm(x)
-            gate, up = call_together((self.gate, self.up), h)
-            return call_add(self.down, _silu_mul(gate, up), x)
+        if tables is not None and x.shape[1] == 1 and x.is_cuda and x.dtype == torch.bfloat16:
+            # one position.  The normalisations and the gate ride in the launches of the projections
+            # that consume them (same bits as their own kernels), rotation, cache update and attention
+            # are one launch: 5 launches per block.
+            q, k, v = call_together((self.query, self.key, self.value), x, input_op=self.attn_norm.as_input_op())
+            if kops.decode_attention_supported(q, cache[0]):
+                a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
+                x = call_add(self.attn_out, a, x)
+                gate, up = call_together((self.gate, self.up), x, input_op=self.ffn_norm.as_input_op())
+                return call_add(self.down, up, x, input_op=("silu_gate", gate))
+        else:
+            h = self.attn_norm(x)
+            # the three projections of h in one launch at decode sizes
+            q, k, v = call_together((self.query, self.key, self.value), h)
         # one rotation over the query and key heads together (half the elementwise launches)
         qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
         q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]

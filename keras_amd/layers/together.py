@@ -51,8 +51,13 @@ def quantize_rows(quantizer, x2):
     return hit[0]
 
 
-def call_together(layers, inputs):
-    """`[layer(inputs) for layer in layers]`.
+def call_together(layers, inputs, input_op=None):
+    """`[layer(op(inputs)) for layer in layers]`.
+
+    input_op: None, `("rms_norm", gain, epsilon)` or `("silu_gate", gate)` -- an elementwise /
+    row-wise operation between two layers of a decoder block (`ops.rmsnorm`, `ops.silu_mul`).  At
+    decode sizes the shared launch applies it to the rows on their way into the kernel, with the
+    bits of the separate launch; otherwise it runs as that launch first.
 
     Weight-only int4 `Dense` / `EinsumDense` layers with one compute dtype, input width and
     group size go to `ops.int4_matmul_multi` (one launch at decode sizes); anything else is
@@ -60,13 +65,15 @@ def call_together(layers, inputs):
     them alike (int8 layers: one quantizer launch instead of one per layer).
     """
     with shared_input_rows():
-        return _call_together(layers, inputs)
+        return _call_together(layers, inputs, input_op)
 
 
-def _call_together(layers, inputs):
+def _call_together(layers, inputs, input_op=None):
     layers = list(layers)
-    if len(layers) < 2:
+    if len(layers) < 2 and input_op is None:
         return [layer(inputs) for layer in layers]
+    if not layers:
+        return []
     if not isinstance(inputs, torch.Tensor):
         inputs = torch.as_tensor(np.asarray(inputs))
     first = layers[0]
@@ -74,6 +81,7 @@ def _call_together(layers, inputs):
         if not layer.built:
             layer.build(tuple(inputs.shape))
     if any(l.device != first.device or l.compute_dtype != first.compute_dtype for l in layers):
+        inputs = kops.apply_input_op(input_op, inputs)
         return [layer(inputs) for layer in layers]
     x = inputs.to(first.device) if inputs.device != first.device else inputs
     cd = to_torch_dtype(first.compute_dtype)
@@ -96,7 +104,16 @@ def _call_together(layers, inputs):
                     for s in specs8)):
         eps, rng = specs8[0]["settings"]
         quantizer = specs8[0]["quantizer"]
-        outs = kops.int8_dense_strip_multi(specs8[0]["x2"], [s["kernel"] for s in specs8], epsilon=eps,
+        x2 = specs8[0]["x2"]
+        if input_op is not None and all(kops.int8_strip_input_op_supported(
+                input_op, x2.shape[0], x2.shape[1], s["kernel"]["units"], rng) for s in specs8):
+            outs = kops.int8_dense_strip_multi(x2, [s["kernel"] for s in specs8], epsilon=eps, value_range=rng,
+                                               input_op=input_op)
+            return [s["finish"](y) for s, y in zip(specs8, outs)]
+        if input_op is not None:
+            # (the op as a launch of its own; the layers then see a new tensor of the same shape)
+            return _call_together(layers, kops.apply_input_op(input_op, x))
+        outs = kops.int8_dense_strip_multi(x2, [s["kernel"] for s in specs8], epsilon=eps,
                                            value_range=rng, quantize=lambda rows: quantize_rows(quantizer, rows))
         return [s["finish"](y) for s, y in zip(specs8, outs)]
     specs = []
@@ -104,17 +121,26 @@ def _call_together(layers, inputs):
         make = getattr(layer, "_int4_together_spec", None)
         spec = make(x) if make is not None else None
         if spec is None:
+            x = kops.apply_input_op(input_op, x)
             return [layer(x) for layer in layers]
         specs.append(spec)
     x2 = specs[0]["x2"]
     if x2.shape[0] > 16:
         # beyond decode sizes nothing is shared: every layer takes its own route for the size
+        x = kops.apply_input_op(input_op, x)
         return [layer(x) for layer in layers]
     if any(s["x2"].shape != x2.shape or s["block_size"] != specs[0]["block_size"] for s in specs):
+        x = kops.apply_input_op(input_op, x)
         return [layer(x) for layer in layers]
+    if input_op is not None and not (
+            all(s.get("strip") is not None for s in specs)
+            and all(kops.int4_strip_input_op_supported(input_op, x2.shape[0], x2.shape[1], s["strip"]["units"],
+                                                       specs[0]["block_size"]) for s in specs)):
+        return _call_together(layers, kops.apply_input_op(input_op, x))
     if all(s.get("strip") is not None for s in specs):
         # every kernel has its strip-linear copy for these rows: one launch, no scratch
-        outs = kops.int4_matmul_strip_multi(x2, [s["strip"] for s in specs], block_size=specs[0]["block_size"])
+        outs = kops.int4_matmul_strip_multi(x2, [s["strip"] for s in specs], block_size=specs[0]["block_size"],
+                                            input_op=input_op)
     else:
         outs = kops.int4_matmul_multi(x2, [s["kernel"] for s in specs], block_size=specs[0]["block_size"])
     return [s["finish"](y) for s, y in zip(specs, outs)]
@@ -131,8 +157,55 @@ def _int8_addend_ok(layer, rows, residual):
     return units % 16 == 0 and (kernel.value.numel() // units) % 8 == 0
 
 
-def call_add(layer, inputs, residual):
-    """`residual + layer(inputs)`.
+def _call_add_with_op(layer, inputs, residual, input_op):
+    """`residual + layer(op(inputs))` in one launch where the layer's decode kernel takes the operation
+    and a row of addends per row; None where it does not."""
+    ok = getattr(layer, "_row_bias_ok", None)
+    if not (isinstance(inputs, torch.Tensor) and isinstance(residual, torch.Tensor) and ok is not None
+            and layer.built and layer.quantization_mode in ("int8", "int4") and not layer.lora_enabled
+            and inputs.is_cuda and inputs.numel() > 0 and residual.device == layer.device
+            and inputs.device == layer.device and inputs.dtype == torch.bfloat16
+            and residual.dtype == torch.bfloat16 and to_torch_dtype(layer.compute_dtype) == torch.bfloat16 and ok()):
+        return None
+    x = inputs.contiguous()
+    lent = residual.reshape(-1)
+    lent = lent if lent.is_contiguous() else lent.contiguous()
+    if layer.quantization_mode == "int4":
+        make = getattr(layer, "_int4_together_spec", None)
+        spec = make(x) if make is not None else None
+        if spec is None or spec.get("strip") is None:
+            return None
+        x2, kernel = spec["x2"], dict(spec["strip"])
+        if kernel.get("bias") is not None or lent.numel() != x2.shape[0] * kernel["units"]:
+            return None
+        if not kops.int4_strip_input_op_supported(input_op, x2.shape[0], x2.shape[1], kernel["units"],
+                                                  spec["block_size"]):
+            return None
+        kernel["bias"] = lent
+        (y,) = kops.int4_matmul_strip_multi(x2, [kernel], block_size=spec["block_size"], input_op=input_op,
+                                            bias_rows=True)
+    else:
+        make = getattr(layer, "_int8_together_spec", None)
+        spec = make(x) if make is not None else None
+        if spec is None:
+            return None
+        x2, kernel = spec["x2"], dict(spec["kernel"])
+        eps, rng = spec["settings"]
+        if kernel.get("bias") is not None or lent.numel() != x2.shape[0] * kernel["units"]:
+            return None
+        if not kops.int8_strip_input_op_supported(input_op, x2.shape[0], x2.shape[1], kernel["units"], rng):
+            return None
+        kernel["bias"] = lent
+        (y,) = kops.int8_dense_strip_multi(x2, [kernel], epsilon=eps, value_range=rng, input_op=input_op,
+                                           bias_rows=True)
+    out = spec["finish"](y)
+    if out.numel() != residual.numel():
+        raise ValueError(f"residual of {tuple(residual.shape)} does not match the layer's output {tuple(out.shape)}")
+    return out.reshape(residual.shape)
+
+
+def call_add(layer, inputs, residual, input_op=None):
+    """`residual + layer(op(inputs))` (input_op as in `call_together`; None: the inputs as they are).
 
     For a quantized `Dense` / `EinsumDense` that has neither bias nor activation the add rides
     in the matmul's bias slot: the kernels add a bias to the rounded product,
@@ -142,6 +215,11 @@ def call_add(layer, inputs, residual):
     quantizer; their decode kernels take a row of addends per row of x.  Anything else is the
     plain sum.
     """
+    if input_op is not None:
+        out = _call_add_with_op(layer, inputs, residual, input_op)
+        if out is not None:
+            return out
+        inputs = kops.apply_input_op(input_op, inputs)
     ok = getattr(layer, "_row_bias_ok", None)
     if (isinstance(inputs, torch.Tensor) and isinstance(residual, torch.Tensor) and ok is not None
             and layer.built and layer.quantization_mode in ("int8", "int4") and not layer.lora_enabled

@@ -294,10 +294,12 @@ def int4_matmul_strip(x, shadow, units, kernel_scale=None, gparams=None, block_s
     return y.reshape(*lead, N)
 
 
-def int4_matmul_strip_multi(x, kernels, block_size=None):
-    """`[x . W_i]` for kernels that share `x[..., K]` (up to 8 bfloat16 rows): one launch for those
+def int4_matmul_strip_multi(x, kernels, block_size=None, input_op=None, bias_rows=False):
+    """`[op(x) . W_i]` for kernels that share `x[..., K]` (up to 16 bfloat16 rows): one launch for those
     whose launch plans agree.  kernels: dicts with `shadow`, `units`, `kernel_scale` (per-channel)
-    or `gparams` (grouped), and optionally `bias` [N]."""
+    or `gparams` (grouped), and optionally `bias` [N] (bias_rows: [M, N], a row per row of x).
+    input_op: None, `("rms_norm", gain, epsilon)` or `("silu_gate", gate)`, applied to the rows inside
+    the kernel (`int4_strip_input_op_supported`), with the bits of `rmsnorm` / `silu_mul`."""
     grouped = block_size is not None and block_size > 0
     K = x.shape[-1]
     lead = x.shape[:-1]
@@ -311,8 +313,9 @@ def int4_matmul_strip_multi(x, kernels, block_size=None):
         N = int(k["units"])
         bias = k.get("bias")
         _lib.require_device(x, k["shadow"], k.get("kernel_scale"), k.get("gparams"), bias)
-        if bias is not None and (bias.numel() != N or bias.dtype != torch.bfloat16):
-            raise ValueError(f"bias must hold {N} bfloat16 values")
+        want = M * N if bias_rows else N
+        if bias is not None and (bias.numel() != want or bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
+            raise ValueError(f"bias must hold {want} bfloat16 values, contiguous")
         if k["shadow"].numel() != lib.k3q_w4s_shadow_bytes(K, N):
             raise ValueError("the strip-linear copy does not belong to a [%d, %d] kernel" % (K, N))
         y = torch.empty((M, N), dtype=x.dtype, device=x.device)
@@ -321,10 +324,85 @@ def int4_matmul_strip_multi(x, kernels, block_size=None):
             N, k["shadow"].data_ptr(), None if grouped else k["kernel_scale"].data_ptr(),
             k["gparams"].data_ptr() if grouped else None,
             bias.data_ptr() if bias is not None else None, y.data_ptr())
-    rc = lib.k3q_gemv_w4s_multi(_lib.ptr(x2), _lib.K3Q_BF16, M, K, len(kernels), ctypes.byref(problems),
-                                int(block_size) if grouped else -1, _lib.stream_ptr(x.device))
-    _lib.check(rc, "k3q_gemv_w4s_multi")
+    if input_op is None and not bias_rows:
+        rc = lib.k3q_gemv_w4s_multi(_lib.ptr(x2), _lib.K3Q_BF16, M, K, len(kernels), ctypes.byref(problems),
+                                    int(block_size) if grouped else -1, _lib.stream_ptr(x.device))
+        _lib.check(rc, "k3q_gemv_w4s_multi")
+    else:
+        pre, keep = _input_op_struct(input_op, M, K, x.device)
+        rc = lib.k3q_gemv_w4s_pre(_lib.ptr(x2), _lib.K3Q_BF16, M, K, ctypes.byref(pre) if pre is not None else None,
+                                  len(kernels), ctypes.byref(problems), int(block_size) if grouped else -1,
+                                  1 if bias_rows else 0, _lib.stream_ptr(x.device))
+        _lib.check(rc, "k3q_gemv_w4s_pre")
+        del keep
     return [y.reshape(*lead, y.shape[1]) for y in outs]
+
+
+# rows up to which the gate silu(g) * u is recomputed by every workgroup of a decode matmul (an exp
+# and a reciprocal per value: beyond, the separate launch is cheaper)
+STRIP_SILU_MAX_ROWS = 2
+
+
+def _input_op_struct(input_op, M, K, device):
+    """`k3q_input_op` for `("rms_norm", gain, epsilon)` / `("silu_gate", gate)`; also returns the
+    tensors that must stay alive across the call."""
+    if input_op is None:
+        return None, None
+    kind = input_op[0]
+    if kind == "rms_norm":
+        gain, eps = input_op[1], float(input_op[2])
+        _lib.require_device(gain)
+        if gain.dtype != torch.bfloat16 or gain.numel() != K:
+            raise ValueError(f"the gain must hold {K} bfloat16 values")
+        gain = gain if gain.is_contiguous() else gain.contiguous()
+        return _lib.InputOp(_lib.K3Q_INPUT_RMS_NORM, eps, gain.data_ptr()), gain
+    if kind == "silu_gate":
+        gate = input_op[1]
+        _lib.require_device(gate)
+        if gate.dtype != torch.bfloat16 or gate.numel() != M * K:
+            raise ValueError(f"the gate must hold {M} x {K} bfloat16 values")
+        gate = gate.reshape(M, K)
+        gate = gate if gate.is_contiguous() else gate.contiguous()
+        return _lib.InputOp(_lib.K3Q_INPUT_SILU_GATE, 0.0, gate.data_ptr()), gate
+    raise ValueError(f"unknown input operation {kind!r}")
+
+
+def apply_input_op(input_op, x):
+    """The operation as a launch of its own: `rmsnorm(x, gain, eps)` or `silu_mul(gate, x)`."""
+    if input_op is None:
+        return x
+    if input_op[0] == "rms_norm":
+        gain, eps = input_op[1], float(input_op[2])
+        if rmsnorm_supported(x, gain):
+            return rmsnorm(x, gain, eps)
+        return torch.nn.functional.rms_norm(x, (x.shape[-1],), gain, eps)
+    if input_op[0] == "silu_gate":
+        gate = input_op[1].reshape(x.shape)
+        if silu_mul_supported(gate, x):
+            return silu_mul(gate, x)
+        return torch.nn.functional.silu(gate) * x
+    raise ValueError(f"unknown input operation {input_op[0]!r}")
+
+
+def _input_op_rows_ok(input_op, M, K):
+    if input_op[0] == "rms_norm":
+        return K % 512 == 0 and K <= 65536
+    return input_op[0] == "silu_gate" and M <= STRIP_SILU_MAX_ROWS
+
+
+def int4_strip_input_op_supported(input_op, M, K, N, block_size=None):
+    """Whether `int4_matmul_strip_multi` folds this operation into its launch for these sizes: x whole
+    in a workgroup's LDS (not staged in halves), whole blocks of 512 for the normalisation, few rows
+    for the gate."""
+    bs = int(block_size) if block_size is not None and block_size > 0 else -1
+    return (_input_op_rows_ok(input_op, M, K) and M * K <= 65536
+            and bool(_lib.load().k3q_gemv_w4s_supported(M, K, N, bs)))
+
+
+def int8_strip_input_op_supported(input_op, M, K, N, value_range=(-127, 127)):
+    """The same for `int8_dense_strip_multi`: sizes at which the kernel quantises the rows itself."""
+    return (_input_op_rows_ok(input_op, M, K) and int8_strip_quantises_inside(M, K, value_range)
+            and bool(_lib.load().k3q_dense_i8_w8s_supported(M, K, N)))
 
 
 def int4_kmajor_copy(kernel_packed, units):
@@ -772,11 +850,13 @@ def int8_dense_strip(x, shadow, units, kernel_scale, bias=None, epsilon=1e-7, va
     return y.reshape(*lead, N)
 
 
-def int8_dense_strip_multi(x, kernels, epsilon=1e-7, value_range=(-127, 127), quantize=None):
-    """`[int8_dense_strip(x, k) for k in kernels]` for layers that share `x[..., K]` (up to 16
+def int8_dense_strip_multi(x, kernels, epsilon=1e-7, value_range=(-127, 127), quantize=None, input_op=None,
+                           bias_rows=False):
+    """`[int8_dense_strip(op(x), k) for k in kernels]` for layers that share `x[..., K]` (up to 16
     bfloat16 rows) and quantise it alike: one launch for those whose launch plans agree, the same
     bits as the separate calls.  kernels: dicts with `shadow`, `units`, `kernel_scale` and
-    optionally `bias` [N]."""
+    optionally `bias` [N] (bias_rows: [M, N]).  input_op: as in `int4_matmul_strip_multi`
+    (`int8_strip_input_op_supported`)."""
     lib = _lib.load()
     K = int(x.shape[-1])
     lead = x.shape[:-1]
@@ -797,14 +877,25 @@ def int8_dense_strip_multi(x, kernels, epsilon=1e-7, value_range=(-127, 127), qu
             raise ValueError("shadow is not int8_strip_copy(kernel) of this [K, N]")
         if ks.dtype != torch.bfloat16 or ks.numel() != N:
             raise ValueError(f"kernel_scale must hold {N} bfloat16 values")
-        if bias is not None and (bias.numel() != N or bias.dtype != torch.bfloat16):
-            raise ValueError(f"bias must hold {N} bfloat16 values")
+        want = M * N if bias_rows else N
+        if bias is not None and (bias.numel() != want or bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
+            raise ValueError(f"bias must hold {want} bfloat16 values, contiguous")
         ks = ks if ks.is_contiguous() else ks.contiguous()
         keep.append(ks)
         y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
         outs.append(y)
         problems[i] = _lib.W8sProblem(N, k["shadow"].data_ptr(), ks.data_ptr(),
                                       bias.data_ptr() if bias is not None else None, y.data_ptr())
+    if input_op is not None or bias_rows:
+        if not int8_strip_quantises_inside(M, K, value_range):
+            raise ValueError("input operations and per-row addends need rows the kernel quantises itself")
+        pre, keep_op = _input_op_struct(input_op, M, K, x.device)
+        rc = lib.k3q_dense_i8_w8s_pre(_lib.ptr(x2), _lib.K3Q_BF16, M, K, ctypes.byref(pre) if pre is not None else None,
+                                      len(kernels), ctypes.byref(problems), float(epsilon), float(value_range[0]),
+                                      float(value_range[1]), 1 if bias_rows else 0, _lib.stream_ptr(x.device))
+        _lib.check(rc, "k3q_dense_i8_w8s_pre")
+        del keep_op
+        return [y.reshape(*lead, y.shape[1]) for y in outs]
     q = s = None
     if not int8_strip_quantises_inside(M, K, value_range):
         if quantize is None:
@@ -876,7 +967,7 @@ def _rows_view(t):
 
 def rmsnorm_supported(x, weight):
     return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-            and x.shape[-1] % 8 == 0 and x.shape[-1] <= 8192 and weight.numel() == x.shape[-1])
+            and x.shape[-1] % 8 == 0 and x.shape[-1] <= 16384 and weight.numel() == x.shape[-1])
 
 
 def rmsnorm(x, weight, epsilon):
