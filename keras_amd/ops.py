@@ -384,9 +384,15 @@ def apply_input_op(input_op, x):
     raise ValueError(f"unknown input operation {input_op[0]!r}")
 
 
+# rows up to which the normalisation is repeated by every workgroup (about ten float operations per
+# value: measured at 8 rows of 4096, 4.9 us more in the projections' launch against 4.3 us for the
+# launch saved; at one row 0.6 us)
+STRIP_RMS_MAX_ROWS = 4
+
+
 def _input_op_rows_ok(input_op, M, K):
     if input_op[0] == "rms_norm":
-        return K % 512 == 0 and K <= 65536
+        return K % 512 == 0 and K <= 65536 and M <= STRIP_RMS_MAX_ROWS
     return input_op[0] == "silu_gate" and M <= STRIP_SILU_MAX_ROWS
 
 

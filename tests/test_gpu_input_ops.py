@@ -40,7 +40,8 @@ def int4_kernels(dev, K, Ns, grouped, g):
 @pytest.mark.parametrize("grouped", [False, True])
 @pytest.mark.parametrize("M,K,Ns", [(1, 4096, (4096, 4096, 4096)), (8, 4096, (14336, 14336)), (3, 8192, (8192,)),
                                     (16, 4096, (4096,)), (1, 14336, (4096,)), (2, 4608, (3072, 4096))])
-def test_int4_rms_norm_inside(dev, M, K, Ns, grouped):
+def test_int4_rms_norm_inside(dev, M, K, Ns, grouped, monkeypatch):
+    monkeypatch.setattr(kops, "STRIP_RMS_MAX_ROWS", 16)  # (the kernel takes any decode size; the op layer is choosier)
     g = torch.Generator().manual_seed(M + K + len(Ns))
     x = (torch.randn(M, K, generator=g) * 2).to(torch.bfloat16).to(dev)
     gain = (torch.rand(K, generator=g) + 0.5).to(torch.bfloat16).to(dev)
