@@ -392,7 +392,9 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         }
         __builtin_amdgcn_sched_barrier(0);
     };
-    // a group's end: the slices of K meet in LDS (fixed order), wave 0 applies the layer's epilogue
+    // a group's end: the slices of K meet in LDS, wave t adds them up for strip t (ascending order of the
+    // waves, its own sums from its registers) and applies the layer's epilogue: the two strips of a
+    // group finish side by side instead of one after the other in wave 0
     auto finish = [&](const int grp, const int turn) {
         if (kGrouped) {
             fold((kD - 1) & 1);
@@ -403,32 +405,40 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
                 for (int rr = 0; rr < 4; ++rr)
                     tot[t][rr] = acc[0][t][rr] - 136.0f * accs[0][rr];
         }
-        float* rbuf = red + (turn & 1) * ((kQ - 1) * kSW * M * kRedStride);  // rows of x only
-        if (q > 0 && j < M) {
+        float* rbuf = red + (turn & 1) * (kQ * kSW * M * kRedStride);  // rows of x only
+        auto slot = [&](const int qq, const int t) { return rbuf + ((qq * kSW + t) * M + j) * kRedStride + 4 * g; };
+        if (j < M) {
 #pragma unroll
             for (int t = 0; t < kSW; ++t)
-                *(v4f*)(rbuf + (((q - 1) * kSW + t) * M + j) * kRedStride + 4 * g) = tot[t];
+                if (q != t) *(v4f*)slot(q, t) = tot[t];
         }
         __syncthreads();
-        if (q == 0 && j < M) {
+        auto finalize = [&](auto t_c) {
+            constexpr int t = decltype(t_c)::value;
+            v4f sum = t == 0 ? tot[0] : *(const v4f*)slot(0, t);
 #pragma unroll
-            for (int t = 0; t < kSW; ++t) {
+            for (int qq = 1; qq < kQ; ++qq) {
+                if (qq == t) sum += tot[t];
+                else sum += *(const v4f*)slot(qq, t);
+            }
+            const int n = (grp * kSW + t) * 16 + 4 * g;
+            if (n >= p.N) return;
+            u32 o[4];
 #pragma unroll
-                for (int qq = 1; qq < kQ; ++qq)
-                    tot[t] += *(const v4f*)(rbuf + (((qq - 1) * kSW + t) * M + j) * kRedStride + 4 * g);
-                const int n = (grp * kSW + t) * 16 + 4 * g;
-                if (n >= p.N) continue;
-                u32 o[4];
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    float v = round_bf16(tot[t][rr]);
-                    if (!kGrouped)
-                        v = round_bf16(v / ((rr & 1) ? bf_hi(esc[t][rr >> 1]) : bf_lo(esc[t][rr >> 1])));
-                    if (p.bias) v = round_bf16(v + ((rr & 1) ? bf_hi(ebi[t][rr >> 1]) : bf_lo(ebi[t][rr >> 1])));
-                    o[rr] = f32_to_bf16_bits(v);
-                }
-                const v2u ov = {o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
-                *(v2u*)(p.y + (int64_t)j * p.N + n) = ov;
+            for (int rr = 0; rr < 4; ++rr) {
+                float v = round_bf16(sum[rr]);
+                if (!kGrouped)
+                    v = round_bf16(v / ((rr & 1) ? bf_hi(esc[t][rr >> 1]) : bf_lo(esc[t][rr >> 1])));
+                if (p.bias) v = round_bf16(v + ((rr & 1) ? bf_hi(ebi[t][rr >> 1]) : bf_lo(ebi[t][rr >> 1])));
+                o[rr] = f32_to_bf16_bits(v);
+            }
+            const v2u ov = {o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+            *(v2u*)(p.y + (int64_t)j * p.N + n) = ov;
+        };
+        if (j < M) {
+            if (q == 0) finalize(std::integral_constant<int, 0>{});
+            if constexpr (kSW == 2) {
+                if (q == 1) finalize(std::integral_constant<int, 1>{});
             }
         }
     };
@@ -586,11 +596,11 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size, bool pre =
     // more groups than the chip holds workgroups: each workgroup takes several, one after the other
     const int64_t turns = (pl.groups + kResident - 1) / kResident;
     pl.blocks = (pl.groups + turns - 1) / turns;
-    const size_t red = (size_t)(turns > 1 ? 2 : 1) * (kQ - 1) * pl.sw * M * kRedStride * 4;
+    const size_t red = (size_t)(turns > 1 ? 2 : 1) * kQ * pl.sw * M * kRedStride * 4;
     const int64_t stage_max = (int64_t)kMaxPieces * 8 * kT;  // elements of x a workgroup stages at a time
     const size_t lds_limit = 160 * 1024;
     // x whole in LDS ...
-    const size_t red_one = (size_t)(kQ - 1) * pl.sw * M * kRedStride * 4;
+    const size_t red_one = (size_t)kQ * pl.sw * M * kRedStride * 4;
     pl.lds = (size_t)((M * (K * 2 + 16) + 255) & ~255) + red;
     pl.lds_two = pl.lds - red + 2 * red_one;
     if (M * K <= stage_max && pl.lds <= lds_limit) {
