@@ -89,9 +89,19 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
     const int stride = n_blocks;
     int lg = block, lu = u_begin;
     const int last_group = p.groups - 1;
+    // Workgroups are dealt round-robin to the 8 XCDs, so XCD x would take the strip groups x, x + 8, ...:
+    // addresses a fixed distance apart, and with groups of 256 KiB (K = 8192, two strips) that lands an
+    // XCD's whole stream on a fraction of the memory channels (measured: odd XCDs finished 1 us after
+    // even ones, 15.2 us per call).  Rotating the assignment within every row of eight groups (XCD x
+    // takes group 8 i + (x + i) % 8) spreads each XCD's addresses again: 13.2 us, and 42.9 -> 39.9 us at
+    // N = 28672.  Smaller groups do not alias and keep the plain order (the rotation costs them 0.1 us).
+    const bool rotate = p.units * kSW >= 256;
+    auto place = [&](const int gi) {
+        return rotate && (gi | 7) < p.groups ? (gi & ~7) | ((gi + (gi >> 3)) & 7) : gi;
+    };
     const v4i* nb[kSW];  // this lane's pieces of the block at the cursor, unit by unit 64 entries apart
     auto at_cursor = [&]() {
-        const int g2 = lg < last_group ? lg : last_group;  // past the end: a valid address, never used
+        const int g2 = place(lg < last_group ? lg : last_group);  // past the end: a valid address, never used
 #pragma unroll
         for (int t = 0; t < kSW; ++t) nb[t] = p.w + ((int64_t)(g2 * kSW + t) * p.units + lu) * 64 + lane;
     };
@@ -290,7 +300,7 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
     for (int grp = block; grp < p.groups; grp += stride, ++turn) {
         // epilogue operands of this group, asked for before the group's units (loads return in
         // order: asked for late they would wait for the next group's first units)
-        const int n0 = grp * kSW * 16;
+        const int n0 = place(grp) * kSW * 16;
         u32 sb_raw[kSW], bias_raw[kSW][4];
 #pragma unroll
         for (int t = 0; t < kSW; ++t) {
