@@ -84,6 +84,27 @@ __device__ __forceinline__ float wave_max(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Eight bfloat16 values of a 16-byte piece -> eight int8 (two dwords), abs-max quantisation with the
+// row's scale s: product, its bfloat16 rounding (one conversion per pair), clip, and rint + int
+// conversion in one addition (1.5 * 2^23 + v leaves rint(v), half to even, in the low mantissa bits:
+// the byte is its two's complement).  The clip comes BEFORE the rounding, which equals the reference's
+// round-then-clip only when the ends of the range are integers: callers check that.
+__device__ __forceinline__ v2u quantize_piece_bf16(const v4u& c, float s, float qlo, float qhi) {
+    u32 t[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const u32 pk = pack_bf16x2(__uint_as_float(c[e] << 16) * s, __uint_as_float(c[e] & 0xffff0000u) * s);
+        const float v0 = fminf(fmaxf(__uint_as_float(pk << 16), qlo), qhi);
+        const float v1 = fminf(fmaxf(__uint_as_float(pk & 0xffff0000u), qlo), qhi);
+        t[2 * e] = __float_as_uint(v0 + 12582912.0f);
+        t[2 * e + 1] = __float_as_uint(v1 + 12582912.0f);
+    }
+    const u32 a0 = __builtin_amdgcn_perm(t[1], t[0], 0x0c0c0400u), a1 = __builtin_amdgcn_perm(t[3], t[2], 0x0c0c0400u);
+    const u32 b0 = __builtin_amdgcn_perm(t[5], t[4], 0x0c0c0400u), b1 = __builtin_amdgcn_perm(t[7], t[6], 0x0c0c0400u);
+    const v2u o = {a0 | (a1 << 16), b0 | (b1 << 16)};
+    return o;
+}
+
 // Sum over the 64 lanes of a wave, in every lane, by the same moves (lanes a move does not write
 // add zero).  The tree is fixed: pairs, quads, halves of a row, rows of 16, then
 // (row 3 + row 2) + (row 1 + row 0) -- kernels that must agree bit for bit on a float sum (a

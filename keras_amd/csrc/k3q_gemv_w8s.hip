@@ -253,27 +253,12 @@ __device__ __forceinline__ void gemv_w8s_body(const W8sParams& p, const int bloc
         __syncthreads();
         if (tid < M) sa[tid] = scale_from_amax_bf16(__uint_as_float(rowmax[tid]), p.eps, p.qhi);
         __syncthreads();
-        // Eight values of a piece -> eight int8: product, its bfloat16 rounding (one conversion per
-        // pair), clip, and rint + int conversion in one addition (1.5 * 2^23 + v leaves rint(v), half to
-        // even, in the low mantissa bits: the byte is its two's complement).  The clip comes first:
-        // the range's ends are integers (the entry point sees to it), so it commutes with rint.
+        // (quantize_piece_bf16: the clip before the rounding, exact between the integer ends of the range
+        // that the entry point insists on)
         auto quantize_piece = [&](int pi, const v4u& c) {
             const int row = (int)__umulhi((u32)pi, (u32)p.row_magic);
             const int col = (pi - row * (K >> 3)) << 3;
-            const float s = sa[row];
-            u32 t[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const u32 pk = pack_bf16x2(__uint_as_float(c[e] << 16) * s, __uint_as_float(c[e] & 0xffff0000u) * s);
-                const float v0 = fminf(fmaxf(__uint_as_float(pk << 16), p.qlo), p.qhi);
-                const float v1 = fminf(fmaxf(__uint_as_float(pk & 0xffff0000u), p.qlo), p.qhi);
-                t[2 * e] = __float_as_uint(v0 + 12582912.0f);
-                t[2 * e + 1] = __float_as_uint(v1 + 12582912.0f);
-            }
-            const u32 a0 = byte_perm(t[1], t[0], 0x0c0c0400u), a1 = byte_perm(t[3], t[2], 0x0c0c0400u);
-            const u32 b0 = byte_perm(t[5], t[4], 0x0c0c0400u), b1 = byte_perm(t[7], t[6], 0x0c0c0400u);
-            const v2u o = {a0 | (a1 << 16), b0 | (b1 << 16)};
-            *(v2u*)(xs + row * pitch + col) = o;
+            *(v2u*)(xs + row * pitch + col) = quantize_piece_bf16(c, sa[row], p.qlo, p.qhi);
         };
         if (kNP > 0) {
 #pragma unroll

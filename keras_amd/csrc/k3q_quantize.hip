@@ -74,7 +74,9 @@ __device__ __forceinline__ float row_max(float v, float* lds) {
 // Fast path.  cols % 16 == 0, rows 16-byte aligned.  A thread owns groups of 16 consecutive
 // elements (32 or 64 bytes of input, one 16-byte store of output); kTpr threads share a row
 // (a wave, or the whole 256-thread block), each keeps up to kGroups groups in registers.
-template <int kDtype, int kTpr, int kGroups>
+// kFast (bfloat16 rows, integer ends of the range): quantize_piece_bf16, 7 instructions per value
+// instead of 11 -- at 4096 x 8192 the kernel's arithmetic is otherwise as long as its memory traffic.
+template <int kDtype, int kTpr, int kGroups, bool kFast = false>
 __global__ __launch_bounds__(256) void quantize_rows_vec(const char* __restrict__ x, int64_t rows,
                                                          int64_t groups_per_row,
                                                          int64_t x_row_bytes, float eps, float qlo,
@@ -127,6 +129,14 @@ __global__ __launch_bounds__(256) void quantize_rows_vec(const char* __restrict_
         const int64_t gi = lane + (int64_t)i * kTpr;
         if (gi < groups_per_row) {
             v4u o;
+            if constexpr (kFast) {
+                static_assert(!kFast || kDtype == K3Q_BF16, "the fast form is for bfloat16 rows");
+                const v2u lo = quantize_piece_bf16(c[i][0], s, qlo, qhi), hi = quantize_piece_bf16(c[i][1], s, qlo, qhi);
+                o[0] = lo[0];
+                o[1] = lo[1];
+                o[2] = hi[0];
+                o[3] = hi[1];
+            } else
 #pragma unroll
             for (int j = 0; j < kCpg; ++j) {
                 float f[kPer];
@@ -178,6 +188,13 @@ void launch_vec(const void* x, int64_t rows, int64_t groups_per_row, int64_t row
                 float qlo, float qhi, int8_t* q, void* scale, hipStream_t s) {
     constexpr int kRowsPerBlock = 256 / kTpr;
     unsigned blocks = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+    if constexpr (kDtype == K3Q_BF16) {
+        if (qlo == rintf(qlo) && qhi == rintf(qhi)) {
+            quantize_rows_vec<kDtype, kTpr, kGroups, true><<<blocks, 256, 0, s>>>(
+                (const char*)x, rows, groups_per_row, row_bytes, eps, qlo, qhi, q, scale);
+            return;
+        }
+    }
     quantize_rows_vec<kDtype, kTpr, kGroups><<<blocks, 256, 0, s>>>(
         (const char*)x, rows, groups_per_row, row_bytes, eps, qlo, qhi, q, scale);
 }
