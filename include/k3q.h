@@ -501,6 +501,18 @@ int k3q_dense_i8_w8s_pre(const void* x, int x_dtype, int64_t M, int64_t K, const
                          int bias_rows, void* stream);
 
 /*
+ * The operation and the activation quantizer of the int8 layers behind it in one launch, for any
+ * number of bfloat16 rows (dim % 8 == 0, dim <= 16384, x / operand / h dense): h = op(x) with the
+ * bits of k3q_rmsnorm / k3q_silu_mul, and q, scale = abs-max quantisation of h over the last axis
+ * with the bits of k3q_absmax_quantize (scale bfloat16 [rows]).  Used where the decode kernels do
+ * not fold the operation in themselves (more than a few rows): one launch instead of two, and h
+ * is not read back.  No counterpart in the reference.
+ */
+int k3q_input_op_quantize(const void* x, int dtype, int64_t rows, int64_t dim, const k3q_input_op* pre,
+                          float epsilon, float range_lo, float range_hi, void* h, int8_t* q, void* scale,
+                          void* stream);
+
+/*
  * One new position of causal self-attention against a key / value cache (the decoder
  * harness's step between the quantized projections): rotate-half RoPE of the new query and
  * key with the table rows of *pos, the new key and value rows written into the caches at

@@ -116,6 +116,8 @@ SIGNATURES = {
         _int, [_ptr, _int, _ptr, _ptr, _i64, _i64, _int, _ptr, _f32, _f32, _f32, _ptr]),
     "k3q_dense_i8_w8s_pre": (
         _int, [_ptr, _int, _i64, _i64, _ptr, _int, _ptr, _f32, _f32, _f32, _int, _ptr]),
+    "k3q_input_op_quantize": (
+        _int, [_ptr, _int, _i64, _i64, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr, _ptr]),
     "k3q_rmsnorm": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _f32, _ptr, _i64, _ptr]),
     "k3q_silu_mul": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "k3q_decode_attention": (

@@ -99,32 +99,33 @@ class DecoderBlock(Layer):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
         (an int64 device tensor [T]); mask [T, maxT]: 0 where a key may be attended to, -inf
         elsewhere; tables: the whole (cos, sin) tables, for the one-position kernel."""
-        if tables is not None and x.shape[1] == 1 and x.is_cuda and x.dtype == torch.bfloat16:
-            # one position.  The normalisations and the gate ride in the launches of the projections
-            # that consume them (same bits as their own kernels), rotation, cache update and attention
-            # are one launch: 5 launches per block.
+        # The normalisations and the gate are handed to the projections that consume them as their
+        # `input_op`: at one position they ride inside the projections' launches, in front of int8
+        # layers they share a launch with the activation quantizer, otherwise they run as their own
+        # kernels (same bits every way).
+        fused = x.is_cuda and x.dtype == torch.bfloat16
+        if fused:
             q, k, v = call_together((self.query, self.key, self.value), x, input_op=self.attn_norm.as_input_op())
-            if kops.decode_attention_supported(q, cache[0]):
-                a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
-                x = call_add(self.attn_out, a, x)
-                gate, up = call_together((self.gate, self.up), x, input_op=self.ffn_norm.as_input_op())
-                return call_add(self.down, up, x, input_op=("silu_gate", gate))
         else:
-            h = self.attn_norm(x)
-            # the three projections of h in one launch at decode sizes
-            q, k, v = call_together((self.query, self.key, self.value), h)
-        # one rotation over the query and key heads together (half the elementwise launches)
-        qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
-        q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
-        kc, vc = cache
-        kc.index_copy_(2, pos, k.transpose(1, 2))
-        vc.index_copy_(2, pos, v.transpose(1, 2))
-        a = torch.nn.functional.scaled_dot_product_attention(
-            q.transpose(1, 2), kc, vc, attn_mask=mask[None, None])
-        # (one row: the residual rides in the projection's bias slot, same bits as the add)
-        x = call_add(self.attn_out, a.transpose(1, 2), x)
-        h = self.ffn_norm(x)
-        gate, up = call_together((self.gate, self.up), h)
+            q, k, v = call_together((self.query, self.key, self.value), self.attn_norm(x))
+        if tables is not None and q.shape[1] == 1 and kops.decode_attention_supported(q, cache[0]):
+            # one position: rotation, cache update and attention in one launch (5 launches per block)
+            a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
+        else:
+            # one rotation over the query and key heads together (half the elementwise launches)
+            qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
+            q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
+            kc, vc = cache
+            kc.index_copy_(2, pos, k.transpose(1, 2))
+            vc.index_copy_(2, pos, v.transpose(1, 2))
+            a = torch.nn.functional.scaled_dot_product_attention(
+                q.transpose(1, 2), kc, vc, attn_mask=mask[None, None]).transpose(1, 2)
+        # (the residual rides in the projection's bias slot where it can, same bits as the add)
+        x = call_add(self.attn_out, a, x)
+        if fused:
+            gate, up = call_together((self.gate, self.up), x, input_op=self.ffn_norm.as_input_op())
+            return call_add(self.down, up, x, input_op=("silu_gate", gate))
+        gate, up = call_together((self.gate, self.up), self.ffn_norm(x))
         return call_add(self.down, _silu_mul(gate, up), x)
 
 

@@ -42,13 +42,39 @@ def quantize_rows(quantizer, x2):
     config = getattr(quantizer, "get_config", None)
     if memo is None or config is None:
         return quantizer(x2, axis=-1)
-    key = (type(quantizer), repr(sorted(config().items())), x2.data_ptr(), tuple(x2.shape),
-           tuple(x2.stride()), x2.dtype, x2._version)
+    key = _quantizer_key(quantizer, x2)
     hit = memo.get(key)
     if hit is None:
         # the memo keeps x2 alive, so its address cannot be handed to another tensor meanwhile
         hit = memo[key] = (quantizer(x2, axis=-1), x2)
     return hit[0]
+
+
+def _quantizer_key(quantizer, x2):
+    return (type(quantizer), repr(sorted(quantizer.get_config().items())), x2.data_ptr(), tuple(x2.shape),
+            tuple(x2.stride()), x2.dtype, x2._version)
+
+
+def apply_input_op_for(layers, input_op, x):
+    """`op(x)` for layers about to be called on it.  Where all of them are int8 layers that quantise
+    their input with the same plain abs-max quantizer, the operation and that quantizer run as ONE
+    launch and the quantised rows are left in the enclosing `shared_input_rows()` for the layers to
+    pick up (same bits as the two launches); otherwise the operation's own launch."""
+    from keras_amd import quantizers
+
+    memo = getattr(_state, "memo", None)
+    if memo is not None and isinstance(x, torch.Tensor) and x.dim() >= 2:
+        qs = [getattr(l, "inputs_quantizer", None) for l in layers]
+        first = qs[0] if qs else None
+        x2 = x.reshape(-1, x.shape[-1])
+        if (first is not None and all(l.quantization_mode == "int8" and type(q) is quantizers.AbsMaxQuantizer
+                                      and q.output_dtype == "int8" and q.axis in (None, (-1,))
+                                      and q.get_config() == first.get_config() for l, q in zip(layers, qs))
+                and kops.input_op_quantize_supported(input_op, x2)):
+            h2, q, s = kops.input_op_quantize(input_op, x2, epsilon=first.epsilon, value_range=first.value_range)
+            memo[_quantizer_key(first, h2)] = ((q, s), h2)
+            return h2.reshape(x.shape)
+    return kops.apply_input_op(input_op, x)
 
 
 def call_together(layers, inputs, input_op=None):
@@ -81,7 +107,7 @@ def _call_together(layers, inputs, input_op=None):
         if not layer.built:
             layer.build(tuple(inputs.shape))
     if any(l.device != first.device or l.compute_dtype != first.compute_dtype for l in layers):
-        inputs = kops.apply_input_op(input_op, inputs)
+        inputs = apply_input_op_for(layers, input_op, inputs)
         return [layer(inputs) for layer in layers]
     x = inputs.to(first.device) if inputs.device != first.device else inputs
     cd = to_torch_dtype(first.compute_dtype)
@@ -112,7 +138,7 @@ def _call_together(layers, inputs, input_op=None):
             return [s["finish"](y) for s, y in zip(specs8, outs)]
         if input_op is not None:
             # (the op as a launch of its own; the layers then see a new tensor of the same shape)
-            return _call_together(layers, kops.apply_input_op(input_op, x))
+            return _call_together(layers, apply_input_op_for(layers, input_op, x))
         outs = kops.int8_dense_strip_multi(x2, [s["kernel"] for s in specs8], epsilon=eps,
                                            value_range=rng, quantize=lambda rows: quantize_rows(quantizer, rows))
         return [s["finish"](y) for s, y in zip(specs8, outs)]
@@ -121,22 +147,22 @@ def _call_together(layers, inputs, input_op=None):
         make = getattr(layer, "_int4_together_spec", None)
         spec = make(x) if make is not None else None
         if spec is None:
-            x = kops.apply_input_op(input_op, x)
+            x = apply_input_op_for(layers, input_op, x)
             return [layer(x) for layer in layers]
         specs.append(spec)
     x2 = specs[0]["x2"]
     if x2.shape[0] > 16:
         # beyond decode sizes nothing is shared: every layer takes its own route for the size
-        x = kops.apply_input_op(input_op, x)
+        x = apply_input_op_for(layers, input_op, x)
         return [layer(x) for layer in layers]
     if any(s["x2"].shape != x2.shape or s["block_size"] != specs[0]["block_size"] for s in specs):
-        x = kops.apply_input_op(input_op, x)
+        x = apply_input_op_for(layers, input_op, x)
         return [layer(x) for layer in layers]
     if input_op is not None and not (
             all(s.get("strip") is not None for s in specs)
             and all(kops.int4_strip_input_op_supported(input_op, x2.shape[0], x2.shape[1], s["strip"]["units"],
                                                        specs[0]["block_size"]) for s in specs)):
-        return _call_together(layers, kops.apply_input_op(input_op, x))
+        return _call_together(layers, apply_input_op_for(layers, input_op, x))
     if all(s.get("strip") is not None for s in specs):
         # every kernel has its strip-linear copy for these rows: one launch, no scratch
         outs = kops.int4_matmul_strip_multi(x2, [s["strip"] for s in specs], block_size=specs[0]["block_size"],
@@ -219,7 +245,8 @@ def call_add(layer, inputs, residual, input_op=None):
         out = _call_add_with_op(layer, inputs, residual, input_op)
         if out is not None:
             return out
-        inputs = kops.apply_input_op(input_op, inputs)
+        with shared_input_rows():
+            return call_add(layer, apply_input_op_for([layer], input_op, inputs), residual)
     ok = getattr(layer, "_row_bias_ok", None)
     if (isinstance(inputs, torch.Tensor) and isinstance(residual, torch.Tensor) and ok is not None
             and layer.built and layer.quantization_mode in ("int8", "int4") and not layer.lora_enabled

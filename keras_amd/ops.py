@@ -390,6 +390,33 @@ def apply_input_op(input_op, x):
 STRIP_RMS_MAX_ROWS = 4
 
 
+def input_op_quantize_supported(input_op, x2):
+    """Whether `input_op_quantize` takes these rows: bfloat16 on the device, dense, rows of whole
+    16-byte pieces up to 16384 values."""
+    K = x2.shape[-1]
+    return (input_op is not None and input_op[0] in ("rms_norm", "silu_gate") and x2.is_cuda
+            and x2.dtype == torch.bfloat16 and x2.dim() == 2 and x2.is_contiguous() and K % 8 == 0 and 0 < K <= 16384
+            and x2.shape[0] > 0)
+
+
+def input_op_quantize(input_op, x2, epsilon=1e-7, value_range=(-127, 127)):
+    """`h = op(x2)` and `q, scale = abs_max_quantize(h, axis=-1)` in one launch, the bits of the
+    separate kernels (`apply_input_op`, `quantizers.abs_max_quantize`).  x2 `[M, K]` bfloat16; returns
+    `(h, q, scale)` with scale `[M, 1]` bfloat16."""
+    _lib.require_device(x2)
+    M, K = (int(d) for d in x2.shape)
+    pre, keep = _input_op_struct(input_op, M, K, x2.device)
+    h = torch.empty_like(x2)
+    q = torch.empty((M, K), dtype=torch.int8, device=x2.device)
+    s = torch.empty((M,), dtype=torch.bfloat16, device=x2.device)
+    rc = _lib.load().k3q_input_op_quantize(_lib.ptr(x2), _lib.K3Q_BF16, M, K, ctypes.byref(pre), float(epsilon),
+                                           float(value_range[0]), float(value_range[1]), _lib.ptr(h), _lib.ptr(q),
+                                           _lib.ptr(s), _lib.stream_ptr(x2.device))
+    _lib.check(rc, "k3q_input_op_quantize")
+    del keep
+    return h, q, s.reshape(M, 1)
+
+
 def _input_op_rows_ok(input_op, M, K):
     if input_op[0] == "rms_norm":
         return K % 512 == 0 and K <= 65536 and M <= STRIP_RMS_MAX_ROWS

@@ -150,3 +150,29 @@ def test_layers_with_input_ops_match_separate_launches(dev, mode, rows):
     got = call_add(down, up, res, input_op=("silu_gate", gate))
     want = call_add(down, kops.silu_mul(gate, up), res)
     assert got.shape == want.shape and torch.equal(bits(got), bits(want))
+
+
+@pytest.mark.parametrize("value_range", [(-127, 127), (-100.5, 90.25)])
+@pytest.mark.parametrize("rows,dim,kind", [(8, 4096, "rms_norm"), (1, 4096, "rms_norm"), (1024, 4096, "rms_norm"),
+                                           (5, 14336, "silu_gate"), (8, 14336, "rms_norm"), (3, 136, "rms_norm"),
+                                           (16, 16384, "silu_gate")])
+def test_input_op_quantize_matches_the_two_launches(dev, rows, dim, kind, value_range):
+    """k3q_input_op_quantize: h, q and scale carry the bits of k3q_rmsnorm / k3q_silu_mul followed by
+    k3q_absmax_quantize."""
+    from keras_amd import quantizers as kq
+
+    g = torch.Generator().manual_seed(rows + dim)
+    x = (torch.randn(rows, dim, generator=g) * 2).to(torch.bfloat16).to(dev)
+    if rows > 2:
+        x[1] = 0  # an all-zero row: scale = range / eps
+    if kind == "rms_norm":
+        op = ("rms_norm", (torch.rand(dim, generator=g) + 0.5).to(torch.bfloat16).to(dev), 1e-6)
+    else:
+        op = ("silu_gate", (torch.randn(rows, dim, generator=g) * 2).to(torch.bfloat16).to(dev))
+    assert kops.input_op_quantize_supported(op, x)
+    h, q, s = kops.input_op_quantize(op, x, epsilon=1e-7, value_range=value_range)
+    want_h = kops.apply_input_op(op, x)
+    want_q, want_s = kq.abs_max_quantize(want_h, axis=-1, value_range=value_range, epsilon=1e-7)
+    assert torch.equal(bits(h), bits(want_h))
+    assert s.shape == want_s.shape and torch.equal(bits(s), bits(want_s))
+    assert torch.equal(q, want_q)
