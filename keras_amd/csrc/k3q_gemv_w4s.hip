@@ -55,7 +55,8 @@ struct W4sParams {
     int64_t bias_stride;     // 0 or N
     int M, K, N, units;      // units = K / 128
     int row_magic;           // ceil(2^32 / pieces per staged row): piece -> row without a division
-    int slice_magic;         // (x staged in halves) ceil(2^32 / pieces per half slice)
+    int slice_magic;         // (x staged in two parts) ceil(2^32 / pieces of a slice's first part); row_magic: of a row's
+    int row_magic2, slice_magic2;  // the same for the second part
     int own_magic[2];        // (waves stage their own slices) ceil(2^32 / pieces per row of a slice): short, long slice
     int own;                 // 1: every wave stages its own slice of x; 0: the workgroup's threads share all of x
     // an operation on x on its way into LDS (kernels built with kPre only):
@@ -102,8 +103,12 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     const int U = (base + (q < extra ? 1 : 0)) * kD;
     const int u0 = (q * base + (q < extra ? q : extra)) * kD;
     const int R = U / kD;  // >= 2 (the launch plan sees to it)
-    const int Uh = kHalves ? U / 2 : U;  // units of a slice whose x is in LDS at a time
-    const int pitch = (kHalves ? K : K * 2) + 16;
+    // kHalves: LDS holds the first Rh rounds' worth of every wave's slice, then the rest (the two parts
+    // are equal when the slice has an even number of rounds)
+    const int Rh = kHalves ? (R + 1) / 2 : R;
+    const int Uh = Rh * kD;    // units of a slice whose x is in LDS at a time (the first part)
+    const int Uh2 = U - Uh;    // (kHalves) the second part
+    const int pitch = (kHalves ? kQ * Uh * 256 : K * 2) + 16;
     // (two buffers, one per parity of the turn, when a workgroup takes several turns)
     float* red = (float*)(w4s_lds + ((M * pitch + 255) & ~255));
 
@@ -115,7 +120,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // (Measured: worth 0.3 us up to 32 KiB of x, a loss beyond.)
     static_assert(!(kPre && kHalves), "no transform of x staged in halves");
     const bool own = !kHalves && !kPre && p.own;
-    const int per_row = kHalves ? K >> 4 : own ? U * 16 : K >> 3;
+    const int per_row = own ? U * 16 : K >> 3;  // (kHalves: per part, below)
     const int pieces = M * per_row;
     const u32 row_magic = own ? (u32)p.own_magic[q < extra ? 1 : 0] : (u32)p.row_magic;
     const int own_col = own ? u0 * 16 : 0;  // first piece of the wave's slice within a row
@@ -123,24 +128,49 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     v4u xst[kNP];
     v4u xop[kPre ? kNP : 1];
     auto stage_load = [&](const int h) {
+        if constexpr (kHalves) {
+            // part h of every wave's slice: row m of LDS = [slice 0's part | slice 1's part | ...]
+            const int uw = h ? Uh2 : Uh, part_row = kQ * uw * 16, part_pieces = M * part_row;
+            const u32 rm = (u32)(h ? p.row_magic2 : p.row_magic), sm = (u32)(h ? p.slice_magic2 : p.slice_magic);
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                int pi = i * kT + tid;
+                pi = pi < part_pieces ? pi : 0;
+                const int m = (int)__umulhi((unsigned)pi, rm);
+                const int c = pi - m * part_row;
+                const int qq = (int)__umulhi((unsigned)c, sm);  // c / (uw * 16): the slice
+                const int cc = c - qq * (uw * 16);
+                xst[i] = *(const v4u*)(p.x + (int64_t)m * K + (int64_t)(qq * U + (h ? Uh : 0)) * 128 + cc * 8);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < kNP; ++i) {
             int pi = own ? i * 64 + lane : i * kT + tid;
             pi = pi < pieces ? pi : 0;
             const int m = (int)__umulhi((unsigned)pi, row_magic);
             const int c = pi - m * per_row;
-            if (kHalves) {
-                const int qq = (int)__umulhi((unsigned)c, (unsigned)p.slice_magic);  // c / (Uh * 16)
-                const int cc = c - qq * (Uh * 16);
-                xst[i] = *(const v4u*)(p.x + (int64_t)m * K + (int64_t)(qq * U + h * Uh) * 128 + cc * 8);
-            } else {
+            {
                 xst[i] = *(const v4u*)(p.x + ((int64_t)m * row_pieces + own_col + c) * 8);
                 if constexpr (kPre)  // the gain's piece of this column, or the second input's piece
                     xop[i] = *(const v4u*)(p.pre_op + (p.pre_kind == 1 ? (int64_t)c : (int64_t)m * row_pieces + c) * 8);
             }
         }
     };
-    auto stage_store = [&]() {
+    auto stage_store = [&](const int h) {
+        if constexpr (kHalves) {
+            const int part_row = kQ * (h ? Uh2 : Uh) * 16, part_pieces = M * part_row;
+            const u32 rm = (u32)(h ? p.row_magic2 : p.row_magic);
+#pragma unroll
+            for (int i = 0; i < kNP; ++i) {
+                const int pi = i * kT + tid;
+                if (pi < part_pieces) {
+                    const int m = (int)__umulhi((unsigned)pi, rm);
+                    *(v4u*)(w4s_lds + m * pitch + (pi - m * part_row) * 16) = xst[i];
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < kNP; ++i) {
             const int pi = own ? i * 64 + lane : i * kT + tid;
@@ -243,10 +273,10 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         }
     }
     // ---- x into LDS: the stores wait for the x loads only (they are the older ones) ----
-    stage_store();
+    stage_store(0);
     if (!own) __syncthreads();  // (own slices: a wave reads back only what it wrote itself)
 
-    const char* xrow = w4s_lds + jj * pitch + (kHalves ? q * Uh : u0) * 256 + g * 16;
+    const char* xrow = w4s_lds + jj * pitch + (kHalves ? q * Uh : u0) * 256 + g * 16;  // (kHalves: of the part in LDS)
     const v4u ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
     // (three MFMAs per step with kSW = 2, two with one strip: a strip's own chain has the others between
@@ -470,7 +500,6 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // falls past the end re-reads the group's first unit: never used)
     begin(grp, grp);
     if constexpr (kHalves) {
-        const int Rh = R / 2;
         for (int r = 0; r < Rh - 1; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
         // the last round on the first halves: the second halves are requested now and written once
         // every wave has read its last fragments of the first (its MFMAs hold them in registers)
@@ -478,9 +507,10 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         __builtin_amdgcn_sched_barrier(0);
         round(bool_constant<false>{}, Rh - 1, bool_constant<true>{});
         __syncthreads();
-        stage_store();
+        stage_store(1);
+        xrow = w4s_lds + jj * pitch + q * Uh2 * 256 + g * 16;
         __syncthreads();
-        read_x(0, 0);  // unit U / 2, the first of the second half (buffer 0: kD is even)
+        read_x(0, 0);  // unit Uh, the first of the second part (buffer 0: kD is even)
         for (int r = Rh; r < R - 1; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
     } else {
         for (int r = 0; r < R - 1; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
@@ -625,12 +655,13 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size, bool pre =
         pl.ok = true;
         return pl;
     }
-    // ... or in two halves: equal slices of whole ring rounds per half, one turn per workgroup
-    pl.lds = (size_t)((M * (K + 16) + 255) & ~255) + red;
-    // (grouped kernels with two strips per wave do not fit the register file next to the staged
-    // half of x: those calls stay with k3q_gemv_w4)
-    if (!pre && M * K / 2 <= stage_max && pl.lds <= lds_limit && turns == 1 && (units % (4 * kQ)) == 0 &&
-        !(grouped && pl.sw == 2)) {
+    // ... or in two parts: equal slices of whole rounds of a ring of two, the first part the larger one
+    // when the rounds are odd; one turn per workgroup
+    const int64_t slice_rounds = units / (2 * kQ);               // rounds of a wave's slice (ring of 2)
+    const int64_t first_units = (slice_rounds + 1) / 2 * 2;      // units of a slice in the first part
+    pl.lds = (size_t)((M * (kQ * first_units * 256 + 16) + 255) & ~255) + red;
+    if (!pre && (units % (2 * kQ)) == 0 && slice_rounds >= 2 && M * kQ * first_units * 128 <= stage_max &&
+        pl.lds <= lds_limit && turns == 1) {
         pl.halves = true;
         pl.d = 2;
         pl.np = 16;
@@ -697,8 +728,17 @@ int fill_params(W4sParams& p, const W4sPlan& pl, const void* x, int64_t M, int64
         }
     }
     p.own = pl.own ? 1 : 0;
-    const uint64_t per_half_slice = (uint64_t)(K / 128 / kQ / 2) * 16;
-    p.slice_magic = pl.halves ? (int)(uint32_t)((((uint64_t)1 << 32) + per_half_slice - 1) / per_half_slice) : 0;
+    p.slice_magic = p.row_magic2 = p.slice_magic2 = 0;
+    if (pl.halves) {
+        // pieces per slice and per row of LDS, first and second part
+        const uint64_t slice_units = (uint64_t)(K / 128) / kQ, rounds = slice_units / 2;
+        const uint64_t first = (rounds + 1) / 2 * 2, second = slice_units - first;
+        auto magic = [](uint64_t d) { return (int)(uint32_t)((((uint64_t)1 << 32) + d - 1) / d); };
+        p.row_magic = magic(kQ * first * 16);
+        p.slice_magic = magic(first * 16);
+        p.row_magic2 = magic(kQ * second * 16);
+        p.slice_magic2 = magic(second * 16);
+    }
     return K3Q_OK;
 }
 

@@ -75,10 +75,7 @@ def run_strip_case(dev, M, K, N, block_size, with_bias, seed=0):
 @pytest.mark.parametrize("M", [1, 4, 8, 9, 16])
 @pytest.mark.parametrize("block_size", [None, 128])
 def test_strip_decode_config(dev, M, block_size):
-    # target configuration 2: K = N = 8192 (grouped kernels above 8 rows stay on the stored-kernel route)
-    if block_size and M > 8:
-        assert not kops.int4_strip_supported(M, 8192, 8192, block_size)
-        return
+    # target configuration 2: K = N = 8192 (above 8 rows x is staged in two parts)
     run_strip_case(dev, M, 8192, 8192, block_size, with_bias=False)
 
 
@@ -88,6 +85,9 @@ def test_strip_decode_config(dev, M, block_size):
     (1, 28672, 4096, None), (4, 5120, 13824, 128), (2, 6144, 6144, None),
     (16, 4096, 4096, 128), (12, 4096, 14336, None), (16, 8192, 4096, 128), (10, 12288, 3072, None),
     (16, 8192, 8192, None), (16, 8192, 4096, 128),
+    # x staged in two unequal parts (a slice of 7 or 5 rounds of the ring)
+    (8, 14336, 4096, 128), (8, 14336, 4096, None), (5, 14336, 4096, 128), (7, 14336, 3584, None),
+    (9, 10240, 4096, 128), (10, 10240, 8192, None), (16, 6144, 4096, 128), (12, 8192, 8192, 128),
 ])
 def test_strip_shapes(dev, M, K, N, block_size):
     run_strip_case(dev, M, K, N, block_size, with_bias=(M % 2 == 1), seed=M)
@@ -96,7 +96,7 @@ def test_strip_shapes(dev, M, K, N, block_size):
 def test_strip_rejects_what_it_does_not_take(dev):
     for M, K, N, bs in [(17, 4096, 4096, None), (16, 14336, 4096, 128), (9, 8192, 16384, None), (1, 4096, 4096, 64),
                         (16, 4096, 32000, 128), (1, 4000, 4096, None),
-                        (1, 4096, 1024, None), (1, 4096, 4104, None), (8, 14336, 4096, 128),
+                        (1, 4096, 1024, None), (1, 4096, 4104, None), (9, 14336, 4096, 128),
                         (1, 1024, 4096, None), (1, 128 * 33, 4096, None), (1, 2048, 4096, None)]:
         assert not kops.int4_strip_supported(M, K, N, bs), (M, K, N, bs)
     lib = _lib.load()
