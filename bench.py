@@ -460,7 +460,10 @@ def main():
                           + ("" if kops.int8_strip_quantises_inside(M8, Kg, (-127, 127)) else " + quantize_rows_vec"),
                           "us_per_call": round(us, 2), "algorithmic_bytes": nbytes,
                           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                                       "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}})
+                                       "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                                       "traffic": measured_traffic(
+                                           "gemv_w8s_M1" if kops.int8_strip_quantises_inside(M8, Kg, (-127, 127))
+                                           else "gemv_w8s_prequantised")}})
             del graph, x8
         read_ref8 = read_reference(s8, Kg * Ng)
         if read_ref8:

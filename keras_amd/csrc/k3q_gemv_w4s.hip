@@ -519,8 +519,13 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     finish(grp, turn);
 }
 
+// One strip per wave and a ring of two: held to 128 registers (four waves per SIMD; they need 129
+// unbounded), so that two workgroups fit a CU.  A launch shared by several problems can have a few
+// workgroups more than the chip has CUs (three problems of 256 groups in three turns: 3 x 86 = 258);
+// with one workgroup per CU the two extra ones would run after all the others (measured: 10.0 ->
+// 14.5 us for the query / key / value launch).  The other forms spill under that bound and keep theirs.
 template <int kSW, int kD, int kNP, bool kGrouped>
-__global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
+__global__ __launch_bounds__(kT, (kSW == 1 && kD == 2) ? 4 : 1) void gemv_w4s(W4sMulti mp) {
     const int bx = blockIdx.x;
     int i = 0;
     while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
@@ -528,7 +533,7 @@ __global__ __launch_bounds__(kT) void gemv_w4s(W4sMulti mp) {
 }
 
 template <int kSW, int kD, int kNP, bool kGrouped>
-__global__ __launch_bounds__(kT) void gemv_w4s_pre(W4sMulti mp) {
+__global__ __launch_bounds__(kT, (kSW == 1 && kD == 2 && kNP <= 8) ? 4 : 1) void gemv_w4s_pre(W4sMulti mp) {
     const int bx = blockIdx.x;
     int i = 0;
     while (i + 1 < mp.count && bx >= mp.first[i + 1]) ++i;
