@@ -618,13 +618,16 @@ struct W4sPlan {
     int sw, d, np;
     int64_t groups;  // strip groups (kSW strips each)
     int64_t blocks;  // workgroups: each takes groups block, block + blocks, ...
+    int64_t resident;  // workgroups of this kernel form the chip holds at once (256 or 512)
     size_t lds;      // dynamic LDS of a launch of this problem alone
     size_t lds_two;  // the same with both reduction buffers: what a launch needs whose workgroups take turns
 };
 
 constexpr int kResident = 256;  // workgroups the chip holds at once: one per CU (registers)
 
-W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size, bool pre = false) {
+// shared: the plan is for a launch that several problems share (the kernels of such launches are
+// held to 128 registers where that costs nothing, the one-problem kernel is not)
+W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size, bool pre = false, bool shared = false) {
     W4sPlan pl{};
     const bool grouped = block_size > 0;
     if (M < 1 || M > kMaxRows || (K % 128) != 0 || (N % 16) != 0) return pl;
@@ -637,9 +640,20 @@ W4sPlan w4s_plan(int64_t M, int64_t K, int64_t N, int64_t block_size, bool pre =
     else if ((units % 2) == 0 && units / 2 >= 2 * kQ) pl.d = 2;
     else return pl;
     pl.sw = strips >= 2 * kResident ? 2 : 1;
+    pl.resident = kResident;
+    // One strip per wave with a ring of two stays within 128 registers, so two workgroups fit a CU --
+    // which a short K needs: its ring holds 2 KiB per wave, 16 KiB per workgroup, and 256 workgroups
+    // would have 4 MiB in flight.  Up to 1024 strips then go one per wave to 512 resident workgroups
+    // (x small enough for two workgroups' LDS, and few enough pieces per thread for that register
+    // budget).
+    if (shared && pl.d == 2 && strips < 4 * kResident && M * K <= 8 * 8 * kT &&
+        (size_t)((M * (K * 2 + 16) + 255) & ~255) + 2 * (size_t)kQ * M * kRedStride * 4 <= 80 * 1024) {
+        pl.sw = 1;
+        pl.resident = 2 * kResident;
+    }
     pl.groups = (strips + pl.sw - 1) / pl.sw;
     // more groups than the chip holds workgroups: each workgroup takes several, one after the other
-    const int64_t turns = (pl.groups + kResident - 1) / kResident;
+    const int64_t turns = (pl.groups + pl.resident - 1) / pl.resident;
     pl.blocks = (pl.groups + turns - 1) / turns;
     const size_t red = (size_t)(turns > 1 ? 2 : 1) * kQ * pl.sw * M * kRedStride * 4;
     const int64_t stage_max = (int64_t)kMaxPieces * 8 * kT;  // elements of x a workgroup stages at a time
@@ -866,10 +880,12 @@ int w4s_run_shared(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_i
         for (; at + n < count && n < kMaxProblems; ++n) {
             const k3q_gemv_w4s_problem& q = problems[at + n];
             if (q.N <= 0) return K3Q_ERR_SHAPE;
-            const W4sPlan pl = w4s_plan(M, K, q.N, block_size, has_pre);
+            const W4sPlan pl = w4s_plan(M, K, q.N, block_size, has_pre, count >= 2);
             if (!pl.ok || (has_pre && pl.halves)) return K3Q_ERR_SHAPE;
             if (n == 0) pl0 = pl;
-            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np || pl.own != pl0.own || pl.halves || pl0.halves) break;
+            else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.np != pl0.np || pl.own != pl0.own || pl.resident != pl0.resident ||
+                     pl.halves || pl0.halves)
+                break;
             const int rc = fill_params(mp.p[n], pl, x, M, K, q.N, q.shadow, q.scale, q.gparams, block_size,
                                        q.bias, bias_rows ? q.N : 0, q.y);
             if (rc != K3Q_OK) return rc;
@@ -884,11 +900,11 @@ int w4s_run_shared(const void* x, int x_dtype, int64_t M, int64_t K, const k3q_i
         // the launch as a whole is cut for the chip: about kResident workgroups, each problem its share;
         // workgroups that take turns need both reduction buffers, and where those do not fit beside x
         // the first problem goes alone
-        int64_t turns = (total + kResident - 1) / kResident;
+        int64_t turns = (total + pl0.resident - 1) / pl0.resident;
         size_t lds = turns > 1 ? pl0.lds_two : pl0.lds;
         if (lds > (size_t)160 * 1024) {
             n = 1;
-            turns = (groups[0] + kResident - 1) / kResident;
+            turns = (groups[0] + pl0.resident - 1) / pl0.resident;
             lds = pl0.lds;
         }
         if (pl0.halves && n != 1) return K3Q_ERR_SHAPE;
