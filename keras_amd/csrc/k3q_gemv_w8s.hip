@@ -412,10 +412,12 @@ struct W8sPlan {
     bool ok;
     int sw, d, np;
     int64_t groups, blocks;
+    int64_t resident;  // workgroups of this kernel form the chip holds at once (256 or 512)
     size_t lds;
 };
 
-W8sPlan w8s_plan(int64_t M, int64_t K, int64_t N) {
+// shared: the plan is for a launch that several problems share
+W8sPlan w8s_plan(int64_t M, int64_t K, int64_t N, bool shared = false) {
     W8sPlan pl{};
     // a wave's 64 pieces of x stay inside a row (K % 512), whole strips (N % 16)
     if (M < 1 || M > kMaxRows8 || K < 1024 || (K % 512) != 0 || (N % 16) != 0 || N < 16) return pl;
@@ -424,8 +426,17 @@ W8sPlan w8s_plan(int64_t M, int64_t K, int64_t N) {
     pl.d = (units / 4 >= 2 * kQ) ? 4 : 2;
     if ((units % pl.d) != 0 || units / pl.d < kQ) return pl;
     pl.sw = strips >= 2 * kResident8 ? 2 : 1;
+    pl.resident = kResident8;
+    // The kernels with few pieces of x per thread stay well within 128 registers, so two workgroups
+    // fit a CU: a shared launch of up to 1024 strips per problem then runs one strip per wave on 512
+    // resident workgroups (twice the requests in flight; x small enough for two workgroups' LDS).
+    if (shared && strips < 4 * kResident8 && M * K / 8 <= 4 * kT &&
+        (size_t)((M * (K + 16) + 255) & ~255) + 2 * kMaxRows8 * 4 + 2 * (size_t)kQ * ((M + 3) / 4) * 16 * 4 * 4 <= 80 * 1024) {
+        pl.sw = 1;
+        pl.resident = 2 * kResident8;
+    }
     pl.groups = (strips + pl.sw - 1) / pl.sw;
-    const int64_t turns = (pl.groups + kResident8 - 1) / kResident8;
+    const int64_t turns = (pl.groups + pl.resident - 1) / pl.resident;
     pl.blocks = (pl.groups + turns - 1) / turns;
     const int64_t pieces = M * K / 8;
     pl.np = pieces <= kT ? 1 : pieces <= 4 * kT ? 4 : pieces <= 16 * kT ? 16 : 0;
@@ -620,14 +631,14 @@ int w8s_run_shared(const void* x, int x_dtype, const int8_t* a, const void* a_sc
         for (; at + n < count && n < kMaxProblems8; ++n) {
             const k3q_w8s_problem& q = problems[at + n];
             if (q.N <= 0) return K3Q_ERR_SHAPE;
-            const W8sPlan pl = w8s_plan(M, K, q.N);
+            const W8sPlan pl = w8s_plan(M, K, q.N, count >= 2);
             if (!pl.ok) return K3Q_ERR_SHAPE;
             if (n == 0) {
                 pl0 = pl;
                 // workgroups of a shared launch may take turns even where a problem alone would not
                 lds_red_one = (size_t)kQ * pl.sw * ((M + 3) / 4) * 16 * 4 * 4;
                 lds_two = (size_t)((M * (K + 16) + 255) & ~255) + 2 * kMaxRows8 * 4 + 2 * lds_red_one;
-            } else if (pl.sw != pl0.sw || pl.d != pl0.d) {
+            } else if (pl.sw != pl0.sw || pl.d != pl0.d || pl.resident != pl0.resident) {
                 break;
             }
             const int rc = fill_params8(mp.p[n], pl, x, a, a_scale, M, K, q.N, q.shadow, q.kernel_scale, q.bias,
@@ -646,11 +657,11 @@ int w8s_run_shared(const void* x, int x_dtype, const int8_t* a, const void* a_sc
         // the launch as a whole is cut for the chip: about kResident8 workgroups, each problem its share;
         // workgroups that take turns need both reduction buffers, and where those do not fit beside x
         // the first problem goes alone, with its own plan
-        int64_t turns = (total + kResident8 - 1) / kResident8;
+        int64_t turns = (total + pl0.resident - 1) / pl0.resident;
         size_t lds = turns > 1 ? lds_two : lds_two - lds_red_one;
         if (lds > (size_t)160 * 1024) {
             n = 1;
-            turns = (groups[0] + kResident8 - 1) / kResident8;
+            turns = (groups[0] + pl0.resident - 1) / pl0.resident;
             lds = pl0.lds;
         }
         int next_block = 0;
