@@ -202,42 +202,45 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         return (const char*)p.gparams + ((int64_t)(place(grp) * kSW + t) * units + u0) * 48;
     };
     const int lane_w = lane * 16, lane_z = 12 * g;
-    const char* wp[kSW];   // the group being computed
-    const char* wn[kSW];   // the group after it (the last group: itself)
-    const char* zp[kSW];
-    const char* zn[kSW];
+    // The weight stream of a wave: unit after unit of its slice, group after group of the workgroup.
+    // The cursor (group, unit) is where the next request goes; the ring is refilled in stream order,
+    // so a request needs no index, and the stream may run any number of groups ahead of the sums (a
+    // slice as short as the ring is one round per group).  Past the workgroup's last group the cursor
+    // stays on it: requested, never used.
+    int cg = block, cu = 0;
+    const char* cw[kSW];
+    const char* cz[kSW];
+    auto at_group = [&]() {
 #pragma unroll
-    for (int t = 0; t < kSW; ++t) {
-        wp[t] = w_base(block, t);
-        zp[t] = z_base(block, t);
-    }
+        for (int t = 0; t < kSW; ++t) {
+            cw[t] = w_base(cg, t);
+            cz[t] = z_base(cg, t);
+        }
+    };
+    at_group();
     v4u W[kD][kSW];
     u32 Z[kGrouped ? kD : 1][kSW][3];
-    // unit u of the group being computed, or (u >= U) unit u - U of the one after it: one
-    // unconditional load either way, the base chosen by a select
-    auto fetch = [&](const int d, const int u) {
-        const bool own = u < U;
-        const int64_t uu = own ? u : u - U;
+    auto fetch = [&](const int d) {
 #pragma unroll
         for (int t = 0; t < kSW; ++t)
-            W[d][t] = __builtin_nontemporal_load((const v4u*)((own ? wp[t] : wn[t]) + uu * 1024 + lane_w));
+            W[d][t] = __builtin_nontemporal_load((const v4u*)(cw[t] + (int64_t)cu * 1024 + lane_w));
         if constexpr (kGrouped) {
 #pragma unroll
             for (int t = 0; t < kSW; ++t) {
-                const u32* z = (const u32*)((own ? zp[t] : zn[t]) + uu * 48 + lane_z);
+                const u32* z = (const u32*)(cz[t] + (int64_t)cu * 48 + lane_z);
                 Z[d][t][0] = z[0];
                 Z[d][t][1] = z[1];
                 Z[d][t][2] = z[2];
             }
         }
+        if (++cu == U) {
+            cu = 0;
+            cg = cg + stride < groups ? cg + stride : cg;
+            at_group();
+        }
     };
 #pragma unroll
-    for (int t = 0; t < kSW; ++t) {
-        wn[t] = wp[t];
-        zn[t] = zp[t];
-    }
-#pragma unroll
-    for (int d = 0; d < kD; ++d) fetch(d, d);
+    for (int d = 0; d < kD; ++d) fetch(d);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (kPre) {
         if (p.pre_kind == 1) {
@@ -362,7 +365,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (do_refill) fetch(dn, i + 1 + kD);
+        if (do_refill) fetch(dn);
         __builtin_amdgcn_sched_barrier(0);
     };
     using std::bool_constant;
@@ -395,7 +398,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
             for (int c = 0; c < 3; ++c) Zk[0][t][c] = Z[0][t][c];
     }
     __builtin_amdgcn_sched_barrier(0);
-    fetch(0, kD);  // (U >= 2 kD)
+    fetch(0);
     __builtin_amdgcn_sched_barrier(0);
 
     u32 esc[kSW][2], ebi[kSW][2];
@@ -403,11 +406,7 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     // requested now rather than at the end of the group's stream
     auto begin = [&](const int grp, const int nxt_grp) {
 #pragma unroll
-        for (int t = 0; t < kSW; ++t) {
-            wn[t] = w_base(nxt_grp, t);
-            zn[t] = z_base(nxt_grp, t);
-            tot[t] = zero4;
-        }
+        for (int t = 0; t < kSW; ++t) tot[t] = zero4;
         if (!kGrouped) {  // (grouped: every unit starts its own accumulators)
             accs[0] = zero4;
 #pragma unroll
@@ -490,11 +489,6 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
         begin(grp, grp + stride);
         for (int r = 0; r < R; ++r) round(bool_constant<false>{}, r, bool_constant<false>{});
         finish(grp, turn);
-#pragma unroll
-        for (int t = 0; t < kSW; ++t) {
-            wp[t] = wn[t];
-            zp[t] = zn[t];
-        }
     }
     // the last group: its last round has nothing to request or convert (the one request before it that
     // falls past the end re-reads the group's first unit: never used)
