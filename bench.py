@@ -8,8 +8,7 @@ de-scale epilogue, at the target shape M=4096, K=N=8192, bfloat16
 activations (inputs and weights already resident in HBM).  `value` is
 2*M*N*K / step time in TOP/s.  The int4 decode GEMV (K=N=8192, M in {1,4,16}),
 the second half of the headline metric, is reported under `int4_gemv` with its own
-HBM roofline (the layer's route: up to 8 rows the strip-linear copy of the kernel, made once
-per layer; 16 rows the stored kernel).  `int8_gemm_sweep` holds the GEMM kernel's time over the
+HBM roofline (the layer's route: the strip-linear copy of the kernel, made once per layer).  `int8_gemm_sweep` holds the GEMM kernel's time over the
 large-M sweep (M in {512, 2048, 4096, 8192} x K=N in {4096, 8192}, plus K=8192, N=28672),
 `einsum_int8` the EinsumDense attention projections (batch 8, t in {1, 512});
 `llama_decode_int4` is the end-to-end greedy decode of a 32-layer Llama-style decoder whose
@@ -164,12 +163,24 @@ def main():
     torch.cuda.synchronize()
     gemm_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
     gemm_tops = ops_per_step / (gemm_ms * 1e-3) / 1e12
-    for i in range(args.steps):
-        ev[2 * i].record()
+    # the quantizer alone: a graph of K launches between two events (a launch of 20 us between events
+    # of its own would be timed together with the host's pause before it)
+    # The launches rotate over five copies of x (320 MiB, more than the 256 MiB memory-side cache holds).
+    xs = [x] + [x.clone() for _ in range(4)]
+    with torch.cuda.stream(side):
         kq.abs_max_quantize(x, axis=-1)
-        ev[2 * i + 1].record()
+        qgraph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(qgraph, stream=side):
+            for i in range(args.steps):
+                kq.abs_max_quantize(xs[i % len(xs)], axis=-1)
     torch.cuda.synchronize()
-    quant_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
+    spin_up(torch, qgraph.replay, 0.05)
+    ev[0].record()
+    qgraph.replay()
+    ev[1].record()
+    torch.cuda.synchronize()
+    quant_ms = ev[0].elapsed_time(ev[1]) / args.steps
+    del qgraph, xs
     quant_bytes = M * K * 2 + M * K + M * 2
 
     # ------------------------------------------------------------------ counter calibration
