@@ -20,6 +20,7 @@ import math
 import torch
 
 from keras_amd import dtype_policies, ops as kops, quantizers
+from keras_amd.layers.dense import int8_strip_route
 from keras_amd.layers.layer import Layer, as_tensor, require_default_g_idx, to_torch_dtype
 from keras_amd.quantization_config import (
     Int4QuantizationConfig,
@@ -560,13 +561,24 @@ class ReversibleEmbedding(Embedding):
                     prepacked=self._cached("prepacked", self.reverse_embeddings,
                                            kops.prepack_int8_kernel))
             return self._soft_cap(logits.reshape(*lead, self.input_dim))
-        q, in_scale = self.inputs_quantizer(x2, axis=-1)
         scale_var = self.embeddings_scale if self.tie_weights else self.reverse_embeddings_scale
         out_dtype = _promote(cd, as_tensor(scale_var).dtype)
         M, N = x2.shape[0], self.input_dim
         exact = self.exact_epilogue
         if exact is None:
             exact = True
+        if (self.tie_weights and exact and out_dtype == torch.bfloat16
+                and int8_strip_route(self.inputs_quantizer, x2, N)):
+            # decode sizes: the table's strip-linear copy as the [dim, vocab] kernel of the projection
+            # (made once, as many bytes as the table): quantizer, exact int8 matmul and de-scale in
+            # one launch, the bits of the route below
+            logits = kops.int8_dense_strip(
+                x2, self._cached("w8s", self._embeddings, lambda t: kops.int8_strip_copy(t.t().contiguous())), N,
+                as_tensor(scale_var), epsilon=self.inputs_quantizer.epsilon,
+                value_range=self.inputs_quantizer.value_range,
+                quantize=lambda rows: self.inputs_quantizer(rows, axis=-1))
+            return self._soft_cap(logits.reshape(*lead, N))
+        q, in_scale = self.inputs_quantizer(x2, axis=-1)
         in_scale = in_scale.to(out_dtype)  # widening an existing value is exact
         round_acc = cd == torch.bfloat16 and out_dtype == torch.float32
         if self.tie_weights:
@@ -590,11 +602,42 @@ class ReversibleEmbedding(Embedding):
             )
         return self._soft_cap(logits.reshape(*lead, N))
 
+    def _tied_strip_operands(self, x2, scale, grouped, block_size):
+        """Operands of `ops.int4_matmul_strip` for the tied int4 table used as the LM head, or None
+        when that route does not take these rows: the table (packed along its last axis, K of the
+        projection) unpacked, transposed and packed again the way a Dense kernel `[dim, vocab]` is,
+        then copied in strip-linear order; grouped scales / zero points transposed to `[groups, vocab]`.
+        Made on first use, kept while the variables do not change."""
+        K, N = self._orig_output_dim, self.input_dim
+        if not (x2.is_cuda and x2.dtype == torch.bfloat16 and scale.dtype == torch.bfloat16
+                and 0 < x2.shape[0] <= kops.STRIP_MAX_ROWS and x2.shape[1] == K
+                and kops.int4_strip_supported(x2.shape[0], K, N, block_size if grouped else None)):
+            return None
+
+        def relay(table):
+            dense = quantizers.unpack_int4(table, K, axis=-1).t().contiguous()  # [dim, vocab] int8
+            return kops.int4_strip_copy(quantizers.pack_int4(dense, axis=-1)[0], N)
+
+        spec = dict(shadow=self._cached("w4s", self._embeddings, relay))
+        if grouped:
+            sv, zv = self.embeddings_scale, self.embeddings_zero
+            stamp = (id(sv), sv.version, id(zv), zv.version)
+            hit = self._cache.get("w4s_params")
+            if hit is None or hit[0] != stamp:
+                value = kops.int4_strip_params(as_tensor(sv).t().contiguous(),
+                                               as_tensor(zv).to(torch.int8).t().contiguous(), K, N, block_size)
+                hit = self._cache["w4s_params"] = (stamp, None, value)
+            spec["gparams"] = hit[2]
+        else:
+            spec["kernel_scale"] = scale if scale.is_contiguous() else scale.contiguous()
+        return spec
+
     def _int4_call(self, inputs, reverse=False, training=None):
         """reversible_embedding.py:298-381.
 
         Tied weights: the packed `[vocab, ceil(dim/2)]` table is the K-contiguous int4 kernel
-        of the projection and is read in place.  Untied weights: `reverse_embeddings` is
+        of the projection and is read in place; at decode sizes (`_tied_strip_operands`) a
+        strip-linear copy of it is streamed by the Dense decode kernel instead.  Untied weights: `reverse_embeddings` is
         packed along its first axis (two k per byte); it is re-packed once, on the device,
         into the Dense layout (two columns per byte, same size) and cached, after which the
         call is a Dense int4 call.  With an activation quantizer (a layer built from a policy
@@ -625,6 +668,12 @@ class ReversibleEmbedding(Embedding):
                     x2, table8, a_scale=in_scale.to(out_dtype), kernel_scale=scale,
                     out_dtype=out_dtype, exact_epilogue=True,
                     round_acc_bf16=(cd == torch.bfloat16 and out_dtype == torch.float32))
+            elif in_scale is None and (strip := self._tied_strip_operands(x2, scale, grouped, block_size)):
+                # decode sizes: the table re-laid once as the [dim, vocab] int4 kernel of the
+                # projection in strip-linear order (as many bytes as the table), streamed by the
+                # Dense decode kernel
+                logits = kops.int4_matmul_strip(x2, strip["shadow"], self.input_dim, block_size=block_size if grouped else None,
+                                                kernel_scale=strip.get("kernel_scale"), gparams=strip.get("gparams"))
             else:
                 logits = kops.int4_matmul_nk(
                     x2 if in_scale is None else x2.to(cd), as_tensor(self._embeddings), scale,

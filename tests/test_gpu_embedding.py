@@ -327,6 +327,37 @@ def test_int4_matmul_nk(dev, x_dtype, scale_dtype, M, V, D, block):
     assert max_rel_err(got, want) <= tol
 
 
+@pytest.mark.parametrize("M", [1, 8, 16])
+@pytest.mark.parametrize("block_size", [128, None])
+def test_reversible_embedding_int4_tied_decode_sizes_take_the_strip_copy(dev, M, block_size):
+    """A tied table wide enough for the Dense decode kernel is re-laid once as that kernel's
+    strip-linear copy; more rows, or other dtypes, keep reading the table in place."""
+    V, D = 3200, 4096
+    layer = build_embedding(ReversibleEmbedding, dev, V, D, "bfloat16", seed=21)
+    t = layer._embeddings.value.cpu()
+    layer.quantize("int4", config=Int4QuantizationConfig(block_size=block_size))
+    qd = ref.embedding_quantize_int4(t.float(), block_size=block_size)
+    x = torch.randn(M, D, generator=torch.Generator().manual_seed(22))
+    y = layer(x, reverse=True)
+    assert "w4s" in layer._cache and ("w4s_params" in layer._cache) == (block_size is not None)
+    want = ref.reversible_embedding_int4_reverse(
+        x.to(torch.bfloat16), qd["embeddings"], qd["embeddings_scale"].to(torch.bfloat16), D,
+        embeddings_zero=qd["embeddings_zero"], g_idx=qd["g_idx"], block_size=block_size,
+        compute_dtype=torch.bfloat16)
+    assert y.dtype == want.dtype and tuple(y.shape) == (M, V)
+    assert max_rel_err(y, want) <= RTOL[torch.bfloat16]
+    # the table read in place (more rows than the decode kernel takes) agrees with it row by row
+    x40 = torch.cat([x, torch.randn(40 - M, D, generator=torch.Generator().manual_seed(23))])
+    y40 = layer(x40, reverse=True)
+    assert max_rel_err(y40[:M], want) <= RTOL[torch.bfloat16]
+    # an assignment to the table makes a new copy
+    before = layer._cache["w4s"][2]
+    layer._embeddings.assign(layer._embeddings.value.clone())
+    y2 = layer(x, reverse=True)
+    assert layer._cache["w4s"][2] is not before
+    assert torch.equal(bits(y2.cpu()), bits(y.cpu()))
+
+
 @pytest.mark.parametrize("policy", ["float32", "bfloat16", "mixed_bfloat16"])
 @pytest.mark.parametrize("block_size", [128, None])
 def test_reversible_embedding_int4_tied(dev, policy, block_size):
