@@ -201,14 +201,14 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     auto z_base = [&](const int grp, const int t) {
         return (const char*)p.gparams + ((int64_t)(place(grp) * kSW + t) * units + u0) * 48;
     };
-    const int lane_w = lane * 16, lane_z = 12 * g;
+    const unsigned lane_w = lane * 16u, lane_z = 12u * g;  // (unsigned: a scalar base + a 32-bit lane offset is one address form)
     // The weight stream of a wave: unit after unit of its slice, group after group of the workgroup.
     // The cursor (group, unit) is where the next request goes; the ring is refilled in stream order,
     // so a request needs no index, and the stream may run any number of groups ahead of the sums (a
     // slice as short as the ring is one round per group).  Past the workgroup's last group the cursor
     // stays on it: requested, never used.
     int cg = block, cu = 0;
-    const char* cw[kSW];
+    const char* cw[kSW];  // where the next request of a strip goes: advanced by a unit per request
     const char* cz[kSW];
     auto at_group = [&]() {
 #pragma unroll
@@ -222,15 +222,18 @@ __device__ __forceinline__ void gemv_w4s_body(const W4sParams& p, const int bloc
     u32 Z[kGrouped ? kD : 1][kSW][3];
     auto fetch = [&](const int d) {
 #pragma unroll
-        for (int t = 0; t < kSW; ++t)
-            W[d][t] = __builtin_nontemporal_load((const v4u*)(cw[t] + (int64_t)cu * 1024 + lane_w));
+        for (int t = 0; t < kSW; ++t) {
+            W[d][t] = __builtin_nontemporal_load((const v4u*)(cw[t] + lane_w));
+            cw[t] += 1024;
+        }
         if constexpr (kGrouped) {
 #pragma unroll
             for (int t = 0; t < kSW; ++t) {
-                const u32* z = (const u32*)(cz[t] + (int64_t)cu * 48 + lane_z);
+                const u32* z = (const u32*)(cz[t] + lane_z);
                 Z[d][t][0] = z[0];
                 Z[d][t][1] = z[1];
                 Z[d][t][2] = z[2];
+                cz[t] += 48;
             }
         }
         if (++cu == U) {
