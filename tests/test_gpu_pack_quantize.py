@@ -83,6 +83,25 @@ def test_abs_max_quantize_last_axis(dev, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_abs_max_quantize_row_lengths_around_the_kernel_forms(dev, dtype):
+    """Row lengths on both sides of every switch between the quantizer's forms (a wave or a
+    workgroup per row, 1 ... 8 groups of 16 values per thread, rows that fill every thread or not),
+    with few and many rows and a zero row."""
+    g = torch.Generator().manual_seed(7)
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    for groups in (1, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049):
+        cols = 16 * groups
+        for rows in (1, 5, 1024 if cols <= 2064 else 9):
+            x = (torch.randn(rows, cols, generator=g) * (0.01 if groups % 2 else 30.0)).to(dtype)
+            if rows > 2:
+                x[1] = 0
+            q_ref, s_ref = ref.abs_max_quantize(x, axis=-1)
+            q, s = kq.abs_max_quantize(x.to(dev), axis=-1)
+            assert torch.equal(q.cpu(), q_ref), (rows, cols)
+            assert torch.equal(s.cpu().view(bits), s_ref.view(bits)), (rows, cols)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_abs_max_quantize_special_rows(dev, dtype):
     x = torch.zeros(6, 64)
     x[1, 3] = 1e-6
