@@ -265,6 +265,9 @@ def test_reversible_embedding_int8_tied(dev, policy, M, V, D):
                                                  compute_dtype=cd)
     assert y.dtype == want.dtype and tuple(y.shape) == (M, V)
     assert torch.equal(bits(y.cpu()), bits(want))
+    # decode sizes of a wide bfloat16 table stream its strip-linear copy (same bits); everything
+    # else reads the table in place
+    assert ("w8s" in layer._cache) == (policy == "bfloat16" and M <= 16 and V == 32000)
     layer.exact_epilogue = False
     assert max_rel_err(layer(x, reverse=True), want) <= RTOL[cd]
     err = (y_float.float().cpu() - y.float().cpu()).abs().max().item()
