@@ -95,10 +95,11 @@ class DecoderBlock(Layer):
         self.down.build((None, ffn_dim))
         self.built = True
 
-    def forward(self, x, cos, sin, cache, pos, mask, tables=None):
+    def forward(self, x, rows, cache, pos, tables=None):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
-        (an int64 device tensor [T]); mask [T, maxT]: 0 where a key may be attended to, -inf
-        elsewhere; tables: the whole (cos, sin) tables, for the one-position kernel."""
+        (an int64 device tensor [T]); rows(): (cos, sin, mask) of these positions -- the table
+        rows and mask [T, maxT], 0 where a key may be attended to, -inf elsewhere -- asked for
+        only by the torch path; tables: the whole (cos, sin) tables, for the one-position kernel."""
         # The normalisations and the gate are handed to the projections that consume them as their
         # `input_op`: at one position they ride inside the projections' launches, in front of int8
         # layers they share a launch with the activation quantizer, otherwise they run as their own
@@ -113,6 +114,7 @@ class DecoderBlock(Layer):
             a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
         else:
             # one rotation over the query and key heads together (half the elementwise launches)
+            cos, sin, mask = rows()
             qk = apply_rope(torch.cat((q, k), dim=2), cos, sin)
             q, k = qk[:, :, : self.n_heads], qk[:, :, self.n_heads:]
             kc, vc = cache
@@ -213,14 +215,23 @@ class LlamaStyleDecoder(Model):
         cd = to_torch_dtype(self.compute_dtype)
         if x.dtype != cd:
             x = x.to(cd)
-        cos = self.cos.index_select(0, pos)
-        sin = self.sin.index_select(0, pos)
-        keys = torch.arange(self.max_len, device=self.device)
-        # additive form once per forward (a boolean mask is converted by every attention call)
-        mask = torch.zeros((pos.shape[0], self.max_len), dtype=cd, device=self.device).masked_fill_(
-            keys[None, :] > pos[:, None], float("-inf"))
+        made = []
+
+        def rows():
+            # table rows and mask of these positions, made once per forward and only if a block
+            # asks (a step on the one-position kernel does not: six small launches less)
+            if not made:
+                cos = self.cos.index_select(0, pos)
+                sin = self.sin.index_select(0, pos)
+                keys = torch.arange(self.max_len, device=self.device)
+                # additive form once per forward (a boolean mask is converted by every attention call)
+                mask = torch.zeros((pos.shape[0], self.max_len), dtype=cd, device=self.device).masked_fill_(
+                    keys[None, :] > pos[:, None], float("-inf"))
+                made.append((cos, sin, mask))
+            return made[0]
+
         for block, kv in zip(self.blocks, cache):
-            x = block.forward(x, cos, sin, kv, pos, mask, tables=(self.cos, self.sin))
+            x = block.forward(x, rows, kv, pos, tables=(self.cos, self.sin))
         if last_only:
             x = x[:, -1:, :]
         return self.token_embedding(self.final_norm(x), reverse=True)
