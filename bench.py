@@ -77,11 +77,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
-    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,xcd,decode,cpu: run the headline "
+    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,decode,cpu: run the headline "
                     "step and only these further sections (for profiler runs); default: all")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
-    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "xcd", "decode", "cpu"}
+    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "decode", "cpu"}
     if unknown:
         sys.exit(f"bench.py: unknown section(s) {sorted(unknown)}")
     want = (lambda name: not only or name in only)
@@ -196,13 +196,13 @@ def main():
 
     # ------------------------------------------------------------------ matrix cores alone
     # What the int8 matrix cores sustain on this board with nothing else running: a loop of
-    # v_mfma_i32_32x32x32_i8 on register-resident operands (libk3q_probe.so, a measurement aid
-    # built beside the product library), about 50 ms per operand kind, clock read in-kernel.
+    # v_mfma_i32_32x32x32_i8 on register-resident operands (bench_probes/libk3q_probe.so, a
+    # measurement aid built beside this file, not part of the product library), about 50 ms per operand kind, clock read in-kernel.
     ceiling = None
     if want("ceiling"):
         import ctypes
 
-        probe_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "keras_amd", "libk3q_probe.so")
+        probe_path = os.path.join(ROOT, "bench_probes", "libk3q_probe.so")
         if os.path.exists(probe_path):
             probe = ctypes.CDLL(probe_path)
             probe.k3q_probe_mfma_i8_only.restype = ctypes.c_double
@@ -388,7 +388,7 @@ def main():
     def load_stream_probe():
         import ctypes
 
-        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "keras_amd", "libk3q_probe.so")
+        path = os.path.join(ROOT, "bench_probes", "libk3q_probe.so")
         if not os.path.exists(path):
             return None
         lib_ = ctypes.CDLL(path)
@@ -425,43 +425,6 @@ def main():
                                  ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
         best["empty_launch_us"] = round(graph_node_us(nothing, 4, 400), 2)
         return best
-
-    # Which XCD reads which addresses: the read-only launch with 256 workgroups of 256 KiB (64 MiB),
-    # the chunk of a workgroup chosen by a table.  Workgroups go round-robin to the 8 XCDs.
-    xcd_table = None
-    if want("xcd"):
-        import ctypes
-
-        lib_ = load_stream_probe()
-        if lib_ is not None:
-            lib_.k3q_probe_stream_read_perm.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p,
-                                                        ctypes.c_void_p, ctypes.c_void_p]
-            W = 256
-            sink = torch.zeros(4096, dtype=torch.int32, device=dev)
-            xcd_table = []
-            for chunk_kib in (128, 256):
-                nb = W * chunk_kib * 1024
-                bufs = [torch.randint(0, 255, (nb,), dtype=torch.uint8, device=dev) for _ in range((448 << 20) // nb)]
-                orders = [("plain: XCD x reads chunks x, x + 8, ...", list(range(W))),
-                          ("rotated: XCD x reads chunk 8 i + (x + i) % 8", [(b & ~7) | ((b + (b >> 3)) & 7) for b in range(W)]),
-                          ("each XCD one contiguous eighth", [(b % 8) * (W // 8) + b // 8 for b in range(W)])]
-                for s_ in (2, 4, 8):
-                    per = [[c for c in range(W) if (c // s_) % 8 == x] for x in range(8)]
-                    bit = (chunk_kib * 1024 * s_).bit_length() - 1
-                    orders.append((f"address bits {bit}-{bit + 2} select the XCD", [per[b % 8][b // 8] for b in range(W)]))
-                for name, order in orders:
-                    table = torch.tensor(order, dtype=torch.int32, device=dev)
-
-                    def call(i):
-                        rc = lib_.k3q_probe_stream_read_perm(ctypes.c_void_p(bufs[i % len(bufs)].data_ptr()), nb, W,
-                                                             ctypes.c_void_p(table.data_ptr()),
-                                                             ctypes.c_void_p(sink.data_ptr()),
-                                                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-                        if rc != 0:
-                            sys.exit("bench.py: the read-only probe did not launch")
-                    xcd_table.append({"chunk_KiB": chunk_kib, "order": name,
-                                      "us_per_launch": round(graph_node_us(call, len(bufs), 4 * len(bufs)), 2)})
-                del bufs
 
     read_ref4 = None
     if want("gemv"):
@@ -524,8 +487,8 @@ def main():
     # Llama-style 32-layer decoder (d_model 4096, 32 heads, SwiGLU 14336, vocab 32000), every
     # weight matrix int4 (grouped, block 128) with synthetic values written on the device;
     # prompt of 128 random ids, greedy decode of 128 steps, prompt and decode steps replayed from
-    # HIP graphs.  Matmuls, embedding lookup and LM head run the k3q kernels; norms, RoPE,
-    # attention and the gating are torch ops.
+    # HIP graphs.  Matmuls, embedding lookup and LM head run the k3q kernels, and so do the
+    # harness's own normalisations, RoPE + cache update + attention and the SwiGLU gate.
     decode = None
     decode_int8 = None
     if want("decode"):
@@ -620,7 +583,6 @@ def main():
         "einsum_int8": einsum,
         "int4_gemv": gemv,
         "read_only_launch_32MiB": read_ref4,
-        "read_only_launch_by_xcd_assignment": xcd_table,
         "int8_decode_dense": gemv8,
         "read_only_launch_64MiB": read_ref8,
         "llama_decode_int4": decode,

@@ -1,5 +1,5 @@
-// Measurement aid, not part of the product library (built into libk3q_probe.so; only bench.py
-// loads it): what a launch that does nothing but READ a buffer costs on this board, and what a
+// Measurement aid, not part of the product library (built into bench_probes/libk3q_probe.so;
+// only bench.py loads it): what a launch that does nothing but READ a buffer costs on this board, and what a
 // launch that does nothing at all costs.  The decode kernels stream a weight matrix once; their
 // time per launch is compared with these two.
 //
@@ -46,31 +46,6 @@ __global__ __launch_bounds__(512) void stream_read(const v4u* src, int steps, un
     }
 }
 
-// The same read with the chunk of a workgroup chosen by a table: workgroups are dealt round-robin
-// to the 8 XCDs, so the table decides which XCD streams which addresses.
-template <int kDepth>
-__global__ __launch_bounds__(512) void stream_read_perm(const v4u* src, const int* chunk_of, int steps,
-                                                       unsigned* out) {
-    const int lane = threadIdx.x & 63;
-    const int wave = chunk_of[blockIdx.x] * 8 + (threadIdx.x >> 6);
-    const v4u* p = src + (int64_t)wave * steps * 64 + lane;
-    v4u r[kDepth];
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) r[d] = __builtin_nontemporal_load(p + (int64_t)d * 64);
-    v4u acc = {0u, 0u, 0u, 0u};
-    for (int base = kDepth; base < steps; base += kDepth) {
-#pragma unroll
-        for (int d = 0; d < kDepth; ++d) {
-            acc ^= r[d];
-            r[d] = __builtin_nontemporal_load(p + (int64_t)(base + d) * 64);
-        }
-    }
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) acc ^= r[d];
-    const unsigned v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
-    if (v == 0x12345u) out[blockIdx.x] = v;  // keeps the loads alive
-}
-
 __global__ void nothing(unsigned* out) {
     if (out == (unsigned*)1) out[0] = 0;  // never true
 }
@@ -99,17 +74,5 @@ extern "C" int k3q_probe_stream_read(const void* src, int64_t bytes, int workgro
 // One workgroup of one wave that does nothing: the cost of a launch itself.
 extern "C" int k3q_probe_empty(void* out, void* stream) {
     nothing<<<1, 64, 0, (hipStream_t)stream>>>((unsigned*)out);
-    return hipGetLastError() == hipSuccess ? 0 : -1;
-}
-
-// As k3q_probe_stream_read with 8 loads of a wave in flight, workgroup b reading chunk chunk_of[b]
-// (a permutation of 0 ... workgroups - 1 in device memory) of `bytes / workgroups` bytes.
-extern "C" int k3q_probe_stream_read_perm(const void* src, int64_t bytes, int workgroups, const int* chunk_of,
-                                          void* out, void* stream) {
-    if (!src || !out || !chunk_of || bytes <= 0 || workgroups <= 0) return -1;
-    const int64_t per_wave = bytes / ((int64_t)workgroups * 8);
-    if (per_wave * workgroups * 8 != bytes || per_wave % 8192 || per_wave < 16384) return -1;
-    stream_read_perm<8><<<workgroups, 512, 0, (hipStream_t)stream>>>((const v4u*)src, chunk_of, (int)(per_wave / 1024),
-                                                                     (unsigned*)out);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }

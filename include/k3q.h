@@ -387,21 +387,6 @@ int k3q_gemv_w4_multi(const void* x, int x_dtype, int64_t M, int64_t K, int coun
                       void* stream);
 
 /*
- * TEST HOOK, not for callers: k3q_gemv_w4_fused with the launch plan overridden, so that the
- * parity tests can run every variant of the kernel (dwords per lane, rows per chunk, waves,
- * slice length) at one shape instead of relying on the shapes that select them:
- * plan = {dwords per lane per k row (1|2), 16-row steps per chunk (1|2),
- * waves per workgroup (1..8), rows of K per wave}; entries <= 0 and a null
- * `plan` keep the built-in choice.  The workspace must then hold
- * ceil(K / (waves * rows per wave)) * min(M, 16) * N floats.  No counterpart in the reference.
- */
-int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
-                     const void* w_packed, const void* scale, const void* zero,
-                     int64_t block_size, const void* bias, void* y, void* workspace,
-                     int64_t workspace_bytes, void* counters, int64_t counters_bytes,
-                     const int* plan, void* stream);
-
-/*
  * Weight-only int4 matmul for decode-sized M with the kernel stored K-contiguous:
  *     y[m,n] = sum_k x[m,k] * W[n,k],  w_packed int8 [N, ceil(K/2)], low nibble = even k
  *   block_size <= 0: scale [N];                         y = T(T(acc) / scale[n])

@@ -133,13 +133,16 @@ SIGNATURES = {
         _int,
         [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr],
     ),
-    "k3q_gemv_w4_plan": (
+}
+
+# test hooks (keras_amd/csrc/k3q_testing.h): exported by the library, not part of the C ABI
+TEST_SIGNATURES = {
+    "k3qt_gemv_w4_plan": (
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
          _ptr, _ptr],
     ),
 }
-
 
 
 class GemvW4Problem(ctypes.Structure):
@@ -187,7 +190,7 @@ def load():
             "(the quantized path has no fallback implementation)"
         )
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (res, args) in SIGNATURES.items():
+    for name, (res, args) in list(SIGNATURES.items()) + list(TEST_SIGNATURES.items()):
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

@@ -12,7 +12,6 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB = os.path.join(PKG, "libk3q.so")
-PROBE_LIB = os.path.join(PKG, "libk3q_probe.so")
 
 SOURCES = [
     "k3q_api.hip",
@@ -70,15 +69,6 @@ def build(verbose=True, jobs=8):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    # the measurement aid bench.py uses: a library of its own, never loaded by the package
-    cmd = [hipcc(), *FLAGS, "-shared", "-o", PROBE_LIB, os.path.join(HERE, "k3q_probe_mfma.hip"),
-           os.path.join(HERE, "k3q_probe_stream.hip")]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
-    if out.returncode != 0:
-        sys.stderr.write(out.stdout.decode())
-        raise RuntimeError("hipcc failed on the probe library")
     return LIB
 
 

@@ -1566,7 +1566,7 @@ extern "C" int k3q_gemv_w4_addend(const void* x, int x_dtype, int64_t M, int64_t
                        workspace_bytes, nullptr, counters, counters_bytes, (hipStream_t)stream, true);
 }
 
-extern "C" int k3q_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+extern "C" int k3qt_gemv_w4_plan(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
                                 const void* w_packed, const void* scale, const void* zero,
                                 int64_t block_size, const void* bias, void* y, void* workspace,
                                 int64_t workspace_bytes, void* counters, int64_t counters_bytes,

@@ -139,7 +139,7 @@ def int4_matmul(x, kernel_packed, kernel_scale, orig_output_dim, kernel_zero=Non
         rc = lib.k3q_gemv_w4_fused(*args, _lib.stream_ptr(x.device))
     else:
         arr = (ctypes.c_int * 4)(*[int(v) for v in plan[:4]])
-        rc = lib.k3q_gemv_w4_plan(*args, arr, _lib.stream_ptr(x.device))
+        rc = lib.k3qt_gemv_w4_plan(*args, arr, _lib.stream_ptr(x.device))
     _lib.check(rc, "k3q_gemv_w4")
     return y.reshape(*lead, N)
 

@@ -26,6 +26,10 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in include/k3q.h but not exported"
     # and the ctypes table binds exactly the declared set
     assert sorted(_lib.SIGNATURES) == names
+    # test hooks live under another prefix and stay out of the ABI header
+    text = open(os.path.join(ROOT, "include", "k3q.h")).read()
+    for name in _lib.TEST_SIGNATURES:
+        assert name.startswith("k3qt_") and hasattr(lib, name) and name not in text
 
 
 def test_version_and_error_strings():

@@ -18,7 +18,7 @@ def make_layer(K, N, block_size, seed, with_bias):
     return qk, bias
 
 
-def run_case(dev, M, K, N, block_size, dtype, with_bias, seed=0, plan=None):
+def run_case(dev, M, K, N, block_size, dtype, with_bias, seed=0, plan=None, two_ulp_case=False):
     qk, bias = make_layer(K, N, block_size, seed, with_bias)
     g = torch.Generator().manual_seed(seed + 1)
     x = torch.randn(M, K, generator=g).to(dtype)
@@ -39,12 +39,15 @@ def run_case(dev, M, K, N, block_size, dtype, with_bias, seed=0, plan=None):
     e_exact = max_rel_err(got, exact)
     e_ref_exact = max_rel_err(want, exact)
     tol = RTOL[dtype]
-    # One bfloat16 ulp of an output in [4, 8) is 0.7 % of max|y| here, so two correctly
-    # rounded chains (the reference rounds every de-quantised weight to bfloat16, the kernel
-    # keeps fp32 until the end) can sit 1.5 ulp apart while each is within 0.7 % of the
-    # float64 value.  Such a case passes only if the kernel is the one closer to that value.
-    assert e_ref <= tol or (e_ref <= 1.5 * tol and e_exact <= e_ref_exact), \
-        f"vs oracle: {e_ref:.3e} > {tol:.0e} (vs float64: kernel {e_exact:.3e}, oracle {e_ref_exact:.3e})"
+    # the stated bound against what the reference returns: 1e-3 (bfloat16: 1e-2) of max|y|.
+    # `two_ulp_case` names a case (listed where it is parametrised) in which one output of the
+    # top binade sits two bfloat16 ulps from the oracle's: there the bound is 1.5e-2 and the
+    # kernel must be the closer of the two to the float64 value.
+    if two_ulp_case:
+        assert tol < e_ref <= 1.5 * tol and e_exact <= e_ref_exact, (e_ref, e_exact, e_ref_exact)
+    else:
+        assert e_ref <= tol, \
+            f"vs oracle: {e_ref:.3e} > {tol:.0e} (vs float64: kernel {e_exact:.3e}, oracle {e_ref_exact:.3e})"
     # the kernel must be at least about as close to the true value as the reference path is
     assert e_exact <= max(2.0 * e_ref_exact, tol / 4), (e_exact, e_ref_exact)
     return e_ref, e_exact
@@ -142,7 +145,14 @@ def test_int4_large_m_off_route(dev, M, K, N, block_size, dtype):
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_int4_mid_rows(dev, M, K, N, block_size, dtype):
-    run_case(dev, M, K, N, block_size, dtype, with_bias=(M % 2 == 0))
+    # The one case of this file outside the 1e-2 bound: 64 bfloat16 rows, K = N = 4096, groups of
+    # 128, seed 0.  One of its 262144 outputs, in [4, 8) where a bfloat16 ulp is 0.7 % of max|y|,
+    # lands two ulps from the oracle's (1.06e-2): the reference rounds every de-quantised weight to
+    # bfloat16 and is 7.2e-3 from the float64 value, the kernel keeps float32 to the end and is 6.0e-3
+    # from it.  If a change of the kernel brings the case inside the bound, the assertion in
+    # run_case fails and this exception is to be deleted.
+    odd = (M, K, N, block_size, dtype) == (64, 4096, 4096, 128, torch.bfloat16)
+    run_case(dev, M, K, N, block_size, dtype, with_bias=(M % 2 == 0), two_ulp_case=odd)
 
 
 def test_int4_single_launch_split_matches_two_launches(dev):
@@ -337,12 +347,12 @@ def run_kmajor_case(dev, M, K, N, block_size, with_bias, seed=90):
     exact = c_w4_matmul_f64(x, qk["kernel"], scale_t, qk["kernel_zero"], block_size, bias_t, N)
     e_ref, e_exact, e_ref_exact = max_rel_err(got, want), max_rel_err(got, exact), max_rel_err(want, exact)
     tol = RTOL[dt]
-    assert e_ref <= tol or (e_ref <= 1.5 * tol and e_exact <= e_ref_exact), (e_ref, e_exact, e_ref_exact)
+    assert e_ref <= tol, (e_ref, e_exact, e_ref_exact)  # the stated bound, unconditionally
     assert e_exact <= max(2.0 * e_ref_exact, tol / 4), (e_exact, e_ref_exact)
     other = kops.int4_matmul(x.to(dev), kernel, scale_t.to(dev), N,
                              kernel_zero=qk["kernel_zero"].to(dev) if grouped else None,
                              block_size=block_size, bias=bias_t.to(dev) if with_bias else None)
-    assert max_rel_err(got, other) <= 1.5 * tol
+    assert max_rel_err(got, other) <= tol
 
 
 @pytest.mark.parametrize("M,K,N,block_size", [(48, 1024, 256, 128), (130, 1536, 96, 192), (64, 512, 64, 64)])

@@ -359,3 +359,238 @@ def test_einsum_int8_descale_approximates_float(equation, kshape, xshape):
     want = torch.einsum(equation, x, kernel)
     assert tuple(y.shape) == tuple(want.shape)
     assert (y - want).pow(2).mean().item() < 1e-3
+
+
+# ---------------------------------------------------------------- EinsumDense int4 (forward), LoRA
+def _nibble(byte, high):
+    """Signed value of one nibble of a stored byte, spelled out (no call into the oracle)."""
+    v = ((int(byte) & 0xFF) >> (4 if high else 0)) & 15
+    return v - 16 if v >= 8 else v
+
+
+def _einsum_int4_kernel_by_loops(qk, block_size):
+    """The float64 kernel an int4 EinsumDense de-quantises to, built weight by weight from the
+    packed bytes: flat row r, flat column c sit in byte [r, c // 2] (even c in the low nibble);
+    the flat matrix is the row-major reshape of the kernel (einsum_dense.py:1388-1398)."""
+    rows, cols = qk["rows"], qk["cols"]
+    packed = qk["kernel"].numpy()
+    scale = qk["kernel_scale"].double().numpy()
+    zero = None if qk["kernel_zero"] is None else qk["kernel_zero"].numpy()
+    flat = np.zeros((rows, cols), np.float64)
+    for r in range(rows):
+        for c in range(cols):
+            v = _nibble(packed[r, c // 2], c % 2 == 1)
+            if block_size in (None, -1):
+                flat[r, c] = v / scale[c]
+            else:
+                gi = r // block_size
+                flat[r, c] = (v - int(zero[gi, c])) * scale[gi, c]
+    out = np.zeros(qk["original_kernel_shape"], np.float64)
+    for i in range(rows * cols):
+        out[np.unravel_index(i, out.shape)] = flat[i // cols, i % cols]
+    return out
+
+
+EINSUM_INT4_CASES = [
+    ("btd,dnh->btnh", (16, 3, 6), (2, 3, 16)),      # contracted axis leads: flat = true [K, N]
+    ("btnh,nhd->btd", (2, 8, 10), (2, 3, 2, 8)),    # two contracted axes lead
+    ("ab,bcd->acd", (16, 3, 4), (5, 16)),
+    ("btd,ndh->btnh", (3, 16, 6), (2, 2, 16)),      # contracted axis in the middle: the reshape mixes
+    ("abc,cd->abd", (16, 7), (2, 3, 16)),           # odd column count: half-filled last byte
+]
+
+
+@pytest.mark.parametrize("equation,kshape,xshape", EINSUM_INT4_CASES)
+@pytest.mark.parametrize("block_size", [None, 8])
+def test_einsum_dense_int4_call_by_loops(equation, kshape, xshape, block_size):
+    g = torch.Generator().manual_seed(23)
+    kernel = torch.rand(kshape, generator=g) - 0.5
+    x = torch.randn(xshape, generator=g)
+    bias_shape = torch.einsum(equation, x, kernel).shape[-1:]
+    bias = torch.randn(bias_shape, generator=g) * 0.1
+    qk = ref.einsum_dense_quantize_int4(kernel, equation, len(xshape), block_size)
+    # rows = product of the kernel axes the output lacks, columns = the rest
+    lhs, out = equation.split("->")
+    kspec = lhs.split(",")[1]
+    rows = int(np.prod([d for c, d in zip(kspec, kshape) if c not in out]))
+    assert qk["rows"] == rows and qk["rows"] * qk["cols"] == int(np.prod(kshape))
+    assert tuple(qk["kernel"].shape) == (rows, (qk["cols"] + 1) // 2)
+    w64 = _einsum_int4_kernel_by_loops(qk, block_size)
+    want = np.einsum(equation, x.double().numpy(), w64) + bias.double().numpy()
+    y = ref.einsum_dense_int4_call(x, qk, equation, bias=bias, block_size=block_size)
+    assert y.dtype == torch.float32 and tuple(y.shape) == want.shape
+    assert np.abs(y.double().numpy() - want).max() / np.abs(want).max() < 1e-5
+    # the de-quantised kernel is the float kernel to within half a step of the column's scale
+    # (grouped: one step of the group's, the value and the zero point being rounded separately),
+    # so a scale applied to the wrong axis fails here
+    if block_size is None:
+        bound = 0.5001 * (1.0 / qk["kernel_scale"].double().numpy())[None, :]
+    else:
+        bound = 1.0001 * np.repeat(qk["kernel_scale"].double().numpy(), block_size, axis=0)[:rows]
+    flat_err = np.abs(w64.reshape(rows, qk["cols"]) - kernel.double().numpy().reshape(rows, qk["cols"]))
+    assert (flat_err <= bound + 1e-7).all()
+    # bfloat16 compute: same quantity within the bfloat16 bound
+    yb = ref.einsum_dense_int4_call(x, qk, equation, bias=bias, compute_dtype="bfloat16", block_size=block_size)
+    assert yb.dtype == torch.bfloat16
+    assert np.abs(yb.double().numpy() - want).max() / np.abs(want).max() < 2e-2
+
+
+@pytest.mark.parametrize("compute_dtype,tol", [("float32", 1e-5), ("bfloat16", 2e-2)])
+def test_dense_lora_term_is_two_matmuls(compute_dtype, tol):
+    g = torch.Generator().manual_seed(29)
+    x = torch.randn(5, 24, generator=g)
+    a = torch.randn(24, 4, generator=g) * 0.3
+    b = torch.randn(4, 9, generator=g) * 0.3
+    got = ref.dense_lora_term(x, a, b, alpha=8.0, rank=4, compute_dtype=compute_dtype)
+    want = np.zeros((5, 9))
+    xa = np.zeros((5, 4))
+    for m in range(5):
+        for r in range(4):
+            xa[m, r] = sum(float(x[m, k]) * float(a[k, r]) for k in range(24))
+    for m in range(5):
+        for n in range(9):
+            want[m, n] = (8.0 / 4) * sum(xa[m, r] * float(b[r, n]) for r in range(4))
+    assert tuple(got.shape) == (5, 9) and got.dtype == getattr(torch, compute_dtype)
+    assert np.abs(got.double().numpy() - want).max() / np.abs(want).max() < tol
+    # alpha / rank is the only scaling: doubling alpha doubles the term, a zero b removes it
+    twice = ref.dense_lora_term(x, a, b, alpha=16.0, rank=4, compute_dtype=compute_dtype)
+    assert torch.equal(twice, 2 * got)
+    assert ref.dense_lora_term(x, a, torch.zeros(4, 9), 8.0, 4, compute_dtype).abs().max().item() == 0
+
+
+def _einsum_int8_dequant_by_loops(equation, q, s):
+    """float64 q / scale with the stored scale indexed by hand: the stored scale broadcasts
+    against the OUTPUT labels (size 1 where the kernel lacks the label), einsum_dense.py:1449-1491."""
+    lhs, out = equation.split("->")
+    kspec = lhs.split(",")[1]
+    s = s.double().numpy()
+    assert s.ndim == len(out), (s.shape, out)
+    w = np.zeros(tuple(q.shape), np.float64)
+    for idx in np.ndindex(*q.shape):
+        pos = dict(zip(kspec, idx))
+        sidx = tuple(pos[c] if (c in kspec and s.shape[i] != 1) else 0 for i, c in enumerate(out))
+        w[idx] = float(q[idx]) / s[sidx]
+    return w
+
+
+@pytest.mark.parametrize("equation,kshape,rank_in,ab_shapes", [
+    ("btd,dnh->btnh", (12, 3, 4), 3, ((12, 2), (2, 3, 4))),
+    ("btnh,nhd->btd", (3, 4, 10), 4, ((3, 4, 2), (2, 10))),
+    ("abcde,afce->acdbf", (1, 6, 2, 8), 5, ((1, 6, 2, 2), (2, 8))),
+    ("ab,bcd->acd", (8, 3, 4), 2, ((8, 2), (2, 3, 4))),
+])
+def test_einsum_merged_lora_kernel_int8(equation, kshape, rank_in, ab_shapes):
+    # lora_kernel_a has the kernel's shape up to its last axis + [rank], lora_kernel_b is
+    # [rank, last axis] (einsum_dense.py:327-360); matmul(a, b) therefore has the kernel's shape
+    g = torch.Generator().manual_seed(31)
+    kernel = torch.rand(kshape, generator=g) - 0.5
+    qk, ks, info = ref.einsum_dense_quantize_int8(kernel, equation, rank_in)
+    rank = 2
+    a = torch.randn(kshape[:-1] + (rank,), generator=g) * 0.05
+    b0 = torch.zeros(rank, kshape[-1])
+    q0, s0, z0 = ref.einsum_dense_merged_lora_kernel("int8", qk, ks, a, b0, 4.0, rank, equation, rank_in)
+    assert z0 is None and torch.equal(q0, qk) and tuple(s0.shape) == tuple(ks.shape)
+    assert torch.allclose(s0, ks, rtol=1e-5, atol=0)
+    b = torch.randn(rank, kshape[-1], generator=g) * 0.05
+    q1, s1, _ = ref.einsum_dense_merged_lora_kernel("int8", qk, ks, a, b, 4.0, rank, equation, rank_in)
+    assert tuple(s1.shape) == tuple(ks.shape) and not torch.equal(q1, qk)
+    old = _einsum_int8_dequant_by_loops(equation, qk, ks)
+    new = _einsum_int8_dequant_by_loops(equation, q1, s1)
+    update = (4.0 / rank) * np.matmul(a.double().numpy(), b.double().numpy())
+    step = np.abs(new / np.where(q1.numpy() == 0, 1, q1.numpy()))  # |1 / scale| wherever q != 0
+    step = np.where(q1.numpy() == 0, step.max(), step)
+    assert (np.abs(new - (old + update)) <= 0.5001 * step + 1e-6).all()
+
+
+@pytest.mark.parametrize("equation,kshape,rank_in", [
+    ("btd,dnh->btnh", (16, 3, 4), 3), ("btnh,nhd->btd", (2, 8, 10), 4), ("btd,ndh->btnh", (3, 16, 4), 3),
+])
+@pytest.mark.parametrize("block_size", [None, 8])
+def test_einsum_merged_lora_kernel_int4(equation, kshape, rank_in, block_size):
+    g = torch.Generator().manual_seed(37)
+    kernel = torch.rand(kshape, generator=g) - 0.5
+    qk = ref.einsum_dense_quantize_int4(kernel, equation, rank_in, block_size)
+    rank = 2
+    a = torch.randn(kshape[:-1] + (rank,), generator=g) * 0.3
+    old = _einsum_int4_kernel_by_loops(qk, block_size)
+    q0, s0, z0 = ref.einsum_dense_merged_lora_kernel(
+        "int4", None, None, a, torch.zeros(rank, kshape[-1]), 4.0, rank, equation, rank_in,
+        qk=qk, block_size=block_size)
+    assert tuple(q0.shape) == tuple(qk["kernel"].shape) and q0.dtype == torch.int8
+    if block_size is None:
+        assert z0 is None and torch.equal(q0, qk["kernel"])
+        assert torch.allclose(s0, qk["kernel_scale"], rtol=1e-5, atol=0)
+    b = torch.randn(rank, kshape[-1], generator=g) * 0.3
+    q1, s1, z1 = ref.einsum_dense_merged_lora_kernel("int4", None, None, a, b, 4.0, rank, equation, rank_in,
+                                                     qk=qk, block_size=block_size)
+    merged = dict(qk, kernel=q1, kernel_scale=s1, kernel_zero=z1)
+    new = _einsum_int4_kernel_by_loops(merged, block_size)
+    update = (4.0 / rank) * np.matmul(a.double().numpy(), b.double().numpy())
+    rows, cols = qk["rows"], qk["cols"]
+    if block_size is None:
+        bound = 0.5001 * (1.0 / s1.double().numpy())[None, :]
+    else:
+        bound = 1.0001 * np.repeat(s1.double().numpy(), block_size, axis=0)[:rows]
+    target = (old + update).reshape(rows, cols)
+    err = np.abs(new.reshape(rows, cols) - target)
+    if block_size is not None:
+        # the zero point is clipped to the int4 range, so a group whose values do not straddle
+        # zero is not representable within a step (quantizers.py:210-222): leave those out
+        grp = target.reshape(rows // block_size, block_size, cols)
+        straddles = (grp.min(axis=1) <= 0) & (grp.max(axis=1) >= 0)
+        assert straddles.mean() > 0.5
+        err = np.where(np.repeat(straddles, block_size, axis=0), err, 0.0)
+    assert (err <= bound + 1e-6).all()
+    assert not torch.equal(q1, qk["kernel"])
+
+
+@pytest.mark.parametrize("mode,block_size", [("int8", None), ("int4", None), ("int4", 8)])
+def test_embedding_merged_lora_table(mode, block_size):
+    g = torch.Generator().manual_seed(41)
+    V, D, rank, alpha = 11, 24, 3, 6.0
+    table = torch.randn(V, D, generator=g) * 0.2
+    a = torch.randn(V, rank, generator=g) * 0.3
+    if mode == "int8":
+        q, s = ref.embedding_quantize_int8(table)
+        zero = g_idx = None
+        kw = dict()
+    else:
+        e = ref.embedding_quantize_int4(table, block_size)
+        q, s, zero, g_idx = e["embeddings"], e["embeddings_scale"], e["embeddings_zero"], e["g_idx"]
+        kw = dict(embeddings_zero=zero, g_idx=g_idx, block_size=block_size, orig_output_dim=D)
+
+    def dequant(q, s, z):
+        """float64 table by loops: row v, column d; int4 byte [v, d // 2], even d low nibble;
+        per-row scale divides, grouped (groups along d) scale multiplies (embedding.py:726-752)."""
+        out = np.zeros((V, D))
+        for v in range(V):
+            for d in range(D):
+                val = int(q[v, d]) if mode == "int8" else _nibble(q[v, d // 2], d % 2 == 1)
+                if block_size is None:
+                    out[v, d] = val / float(s[v])
+                else:
+                    out[v, d] = (val - int(z[v, d // block_size])) * float(s[v, d // block_size])
+        return out
+
+    q0, s0, z0 = ref.embedding_merged_lora_table(mode, q, s, a, torch.zeros(rank, D), alpha, rank, **kw)
+    assert tuple(q0.shape) == tuple(q.shape) and q0.dtype == torch.int8 and tuple(s0.shape) == tuple(s.shape)
+    if block_size is None:
+        assert z0 is None and torch.equal(q0, q) and torch.allclose(s0, s, rtol=1e-5, atol=0)
+    else:
+        assert tuple(z0.shape) == tuple(zero.shape) and z0.dtype == torch.int8
+    b = torch.randn(rank, D, generator=g) * 0.3
+    q1, s1, z1 = ref.embedding_merged_lora_table(mode, q, s, a, b, alpha, rank, **kw)
+    target = dequant(q, s, zero) + (alpha / rank) * (a.double().numpy() @ b.double().numpy())
+    got = dequant(q1, s1, z1)
+    if block_size is None:
+        bound = 0.5001 * (1.0 / s1.double().numpy())[:, None]
+    else:
+        bound = 1.0001 * np.repeat(s1.double().numpy(), block_size, axis=1)[:, :D]
+    err = np.abs(got - target)
+    if block_size is not None:
+        grp = target.reshape(V, D // block_size, block_size)
+        straddles = (grp.min(axis=2) <= 0) & (grp.max(axis=2) >= 0)
+        assert straddles.mean() > 0.5
+        err = np.where(np.repeat(straddles, block_size, axis=1), err, 0.0)
+    assert (err <= bound + 1e-6).all()
+    assert not torch.equal(q1, q)
