@@ -419,7 +419,9 @@ def dense_int4_call(inputs, kernel, kernel_scale, orig_output_dim,
 # --------------------------------------------------------------------------
 def dense_lora_term(inputs, lora_a, lora_b, alpha, rank, compute_dtype=None):
     """keras/src/layers/core/dense.py:977-980 / :1086-1089: what a quantized call adds when LoRA
-    is enabled, before the bias (the float32 LoRA variables are read in the compute dtype)."""
+    is enabled, before the bias (the float32 LoRA variables are read in the compute dtype).
+    Pinned by: the two matrix products as scalar float64 loops, linearity in alpha, a zero `b`
+    (tests/test_oracle.py::test_dense_lora_term_is_two_matmuls)."""
     cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
     x = torch.matmul(inputs.to(cd), _read_var(lora_a, cd))
     x = torch.matmul(x, _read_var(lora_b, cd))
@@ -623,7 +625,12 @@ def einsum_dense_merged_lora_kernel(mode, kernel, kernel_scale, lora_a, lora_b, 
     """keras/src/layers/core/einsum_dense.py:1536-1623: de-quantise (int8: kernel over its scale
     taken back through `_adjust_scale_for_dequant`; int4: `qk` as `einsum_dense_quantize_int4`
     returns it, as Dense on the flat matrix), add (alpha / rank) * a . b, quantise again as
-    `quantize()` does.  Pinned like `dense_merged_lora_kernel` (zero update = identity)."""
+    `quantize()` does.  Pinned by (tests/test_oracle.py::test_einsum_merged_lora_kernel_int8 /
+    _int4): a zero update returns the integers and scales it started from; a real update
+    de-quantises -- weight by weight, the stored scale indexed by hand through the output labels,
+    the int4 nibbles taken from the packed bytes by loops -- to old + update within half a step
+    (grouped: one step), for equations with leading, double and non-leading contracted axes and
+    the shared-label equation of einsum_dense_test.py:598-629."""
     cd = _tdtype(compute_dtype)
     info = einsum_quantization_info(equation, input_rank)
     update = (alpha / rank) * torch.matmul(lora_a, lora_b)
@@ -666,7 +673,12 @@ def einsum_dense_quantize_int4(kernel, equation, input_rank, block_size=128):
 
 def einsum_dense_int4_call(inputs, qk, equation, bias=None, compute_dtype=None,
                            block_size=128):
-    """keras/src/layers/core/einsum_dense.py:1120-1261 (forward, weight-only)."""
+    """keras/src/layers/core/einsum_dense.py:1120-1261 (forward, weight-only).
+    Pinned by tests/test_oracle.py::test_einsum_dense_int4_call_by_loops: a float64 kernel built
+    weight by weight from the packed bytes (nibble order, flat row-major position, per-column or
+    per-(group, column) scale and zero point all spelled out) and contracted with numpy's float64
+    einsum, for five equations including a non-leading contracted axis and an odd column count;
+    the de-quantised kernel is also held to the float kernel within a step."""
     cd = _tdtype(compute_dtype) if compute_dtype is not None else inputs.dtype
     inputs = inputs.to(cd)
     ks = _read_var(qk["kernel_scale"], cd)
@@ -762,7 +774,9 @@ def embedding_merged_lora_table(mode, embeddings, embeddings_scale, lora_a, lora
     """keras/src/layers/core/embedding.py:721-818: de-quantise the table (rows over their scales, or
     `dequantize_with_sz_map` along the output axis), add (alpha / rank) * a . b, quantise again per
     row (grouped: through the transpose, as `quantize()` does).  -> (table, scale, zero) as saved.
-    Pinned like `dense_merged_lora_kernel`: a zero update is the identity on the integers."""
+    Pinned by tests/test_oracle.py::test_embedding_merged_lora_table: a zero update is the identity
+    on the integers and scales; a real update de-quantises (per element, by loops over the stored
+    bytes, groups along the output axis) to old + update within half a step (grouped: one)."""
     cd = _tdtype(compute_dtype)
     grouped = block_size is not None and block_size != -1
     if mode == "int4":
