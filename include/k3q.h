@@ -261,7 +261,9 @@ int k3q_gemv_w4_addend(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
  * A shape whose K split needs more than k3q_gemv_w4_static_max_bytes() of partials
  * (K split x min(M, 16) x N floats) is rejected with K3Q_ERR_WORKSPACE and nothing is launched.
  * Every call on a GPU shares that GPU's array: calls ordered on one stream are fine, calls
- * that overlap in time on one GPU (two streams, two host threads) race on it.
+ * that overlap in time on one GPU (two streams, two host threads) race on it.  The current
+ * device must be the device of `stream`.  The first call on a device may itself be under stream
+ * capture (it adds only the matmul's own nodes to the graph).
  * No counterpart in the reference (torch's matmul owns its own scratch there).
  */
 int64_t k3q_gemv_w4_static_max_bytes(void);
@@ -286,7 +288,9 @@ int k3q_gemv_w4_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
  *            4 bytes zero + 128};                                  y = T(x . ((W - zero) * scale)) (+ bias)
  *   bias: bfloat16 [N] (bias_stride 0) or an [M, N] addend (bias_stride N), or null.
  * Takes (k3q_gemv_w4s_supported): bfloat16 x, 1 <= M <= 16 while the rows fit a workgroup's LDS
- * (M * K <= 65536; up to twice that, staged in two halves, when K % 4096 == 0 and N <= 8192),
+ * (M * K <= 65536 values and M * (2 K + 16) bytes + the cross-wave sums within 160 KiB; beyond that x is
+ * staged in two parts of every wave's slice, the first the larger, when K % 2048 == 0, K >= 4096, that
+ * part fits the same limits and every workgroup has one strip group: N <= 8192),
  * K % 256 == 0, K >= 4096, N % 16 == 0, N >= 3072, block_size <= 0 or == 128; anything else
  * K3Q_ERR_SHAPE (callers keep k3q_gemv_w4 for those).  k3q_gemv_w4s_multi: several kernels against one x (same M, K,
  * block_size), one launch for those whose launch plans agree.
@@ -505,13 +509,17 @@ int k3q_input_op_quantize(const void* x, int dtype, int64_t rows, int64_t dim, c
  * q, k, v, out: [B, H, 128]; cos_table, sin_table: [max_len, 128] (sin with the sign of the
  * rotated half folded in); k_cache, v_cache: [B, H, max_len, 128]; pos: one int64 in device
  * memory, read by the kernel (a captured graph replays with the value it then holds).
+ * A position outside [0, max_len) writes nothing to the caches, gives zero output rows and sets
+ * *oob_flag (one int32 in device memory, may be null; the kernel never clears it) to 1: the torch
+ * ops this stands for raise there, and the caller checks the flag when it next synchronises.
  * No counterpart in the reference's quantized layers: it stands for the torch ops (two
  * multiplies and an add per rotation, two index_copy, scaled_dot_product_attention) that a
  * Keras decoder runs between its Dense / EinsumDense calls.
  */
 int k3q_decode_attention(const void* q, const void* k, const void* v, int dtype, int64_t B, int64_t H,
                          int64_t head_dim, int64_t max_len, const void* cos_table, const void* sin_table,
-                         const int64_t* pos, void* k_cache, void* v_cache, void* out, void* stream);
+                         const int64_t* pos, void* k_cache, void* v_cache, void* out, int* oob_flag,
+                         void* stream);
 
 /*
  * Two more pieces of the decoder harness's glue (no counterpart in the quantized layers; they

@@ -122,7 +122,7 @@ SIGNATURES = {
     "k3q_silu_mul": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr]),
     "k3q_decode_attention": (
         _int,
-        [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr],
+        [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr],
     ),
     "k3q_gemm_w4_kmajor_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "k3q_gemm_w4_kmajor": (

@@ -23,6 +23,7 @@ struct AttnParams {
     const int64_t* pos;             // device: the position of this step
     uint16_t *kc, *vc;              // [B, H, max_len, 128]
     uint16_t* out;                  // [B, H, 128]
+    int* oob;                       // device flag, may be null: set to 1 when the position is outside the cache
     int H, max_len;
     float scale;
 };
@@ -42,8 +43,16 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bh = blockIdx.x;
-    int pos = (int)p.pos[0];
-    pos = pos < 0 ? 0 : (pos >= p.max_len ? p.max_len - 1 : pos);
+    // A position outside the cache (the torch ops this stands for raise there): nothing is written
+    // to the caches, the output rows are zero and the caller's flag is raised.  Every thread reads
+    // the same position, so the whole workgroup leaves here before its first barrier.
+    const int64_t pos64 = p.pos[0];
+    if (pos64 < 0 || pos64 >= p.max_len) {
+        if (tid < kHd) p.out[(int64_t)bh * kHd + tid] = 0;
+        if (tid == 0 && p.oob) p.oob[0] = 1;
+        return;
+    }
+    const int pos = (int)pos64;
     const int64_t row0 = (int64_t)bh * p.max_len;  // first cache row of this (sequence, head)
 
     // ---- rotate q and k, write the new cache rows ----
@@ -188,7 +197,7 @@ using namespace k3q;
 extern "C" int k3q_decode_attention(const void* q, const void* k, const void* v, int dtype, int64_t B,
                                     int64_t H, int64_t head_dim, int64_t max_len, const void* cos_table,
                                     const void* sin_table, const int64_t* pos, void* k_cache,
-                                    void* v_cache, void* out, void* stream) {
+                                    void* v_cache, void* out, int* oob_flag, void* stream) {
     if (dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (B < 0 || H <= 0 || head_dim != kHd || max_len <= 0 || max_len > 32768 || B * H >= (1 << 30))
         return K3Q_ERR_SHAPE;
@@ -206,6 +215,7 @@ extern "C" int k3q_decode_attention(const void* q, const void* k, const void* v,
     p.kc = (uint16_t*)k_cache;
     p.vc = (uint16_t*)v_cache;
     p.out = (uint16_t*)out;
+    p.oob = oob_flag;
     p.H = (int)H;
     p.max_len = (int)max_len;
     p.scale = 0.08838834764831845f;  // 1 / sqrt(128)

@@ -1763,19 +1763,33 @@ __global__ void clear_words(unsigned* p, int n) {
     if (i < n) p[i] = 0u;
 }
 
-// Address of this device's copy of `scratch`; on the first call on a device its counters are
-// also cleared on `s` (a fill kernel, not a memset node: the call may be under graph capture).
+// Address of this device's copy of `scratch` ("this device" = the current one, which a launch on
+// `s` requires to be the device of `s` anyway).  The look-up happens on the first call on a device
+// and that call may already be under stream capture: the symbol query is not a stream operation,
+// so the thread's capture mode is relaxed around it (under the strict modes a capture refuses
+// every call that is not known to be safe, and is invalidated by it).  On a first call outside
+// capture the counters are also cleared on `s` by a fill kernel; a first call under capture relies
+// on what the language guarantees -- a `__device__` array without initialiser is zero when the
+// code object is loaded -- and adds no node of its own to the caller's graph.  Every call leaves
+// the counters at zero again.
 int static_scratch(hipStream_t s, unsigned char** out) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) return K3Q_ERR_LAUNCH;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_scratch_ptr[dev]) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capturing) != hipSuccess) return K3Q_ERR_LAUNCH;
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        if (hipThreadExchangeStreamCaptureMode(&mode) != hipSuccess) return K3Q_ERR_LAUNCH;
         unsigned char* ptr = nullptr;
-        if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr)
-            return K3Q_ERR_LAUNCH;
-        const int words = (int)(kStaticCounterBytes / 4);
-        clear_words<<<(words + 255) / 256, 256, 0, s>>>((unsigned*)ptr, words);
-        if (hipGetLastError() != hipSuccess) return K3Q_ERR_LAUNCH;
+        const hipError_t found = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (hipThreadExchangeStreamCaptureMode(&mode) != hipSuccess) return K3Q_ERR_LAUNCH;
+        if (found != hipSuccess || !ptr) return K3Q_ERR_LAUNCH;
+        if (capturing == hipStreamCaptureStatusNone) {
+            const int words = (int)(kStaticCounterBytes / 4);
+            clear_words<<<(words + 255) / 256, 256, 0, s>>>((unsigned*)ptr, words);
+            if (hipGetLastError() != hipSuccess) return K3Q_ERR_LAUNCH;
+        }
         g_scratch_ptr[dev] = ptr;
     }
     *out = g_scratch_ptr[dev];

@@ -1,4 +1,4 @@
-// Weight-only int4 decode matmul from a strip-linear copy of the kernel: y[M,N] = x[M,K] . W4[K,N], M <= 8.
+// Weight-only int4 decode matmul from a strip-linear copy of the kernel: y[M,N] = x[M,K] . W4[K,N], M <= 16.
 //
 // The layer's stored kernel ([K, ceil(N/2)] bytes, two output columns per byte) makes a workgroup
 // read 128-byte pieces at a 4 KiB stride and needs a split of K over workgroups to fill the chip.

@@ -95,11 +95,12 @@ class DecoderBlock(Layer):
         self.down.build((None, ffn_dim))
         self.built = True
 
-    def forward(self, x, rows, cache, pos, tables=None):
+    def forward(self, x, rows, cache, pos, tables=None, oob_flag=None):
         """x [B, T, D].  cache: (k, v) each [B, H, maxT, hd], written at positions `pos`
         (an int64 device tensor [T]); rows(): (cos, sin, mask) of these positions -- the table
         rows and mask [T, maxT], 0 where a key may be attended to, -inf elsewhere -- asked for
-        only by the torch path; tables: the whole (cos, sin) tables, for the one-position kernel."""
+        only by the torch path; tables: the whole (cos, sin) tables, for the one-position kernel;
+        oob_flag: the int32 device flag that kernel raises for a position outside the cache."""
         # The normalisations and the gate are handed to the projections that consume them as their
         # `input_op`: at one position they ride inside the projections' launches, in front of int8
         # layers they share a launch with the activation quantizer, otherwise they run as their own
@@ -111,7 +112,7 @@ class DecoderBlock(Layer):
             q, k, v = call_together((self.query, self.key, self.value), self.attn_norm(x))
         if tables is not None and q.shape[1] == 1 and kops.decode_attention_supported(q, cache[0]):
             # one position: rotation, cache update and attention in one launch (5 launches per block)
-            a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1])
+            a = kops.decode_attention(q, k, v, tables[0], tables[1], pos, cache[0], cache[1], oob_flag=oob_flag)
         else:
             # one rotation over the query and key heads together (half the elementwise launches)
             cos, sin, mask = rows()
@@ -173,6 +174,16 @@ class LlamaStyleDecoder(Model):
         self.cos, self.sin = rope_tables(self.head_dim, max_len, self.device,
                                          dtype=to_torch_dtype(self.compute_dtype))
         self._graphs = {}
+        # raised by the one-position attention kernel when a step's position is outside the cache
+        # (the torch path's index_copy_ raises there); read by check_positions()
+        self._pos_oob = torch.zeros(1, dtype=torch.int32, device=self.device)
+
+    def check_positions(self):
+        """Raise IndexError if any decode step since the last check ran at a position outside
+        the cache (synchronises)."""
+        if int(self._pos_oob.item()):
+            self._pos_oob.zero_()
+            raise IndexError(f"a decode step ran at a position outside the cache of {self.max_len} rows")
 
     # ---- synthetic quantized weights ---------------------------------------------------
     def randomize_quantized_weights(self, seed=0):
@@ -231,7 +242,7 @@ class LlamaStyleDecoder(Model):
             return made[0]
 
         for block, kv in zip(self.blocks, cache):
-            x = block.forward(x, rows, kv, pos, tables=(self.cos, self.sin))
+            x = block.forward(x, rows, kv, pos, tables=(self.cos, self.sin), oob_flag=self._pos_oob)
         if last_only:
             x = x[:, -1:, :]
         return self.token_embedding(self.final_norm(x), reverse=True)
@@ -330,6 +341,7 @@ class LlamaStyleDecoder(Model):
             torch.cuda.synchronize(self.device)
             stats.update(prefill_ms=ev[0].elapsed_time(ev[1]), decode_ms=ev[2].elapsed_time(ev[3]),
                          decode_steps=timed, batch=B)
+        self.check_positions()
         return result
 
     def generate(self, prompt, steps, use_graph=True, stats=None):
@@ -376,4 +388,5 @@ class LlamaStyleDecoder(Model):
             torch.cuda.synchronize(self.device)
             stats.update(prefill_ms=ev[0].elapsed_time(ev[1]), decode_ms=ev[2].elapsed_time(ev[3]),
                          decode_steps=timed, batch=B)
+        self.check_positions()
         return out_buf

@@ -952,13 +952,16 @@ def decode_attention_supported(q, cache_k):
             and q.shape[-1] == 128 and cache_k.dtype == torch.bfloat16 and cache_k.shape[2] <= 32768)
 
 
-def decode_attention(q, k, v, cos_table, sin_table, pos, cache_k, cache_v):
+def decode_attention(q, k, v, cos_table, sin_table, pos, cache_k, cache_v, oob_flag=None):
     """One decode position of causal self-attention: q, k, v `[B, 1, H, 128]` bfloat16 (as the
     projections give them), `cos_table` / `sin_table` `[max_len, 128]`, `pos` an int64 device
     tensor holding the position, the caches `[B, H, max_len, 128]` (row `pos` is written).
     Returns `[B, 1, H, 128]`.  What it replaces in a decoder step: the rotation of q and k,
     two `index_copy_` into the caches and `scaled_dot_product_attention` under a mask that
-    admits keys `<= pos`."""
+    admits keys `<= pos`.  A position outside `[0, max_len)` (where `index_copy_` raises) leaves
+    the caches alone, returns zero rows and sets `oob_flag` (an int32 device tensor of one element
+    that the caller reads when it synchronises anyway; without one the call checks a flag of its
+    own, which costs a synchronisation)."""
     _lib.require_device(q, k, v, cos_table, sin_table, pos, cache_k, cache_v)
     lib = _lib.load()
     B, T, H, hd = q.shape
@@ -980,11 +983,20 @@ def decode_attention(q, k, v, cos_table, sin_table, pos, cache_k, cache_v):
     cos_table = cos_table if cos_table.is_contiguous() else cos_table.contiguous()
     sin_table = sin_table if sin_table.is_contiguous() else sin_table.contiguous()
     out = torch.empty((B, 1, H, hd), dtype=torch.bfloat16, device=q.device)
+    own_flag = oob_flag is None and not torch.cuda.is_current_stream_capturing()
+    if own_flag:
+        oob_flag = torch.zeros(1, dtype=torch.int32, device=q.device)
+    if oob_flag is not None:
+        _lib.require_device(oob_flag)
+        if oob_flag.dtype != torch.int32 or oob_flag.numel() != 1:
+            raise ValueError("oob_flag must be one int32 value on the device")
     rc = lib.k3q_decode_attention(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.dtype_code(q.dtype), B, H, hd,
                                   max_len, _lib.ptr(cos_table), _lib.ptr(sin_table), _lib.ptr(pos),
-                                  _lib.ptr(cache_k), _lib.ptr(cache_v), _lib.ptr(out),
+                                  _lib.ptr(cache_k), _lib.ptr(cache_v), _lib.ptr(out), _lib.ptr(oob_flag),
                                   _lib.stream_ptr(q.device))
     _lib.check(rc, "k3q_decode_attention")
+    if own_flag and int(oob_flag.item()):
+        raise IndexError(f"decode_attention: position {int(pos.item())} is outside the cache of {max_len} rows")
     return out
 
 

@@ -150,3 +150,31 @@ def test_silu_mul_matches_torch(dev, rows, dim):
     assert (diff <= want.float().abs() * 2 ** -7 + 1e-30).all()
     assert (diff > 0).float().mean().item() < 0.01
     assert torch.equal(kops.silu_mul(gate.contiguous(), up.contiguous()).view(torch.int16), got.view(torch.int16))
+
+
+@pytest.mark.parametrize("bad", [-1, 16, 1 << 40])
+def test_decode_attention_position_outside_the_cache(dev, bad):
+    # where the torch ops (index_copy_ into the caches) raise, the kernel writes nothing to the
+    # caches, returns zero rows and raises the caller's flag; without a flag the call raises itself
+    hd, max_len = 128, 16
+    g = torch.Generator().manual_seed(3)
+    r = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(dev)
+    cos_t, sin_t = rope_tables(hd, max_len, dev, dtype=torch.bfloat16)
+    q, k, v = r(2, 1, 4, hd), r(2, 1, 4, hd), r(2, 1, 4, hd)
+    kc, vc = r(2, 4, max_len, hd), r(2, 4, max_len, hd)
+    kc0, vc0 = kc.clone(), vc.clone()
+    pos = torch.full((1,), bad, dtype=torch.int64, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = kops.decode_attention(q, k, v, cos_t, sin_t, pos, kc, vc, oob_flag=flag)
+    torch.cuda.synchronize()
+    assert flag.item() == 1 and out.abs().max().item() == 0
+    assert torch.equal(kc.view(torch.int16), kc0.view(torch.int16))
+    assert torch.equal(vc.view(torch.int16), vc0.view(torch.int16))
+    with pytest.raises(IndexError):
+        kops.decode_attention(q, k, v, cos_t, sin_t, pos, kc, vc)
+    # a position inside leaves a raised flag alone and a clear one clear
+    pos.fill_(max_len - 1)
+    flag.zero_()
+    kops.decode_attention(q, k, v, cos_t, sin_t, pos, kc, vc, oob_flag=flag)
+    assert flag.item() == 0
+    assert not torch.equal(kc.view(torch.int16), kc0.view(torch.int16))
