@@ -61,6 +61,33 @@ int k3q_absmax_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols,
                         int8_t* q, void* scale, void* stream);
 
 /*
+ * The weight quantizers of `quantize()` for kernels that live on the device.  The reference
+ * runs them in numpy on the host (`to_numpy=True`); these repeat its float32 operations one
+ * by one, so q, scale and zero are the bits numpy produces (bfloat16 inputs are widened to
+ * float32 first and the scale is rounded back to bfloat16 at the end).
+ *
+ * k3q_weight_absmax_quantize replaces keras/src/quantizers/quantizers.py:95-109 for a reduction
+ * over the middle axis of a contiguous x [outer, R, inner] (Dense: axis 0 of [K, N] is outer 1,
+ * R = K, inner = N; EinsumDense: its kernel's reduced axes):
+ *     scale[o, i] = hi / (max_r |x[o, r, i]| + eps);  q = int8(clip(rint(x * scale), lo, hi))
+ * q: [outer, R, inner] int8; scale: [outer, inner] of x_dtype; amax_workspace: outer * inner
+ * 32-bit words of scratch (cleared by the call).  outer <= 65535, R <= 65535 * 256.
+ *
+ * k3q_weight_quantize_grouped replaces the numpy variant of
+ * abs_max_quantize_grouped_with_zero_point, quantizers.py:182-234, for x [K, N]: groups of
+ * `block_size` rows (the last one zero-padded), per (group, column)
+ *     scale = ((max - min) + eps) / (hi - lo);  zero = clip(rint(-min / scale) + lo, lo, hi)
+ *     q = int8(clip(rint(x / scale) + zero, lo, hi))
+ * q: [K, N] int8; scale: [ceil(K / block_size), N] of x_dtype; zero: the same shape, int8.
+ */
+int k3q_weight_absmax_quantize(const void* x, int x_dtype, int64_t outer, int64_t R, int64_t inner,
+                               float epsilon, float range_lo, float range_hi, int8_t* q, void* scale,
+                               void* amax_workspace, void* stream);
+int k3q_weight_quantize_grouped(const void* x, int x_dtype, int64_t K, int64_t N, int64_t block_size,
+                                float epsilon, float range_lo, float range_hi, int8_t* q, void* scale,
+                                int8_t* zero, void* stream);
+
+/*
  * pack_int4 along the middle axis of a contiguous [outer, len, inner] int8 or
  * uint8 tensor -> [outer, ceil(len/2), inner]; byte = (lo & 15) | ((hi & 15) << 4),
  * an odd `len` is padded with one zero slice.

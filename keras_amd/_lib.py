@@ -40,6 +40,10 @@ SIGNATURES = {
         _int,
         [_ptr, _int, _i64, _i64, _i64, _f32, _f32, _f32, _ptr, _ptr, _ptr],
     ),
+    "k3q_weight_absmax_quantize": (
+        _int, [_ptr, _int, _i64, _i64, _i64, _f32, _f32, _f32, _ptr, _ptr, _ptr, _ptr]),
+    "k3q_weight_quantize_grouped": (
+        _int, [_ptr, _int, _i64, _i64, _i64, _f32, _f32, _f32, _ptr, _ptr, _ptr, _ptr]),
     "k3q_pack_int4": (_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr]),
     "k3q_unpack_int4": (_int, [_ptr, _i64, _i64, _i64, _i64, _int, _ptr, _ptr]),
     "k3q_gemm_i8_workspace_bytes": (_i64, [_i64, _i64, _i64]),

@@ -17,6 +17,7 @@ SOURCES = [
     "k3q_api.hip",
     "k3q_pack.hip",
     "k3q_quantize.hip",
+    "k3q_weight_quantize.hip",
     "k3q_gemv_w4.hip",
     "k3q_gemv_w4s.hip",
     "k3q_gemv_w4_nk.hip",

@@ -10,10 +10,13 @@ through the k3q C ABI.
   pack_int4 / unpack_int4                   quantizers.py:623-900
   dequantize_with_sz_map                    quantizers.py:1631-1668
 
-`to_numpy=True` keeps the reference's meaning: the arithmetic is done with
-numpy on the host (the reference does this on purpose, to keep the float
-kernel off the device while a model is being converted) and the results are
-moved to the device of the input.
+`to_numpy=True` keeps the reference's meaning for host tensors and arrays: the
+arithmetic is done with numpy on the host (the reference does this on purpose,
+to keep the float kernel off the device while a model is being converted) and
+the results are moved to the device of the input.  A float32 / bfloat16 tensor
+that already lives on a HIP device is quantised where it is, by kernels that
+repeat numpy's float32 operations one by one (k3q_weight_quantize.hip): the same
+integers, scales and zero points, bit for bit, without the trip to the host.
 """
 
 import math
@@ -71,6 +74,8 @@ def abs_max_quantize(
         raise NotImplementedError(
             f"abs_max_quantize on this path produces int8 only, got dtype={dtype}"
         )
+    if to_numpy and _on_device(inputs) and len(_standardize_axis(axis, inputs.dim())) > 0:
+        return _abs_max_quantize_numpy_bits(inputs, axis, value_range, epsilon)
     if to_numpy:
         # reference: quantizers.py:95-109
         device = inputs.device if isinstance(inputs, torch.Tensor) else None
@@ -128,6 +133,55 @@ def abs_max_quantize(
         inv = [perm.index(i) for i in range(rank)]
         q = q2.reshape([x.shape[i] for i in perm]).permute(inv)
     return q, s1.reshape(scale_shape)
+
+
+def _on_device(x):
+    return isinstance(x, torch.Tensor) and x.is_cuda and x.dtype in (torch.float32, torch.bfloat16)
+
+
+def _abs_max_quantize_numpy_bits(x, axis, value_range, epsilon):
+    """The `to_numpy=True` result (quantizers.py:95-109: float32 numpy arithmetic, scale cast back
+    to the input's dtype) for a tensor that lives on the device, computed there."""
+    _check_int8_range(value_range, "int8")
+    rank = x.dim()
+    ax = _standardize_axis(axis, rank)
+    scale_shape = [1 if i in ax else x.shape[i] for i in range(rank)]
+    if x.numel() == 0:
+        raise ValueError("Cannot compute the max of an empty tensor.")
+    if ax[-1] == rank - 1 and ax == tuple(range(ax[0], rank)):
+        # trailing axes: the row kernel in float32 is the same operation sequence
+        q, s = abs_max_quantize(x.float() if x.dtype != torch.float32 else x, ax, value_range, "int8",
+                                epsilon, to_numpy=False)
+        return q, s.to(x.dtype)
+    run = ax == tuple(range(ax[0], ax[-1] + 1))
+    if run:
+        src, perm = x.contiguous(), None
+    else:
+        # reduced axes that are not neighbours: bring them together in front of the trailing kept axes
+        kept = [i for i in range(rank) if i not in ax]
+        head = [i for i in kept if i < ax[0]]
+        perm = head + list(ax) + [i for i in kept if i > ax[0]]
+        src = x.permute(perm).contiguous()
+    shape = list(src.shape)
+    a0 = ax[0] if run else len([i for i in range(rank) if i not in ax and i < ax[0]])
+    outer = int(np.prod(shape[:a0], dtype=np.int64)) if a0 else 1
+    R = int(np.prod(shape[a0:a0 + len(ax)], dtype=np.int64))
+    inner = int(np.prod(shape[a0 + len(ax):], dtype=np.int64))
+    q = torch.empty(shape, dtype=torch.int8, device=x.device)
+    s = torch.empty((outer * inner,), dtype=x.dtype, device=x.device)
+    ws = torch.empty((outer * inner,), dtype=torch.int32, device=x.device)
+    rc = _lib.load().k3q_weight_absmax_quantize(
+        _lib.ptr(src), _lib.dtype_code(x.dtype), outer, R, inner, float(epsilon),
+        float(value_range[0]), float(value_range[1]), _lib.ptr(q), _lib.ptr(s), _lib.ptr(ws),
+        _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_weight_absmax_quantize")
+    if perm is not None:
+        inv = [perm.index(i) for i in range(rank)]
+        q = q.permute(inv)
+        kept_shape = [shape[i] for i in range(len(shape)) if not (a0 <= i < a0 + len(ax))]
+        kept_axes = [p_ for i, p_ in enumerate(perm) if not (a0 <= i < a0 + len(ax))]
+        s = s.reshape(kept_shape).permute(sorted(range(len(kept_axes)), key=kept_axes.__getitem__))
+    return q, s.reshape(scale_shape)
 
 
 class Quantizer:
@@ -195,14 +249,35 @@ def abs_max_quantize_grouped_with_zero_point(
 ):
     """Grouped asymmetric quantisation of a `[input_dim, output_dim]` kernel.
 
-    Host (numpy) variant, the one `Dense.quantize` / `EinsumDense.quantize`
-    call (quantizers.py:179-234).  Returns `(q int8 [K,N], scale [G,N],
-    zero int8 [G,N])` on the device of `inputs`.
+    The numpy variant, the one `Dense.quantize` / `EinsumDense.quantize` call
+    (quantizers.py:179-234): on the host for host inputs, on the device -- the same
+    float32 operations, the same bits -- for a float32 / bfloat16 tensor that lives
+    there.  Returns `(q int8 [K,N], scale [G,N], zero int8 [G,N])` on the device of
+    `inputs`.
     """
     if not to_numpy:
         raise NotImplementedError(
-            "only the host variant (to_numpy=True) is on the inference path"
+            "only the numpy variant (to_numpy=True) is on the inference path: the tensor variant "
+            "(quantizers.py:237-306) goes through the GPTQ parameter search, which the layers never call"
         )
+    if _on_device(inputs):
+        if inputs.dim() != 2:
+            raise ValueError(f"expected a [input_dim, output_dim] kernel, got shape {tuple(inputs.shape)}")
+        if dtype != "int8":
+            raise NotImplementedError(f"the grouped quantizer produces int8 storage only, got dtype={dtype}")
+        _check_int8_range(value_range, dtype)
+        x = inputs.contiguous()
+        K, N = x.shape
+        G = math.ceil(K / block_size)
+        q = torch.empty((K, N), dtype=torch.int8, device=x.device)
+        st = torch.empty((G, N), dtype=x.dtype, device=x.device)
+        zt = torch.empty((G, N), dtype=torch.int8, device=x.device)
+        rc = _lib.load().k3q_weight_quantize_grouped(
+            _lib.ptr(x), _lib.dtype_code(x.dtype), K, N, int(block_size), float(epsilon),
+            float(value_range[0]), float(value_range[1]), _lib.ptr(q), _lib.ptr(st), _lib.ptr(zt),
+            _lib.stream_ptr(x.device))
+        _lib.check(rc, "k3q_weight_quantize_grouped")
+        return q, st, zt
     device = inputs.device if isinstance(inputs, torch.Tensor) else None
     original_dtype = inputs.dtype if isinstance(inputs, torch.Tensor) else None
     arr = _to_host_array(inputs)
