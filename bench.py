@@ -11,9 +11,11 @@ the second half of the headline metric, is reported under `int4_gemv` with its o
 HBM roofline (the layer's route: the strip-linear copy of the kernel, made once per layer).  `int8_gemm_sweep` holds the GEMM kernel's time over the
 large-M sweep (M in {512, 2048, 4096, 8192} x K=N in {4096, 8192}, plus K=8192, N=28672),
 `einsum_int8` the EinsumDense attention projections (batch 8, t in {1, 512});
-`llama_decode_int4` is the end-to-end greedy decode of a 32-layer Llama-style decoder whose
-weight matrices are all int4 (tokens/s at batch 1 and 8), `llama_decode_int8` the same with
-int8 layers.
+`pack_unpack` the standalone pack_int4 / unpack_int4 kernels at 8192 x 8192 values on both axes,
+`embedding_lookup` the quantized lookup of 32768 ids; `llama_decode_int4` is configuration 5 end to
+end: a 32-layer Llama-style decoder with random float weights, `model.quantize("int4")` (seconds
+reported), 128-token prompts and 128 greedy steps (tokens/s at batch 1 and 8, resident weight
+bytes), `llama_decode_int8` the same with `model.quantize("int8")`.
 The CPU oracle (a restatement of the reference's torch-CPU op sequence) is timed
 on the host cores on a bounded sample as `cpu_baseline`.
 
@@ -77,11 +79,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
-    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,decode,cpu: run the headline "
+    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,pack,embed,decode,cpu: run the headline "
                     "step and only these further sections (for profiler runs); default: all")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
-    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "decode", "cpu"}
+    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "pack", "embed", "decode", "cpu"}
     if unknown:
         sys.exit(f"bench.py: unknown section(s) {sorted(unknown)}")
     want = (lambda name: not only or name in only)
@@ -483,12 +485,58 @@ def main():
         del s8
         torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ pack / unpack int4
+    # The standalone kernels at the config-2 kernel size (8192 x 8192 int4 values), along the last
+    # axis (what Dense / EinsumDense store) and along axis 0; HBM-bound, 1.5 bytes per value (one
+    # unpacked byte + half a packed one).  Cold: the calls rotate over five tensors of 64 MiB
+    # (packing) or 32 MiB + 64 MiB of fresh output (unpacking), more than the 256 MiB memory-side
+    # cache holds; each call is a graph node.
+    pack_rows = []
+    if want("pack"):
+        n_val = Kg * Ng
+        unpacked = [torch.randint(-8, 8, (Kg, Ng), dtype=torch.int8, device=dev) for _ in range(5)]
+        for axis in (-1, 0):
+            packed = [kq.pack_int4(u, axis=axis)[0] for u in unpacked]
+            for name, call in (("pack_int4", lambda i: kq.pack_int4(unpacked[i % 5], axis=axis)),
+                               ("unpack_int4", lambda i: kq.unpack_int4(packed[i % 5], Kg if axis == 0 else Ng, axis=axis))):
+                us_ = graph_node_us(call, 5, 20)
+                gbs_ = 1.5 * n_val / us_ / 1e3
+                pack_rows.append({"op": name, "axis": axis, "values": n_val, "us_per_call": round(us_, 2),
+                                  "algorithmic_bytes": int(1.5 * n_val),
+                                  "roofline": {"bound": "hbm", "achieved": round(gbs_, 1), "peak": HBM_PEAK_GBS,
+                                               "unit": "GB/s", "frac": round(gbs_ / HBM_PEAK_GBS, 4), "traffic": None}})
+            del packed
+        del unpacked
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ quantized embedding lookup
+    # 32768 random ids into an int8 table of 32000 x 4096 with float32 per-row scales (what a
+    # float32 or mixed_bfloat16 layer stores): 1 byte read and 4 written per element, plus the ids and
+    # a scale per row; the output of a call (512 MiB) is more than the memory-side cache holds.
+    embed_row = None
+    if want("embed"):
+        vocab_, dim_, count_ = 32000, 4096, 32768
+        table_ = torch.randint(-127, 128, (vocab_, dim_), dtype=torch.int8, device=dev)
+        tscale_ = (torch.rand(vocab_, device=dev) * 50 + 50)
+        ids_ = torch.randint(0, vocab_, (count_,), device=dev)
+        us_ = graph_node_us(lambda i: kops.embedding_lookup(ids_, table_, tscale_, dim_, check_ids=False), 2, 8)
+        nbytes_ = count_ * dim_ * 5 + count_ * (8 + 4)
+        embed_row = {"ids": count_, "vocab": vocab_, "dim": dim_, "table": "int8", "out": "float32",
+                     "us_per_call": round(us_, 1), "algorithmic_bytes": nbytes_,
+                     "roofline": {"bound": "hbm", "achieved": round(nbytes_ / us_ / 1e3, 1), "peak": HBM_PEAK_GBS,
+                                  "unit": "GB/s", "frac": round(nbytes_ / us_ / 1e3 / HBM_PEAK_GBS, 4), "traffic": None}}
+        del table_, tscale_, ids_
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ end-to-end decode
-    # Llama-style 32-layer decoder (d_model 4096, 32 heads, SwiGLU 14336, vocab 32000), every
-    # weight matrix int4 (grouped, block 128) with synthetic values written on the device;
-    # prompt of 128 random ids, greedy decode of 128 steps, prompt and decode steps replayed from
-    # HIP graphs.  Matmuls, embedding lookup and LM head run the k3q kernels, and so do the
-    # harness's own normalisations, RoPE + cache update + attention and the SwiGLU gate.
+    # Configuration 5 as written: a Llama-style 32-layer decoder (d_model 4096, 32 heads, SwiGLU
+    # 14336, vocab 32000) built from the layer mirrors with random float weights (mixed_bfloat16:
+    # float32 variables, bfloat16 compute; drawn on the device), converted with
+    # `model.quantize("int4")` (grouped, block 128; the weight quantizers run on the device with the
+    # bits of the reference's numpy path) or `model.quantize("int8")`, then 128 random prompt ids at
+    # batch 1 and 8 and 128 greedy steps, prompt and decode steps replayed from HIP graphs.  Matmuls,
+    # embedding lookup and LM head run the k3q kernels, and so do the harness's own normalisations,
+    # RoPE + cache update + attention and the SwiGLU gate.
     decode = None
     decode_int8 = None
     if want("decode"):
@@ -498,28 +546,45 @@ def main():
         del packs, strips
         torch.cuda.empty_cache()
 
-        def decode_figures(policy):
-            model = LlamaStyleDecoder(max_len=256, dtype="bfloat16", device=dev, layer_policy=policy)
-            model.randomize_quantized_weights()
-            out = []
+        def decode_figures(mode):
+            import warnings
+
+            torch.cuda.synchronize()
+            t0_ = time.perf_counter()
+            model = LlamaStyleDecoder(max_len=256, dtype="mixed_bfloat16", device=dev, init_on_device=True)
+            torch.cuda.synchronize()
+            t1_ = time.perf_counter()
+            with warnings.catch_warnings():
+                warnings.simplefilter("ignore")  # (the norms have no quantized form: reported, not an error)
+                report = model.quantize(mode)
+            torch.cuda.synchronize()
+            t2_ = time.perf_counter()
+            torch.cuda.empty_cache()
+            rows = []
             for batch in (1, 8):
                 prompt = torch.randint(0, model.vocab, (batch, 128), generator=g)
                 model.generate(prompt, 8)  # first-call set-up: the graphs of this shape are captured
                 st = {}
                 model.generate(prompt, 128, stats=st)
-                out.append({
+                rows.append({
                     "batch": batch, "prompt": 128, "steps": 128,
                     "prefill_ms": round(st["prefill_ms"], 2),
                     "decode_ms_per_step": round(st["decode_ms"] / st["decode_steps"], 3),
                     "tokens_per_s": round(batch * st["decode_steps"] / st["decode_ms"] * 1e3, 1),
                 })
+            resident = model.resident_bytes()
+            out = {"policy": "mixed_bfloat16", "mode": mode, "init_float_weights_s": round(t1_ - t0_, 2),
+                   "quantize_s": round(t2_ - t1_, 3), "layers_quantized": report.num_quantized,
+                   # after a prompt and decode steps at both batch sizes: what the reference's layers
+                   # store, and the copies this build keeps beside them for its kernels
+                   "weights_resident_bytes": resident, "runs": rows}
             del model
             torch.cuda.empty_cache()
             return out
 
-        decode = decode_figures("int4/128_from_bfloat16")
+        decode = decode_figures("int4")
         # the same decoder with int8 layers (dynamic per-row activation quantisation)
-        decode_int8 = decode_figures("int8_from_bfloat16")
+        decode_int8 = decode_figures("int8")
 
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu = None
@@ -585,6 +650,8 @@ def main():
         "read_only_launch_32MiB": read_ref4,
         "int8_decode_dense": gemv8,
         "read_only_launch_64MiB": read_ref8,
+        "pack_unpack": pack_rows,
+        "embedding_lookup": embed_row,
         "llama_decode_int4": decode,
         "llama_decode_int8": decode_int8,
         "cpu_baseline": cpu,

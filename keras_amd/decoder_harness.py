@@ -134,23 +134,27 @@ class DecoderBlock(Layer):
 
 class LlamaStyleDecoder(Model):
     def __init__(self, vocab=32000, d_model=4096, n_heads=32, ffn_dim=14336, n_layers=32,
-                 max_len=256, dtype="bfloat16", device=None, seed=0, layer_policy=None):
+                 max_len=256, dtype="bfloat16", device=None, seed=0, layer_policy=None,
+                 init_on_device=False):
         """layer_policy: dtype-policy name for the weight-carrying layers, e.g.
         "int4/128_from_bfloat16": the layers are then built already quantized (zero
         weights, to be filled by `load_own_variables` or `randomize_quantized_weights`)
-        instead of being built in float and converted."""
+        instead of being built in float and converted.
+        init_on_device: draw the random initial weights with the device's generator instead of
+        the host's (seconds instead of half a minute at full size; another stream of numbers)."""
         super().__init__(dtype=dtype, name="llama_style_decoder", device=device)
         self.vocab, self.d_model, self.n_heads = vocab, d_model, n_heads
         self.head_dim = d_model // n_heads
         self.max_len = max_len
-        gen = torch.Generator().manual_seed(seed)
+        gen_device = self.device if init_on_device else torch.device("cpu")
+        gen = torch.Generator(device=gen_device).manual_seed(seed)
         wdtype = layer_policy or dtype
 
         def init(shape, dt):
             # N(0, 1/fan_in); the output projection [heads, head_dim, d_model] contracts its
             # two leading axes, every other kernel its first
             fan_in = shape[0] * shape[1] if len(shape) == 3 and shape[0] == n_heads else shape[0]
-            return (torch.randn(shape, generator=gen) * (1.0 / math.sqrt(fan_in))).to(dt)
+            return (torch.randn(shape, generator=gen, device=gen_device) * (1.0 / math.sqrt(fan_in))).to(dt)
 
         # A layer built straight from an int4 policy has no config and would fall back to the
         # default activation quantizer (reversible_embedding.py:229-233); pass the config that
@@ -162,7 +166,7 @@ class LlamaStyleDecoder(Model):
         self.token_embedding = ReversibleEmbedding(
             vocab, d_model, dtype=wdtype, device=self.device, name="token_embedding",
             quantization_config=emb_config,
-            embeddings_initializer=lambda s, dt: (torch.randn(s, generator=gen) * 0.02).to(dt))
+            embeddings_initializer=lambda s, dt: (torch.randn(s, generator=gen, device=gen_device) * 0.02).to(dt))
         self.token_embedding.build()
         self.token_embedding.check_ids = False
         self.blocks = [

@@ -180,8 +180,51 @@ class Layer:
         t = as_tensor(var)
         cd = to_torch_dtype(self.compute_dtype)
         if t.dtype.is_floating_point and t.dtype != cd:
-            return t.to(cd)
+            # the cast copy is kept while the variable holds the same value (assign() bumps the
+            # variable's version, an in-place write the tensor's): a decode step reads the same
+            # gains and scales thousands of times
+            cache = self.__dict__.setdefault("_read_cache", {})
+            stamp = (var.version, t.data_ptr(), t._version, cd)
+            hit = cache.get(id(var))
+            if hit is not None and hit[0] == stamp and hit[1] is var:
+                return hit[2]
+            value = t.to(cd)
+            cache[id(var)] = (stamp, var, value)
+            return value
         return t
+
+    def resident_bytes(self):
+        """Device memory this layer holds, split into what the reference's layer stores and what
+        this build derives from it: `{"stored": bytes of the variables, "derived": bytes of the
+        copies kept for the kernels (strip-linear / K-contiguous / prepacked kernels, cast
+        scales)}`.  Storage shared by several tensors is counted once.  No counterpart in the
+        reference."""
+        seen, stored = set(), 0
+        for var in getattr(self, "_variables", []):
+            t = as_tensor(var)
+            key = t.untyped_storage().data_ptr()
+            if key not in seen:
+                seen.add(key)
+                stored += t.untyped_storage().nbytes()
+        derived = 0
+
+        def visit(value):
+            nonlocal derived
+            if isinstance(value, torch.Tensor):
+                key = value.untyped_storage().data_ptr()
+                if value.is_cuda and key not in seen:
+                    seen.add(key)
+                    derived += value.untyped_storage().nbytes()
+            elif isinstance(value, (list, tuple)):
+                for v in value:
+                    visit(v)
+            elif isinstance(value, dict):
+                for v in value.values():
+                    visit(v)
+
+        visit(self.__dict__.get("_cache", {}))
+        visit(self.__dict__.get("_read_cache", {}))
+        return {"stored": stored, "derived": derived}
 
     # ---- config ---------------------------------------------------------------
     @classmethod

@@ -144,6 +144,15 @@ class Model(Layer):
         layers = _sublayers(self, seen)
         return ([self] if include_self else []) + layers
 
+    def resident_bytes(self):
+        """`Layer.resident_bytes` summed over the model and every layer below it."""
+        total = {"stored": 0, "derived": 0}
+        for layer in self._flatten_layers(include_self=True):
+            part = Layer.resident_bytes(layer)
+            total["stored"] += part["stored"]
+            total["derived"] += part["derived"]
+        return total
+
     @property
     def layers(self):
         """The layers held directly by this model, containers flattened, sublayers of layers

@@ -36,6 +36,21 @@ def test_pack_unpack_matches_oracle(dev, shape, axis, dtype):
     assert torch.equal(u_gpu.cpu(), arr)
 
 
+@pytest.mark.parametrize("axis", [-1, 0])
+def test_pack_unpack_config2_kernel_size(dev, axis):
+    # the 8192 x 8192 kernel of configuration 2, packed along the last axis (the layers' layout)
+    # and along axis 0 (K-packed, what the configuration's wording describes), int8 storage
+    g = torch.Generator().manual_seed(8192 + axis)
+    arr = torch.randint(-8, 8, (8192, 8192), generator=g, dtype=torch.int8)
+    p_ref, shape_ref, n_ref = ref.pack_int4(arr, axis=axis)
+    p_gpu, shape_gpu, n_gpu = kq.pack_int4(arr.to(dev), axis=axis)
+    assert shape_gpu == shape_ref == ((8192, 4096) if axis == -1 else (4096, 8192)) and n_gpu == n_ref == 8192
+    assert torch.equal(p_gpu.cpu(), p_ref)
+    u_gpu = kq.unpack_int4(p_gpu, n_gpu, axis=axis)
+    assert torch.equal(u_gpu.cpu(), arr)
+    assert torch.equal(ref.unpack_int4(p_ref, n_ref, axis=axis), arr)
+
+
 def test_unpack_all_bytes(dev):
     b = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(torch.int8).reshape(16, 16)
     for axis in (0, 1):
