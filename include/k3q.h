@@ -393,6 +393,18 @@ int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t
                        void* stream);
 
 /*
+ * k3q_gemm_w4_kmajor from the strip-linear copy that the decode kernels stream (k3q_w4s_pack)
+ * instead of a K-contiguous copy of its own: same tiles, same sums in another order of k inside
+ * each unit of 128 (results within the float tolerance of k3q_gemm_w4_kmajor, not its bits), so a
+ * layer keeps ONE derived copy of its kernel for 1 ... 512 rows.  Same arguments and workspace
+ * (k3q_gemm_w4_kmajor_workspace_bytes); block_size <= 0 or a multiple of 128, else K3Q_ERR_SHAPE.
+ */
+int k3q_gemm_w4_strip(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                      const void* w_strip, const void* scale, const void* zero,
+                      int64_t block_size, const void* bias, void* y, void* workspace,
+                      int64_t workspace_bytes, void* stream);
+
+/*
  * Several weight-only int4 matmuls against ONE x, each as k3q_gemv_w4_fused computes it (same
  * bits), in one launch when they are decode-sized (M <= 16) and their launch plans agree
  * (e.g. kernels of one shape: the query / key / value projections of an attention block, the

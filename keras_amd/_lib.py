@@ -133,6 +133,10 @@ SIGNATURES = {
         _int,
         [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr],
     ),
+    "k3q_gemm_w4_strip": (
+        _int,
+        [_ptr, _int, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _ptr],
+    ),
     "k3q_gemv_w4_multi": (
         _int,
         [_ptr, _int, _i64, _i64, _int, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr],

@@ -1168,6 +1168,8 @@ struct KmParams {
     int64_t M, N, K;
     int gsize;              // values of K per group (multiple of kKmStage)
     int klen;               // values of K per split (multiple of gsize)
+    int strip;              // 1: `shadow` is the strip-linear copy of the decode kernels (k3q_w4s_pack), see below
+    int units;              // (strip) K / 128
 };
 
 // sx[g][m] = sum of x[m, g*gsize .. (g+1)*gsize): one wave per (g, m), fixed order.  Stored as
@@ -1241,15 +1243,32 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
         const int ch = (lane & 7) ^ km_swz(row);
         int64_t grow = m0 + row;
         if (grow >= p.M) grow = p.M - 1;
-        a_src[j] = (const char*)(p.x + grow * p.K + k_begin) + ch * 16;
+        // (strip: position 4 g + s of the stage's x row holds chunk 4 s + 2 h + g of the unit's sixteen)
+        a_src[j] = (const char*)(p.x + grow * p.K + k_begin) + (p.strip ? 4 * (ch & 3) + (ch >> 2) : ch) * 16;
     }
+    // The same kernel reads the decode kernels' strip-linear copy instead of a K-contiguous one
+    // (p.strip): [strip = n / 16][unit = k / 128][lane' = i + 16 g'][4 dwords], dword s of lane' the
+    // eight k = 128 unit + 32 s + 8 g' + e.  A stage is then HALF A UNIT in another sense than 64
+    // consecutive k: stage h of a unit takes the pieces g' = 2 h and 2 h + 1 of every column -- a
+    // column's two 16-byte pieces of the stage, 512 contiguous bytes per strip and instruction --
+    // i.e. the sixteen k = 32 s + 16 h ... + 15 for s = 0 ... 3.  MFMA step s of the stage contracts
+    // exactly those sixteen (lanes 0 ... 31 the first eight, lanes 32 ... 63 the second), so only the
+    // SOURCE addresses change: the kernel rows advance by 512 bytes per stage, and the x tile takes
+    // the matching four runs of 32 bytes of the unit's 256 (advancing by 32, then by 224).  A sum
+    // over a group of 128 (= a unit) does not care in which order its k arrive; groups of 64 would
+    // be split across stages and keep the K-contiguous copy.
+    int x_step = p.strip ? 32 : 128;
+    const int w_step = p.strip ? 512 : 32;
     // kernel rows: one instruction per wave and stage = 32 rows x 32 bytes, two lanes per row
     const char* w_src;
     {
         // (narrow tiles: waves 4 ... 7 fetch the rows of waves 0 ... 3 again, into the unused half)
         int64_t n = n0 + (kBN == 128 ? (wave & 3) : wave) * 32 + (lane >> 1);
         if (n >= p.N) n = p.N - 1;
-        w_src = (const char*)p.shadow + n * (p.K / 2) + k_begin / 2 + (lane & 1) * 16;
+        if (p.strip)
+            w_src = (const char*)p.shadow + ((n >> 4) * p.units + k_begin / 128) * 1024 + (n & 15) * 16 + (lane & 1) * 256;
+        else
+            w_src = (const char*)p.shadow + n * (p.K / 2) + k_begin / 2 + (lane & 1) * 16;
     }
     // group parameters, four bytes per lane: waves 0, 1 the scales, wave 2 the zero points,
     // waves 3 ... 6 the sums of x (two dwords per row); the last fetches a spare copy so that
@@ -1309,12 +1328,13 @@ __global__ __launch_bounds__(kKmThreads) void gemm_w4_kmajor(KmParams p) {
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)a_src[j],
                 (__attribute__((address_space(3))) void*)(base + (kXOps * wave + j) * 1024), 16, 0, 0);
-            a_src[j] += 128;
+            a_src[j] += x_step;
         }
+        if (p.strip) x_step = 256 - x_step;
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)w_src,
             (__attribute__((address_space(3))) void*)(base + kKmXBytes + wave * 1024), 16, 0, 0);
-        w_src += 32;
+        w_src += w_step;
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void*)par_src,
             (__attribute__((address_space(3))) void*)(base + kKmXBytes + kKmWBytes + par_dst), 4, 0, 0);
@@ -1660,10 +1680,10 @@ extern "C" int64_t k3q_gemm_w4_kmajor_workspace_bytes(int64_t M, int64_t K, int6
     return ((K / gsize) * M * 8 + 255) / 256 * 256 + (int64_t)pl.ks * M * N * 4;
 }
 
-extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
-                                  const void* w_kmajor, const void* scale, const void* zero,
-                                  int64_t block_size, const void* bias, void* y, void* workspace,
-                                  int64_t workspace_bytes, void* stream) {
+static int run_gemm_w4_tiles(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                             const void* w_kmajor, bool strip, const void* scale, const void* zero,
+                             int64_t block_size, const void* bias, void* y, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
     if (x_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (M < 0 || K <= 0 || N <= 0) return K3Q_ERR_SHAPE;
     if (M == 0) return K3Q_OK;
@@ -1671,6 +1691,7 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     const bool grouped = block_size > 0;
     if (grouped && !zero) return K3Q_ERR_NULL;
     if (!kmajor_ok(M, K, N, block_size)) return K3Q_ERR_SHAPE;
+    if (strip && block_size > 0 && (block_size % 128) != 0) return K3Q_ERR_SHAPE;
     if (!aligned_to(x, 16) || !aligned_to(w_kmajor, 16) || !aligned_to(scale, 8) ||
         (zero && !aligned_to(zero, 4)) || !aligned_to(y, 8) || (bias && !aligned_to(bias, 2)))
         return K3Q_ERR_ALIGN;
@@ -1698,6 +1719,8 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     kp.K = K;
     kp.gsize = (int)gsize;
     kp.klen = (int)pl.klen;
+    kp.strip = strip ? 1 : 0;
+    kp.units = (int)(K / 128);
     dim3 grid((unsigned)((N + pl.bn - 1) / pl.bn), (unsigned)((M + pl.bm - 1) / pl.bm), (unsigned)pl.ks);
     constexpr int kDepth = 4;
     const size_t lds = (size_t)kDepth * kKmSlotBytes;
@@ -1740,6 +1763,22 @@ extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t
     else
         gemv_w4_reduce<true, false><<<rgrid, 256, 0, s>>>(gp, pl.ks);
     return launch_status();
+}
+
+extern "C" int k3q_gemm_w4_kmajor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                  const void* w_kmajor, const void* scale, const void* zero,
+                                  int64_t block_size, const void* bias, void* y, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+    return run_gemm_w4_tiles(x, x_dtype, M, K, N, w_kmajor, false, scale, zero, block_size, bias, y, workspace,
+                             workspace_bytes, stream);
+}
+
+extern "C" int k3q_gemm_w4_strip(const void* x, int x_dtype, int64_t M, int64_t K, int64_t N,
+                                 const void* w_strip, const void* scale, const void* zero,
+                                 int64_t block_size, const void* bias, void* y, void* workspace,
+                                 int64_t workspace_bytes, void* stream) {
+    return run_gemm_w4_tiles(x, x_dtype, M, K, N, w_strip, true, scale, zero, block_size, bias, y, workspace,
+                             workspace_bytes, stream);
 }
 
 // ---- the decode-sized call for callers that cannot allocate -----------------------------

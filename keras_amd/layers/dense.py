@@ -455,13 +455,21 @@ class Dense(Layer):
             # a few dozen to a hundred-odd rows: from the K-contiguous copy of the kernel (made
             # on first use, kept while the kernel does not change), read once as int4
             units = self._orig_output_dim
-            y = kops.int4_matmul_kmajor(
-                inputs, self._cached("kmajor", self._kernel, lambda t: kops.int4_kmajor_copy(t, units)),
-                self._read_cached("kernel_scale", self.kernel_scale),
-                kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
-                block_size=block_size if grouped else None,
-                bias=self._call_bias(),
-            )
+            if kops.int4_tiles_strip_supported(rows, inputs.shape[-1], units, block_size if grouped else None):
+                # ... from the SAME strip-linear copy the decode kernel streams: one derived copy per layer
+                y = kops.int4_matmul_tiles_strip(
+                    inputs, self._cached("w4s", self._kernel, lambda t: kops.int4_strip_copy(t, units)), units,
+                    self._read_cached("kernel_scale", self.kernel_scale),
+                    kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+                    block_size=block_size if grouped else None, bias=self._call_bias())
+            else:
+                y = kops.int4_matmul_kmajor(
+                    inputs, self._cached("kmajor", self._kernel, lambda t: kops.int4_kmajor_copy(t, units)),
+                    self._read_cached("kernel_scale", self.kernel_scale),
+                    kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+                    block_size=block_size if grouped else None,
+                    bias=self._call_bias(),
+                )
         else:
             y = kops.int4_matmul(
                 inputs, as_tensor(self._kernel),

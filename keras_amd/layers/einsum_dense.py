@@ -793,12 +793,19 @@ class EinsumDense(Layer):
         if (x2.dtype == torch.bfloat16 and kmajor_rows(x2.shape[0], units, x2.shape[1])
                 and kops.int4_kmajor_supported(x2.shape[0], x2.shape[1], units,
                                                block_size if grouped else None)):
-            # as Dense: from the K-contiguous copy of the kernel, read once as int4
-            y2 = kops.int4_matmul_kmajor(
-                x2, self._cached("kmajor", self._kernel, lambda t: kops.int4_kmajor_copy(t, units)),
-                self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).contiguous()),
-                kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
-                block_size=block_size if grouped else None, bias=bias)
+            # as Dense: the int4 tile kernel, from the strip-linear copy the decode kernel streams
+            # where it takes the shape, else from a K-contiguous copy; the kernel is read once as int4
+            scale_cd = self._cached("kernel_scale", self.kernel_scale, lambda t: t.to(cd).contiguous())
+            if kops.int4_tiles_strip_supported(x2.shape[0], x2.shape[1], units, block_size if grouped else None):
+                y2 = kops.int4_matmul_tiles_strip(
+                    x2, self._cached("w4s", self._kernel, lambda t: kops.int4_strip_copy(t, units)), units,
+                    scale_cd, kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+                    block_size=block_size if grouped else None, bias=bias)
+            else:
+                y2 = kops.int4_matmul_kmajor(
+                    x2, self._cached("kmajor", self._kernel, lambda t: kops.int4_kmajor_copy(t, units)),
+                    scale_cd, kernel_zero=as_tensor(self.kernel_zero) if grouped else None,
+                    block_size=block_size if grouped else None, bias=bias)
             return self._finish(y2, free_shape, gv, fused)
         y2 = kops.int4_matmul(
             x2, as_tensor(self._kernel),

@@ -496,6 +496,47 @@ def int4_matmul_kmajor(x, kernel_kmajor, kernel_scale, kernel_zero=None, block_s
     return y.reshape(*lead, N)
 
 
+def int4_tiles_strip_supported(M, K, N, block_size=None):
+    """Whether `int4_matmul_tiles_strip` takes M bfloat16 rows against a [K, N] kernel's strip copy."""
+    grouped = block_size is not None and block_size > 0
+    return (int4_kmajor_supported(M, K, N, block_size) and (not grouped or block_size % 128 == 0)
+            and _lib.load().k3q_w4s_shadow_bytes(int(K), int(N)) > 0)
+
+
+def int4_matmul_tiles_strip(x, shadow, units, kernel_scale, kernel_zero=None, block_size=None, bias=None):
+    """`x[..., K] . W4` for 17 ... 512 bfloat16 rows on the int4 tile kernel, reading the SAME
+    strip-linear copy (`int4_strip_copy`) that the decode kernel streams: a layer then keeps one derived
+    copy of its kernel for every row count up to 512.  kernel_scale `[N]` or `[G, N]` and
+    kernel_zero `[G, N]` as stored (bfloat16 scales).  Reference: keras/src/layers/core/dense.py:988-1095."""
+    _lib.require_device(x, shadow, kernel_scale, kernel_zero, bias)
+    if x.dtype != torch.bfloat16 or kernel_scale.dtype != torch.bfloat16:
+        raise TypeError("the int4 tile route computes in bfloat16")
+    grouped = block_size is not None and block_size > 0
+    N, K = int(units), x.shape[-1]
+    lib = _lib.load()
+    if shadow.numel() != lib.k3q_w4s_shadow_bytes(K, N):
+        raise ValueError("the strip-linear copy does not belong to a [%d, %d] kernel" % (K, N))
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, K)
+    x2 = x2 if x2.is_contiguous() else x2.contiguous()
+    M = x2.shape[0]
+    if bias is not None and bias.numel() != N:
+        raise ValueError(f"bias holds {bias.numel()} values, the layer has {N} units")
+    bs = int(block_size) if grouped else -1
+    nbytes = lib.k3q_gemm_w4_kmajor_workspace_bytes(M, K, N, bs)
+    if nbytes <= 0 or not int4_tiles_strip_supported(M, K, N, block_size):
+        raise ValueError(f"the int4 tile route does not take M={M}, K={K}, N={N}, block_size={block_size}")
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    ws = _workspace(x.device, nbytes)
+    ks = kernel_scale if kernel_scale.is_contiguous() else kernel_scale.contiguous()
+    rc = lib.k3q_gemm_w4_strip(_lib.ptr(x2), _lib.dtype_code(x.dtype), M, K, N, _lib.ptr(shadow),
+                               _lib.ptr(ks), _lib.ptr(kernel_zero) if grouped else None, bs,
+                               _lib.ptr(bias), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
+                               _lib.stream_ptr(x.device))
+    _lib.check(rc, "k3q_gemm_w4_strip")
+    return y.reshape(*lead, N)
+
+
 GEMM_EXACT_EPILOGUE = 1
 # up to this many rows the int8 matmul streams the [K, N] kernel in place; above, the prepacked
 # copy on 128-row MFMA tiles (K split over workgroups while the tiles are few) is faster
