@@ -115,13 +115,15 @@ def main():
     wq, wscale = kq.abs_max_quantize(kernel_f, axis=0, to_numpy=True)  # one-time, host side
     wq = wq.to(dev)
     wscale_t = wscale.reshape(-1).to(torch.bfloat16).to(dev)
-    prepacked = kops.prepack_int8_kernel(wq)  # one-time [N,K] shadow copy of the int8 kernel
+    # what an int8 layer keeps beside its stored kernel: the strip-linear copy, read by the decode
+    # kernel and, as its B operand, by the tile GEMM (one-time, per layer)
+    strip8 = kops.int8_strip_copy(wq)
     del kernel_f
 
     def step():
         q, s = kq.abs_max_quantize(x, axis=-1)
         return kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
-                                prepacked=prepacked, exact_epilogue=True)
+                                strip=strip8, exact_epilogue=True)
 
     # W untimed warm-up steps, then exactly K timed steps.  The K steps are recorded once
     # into a HIP graph and replayed, so that the clock sees the kernels and not the Python
@@ -154,13 +156,13 @@ def main():
     def gemm_burst():
         for _ in range(20):
             kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
-                             prepacked=prepacked, exact_epilogue=True)
+                             strip=strip8, exact_epilogue=True)
 
     spin_up(torch, gemm_burst)
     for i in range(args.steps):
         ev[2 * i].record()
         kops.int8_matmul(q, wq, a_scale=s, kernel_scale=wscale_t, out_dtype=torch.bfloat16,
-                         prepacked=prepacked, exact_epilogue=True)
+                         strip=strip8, exact_epilogue=True)
         ev[2 * i + 1].record()
     torch.cuda.synchronize()
     gemm_ms = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
@@ -245,16 +247,16 @@ def main():
     sweep = []
     for (Ks, Ns) in ((4096, 4096), (8192, 8192), (8192, 28672)) if want("sweep") else ():
         if (Ks, Ns) == (K, N):
-            ws_, wp_, sc_ = wq, prepacked, wscale_t
+            ws_, wp_, sc_ = wq, strip8, wscale_t
         else:
             ws_ = torch.randint(-127, 128, (Ks, Ns), device=dev, dtype=torch.int8)
-            wp_ = kops.prepack_int8_kernel(ws_)
+            wp_ = kops.int8_strip_copy(ws_)
             sc_ = (torch.rand(Ns, device=dev) * 100 + 100).to(torch.bfloat16)
         for Ms in (512, 2048, 4096, 8192):
             xs = torch.randn(Ms, Ks, device=dev).to(torch.bfloat16)
             qs, ss = kq.abs_max_quantize(xs, axis=-1)
             us_ = kernel_us(lambda: kops.int8_matmul(qs, ws_, a_scale=ss, kernel_scale=sc_,
-                                                     out_dtype=torch.bfloat16, prepacked=wp_,
+                                                     out_dtype=torch.bfloat16, strip=wp_,
                                                      exact_epilogue=True), 10 if Ms * Ns > 1 << 27 else 30)
             tops_ = 2.0 * Ms * Ns * Ks / us_ / 1e6
             sweep.append({"M": Ms, "K": Ks, "N": Ns, "us_per_launch": round(us_, 1),
@@ -630,7 +632,7 @@ def main():
         "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": f"Dense int8 forward M={M} K={K} N={N}, bf16 activations ~N(0,1), "
-                               "glorot-uniform kernel quantized per channel, kernel prepacked once"},
+                               "glorot-uniform kernel quantized per channel, tile GEMM fed from the layer's strip-linear copy of the kernel"},
         "roofline": {"bound": "mfma", "achieved": round(gemm_tops, 1), "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 4),
                      "traffic": measured_traffic("gemm_mfma_i8_M4096_K8192_N8192"), "kernel": "gemm_mfma<int8>",

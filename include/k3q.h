@@ -110,7 +110,10 @@ int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len, int64_t i
  *     y[m,n]   = T(T(acc[m,n]) / T(b_scale[n] * a_scale[m]))  (+ bias[n])
  * a: [M,K] int8 (the quantised activations).  b: the layer's int8 kernel, either
  * as the variable stores it, [K,N] (b_layout 0), or as the [N,K] shadow copy made
- * by k3q_prepack_kernel_i8 (b_layout 1).  a_scale [M], b_scale [N], bias [N] are
+ * by k3q_prepack_kernel_i8 (b_layout 1), or as the strip-linear copy that the int8 decode
+ * kernel streams (k3q_w8s_pack; b_layout 2: MFMA tile kernel only, K % 128 == 0, the same
+ * accumulators and bits -- a layer then keeps ONE derived copy of its kernel for every row
+ * count; K3Q_ERR_SHAPE where the tile kernel does not apply).  a_scale [M], b_scale [N], bias [N] are
  * of out_dtype; a null scale counts as 1, a null bias as absent.  y: out_dtype
  * [M,N] or null.  acc_out: int32 [M,N] or null (the raw accumulators, for
  * bit-exact checks).  At least one of y / acc_out must be given.

@@ -71,6 +71,11 @@ struct GemmParams {
     int64_t row_bytes;      // bytes per row of a and bt: K (int8) or 2K (bfloat16 operands)
     int tiles_m, tiles_n;
     int flags;
+    // bt is not [N, K] rows but the strip-linear copy of the int8 decode kernel (k3q_w8s_pack):
+    // [strip = n / 16][unit = k / 64][lane' = n % 16 + 16 g][16 bytes k = 64 unit + 16 g ...].  Only the
+    // SOURCE addresses of the B tile's DMA change: a row's 16-byte chunk c of stage kt lies at
+    // ((strip * units + 2 kt + c / 4) * 64 + n % 16 + 16 (c % 4)) * 16, i.e. a stage is 2 KiB further on.
+    int b_strip, b_units;
     // split of K over workgroups (problems with few tiles and a long K): split sp takes the
     // stages [sp * kt_split, min((sp + 1) * kt_split, stages)) and stores its raw
     // accumulators to part[sp][M][N] (int32 or float32); gemm_split_reduce sums them in
@@ -176,7 +181,13 @@ __device__ __forceinline__ float descale_f(float acc, float sb, float bv, bool h
     return r;
 }
 
-template <class T, int kKind, bool kBF16, bool kExact>
+// kBStrip: the B operand is the strip-linear copy of the int8 decode kernel (GemmParams::b_strip).
+// Read row by row, that copy would make every group of 16 lanes of a DMA instruction touch eight
+// cache lines instead of two, so the B tile then lies in LDS as [8-row block][chunk][row] instead
+// of [row][chunk]: the eight rows of a block fetch one chunk from 128 contiguous bytes of the copy.
+// The chunk position is flipped in every second block (neighbouring blocks then sit in different
+// halves of the banks for one fragment read), and a K step is still one XOR on the fragment address.
+template <class T, int kKind, bool kBF16, bool kExact, bool kBStrip = false>
 __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
     constexpr int kBM = T::kBM, kBN = T::kBN, kWavesN = T::kWavesN, kThreads = T::kThreads;
     constexpr int kWN = T::kWN, kWM = T::kWM, kNBlk = T::kNBlk, kMBlk = T::kMBlk;
@@ -221,20 +232,29 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         for (int d = 0; d < kDmaPerWave; ++d) {
             const int inst = wave * kDmaPerWave + d;
             const bool is_b = inst >= kDmaA;
-            const int row = (is_b ? inst - kDmaA : inst) * 8 + lane / kRowChunks;
-            const int chunk = (lane & (kRowChunks - 1)) ^ swz(row);
+            const bool strip_b = kBStrip && is_b;
+            const int blk = is_b ? inst - kDmaA : inst;  // the 8-row block this instruction fills
+            const int row = blk * 8 + (strip_b ? lane & 7 : lane / kRowChunks);
+            const int chunk = strip_b ? (lane >> 3) ^ (blk & 1) : (lane & (kRowChunks - 1)) ^ swz(row);
             int64_t grow = (is_b ? n0 : m0) + row;
             const int64_t lim = (is_b ? p.N : p.M) - 1;
             grow = grow < lim ? grow : lim;
-            src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16 +
-                     (int64_t)sp * p.kt_split * kBK;
+            if (strip_b)
+                src[d] = (const char*)p.bt + ((grow >> 4) * p.b_units + (chunk >> 2)) * 1024 +
+                         ((grow & 15) + 16 * (chunk & 3)) * 16 + (int64_t)sp * p.kt_split * 2048;
+            else
+                src[d] = (const char*)(is_b ? p.bt : p.a) + grow * p.row_bytes + chunk * 16 +
+                         (int64_t)sp * p.kt_split * kBK;
         }
+        // (all DMA instructions of a wave belong to the same operand: kDmaA is a multiple of kDmaPerWave)
+        static_assert(kDmaA % kDmaPerWave == 0, "a wave's DMA instructions fill one operand");
+        const int kstep = (kBStrip && wave * kDmaPerWave >= kDmaA) ? 2048 : kBK;
         auto issue_stage = [&](int kt) {
             char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
 #pragma unroll
             for (int d = 0; d < kDmaPerWave; ++d) {
                 __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
+                    (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kstep),
                     (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
             }
         };
@@ -253,9 +273,11 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         const int lane_chunk = (fg ^ swz(fi)) << 4;
         int ra = (wm * kWM + fi) * kBK + lane_chunk;
         int rb = kATileBytes + (wn * kWN + fi) * kBK + lane_chunk;
+        if (kBStrip)  // [block][chunk position][row]: chunk 2 ks + g of row i at position (2 ks + g) ^ (block & 1)
+            rb = kATileBytes + ((wn * kWN + fi) >> 3) * 1024 + ((fg ^ ((fi >> 3) & 1)) << 7) + (fi & 7) * 16;
         v4i af[2][kMBlk], bf[2][kNBlk];
         auto read_frags = [&](int fb, int ks) {
-            const char* pb = lds + (rb ^ (32 * ks));
+            const char* pb = lds + (rb ^ ((kBStrip ? 256 : 32) * ks));
 #pragma unroll
             for (int nb = 0; nb < kNBlk; ++nb) bf[fb][nb] = *(const v4i*)(pb + nb * 32 * kBK);
             const char* pa = lds + (ra ^ (32 * ks));
@@ -300,7 +322,7 @@ __global__ __launch_bounds__(T::kThreads) void gemm_mfma(GemmParams p) {
         auto issue_one = [&](int kt, int d) {
             char* dst = lds + (kt % kStages) * kStageBytes + wave * kDmaPerWave * 1024;
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kBK),
+                (const __attribute__((address_space(1))) void*)(src[d] + (int64_t)kt * kstep),
                 (__attribute__((address_space(3))) void*)(dst + d * 1024), 16, 0, 0);
         };
         auto mma_half = [&](int ks, int half, int kt) {
@@ -819,11 +841,11 @@ inline int64_t split_workspace_bytes(int64_t M, int64_t N, int64_t row_bytes) {
     return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
 }
 
-template <class T, int kKind, bool kBF16, bool kExact>
+template <class T, int kKind, bool kBF16, bool kExact, bool kBStrip = false>
 int launch_tile(GemmParams p, hipStream_t s) {
     // more than 64 KiB of dynamic LDS needs the attribute raised once per kernel
     static const bool raised =
-        hipFuncSetAttribute((const void*)gemm_mfma<T, kKind, kBF16, kExact>,
+        hipFuncSetAttribute((const void*)gemm_mfma<T, kKind, kBF16, kExact, kBStrip>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, T::kLdsBytes) == hipSuccess;
     if (!raised) return K3Q_ERR_LAUNCH;
     p.tiles_m = (int)((p.M + T::kBM - 1) / T::kBM);
@@ -844,7 +866,7 @@ int launch_tile(GemmParams p, hipStream_t s) {
     const int64_t total = tiles * p.splits;
     int64_t grid = ((total + 7) / 8) * 8;
     if (resident >= 8 && grid > resident) grid = resident;
-    gemm_mfma<T, kKind, kBF16, kExact><<<(unsigned)grid, T::kThreads, T::kLdsBytes, s>>>(p);
+    gemm_mfma<T, kKind, kBF16, kExact, kBStrip><<<(unsigned)grid, T::kThreads, T::kLdsBytes, s>>>(p);
     if (p.splits > 1) {
         const int64_t threads = p.M * (p.N / 4);
         gemm_split_reduce<kKind, kBF16, kExact><<<(unsigned)((threads + 255) / 256), 256, 0, s>>>(p);
@@ -860,6 +882,12 @@ template <int kKind, bool kBF16, bool kExact>
 int launch_mfma(const GemmParams& p, hipStream_t s) {
     const int64_t large_tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
     const bool large = large_tiles >= kLargeTileMinTiles;
+    if constexpr (kKind == kKindI8) {
+        if (p.b_strip) {
+            if (large) return launch_tile<TileLarge, kKind, kBF16, kExact, true>(p, s);
+            return launch_tile<TileSmall, kKind, kBF16, kExact, true>(p, s);
+        }
+    }
     if (large) return launch_tile<TileLarge, kKind, kBF16, kExact>(p, s);
     return launch_tile<TileSmall, kKind, kBF16, kExact>(p, s);
 }
@@ -947,7 +975,7 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
                            int64_t workspace_bytes, void* stream) {
     if (out_dtype != K3Q_F32 && out_dtype != K3Q_BF16) return K3Q_ERR_DTYPE;
     if (M < 0 || N <= 0 || K <= 0) return K3Q_ERR_SHAPE;
-    if (b_layout != 0 && b_layout != 1) return K3Q_ERR_SHAPE;
+    if (b_layout != 0 && b_layout != 1 && b_layout != 2) return K3Q_ERR_SHAPE;
     if (M == 0) return K3Q_OK;
     if (!a || !b || (!y && !acc_out)) return K3Q_ERR_NULL;
     hipStream_t s = (hipStream_t)stream;
@@ -989,7 +1017,13 @@ extern "C" int k3q_gemm_i8(const int8_t* a, const int8_t* b, int b_layout, int64
                                      workspace, workspace_bytes, s);
     char* scratch = (workspace && aligned_to(workspace, 16)) ? (char*)workspace : nullptr;
     int64_t scratch_bytes = scratch ? workspace_bytes : 0;
-    if (fast && padded) {
+    if (b_layout == 2) {
+        // the strip-linear copy of the decode kernel as the tiles' B operand: the tile kernel or nothing
+        if (!fast || padded) return K3Q_ERR_SHAPE;
+        p.bt = b;
+        p.b_strip = 1;
+        p.b_units = (int)(K / 64);
+    } else if (fast && padded) {
         int8_t* a_pad = (int8_t*)scratch;
         int8_t* b_pad = a_pad + M * Kpad;
         pad_rows_i8<<<(unsigned)((M * (Kpad / 16) + 255) / 256), 256, 0, s>>>(a, a_pad, M, K, Kpad);

@@ -359,6 +359,14 @@ class Dense(Layer):
             spec["kernel_scale"] = self._read_cached("kernel_scale", self.kernel_scale)
         return spec
 
+    def _tile_operand(self, input_dim):
+        """The derived copy of the int8 kernel that the tile GEMM reads, as a keyword of
+        `ops.int8_matmul`: the decode kernel's strip-linear copy where the tile kernel can take it
+        (one derived copy per layer; same bits and speed as from a [N, K] copy), else the [N, K] copy."""
+        if input_dim % 128 == 0:
+            return dict(strip=self._cached("w8s", self._kernel, kops.int8_strip_copy))
+        return dict(prepacked=self._cached("prepacked", self._kernel, kops.prepack_int8_kernel))
+
     # ---- quantized forward --------------------------------------------------------
     def _int8_call(self, inputs, training=None):
         """keras/src/layers/core/dense.py:938-986: quantise rows, int8 GEMM, de-scale, bias."""
@@ -398,8 +406,7 @@ class Dense(Layer):
             kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
             bias=self._call_bias(),
             out_dtype=to_torch_dtype(self.compute_dtype),
-            prepacked=self._cached("prepacked", self._kernel, kops.prepack_int8_kernel),
-            exact_epilogue=exact,
+            exact_epilogue=exact, **self._tile_operand(x2.shape[1]),
         )
         y = y.reshape(*lead, N)
         if self.activation is not None:
@@ -424,12 +431,25 @@ class Dense(Layer):
             lead = inputs.shape[:-1]
             x2 = inputs.reshape(-1, inputs.shape[-1])
             q, scale = quantize_rows(self.inputs_quantizer, x2)
-            unpacked = quantizers.unpack_int4(as_tensor(self._kernel), self._orig_output_dim, axis=-1)
+            units = self._orig_output_dim
+            operand = {}
+            if x2.shape[1] % 128 == 0 and x2.shape[0] > kops.SKINNY_MAX_ROWS:
+                # the tile GEMM reads a strip-linear int8 copy of the unpacked kernel, made once and kept
+                # while the kernel does not change (one byte per weight beside the stored half byte: this
+                # configuration, which the reference does not default to, holds 3x the stored bytes)
+                # instead of unpacking the whole kernel into scratch on every call
+                unpacked = None
+                operand = dict(strip=self._cached(
+                    "w8s_unpacked", self._kernel,
+                    lambda t: kops.int8_strip_copy(quantizers.unpack_int4(t, units, axis=-1))))
+            else:
+                unpacked = quantizers.unpack_int4(as_tensor(self._kernel), units, axis=-1)
             y = kops.int8_matmul(
                 q, unpacked, a_scale=scale,
                 kernel_scale=self._read_cached("kernel_scale", self.kernel_scale),
                 bias=self._call_bias(),
-                out_dtype=to_torch_dtype(self.compute_dtype), exact_epilogue=True,
+                out_dtype=to_torch_dtype(self.compute_dtype), exact_epilogue=True, kernel_shape=(x2.shape[1], units),
+                **operand,
             )
             y = y.reshape(*lead, self._orig_output_dim)
             if self.activation is not None:

@@ -614,7 +614,6 @@ class EinsumDense(Layer):
 
         k2 = self._cached("kernel2d", self._kernel, kernel_matrix)
         n = k2.shape[1]
-        pre = self._cached("prepacked", self._kernel, lambda t: kops.prepack_int8_kernel(kernel_matrix(t)))
         bias, fused = self._fusable_bias(gv, n)
         if not self.inputs_quantizer:
             # Weight-only (einsum_dense.py:1085-1101).  The torch backend divides every weight
@@ -625,7 +624,8 @@ class EinsumDense(Layer):
                 x2, k2,
                 self._cached("kernel_scale", self.kernel_scale,
                              lambda t: t.to(cd).reshape(-1).contiguous()),
-                bias=bias, prepacked=pre)
+                bias=bias,
+                prepacked=self._cached("prepacked", self._kernel, lambda t: kops.prepack_int8_kernel(kernel_matrix(t))))
             return self._finish(y2, free_shape, gv, fused)
         exact = self.exact_epilogue
         if exact is None:
@@ -644,7 +644,13 @@ class EinsumDense(Layer):
             q, k2, a_scale=scale,
             kernel_scale=self._cached("kernel_scale", self.kernel_scale,
                                       lambda t: t.to(cd).reshape(-1).contiguous()),
-            bias=bias, out_dtype=cd, prepacked=pre, exact_epilogue=exact,
+            bias=bias, out_dtype=cd, exact_epilogue=exact,
+            # the tile GEMM's operand: the decode kernel's strip-linear copy where it can take it
+            # (one derived copy per layer), else the [N, K] copy
+            **(dict(strip=self._cached("w8s", self._kernel, lambda t: kops.int8_strip_copy(kernel_matrix(t))))
+               if x2.shape[1] % 128 == 0 else
+               dict(prepacked=self._cached("prepacked", self._kernel,
+                                           lambda t: kops.prepack_int8_kernel(kernel_matrix(t))))),
         )
         return self._finish(y2, free_shape, gv, fused)
 

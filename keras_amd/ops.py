@@ -562,21 +562,32 @@ def prepack_int8_kernel(kernel):
 
 
 def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype=None,
-                prepacked=None, exact_epilogue=False, want_acc=False, want_y=True):
+                prepacked=None, exact_epilogue=False, want_acc=False, want_y=True, strip=None,
+                kernel_shape=None):
     """`a[M, K] int8 . kernel[K, N] int8` with the de-scale epilogue fused.
 
     Returns y (out_dtype [M, N]); with want_acc also the int32 accumulators.
     `prepacked` is the cached result of `prepack_int8_kernel(kernel)`; without it
-    the [N, K] copy is rebuilt in scratch memory on every call.
+    the [N, K] copy is rebuilt in scratch memory on every call.  `strip` is the cached
+    `int8_strip_copy(kernel)` of the decode kernel: with K % 128 == 0 the tile kernel reads
+    that copy instead (the same bits), so a layer need not keep a prepacked one beside it.
+    `kernel` may be None when `strip` serves the call (more than 8 rows, K % 128 == 0) and
+    `kernel_shape = (K, N)` is given.
     Reference: keras/src/layers/core/dense.py:961-983.
     """
-    _lib.require_device(a, kernel, a_scale, kernel_scale, bias, prepacked)
-    if a.dtype != torch.int8 or kernel.dtype != torch.int8:
+    _lib.require_device(a, kernel, a_scale, kernel_scale, bias, prepacked, strip)
+    if a.dtype != torch.int8 or (kernel is not None and kernel.dtype != torch.int8):
         raise TypeError("int8_matmul takes int8 operands")
     M, K = a.shape
-    if kernel.shape[0] != K:
-        raise ValueError(f"inner dimensions differ: {a.shape} x {kernel.shape}")
-    N = kernel.shape[1]
+    if kernel is None:
+        if strip is None or kernel_shape is None or kernel_shape[0] != K or K % 128 or M <= SKINNY_MAX_ROWS:
+            raise ValueError("without the stored kernel the call needs its strip-linear copy, kernel_shape, "
+                             "K % 128 == 0 and more than %d rows" % SKINNY_MAX_ROWS)
+        N = int(kernel_shape[1])
+    else:
+        if kernel.shape[0] != K:
+            raise ValueError(f"inner dimensions differ: {a.shape} x {kernel.shape}")
+        N = kernel.shape[1]
     if out_dtype is None:
         out_dtype = a_scale.dtype if a_scale is not None else torch.float32
     code = _lib.dtype_code(out_dtype)
@@ -592,7 +603,12 @@ def int8_matmul(a, kernel, a_scale=None, kernel_scale=None, bias=None, out_dtype
     lib = _lib.load()
     skinny = M <= SKINNY_MAX_ROWS and N % 16 == 0 and K % 8 == 0
     nbytes = lib.k3q_gemm_i8_workspace_bytes(M, N, K)
-    if prepacked is not None and not skinny:
+    if strip is not None and not skinny and K % 128 == 0:
+        if strip.numel() != lib.k3q_w8s_shadow_bytes(K, N):
+            raise ValueError("the strip-linear copy does not belong to a [%d, %d] kernel" % (K, N))
+        b, layout = strip, 2
+        nbytes = max(0, nbytes - (N * K + 15) // 16 * 16)  # (room for the partials of a K split only)
+    elif prepacked is not None and not skinny:
         # no per-call [N,K] copy: only the part of the scratch beyond it (partial sums of a
         # K split, taken for few-tile problems) is of use; a K that is not a multiple of 128
         # keeps all of it (both operands are zero-padded into it)

@@ -28,11 +28,14 @@ def run_dense_int8(dev, M, K, N, dtype, prepack, exact, seed=0, with_bias=True, 
     q, s = kq.abs_max_quantize(x.to(dev), axis=-1)
     assert torch.equal(q.cpu(), inter["q"])
     qk_d = qk.to(dev)
-    pre = kops.prepack_int8_kernel(qk_d) if prepack else None
+    # prepack: True = the [N, K] copy, "strip" = the decode kernel's strip-linear copy as the tiles'
+    # operand (K % 128 == 0; other shapes fall back to the stored kernel), False = the stored kernel
+    pre = kops.prepack_int8_kernel(qk_d) if prepack is True else None
+    strip = kops.int8_strip_copy(qk_d) if prepack == "strip" and K % 64 == 0 else None
     y, acc = kops.int8_matmul(
         q, qk_d, a_scale=s, kernel_scale=ks.to(dtype).to(dev),
         bias=bias.to(dtype).to(dev) if bias is not None else None, out_dtype=dtype,
-        prepacked=pre, exact_epilogue=exact, want_acc=True)
+        prepacked=pre, strip=strip, exact_epilogue=exact, want_acc=True)
     torch.cuda.synchronize()
     assert torch.equal(acc.cpu(), inter["acc"]), "int32 accumulators differ from the reference"
     if exact:
@@ -61,7 +64,7 @@ SHAPES = [
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("prepack", [True, False])
+@pytest.mark.parametrize("prepack", [True, False, "strip"])
 def test_dense_int8_exact_epilogue(dev, M, K, N, dtype, prepack):
     run_dense_int8(dev, M, K, N, dtype, prepack, exact=True)
 
@@ -94,6 +97,7 @@ def test_dense_int8_wide_range_scales(dev, M, K, N, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_dense_int8_split_k(dev, M, K, N, dtype):
     run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=True)
+    run_dense_int8(dev, M, K, N, dtype, prepack="strip", exact=True, seed=4)
     run_dense_int8(dev, M, K, N, dtype, prepack=False, exact=True, seed=5, with_bias=False)
     run_dense_int8(dev, M, K, N, dtype, prepack=True, exact=False, seed=6)
 
