@@ -420,12 +420,9 @@ class Dense(Layer):
             return self._quantized_call_with_lora(self._int4_call, inputs)
         block_size = getattr(self, "_int4_block_size", None)
         grouped = block_size is not None and block_size > 0
-        if self.inputs_quantizer:
-            if grouped:
-                raise NotImplementedError(
-                    "Grouped int4 with an activation quantizer has no counterpart in the "
-                    "reference (dense.py:1040-1084 ignores the quantizer there)."
-                )
+        # (a grouped kernel ignores an activation quantizer, as the reference's sub-channel branch
+        # does: dense.py:1040-1084 never reads it)
+        if self.inputs_quantizer and not grouped:
             # activation-quantized, per-channel (dense.py:1023-1031): int8 rows against the
             # nibbles unpacked to int8 in scratch, exact int32 accumulation, one de-scale
             lead = inputs.shape[:-1]

@@ -205,9 +205,11 @@ class _BatchedView:
     def __init__(self, i_spec, k_spec, o_spec):
         si, sk, so = set(i_spec), set(k_spec), set(o_spec)
         if sk - si - so:
+            # (unreachable through build(): a kernel label that neither the input nor the output
+            # carries has no size, and `analyze_einsum_shapes` raises ValueError for it, as the
+            # reference does, keras/src/layers/core/einsum_dense.py:1854-1866)
             raise NotImplementedError(
-                f"labels {sorted(sk - si - so)} are summed out of the kernel alone: not lowered to "
-                "the quantized GEMM")
+                f"labels {sorted(sk - si - so)} are summed out of the kernel alone: the layer cannot be built")
         self.i_spec, self.k_spec, self.o_spec = i_spec, k_spec, o_spec
         self.batch = [c for c in i_spec if c in sk and c in so]
         self.free = [c for c in i_spec if c in so and c not in sk]
@@ -726,8 +728,6 @@ class EinsumDense(Layer):
         cd = to_torch_dtype(self.compute_dtype)
         block_size = self._int4_block_size
         grouped = block_size is not None and block_size > 0
-        if self.inputs_quantizer:
-            raise NotImplementedError("activation-quantized int4 is built for GEMM-shaped equations only")
         variables = [self._kernel, self.kernel_scale] + ([self.kernel_zero, self.g_idx] if grouped else [])
         stamp = tuple((id(v), v.version) for v in variables) + (cd,)
         hit = self._cache.get("int4_float_kernel")
@@ -740,7 +740,23 @@ class EinsumDense(Layer):
             else:
                 fk = torch.divide(unpacked.to(cd), scale)
             hit = self._cache["int4_float_kernel"] = (stamp, fk.reshape(self.original_kernel_shape))
-        y = torch.einsum(self.equation, inputs.to(cd), hit[1])
+        if self.inputs_quantizer and not grouped:
+            # einsum_dense.py:1163-1184 (a grouped kernel never reads the quantizer, :1188-1261): rows
+            # quantised over the labels the output lacks, cast back to the compute dtype, contracted
+            # against the float kernel, divided by the input scale in the shape the reference's
+            # transpose / expand / squeeze bookkeeping gives it
+            bv = self._batched
+            size = dict(zip(bv.i_spec, inputs.shape))
+            prod = lambda labels: math.prod(size[c] for c in labels)
+            q_labels = bv.rows + bv.reduced
+            x2 = inputs.to(cd).permute([bv.i_spec.index(c) for c in q_labels]).reshape(prod(bv.rows), prod(bv.reduced))
+            q2, scale = quantize_rows(self.inputs_quantizer, x2.contiguous())
+            s_in = scale.reshape([1 if c in bv.reduced else size[c] for c in bv.i_spec])
+            q = q2.reshape([size[c] for c in q_labels]).permute([q_labels.index(c) for c in bv.i_spec])
+            y = torch.einsum(self.equation, q.to(cd), hit[1])
+            y = torch.divide(y, _adjust_scale(s_in, self._quant_info["input"]))
+        else:
+            y = torch.einsum(self.equation, inputs.to(cd), hit[1])
         if self.bias is not None:
             y = torch.add(y, self.read(self.bias))
         if self.activation is not None:
@@ -763,12 +779,9 @@ class EinsumDense(Layer):
         bias, fused = self._fusable_bias(gv, self._int4_unpacked_column_size)
         if grouped:
             require_default_g_idx(self, block_size)  # (the de-quantised route above reads g_idx)
-        if self.inputs_quantizer:
-            if grouped:
-                raise NotImplementedError(
-                    "Grouped int4 with an activation quantizer has no counterpart in the "
-                    "reference (einsum_dense.py:1188-1261 ignores the quantizer there)."
-                )
+        # (a grouped kernel ignores an activation quantizer, as the reference's sub-channel branch
+        # does: einsum_dense.py:1188-1261 never reads it)
+        if self.inputs_quantizer and not grouped:
             # Activation-quantized, per-channel (einsum_dense.py:1163-1187).  The torch
             # backend contracts the quantised rows, cast back to float, with the kernel
             # divided by its scale weight by weight; here the contraction is the exact int32
@@ -922,12 +935,7 @@ class EinsumDense(Layer):
         if x2.dtype not in (torch.bfloat16, torch.float32):
             raise TypeError(f"int4 EinsumDense computes in bfloat16 or float32, got {x2.dtype}")
         wt, parts = self._int4_dequantized_kernel(gv, cd, grouped)
-        if self.inputs_quantizer:
-            if grouped:
-                raise NotImplementedError(
-                    "Grouped int4 with an activation quantizer has no counterpart in the "
-                    "reference (einsum_dense.py:1188-1261 ignores the quantizer there)."
-                )
+        if self.inputs_quantizer and not grouped:
             # einsum_dense.py:1163-1184: quantised rows, cast back to float, against the float
             # kernel; then the division by the input scale, then the bias
             q, scale = quantize_rows(self.inputs_quantizer, x2)

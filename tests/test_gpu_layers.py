@@ -733,3 +733,67 @@ def test_call_add_is_the_separate_add(dev, mode, dtype):
     plain = down(h)
     ka.layers.call_add(down, h, torch.ones((1, 1, 256), dtype=cd, device=dev))
     assert torch.equal(down(h), plain)
+
+
+@pytest.mark.parametrize("equation,output_shape,input_shape,bias_axes", GENERAL[:5])
+@pytest.mark.parametrize("policy", ["float32", "mixed_bfloat16"])
+def test_einsum_dense_int4_activation_quantized_general_equations(dev, equation, output_shape, input_shape,
+                                                                  bias_axes, policy):
+    # equations outside the [M, K] x [K, N] view (labels shared by all three operands, no summed
+    # label, a label only the input carries) with a per-channel int4 kernel AND an activation
+    # quantizer: the reference's torch branch (einsum_dense.py:1163-1184) -- rows quantised over the
+    # labels the output lacks, cast back, float einsum against the de-quantised kernel, division by
+    # the adjusted input scale
+    g = torch.Generator().manual_seed(97)
+    layer = EinsumDense(equation, output_shape, bias_axes=bias_axes, dtype=policy, device=dev,
+                        kernel_initializer=lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d),
+                        bias_initializer=lambda s, d: torch.randn(s, generator=g).to(d))
+    layer.build(input_shape)
+    cd = TORCH[layer.compute_dtype]
+    kernel_f = layer._kernel.value.cpu()
+    bias_f = layer.bias.value.cpu() if layer.bias is not None else None
+    x = torch.rand(input_shape, generator=g) - 0.3
+    config = ka.Int4QuantizationConfig(block_size=None, activation_quantizer=ka.quantizers.AbsMaxQuantizer())
+    layer.quantize("int4", config=config)
+    assert layer.inputs_quantizer is not None
+    qk = ref.einsum_dense_quantize_int4(kernel_f, equation, len(input_shape), None)
+    assert torch.equal(layer._kernel.value.cpu(), qk["kernel"])
+    y = layer(x)
+    want = ref.einsum_dense_int4_activation_quantized_call(x.to(cd), qk, equation, bias=bias_f, compute_dtype=cd)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    assert max_rel_err(y, want) <= RTOL[cd]
+
+
+@pytest.mark.parametrize("kind", ["dense", "einsum", "einsum_non_leading"])
+def test_grouped_int4_ignores_an_activation_quantizer(dev, kind):
+    # the reference's sub-channel branches never read `inputs_quantizer` (dense.py:1040-1084,
+    # einsum_dense.py:1188-1261): a grouped int4 layer configured with one is the weight-only layer
+    g = torch.Generator().manual_seed(96)
+    init = lambda s, d: (torch.rand(s, generator=g) - 0.5).to(d)
+    if kind == "dense":
+        layer = Dense(96, dtype="mixed_bfloat16", device=dev, kernel_initializer=init, use_bias=False)
+        shape, eq = (5, 256), None
+    elif kind == "einsum":
+        layer = EinsumDense("btd,dnh->btnh", (None, 4, 24), dtype="mixed_bfloat16", device=dev, kernel_initializer=init)
+        shape, eq = (2, 3, 256), "btd,dnh->btnh"
+    else:
+        layer = EinsumDense("btd,ndh->btnh", (None, 4, 24), dtype="mixed_bfloat16", device=dev, kernel_initializer=init)
+        shape, eq = (2, 3, 256), "btd,ndh->btnh"
+    layer.build(shape)
+    kernel_f = layer._kernel.value.cpu()
+    x = torch.rand(shape, generator=g) - 0.5
+    # (Int4QuantizationConfig refuses the combination, as the reference's does, so the quantizer is
+    # attached by hand -- what a subclass or a hand-edited layer could carry)
+    layer.quantize("int4", config=ka.Int4QuantizationConfig(block_size=128))
+    layer.inputs_quantizer = ka.quantizers.AbsMaxQuantizer()
+    y = layer(x)
+    cd = torch.bfloat16
+    if eq is None:
+        q4 = ref.dense_quantize_int4(kernel_f, 128)
+        want = ref.dense_int4_call(x.to(cd), q4["kernel"], q4["kernel_scale"], 96, kernel_zero=q4["kernel_zero"],
+                                   g_idx=q4["g_idx"], block_size=128, compute_dtype=cd)
+    else:
+        qk = ref.einsum_dense_quantize_int4(kernel_f, eq, 3, 128)
+        want = ref.einsum_dense_int4_call(x.to(cd), qk, eq, compute_dtype=cd, block_size=128)
+    assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
+    assert max_rel_err(y, want) <= RTOL[cd]
