@@ -521,6 +521,12 @@ class EinsumDense(Layer):
         if hit is not None and hit[0] == var.version and hit[1] is var:
             return hit[2]
         value = make(as_tensor(var))
+        if (hit is not None and isinstance(hit[2], torch.Tensor) and isinstance(value, torch.Tensor)
+                and hit[2].shape == value.shape and hit[2].dtype == value.dtype and hit[2].device == value.device):
+            # a rebuilt copy keeps its address: a captured HIP graph that holds the old copy's address
+            # goes on reading live memory (the new values) instead of memory that was freed
+            hit[2].copy_(value)
+            value = hit[2]
         self._cache[key] = (var.version, var, value)
         return value
 

@@ -353,11 +353,11 @@ def test_reversible_embedding_int4_tied_decode_sizes_take_the_strip_copy(dev, M,
     x40 = torch.cat([x, torch.randn(40 - M, D, generator=torch.Generator().manual_seed(23))])
     y40 = layer(x40, reverse=True)
     assert max_rel_err(y40[:M], want) <= RTOL[torch.bfloat16]
-    # an assignment to the table makes a new copy
-    before = layer._cache["w4s"][2]
+    # an assignment to the table rebuilds the copy (in place: its address stays what captured graphs hold)
+    before, stamp = layer._cache["w4s"][2].data_ptr(), layer._cache["w4s"][0]
     layer._embeddings.assign(layer._embeddings.value.clone())
     y2 = layer(x, reverse=True)
-    assert layer._cache["w4s"][2] is not before
+    assert layer._cache["w4s"][0] != stamp and layer._cache["w4s"][2].data_ptr() == before
     assert torch.equal(bits(y2.cpu()), bits(y.cpu()))
 
 

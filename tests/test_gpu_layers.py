@@ -797,3 +797,24 @@ def test_grouped_int4_ignores_an_activation_quantizer(dev, kind):
         want = ref.einsum_dense_int4_call(x.to(cd), qk, eq, compute_dtype=cd, block_size=128)
     assert tuple(y.shape) == tuple(want.shape) and y.dtype == cd
     assert max_rel_err(y, want) <= RTOL[cd]
+
+
+@pytest.mark.parametrize("mode", ["int8", "int4"])
+def test_derived_copy_keeps_its_address_when_the_kernel_is_assigned(dev, mode):
+    # the strip-linear copy is rebuilt in place when the kernel variable is assigned: a captured
+    # graph that holds the copy's address then reads the new values, not freed memory
+    layer = build_dense(dev, 4096, 4096, "mixed_bfloat16", seed=11, use_bias=False)
+    other = build_dense(dev, 4096, 4096, "mixed_bfloat16", seed=12, use_bias=False)
+    layer.quantize(mode)
+    other.quantize(mode)
+    x = torch.randn(2, 4096, generator=torch.Generator().manual_seed(13)).to(torch.bfloat16).to(dev)
+    y0 = layer(x)
+    key = "w8s" if mode == "int8" else "w4s"
+    copy0 = layer._cache[key][2]
+    address = copy0.data_ptr()
+    for name in ("_kernel", "kernel_scale") + (("kernel_zero",) if mode == "int4" else ()):
+        getattr(layer, name).assign(getattr(other, name).value)
+    y1 = layer(x)
+    assert layer._cache[key][2].data_ptr() == address
+    assert torch.equal(bits(y1.cpu()), bits(other(x).cpu()))
+    assert not torch.equal(bits(y1.cpu()), bits(y0.cpu()))
