@@ -79,11 +79,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
-    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,pack,embed,decode,cpu: run the headline "
+    ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,pack,wq,embed,decode,cpu: run the headline "
                     "step and only these further sections (for profiler runs); default: all")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
-    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "pack", "embed", "decode", "cpu"}
+    unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "pack", "wq", "embed", "decode", "cpu"}
     if unknown:
         sys.exit(f"bench.py: unknown section(s) {sorted(unknown)}")
     want = (lambda name: not only or name in only)
@@ -511,6 +511,34 @@ def main():
         del unpacked
         torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ weight quantizers on the device
+    # What `quantize()` runs on a float32 kernel that lives on the device (the bits of the reference's
+    # numpy path): per-column abs-max (int8 and per-channel int4) and the grouped min / max quantizer
+    # (block 128), 8192 x 8192 float32; algorithmic bytes: 4 read + 1 written per weight (the kernels
+    # make two passes over x; the second finds most of it in the caches).  Rotating over two kernels
+    # of 256 MiB.
+    wq_rows = []
+    if want("wq"):
+        wf = [torch.randn(Kg, Ng, device=dev) * 0.02 for _ in range(2)]
+        for name, call in (("abs_max_quantize axis=0 (int8)", lambda i: kq.abs_max_quantize(wf[i % 2], axis=0, to_numpy=True)),
+                           ("abs_max_quantize_grouped_with_zero_point block 128 (int4)",
+                            lambda i: kq.abs_max_quantize_grouped_with_zero_point(wf[i % 2], 128, to_numpy=True))):
+            call(0)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(6):
+                call(i)
+            e1.record()
+            torch.cuda.synchronize()
+            us_ = e0.elapsed_time(e1) / 6 * 1e3
+            nb_ = 5 * Kg * Ng
+            wq_rows.append({"op": name, "shape": [Kg, Ng], "us_per_call": round(us_, 1), "algorithmic_bytes": nb_,
+                            "roofline": {"bound": "hbm", "achieved": round(nb_ / us_ / 1e3, 1), "peak": HBM_PEAK_GBS,
+                                         "unit": "GB/s", "frac": round(nb_ / us_ / 1e3 / HBM_PEAK_GBS, 4), "traffic": None}})
+        del wf
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ quantized embedding lookup
     # 32768 random ids into an int8 table of 32000 x 4096 with float32 per-row scales (what a
     # float32 or mixed_bfloat16 layer stores): 1 byte read and 4 written per element, plus the ids and
@@ -653,6 +681,7 @@ def main():
         "int8_decode_dense": gemv8,
         "read_only_launch_64MiB": read_ref8,
         "pack_unpack": pack_rows,
+        "weight_quantizers": wq_rows,
         "embedding_lookup": embed_row,
         "llama_decode_int4": decode,
         "llama_decode_int8": decode_int8,

@@ -224,3 +224,27 @@ def test_einsum_errors():
         EinsumDense("ab,bc,cd->ad", 4, device="cpu").build((2, 3))
     with pytest.raises(ValueError, match="Bias dimension"):
         EinsumDense("ab,bc->ac", 4, bias_axes="z", device="cpu").build((2, 3))
+
+
+def test_autocast_reads_are_cached_until_the_variable_changes():
+    # Layer.read under a mixed policy: the cast copy is made once, rebuilt after assign() and after
+    # an in-place write to the stored tensor
+    layer = Dense(8, dtype="mixed_bfloat16", device="cpu", use_bias=True)
+    layer.build((None, 4))
+    first = layer.read(layer.bias)
+    assert first.dtype == torch.bfloat16 and layer.read(layer.bias) is first
+    layer.bias.assign(torch.ones(8))
+    second = layer.read(layer.bias)
+    assert second is not first and second.float().sum().item() == 8
+    layer.bias.value.mul_(2)
+    third = layer.read(layer.bias)
+    assert third is not second and third.float().sum().item() == 16
+    same = Dense(8, dtype="float32", device="cpu")
+    same.build((None, 4))
+    assert same.read(same.bias) is same.bias.value  # nothing to cast: the stored tensor itself
+
+
+def test_resident_bytes_counts_variables_once():
+    layer = Dense(8, dtype="float32", device="cpu")
+    layer.build((None, 4))
+    assert layer.resident_bytes() == {"stored": 4 * 8 * 4 + 8 * 4, "derived": 0}
