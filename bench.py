@@ -527,11 +527,11 @@ def main():
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            for i in range(6):
+            for i in range(20):
                 call(i)
             e1.record()
             torch.cuda.synchronize()
-            us_ = e0.elapsed_time(e1) / 6 * 1e3
+            us_ = e0.elapsed_time(e1) / 20 * 1e3
             nb_ = 5 * Kg * Ng
             wq_rows.append({"op": name, "shape": [Kg, Ng], "us_per_call": round(us_, 1), "algorithmic_bytes": nb_,
                             "roofline": {"bound": "hbm", "achieved": round(nb_ / us_ / 1e3, 1), "peak": HBM_PEAK_GBS,

@@ -1,8 +1,8 @@
 // int4 <-> int8 nibble packing along the middle axis of [outer, len, inner].
 //
 // Both directions are pure HBM streams (1.5 bytes moved per int4 value), so
-// the fast paths do nothing but 16-byte loads, a handful of bit operations per
-// dword and 16-byte stores.  inner == 1 is the "pack along the last axis" case
+// the fast paths do nothing but 8- or 16-byte loads, a handful of bit operations
+// per dword and 16-byte stores that fill whole cache lines per instruction.  inner == 1 is the "pack along the last axis" case
 // (the two nibbles of a byte are neighbours in memory and must be interleaved
 // with byte permutes); inner > 1 is the "pack along a leading axis" case (the
 // two nibbles go to two different rows, no interleave).
@@ -29,29 +29,27 @@ __device__ __forceinline__ void split_dword(u32 w, u32& lo, u32& hi) {
 }
 
 // ---- unpack, nibbles adjacent along the packed axis (inner == 1) ----------
+// A thread turns 8 packed bytes into one 16-byte store, twice: the stores of a wave are then 1 KiB
+// of consecutive addresses each (16 packed bytes -> two neighbouring stores per thread would leave
+// every store instruction filling half of each cache line, and memory sees the partial writes).
 template <bool kSigned>
-__global__ __launch_bounds__(kThreads) void unpack_last_vec(const v4u* __restrict__ in,
-                                                            v4u* __restrict__ out, int64_t n_chunks) {
-    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (i >= n_chunks) return;
-    v4u w = __builtin_nontemporal_load(in + i);
-    v4u o0, o1;
+__global__ __launch_bounds__(kThreads) void unpack_last_vec(const v2u* __restrict__ in,
+                                                            v4u* __restrict__ out, int64_t n_half) {
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        u32 lo, hi;
-        split_dword<kSigned>(w[d], lo, hi);
-        u32 a = byte_perm(hi, lo, 0x05010400u);  // lo0 hi0 lo1 hi1
-        u32 b = byte_perm(hi, lo, 0x07030602u);  // lo2 hi2 lo3 hi3
-        if (d < 2) {
-            o0[2 * d] = a;
-            o0[2 * d + 1] = b;
-        } else {
-            o1[2 * (d - 2)] = a;
-            o1[2 * (d - 2) + 1] = b;
+    for (int h = 0; h < 2; ++h) {
+        const int64_t i = ((int64_t)blockIdx.x * 2 + h) * kThreads + threadIdx.x;
+        if (i >= n_half) return;
+        const v2u w = __builtin_nontemporal_load(in + i);
+        v4u o;
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            u32 lo, hi;
+            split_dword<kSigned>(w[d], lo, hi);
+            o[2 * d] = byte_perm(hi, lo, 0x05010400u);      // lo0 hi0 lo1 hi1
+            o[2 * d + 1] = byte_perm(hi, lo, 0x07030602u);  // lo2 hi2 lo3 hi3
         }
+        __builtin_nontemporal_store(o, out + i);
     }
-    __builtin_nontemporal_store(o0, out + 2 * i);
-    __builtin_nontemporal_store(o1, out + 2 * i + 1);
 }
 
 // ---- unpack, nibbles go to rows 2j and 2j+1 (inner % 16 == 0) -------------
@@ -208,11 +206,11 @@ extern "C" int k3q_unpack_int4(const void* in, int64_t outer, int64_t packed_len
     bool al = aligned_to(in, 16) && aligned_to(out, 16);
     bool full = (used_plen == packed_len);
     if (inner == 1 && full && orig_len == 2 * packed_len && (total % 16) == 0 && al) {
-        int64_t n = total / 16;
+        int64_t n = total / 8;  // 8 packed bytes per store
         if (is_signed)
-            unpack_last_vec<true><<<blocks_for(n), kThreads, 0, s>>>((const v4u*)in, (v4u*)out, n);
+            unpack_last_vec<true><<<blocks_for((n + 1) / 2), kThreads, 0, s>>>((const v2u*)in, (v4u*)out, n);
         else
-            unpack_last_vec<false><<<blocks_for(n), kThreads, 0, s>>>((const v4u*)in, (v4u*)out, n);
+            unpack_last_vec<false><<<blocks_for((n + 1) / 2), kThreads, 0, s>>>((const v2u*)in, (v4u*)out, n);
     } else if (inner > 1 && (inner % 16) == 0 && full && al) {
         int64_t n = total / 16;
         if (is_signed)

@@ -11,8 +11,12 @@
 // What makes the bits equal: every step is one IEEE float32 operation in numpy and here (compiled
 // with -ffp-contract=off, `/` is the correctly rounded division, rintf rounds half to even as
 // np.round does); bfloat16 inputs are widened first, as the reference's conversion to numpy does.
-// Both are two passes over x (the second finds it in the cache for the tile sizes used here): HBM
-// reads x once or twice and writes one byte per element.
+// Both are two passes over x, and both read it from memory twice (a column's maximum needs all of
+// the column first; the groups resident on the chip at one time are larger than its caches).  The
+// grouped kernel is bound by its arithmetic, not by the second read: the correctly rounded
+// division and the NaN-aware min / max come to ~45 vector instructions per element, and a
+// variant that kept a group's rows in registers between the passes (half the reads) measured
+// 117 us against 111 us for 8192 x 8192 float32, block 128.
 #include "k3q_common.h"
 
 namespace k3q {
