@@ -506,7 +506,9 @@ def main():
                 pack_rows.append({"op": name, "axis": axis, "values": n_val, "us_per_call": round(us_, 2),
                                   "algorithmic_bytes": int(1.5 * n_val),
                                   "roofline": {"bound": "hbm", "achieved": round(gbs_, 1), "peak": HBM_PEAK_GBS,
-                                               "unit": "GB/s", "frac": round(gbs_ / HBM_PEAK_GBS, 4), "traffic": None}})
+                                               "unit": "GB/s", "frac": round(gbs_ / HBM_PEAK_GBS, 4),
+                                               "traffic": measured_traffic(
+                                                   f"{name}_{'last_axis' if axis == -1 else 'axis0'}_64M")}})
             del packed
         del unpacked
         torch.cuda.empty_cache()
@@ -514,15 +516,18 @@ def main():
     # ------------------------------------------------------------------ weight quantizers on the device
     # What `quantize()` runs on a float32 kernel that lives on the device (the bits of the reference's
     # numpy path): per-column abs-max (int8 and per-channel int4) and the grouped min / max quantizer
-    # (block 128), 8192 x 8192 float32; algorithmic bytes: 4 read + 1 written per weight (the kernels
-    # make two passes over x; the second finds most of it in the caches).  Rotating over two kernels
-    # of 256 MiB.
+    # (block 128), 8192 x 8192 float32; algorithmic bytes: 4 read + 1 written per weight.  The kernels
+    # make two passes over x and memory sees both (`traffic`): a column's maximum needs the whole
+    # column first, and the grouped kernel is bound by its arithmetic, not by the second read.
+    # Rotating over two kernels of 256 MiB; eager calls, so host time per call counts as well.
     wq_rows = []
     if want("wq"):
         wf = [torch.randn(Kg, Ng, device=dev) * 0.02 for _ in range(2)]
-        for name, call in (("abs_max_quantize axis=0 (int8)", lambda i: kq.abs_max_quantize(wf[i % 2], axis=0, to_numpy=True)),
-                           ("abs_max_quantize_grouped_with_zero_point block 128 (int4)",
-                            lambda i: kq.abs_max_quantize_grouped_with_zero_point(wf[i % 2], 128, to_numpy=True))):
+        for name, key, call in (("abs_max_quantize axis=0 (int8)", "absmax_reduce_f32_8192x8192",
+                                 lambda i: kq.abs_max_quantize(wf[i % 2], axis=0, to_numpy=True)),
+                                ("abs_max_quantize_grouped_with_zero_point block 128 (int4)",
+                                 "grouped_zp_f32_8192x8192_block128",
+                                 lambda i: kq.abs_max_quantize_grouped_with_zero_point(wf[i % 2], 128, to_numpy=True))):
             call(0)
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -535,7 +540,8 @@ def main():
             nb_ = 5 * Kg * Ng
             wq_rows.append({"op": name, "shape": [Kg, Ng], "us_per_call": round(us_, 1), "algorithmic_bytes": nb_,
                             "roofline": {"bound": "hbm", "achieved": round(nb_ / us_ / 1e3, 1), "peak": HBM_PEAK_GBS,
-                                         "unit": "GB/s", "frac": round(nb_ / us_ / 1e3 / HBM_PEAK_GBS, 4), "traffic": None}})
+                                         "unit": "GB/s", "frac": round(nb_ / us_ / 1e3 / HBM_PEAK_GBS, 4),
+                                         "traffic": measured_traffic(key)}})
         del wf
         torch.cuda.empty_cache()
 
@@ -554,7 +560,8 @@ def main():
         embed_row = {"ids": count_, "vocab": vocab_, "dim": dim_, "table": "int8", "out": "float32",
                      "us_per_call": round(us_, 1), "algorithmic_bytes": nbytes_,
                      "roofline": {"bound": "hbm", "achieved": round(nbytes_ / us_ / 1e3, 1), "peak": HBM_PEAK_GBS,
-                                  "unit": "GB/s", "frac": round(nbytes_ / us_ / 1e3 / HBM_PEAK_GBS, 4), "traffic": None}}
+                                  "unit": "GB/s", "frac": round(nbytes_ / us_ / 1e3 / HBM_PEAK_GBS, 4),
+                                  "traffic": measured_traffic("embedding_rows_int8_32768x4096_f32")}}
         del table_, tscale_, ids_
         torch.cuda.empty_cache()
 
