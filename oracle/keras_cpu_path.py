@@ -6,7 +6,15 @@ on ``KERAS_BACKEND=torch`` with tensors on the CPU, so integer results are the
 reference's results and float results carry the reference's per-op rounding.
 
 Pinning status (what makes each function trustworthy without importing the
-reference) is listed per function; ``tests/test_oracle_*.py`` holds the checks.
+reference) is listed per function; ``tests/test_oracle*.py`` holds the checks.
+
+PARITY UNPINNED: the ``to_numpy=True`` weight quantizers on bfloat16
+*variables* (a pure ``bfloat16`` dtype policy).  The reference converts such a
+variable to a numpy array of ``ml_dtypes.bfloat16``, and numpy then rounds every
+step to bfloat16; ``ml_dtypes`` is not installed here and nothing in the
+reference's tests holds outputs for that case, so this file widens the variable
+to float32 first and computes as for a float32 variable.  float32 variables
+(the default and ``mixed_bfloat16`` policies) are not affected.
 
 Reference citations are relative to the keras-team/keras 3.16.0 tree.
 """
