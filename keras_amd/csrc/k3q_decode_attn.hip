@@ -8,6 +8,9 @@
 // through LDS (one float per cache row), softmax in float32, the value sum is reduced over
 // the 4 row slots of a wave by lane exchange and over the waves through LDS.
 // The position is read from device memory, so a captured graph replays with a new one.
+// Two dependent rounds of loads: the position with the new query / key / value rows, then the
+// rotation's table entries with the cached rows below the position; the new rows are used from
+// LDS, so nothing waits for their stores into the cache to be acknowledged.
 #include "k3q_common.h"
 
 namespace k3q {
@@ -28,9 +31,13 @@ struct AttnParams {
     float scale;
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+// every lane of a row of 16 gets the row's sum: x ^ 1, x ^ 2, then the other quad of the half row,
+// then the other half (the same pairs, in the same order, as a butterfly over 1, 2, 4, 8)
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xf>(v);  // row_half_mirror
+    v += dpp_move<0x140, 0xf>(v);  // row_mirror
     return v;
 }
 
@@ -39,10 +46,24 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
     float* qs = attn_lds;                   // [128] rotated query, pre-scaled
     float* red = qs + kHd;                  // [2 * kAW]
     float* oacc = red + 2 * kAW;            // [kAW][128]
-    float* sc = oacc + kAW * kHd;           // [max_len]
+    uint16_t* knew = (uint16_t*)(oacc + kAW * kHd);  // [128] the new key row as it goes into the cache
+    uint16_t* vnew = knew + kHd;            // [128] the new value row
+    float* sc = (float*)(vnew + kHd);       // [max_len]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bh = blockIdx.x;
+    // The loads that do not depend on the position go out together with the position itself:
+    // the new query / key elements (with their rotate-half partners) and the new value row.
+    const int d = tid & (kHd - 1);
+    float x = 0.f, sw = 0.f;
+    v4u vrow = {0u, 0u, 0u, 0u};
+    if (tid < 2 * kHd) {
+        const uint16_t* src = (tid < kHd ? p.q : p.k) + (int64_t)bh * kHd;
+        x = bf16_bits_to_f32(src[d]);
+        sw = bf16_bits_to_f32(src[d ^ (kHd / 2)]);
+    } else if (tid < 2 * kHd + 16) {
+        vrow = ((const v4u*)(p.v + (int64_t)bh * kHd))[tid - 2 * kHd];
+    }
     // A position outside the cache (the torch ops this stands for raise there): nothing is written
     // to the caches, the output rows are zero and the caller's flag is raised.  Every thread reads
     // the same position, so the whole workgroup leaves here before its first barrier.
@@ -55,71 +76,97 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
     const int pos = (int)pos64;
     const int64_t row0 = (int64_t)bh * p.max_len;  // first cache row of this (sequence, head)
 
-    // ---- rotate q and k, write the new cache rows ----
+    // ---- second round of loads: the rotation's table entries and the cached rows ----
+    // Rows 0 ... pos-1 are in the cache already, so their loads need not wait for the new row to be
+    // written: row pos itself is taken from LDS below.  Blocks of 4 cache rows go to the waves
+    // round-robin; a wave asks for kU blocks of keys at once and -- for its first kU blocks -- for
+    // the value rows too, before the softmax, so that the weighted sum finds them in registers
+    // (the value rows do not depend on the scores).
+    float cs = 0.f, sn = 0.f;
     if (tid < 2 * kHd) {
-        const int d = tid & (kHd - 1);
-        const uint16_t* src = (tid < kHd ? p.q : p.k) + (int64_t)bh * kHd;
-        const float x = bf16_bits_to_f32(src[d]), sw = bf16_bits_to_f32(src[d ^ (kHd / 2)]);
-        const float c = bf16_bits_to_f32(p.cos_t[(int64_t)pos * kHd + d]);
-        const float s = bf16_bits_to_f32(p.sin_t[(int64_t)pos * kHd + d]);
-        // the rounding steps of x * cos + swapped * sin evaluated in bfloat16
-        const float r = round_bf16(round_bf16(x * c) + round_bf16(sw * s));
-        if (tid < kHd) qs[d] = r * p.scale;
-        else p.kc[(row0 + pos) * kHd + d] = (uint16_t)f32_to_bf16_bits(r);
-    } else if (tid < 2 * kHd + 16) {
-        const int c = tid - 2 * kHd;
-        ((v4u*)(p.vc + (row0 + pos) * kHd))[c] = ((const v4u*)(p.v + (int64_t)bh * kHd))[c];
+        cs = bf16_bits_to_f32(p.cos_t[(int64_t)pos * kHd + d]);
+        sn = bf16_bits_to_f32(p.sin_t[(int64_t)pos * kHd + d]);
     }
-    __syncthreads();  // the new rows are written (and acknowledged) before any wave reads the cache
-
-    // ---- scores ----
-    // Blocks of 4 cache rows go to the waves round-robin; a wave asks for kU blocks of keys at once
-    // and -- for its first kU blocks -- for the value rows too, before the softmax, so that the
-    // weighted sum below finds them in registers (the value rows do not depend on the scores).
     const int n = pos + 1;
     const int nblk = (n + 3) >> 2;
     const int sub = lane >> 4, dl = (lane & 15) * 8;
+    const int last_old = pos > 0 ? pos - 1 : 0;  // a row that is safe to read for lanes without a cached row
     constexpr int kU = 8;
+    v4u kk0[kU], vv0[kU];
+    if (wave < nblk) {
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (wave + u * kAW) + sub;
+            kk0[u] = *(const v4u*)(p.kc + (row0 + (j < pos ? j : last_old)) * kHd + dl);
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (wave + u * kAW) + sub;
+            vv0[u] = *(const v4u*)(p.vc + (row0 + (j < pos ? j : last_old)) * kHd + dl);
+        }
+    }
+
+    // ---- rotate q and k; the new rows go to the cache and, for this launch, to LDS ----
+    if (tid < 2 * kHd) {
+        // the rounding steps of x * cos + swapped * sin evaluated in bfloat16
+        const float r = round_bf16(round_bf16(x * cs) + round_bf16(sw * sn));
+        if (tid < kHd) {
+            qs[d] = r * p.scale;
+        } else {
+            const uint16_t bits = (uint16_t)f32_to_bf16_bits(r);
+            knew[d] = bits;
+            p.kc[(row0 + pos) * kHd + d] = bits;
+        }
+    } else if (tid < 2 * kHd + 16) {
+        const int c = tid - 2 * kHd;
+        ((v4u*)vnew)[c] = vrow;
+        ((v4u*)(p.vc + (row0 + pos) * kHd))[c] = vrow;
+    }
+    __syncthreads();
+
+    // ---- scores ----
     float qv[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) qv[e] = qs[dl + e];
     float mx = -INFINITY;
-    v4u vv0[kU];
     for (int kb0 = wave; kb0 < nblk; kb0 += kAW * kU) {
         v4u kk[kU];
-#pragma unroll
-        for (int u = 0; u < kU; ++u) {
-            const int j = 4 * (kb0 + u * kAW) + sub;
-            kk[u] = *(const v4u*)(p.kc + (row0 + (j < n ? j : pos)) * kHd + dl);
-        }
         if (kb0 == wave) {
+#pragma unroll
+            for (int u = 0; u < kU; ++u) kk[u] = kk0[u];
+        } else {
 #pragma unroll
             for (int u = 0; u < kU; ++u) {
                 const int j = 4 * (kb0 + u * kAW) + sub;
-                vv0[u] = *(const v4u*)(p.vc + (row0 + (j < n ? j : pos)) * kHd + dl);
+                kk[u] = *(const v4u*)(p.kc + (row0 + (j < pos ? j : last_old)) * kHd + dl);
             }
         }
+        float dot[kU];
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             const int j = 4 * (kb0 + u * kAW) + sub;
-            float dot = 0.f;
+            if (j == pos) kk[u] = *(const v4u*)(knew + dl);
+            dot[u] = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                dot += qv[2 * e] * __uint_as_float(kk[u][e] << 16);
-                dot += qv[2 * e + 1] * __uint_as_float(kk[u][e] & 0xffff0000u);
+                dot[u] += qv[2 * e] * __uint_as_float(kk[u][e] << 16);
+                dot[u] += qv[2 * e + 1] * __uint_as_float(kk[u][e] & 0xffff0000u);
             }
-            dot += __shfl_xor(dot, 1, kWave);
-            dot += __shfl_xor(dot, 2, kWave);
-            dot += __shfl_xor(dot, 4, kWave);
-            dot += __shfl_xor(dot, 8, kWave);
+        }
+        // sum over the 16 lanes of a row, as lane exchanges inside the vector unit (through LDS
+        // permutes the kU dependent chains of four exchanges took 2 us of the launch's 8)
+#pragma unroll
+        for (int u = 0; u < kU; ++u) dot[u] = row16_sum(dot[u]);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+            const int j = 4 * (kb0 + u * kAW) + sub;
             if (j < n) {
-                mx = fmaxf(mx, dot);
-                if ((lane & 15) == 0) sc[j] = dot;
+                mx = fmaxf(mx, dot[u]);
+                if ((lane & 15) == 0) sc[j] = dot[u];
             }
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
     __syncthreads();
     float gmx = red[0];
@@ -155,6 +202,7 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             const int j = 4 * (wave + u * kAW) + sub;
+            if (j == pos) vv0[u] = *(const v4u*)(vnew + dl);
             add_row(vv0[u], j < n ? sc[j] : 0.f);
         }
     }
@@ -163,11 +211,12 @@ __global__ __launch_bounds__(kAT) void decode_attention(AttnParams p) {
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             const int j = 4 * (kb0 + u * kAW) + sub;
-            vv[u] = *(const v4u*)(p.vc + (row0 + (j < n ? j : pos)) * kHd + dl);
+            vv[u] = *(const v4u*)(p.vc + (row0 + (j < pos ? j : last_old)) * kHd + dl);
         }
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
             const int j = 4 * (kb0 + u * kAW) + sub;
+            if (j == pos) vv[u] = *(const v4u*)(vnew + dl);
             add_row(vv[u], j < n ? sc[j] : 0.f);
         }
     }
@@ -219,7 +268,7 @@ extern "C" int k3q_decode_attention(const void* q, const void* k, const void* v,
     p.H = (int)H;
     p.max_len = (int)max_len;
     p.scale = 0.08838834764831845f;  // 1 / sqrt(128)
-    const size_t lds = (size_t)(kHd + 2 * kAW + kAW * kHd + max_len) * sizeof(float);
+    const size_t lds = (size_t)(kHd + 2 * kAW + kAW * kHd + kHd + max_len) * sizeof(float);  // as laid out in the kernel
     if (lds > 64 * 1024) {
         static const bool raised = hipFuncSetAttribute((const void*)decode_attention,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize,
