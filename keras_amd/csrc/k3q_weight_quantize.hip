@@ -11,12 +11,10 @@
 // What makes the bits equal: every step is one IEEE float32 operation in numpy and here (compiled
 // with -ffp-contract=off, `/` is the correctly rounded division, rintf rounds half to even as
 // np.round does); bfloat16 inputs are widened first, as the reference's conversion to numpy does.
-// Both are two passes over x, and both read it from memory twice (a column's maximum needs all of
-// the column first; the groups resident on the chip at one time are larger than its caches).  The
-// grouped kernel is bound by its arithmetic, not by the second read: the correctly rounded
-// division and the NaN-aware min / max come to ~45 vector instructions per element, and a
-// variant that kept a group's rows in registers between the passes (half the reads) measured
-// 117 us against 111 us for 8192 x 8192 float32, block 128.
+// The abs-max form reads x from memory twice (a column's maximum needs all of the column before the
+// first integer, and the kernel is larger than the chip's caches).  Groups of up to 128 rows keep
+// their rows in registers between the min / max and the integers (grouped_zp_held: one read); larger
+// groups take the generic two-pass kernel.
 #include "k3q_common.h"
 
 namespace k3q {
@@ -213,6 +211,119 @@ __global__ __launch_bounds__(kWqT) void grouped_zp(GroupedParams p) {
     }
 }
 
+// rintf(x / s) with the division's own rounding, for a column scale s > 0 whose reciprocal
+// (correctly rounded) is at hand.  r = x * (1 / s) lies within 3 * 2^-24 |r| of the correctly rounded
+// quotient t, so rint(t) = rint(r) unless r is that close to a half-integer; there (and for
+// anything that is not a number) the division is done.  The margin used is 2^-20 |r|.
+__device__ __forceinline__ float rint_quotient(float x, float s, float inv_s) {
+    const float r = x * inv_s;
+    float n = rintf(r);
+    const float d = fabsf(r - n);
+    if (!(0.5f - d > fabsf(r) * 0x1p-20f)) n = rintf(x / s);
+    return n;
+}
+
+// The same for groups of up to kHeldY * kHeldRows rows with N a multiple of 4.  A thread keeps its
+// rows in registers between the two passes, so memory sees x once (the groups resident on the chip
+// at one time are far larger than its caches, and the generic kernel's second read comes from
+// memory again); the integers come from rint_quotient.  A workgroup walks work items (column
+// tile, group) at a stride of the grid and asks for the next item's rows before it works on the
+// current one: with one item per workgroup the whole chip alternates between loading and computing
+// (the registers allow one or two workgroups per CU), and neither memory nor the vector units see
+// more than half of the time.
+constexpr int kHeldY = 8, kHeldRows = 16;
+template <bool kBF16>
+__global__ __launch_bounds__(kWqX * kHeldY) void grouped_zp_held(GroupedParams p, int col_tiles, int items) {
+    __shared__ float lo_s[2][kHeldY][kWqX * 4], hi_s[2][kHeldY][kWqX * 4];
+    const int tx = threadIdx.x % kWqX, ty = threadIdx.x / kWqX;
+    auto load_item = [&](const int item, float (&rows)[kHeldRows][4]) {
+        const int64_t g = item / col_tiles;
+        const int64_t col = ((int64_t)(item - g * col_tiles) * kWqX + tx) * 4;
+        const int64_t r0 = g * p.block;
+#pragma unroll
+        for (int j = 0; j < kHeldRows; ++j) {
+            const int i = ty + j * kHeldY;
+            if (item < items && col < p.N && i < p.block && r0 + i < p.K) {
+                load_vals<kBF16, 4>(p.x, (r0 + i) * p.N + col, rows[j]);
+            } else {  // rows past K count as zeros; rows past the group do not count (skipped below)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) rows[j][e] = 0.f;
+            }
+        }
+    };
+    auto work = [&](const int item, const int par, const float (&rows)[kHeldRows][4]) {
+        const int64_t g = item / col_tiles;
+        const int64_t col = ((int64_t)(item - g * col_tiles) * kWqX + tx) * 4;
+        const int64_t r0 = g * p.block;
+        float lo[4], hi[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo[e] = INFINITY;
+            hi[e] = -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < kHeldRows; ++j)
+            if (ty + j * kHeldY < p.block) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    lo[e] = fminf(lo[e], rows[j][e]);
+                    hi[e] = fmaxf(hi[e], rows[j][e]);
+                }
+            }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo_s[par][ty][tx * 4 + e] = lo[e];
+            hi_s[par][ty][tx * 4 + e] = hi[e];
+        }
+        __syncthreads();  // (the buffers alternate, so the item after the next may overwrite this one's)
+        if (col >= p.N) return;
+        float scale[4], inv[4], zero[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float l = lo_s[par][0][tx * 4 + e], h = hi_s[par][0][tx * 4 + e];
+#pragma unroll
+            for (int y = 1; y < kHeldY; ++y) {
+                l = fminf(l, lo_s[par][y][tx * 4 + e]);
+                h = fmaxf(h, hi_s[par][y][tx * 4 + e]);
+            }
+            scale[e] = ((h - l) + p.eps) / p.levels;
+            inv[e] = 1.0f / scale[e];
+            zero[e] = fminf(fmaxf(rintf(-l / scale[e]) + p.qmin, p.qmin), p.qmax);
+        }
+        if (ty == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                store_scale<kBF16>(p.scale, g * p.N + col + e, scale[e]);
+                p.zero[g * p.N + col + e] = (int8_t)(int)zero[e];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kHeldRows; ++j) {
+            const int i = ty + j * kHeldY;
+            if (i < p.block && r0 + i < p.K) {
+                int v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    v[e] = (int)__builtin_amdgcn_fmed3f(rint_quotient(rows[j][e], scale[e], inv[e]) + zero[e], p.qmin, p.qmax);
+                store_q<4>(p.q, (r0 + i) * p.N + col, v);
+            }
+        }
+    };
+    float a[kHeldRows][4], b[kHeldRows][4];
+    const int step = gridDim.x;
+    int item = blockIdx.x;
+    load_item(item, a);
+    while (item < items) {  // (uniform over the workgroup: every thread meets every barrier)
+        load_item(item + step, b);
+        work(item, 0, a);
+        item += step;
+        if (item >= items) break;
+        load_item(item + step, a);
+        work(item, 1, b);
+        item += step;
+    }
+}
+
 __global__ void clear_u32(u32* p, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -294,6 +405,16 @@ extern "C" int k3q_weight_quantize_grouped(const void* x, int x_dtype, int64_t K
     const int v = vec ? 4 : 1;
     dim3 grid((unsigned)((N + (int64_t)kWqX * v - 1) / ((int64_t)kWqX * v)), (unsigned)groups);
     hipStream_t s = (hipStream_t)stream;
+    // the held form's quotient needs a finite positive scale and its reciprocal: an epsilon > 0 gives
+    // both for any finite kernel
+    const int64_t col_tiles = grid.x, items = col_tiles * groups;
+    const bool held = vec && block_size <= (int64_t)kHeldY * kHeldRows && epsilon > 0.f && items < (1ll << 30);
+    if (held) {
+        const unsigned blocks = (unsigned)(items < 256 ? items : 256);  // one resident workgroup per CU
+        if (bf) grouped_zp_held<true><<<blocks, kWqX * kHeldY, 0, s>>>(p, (int)col_tiles, (int)items);
+        else grouped_zp_held<false><<<blocks, kWqX * kHeldY, 0, s>>>(p, (int)col_tiles, (int)items);
+        return launch_status();
+    }
     if (bf && vec) grouped_zp<true, 4><<<grid, kWqT, 0, s>>>(p);
     else if (bf) grouped_zp<true, 1><<<grid, kWqT, 0, s>>>(p);
     else if (vec) grouped_zp<false, 4><<<grid, kWqT, 0, s>>>(p);
