@@ -76,6 +76,48 @@ def test_device_grouped_weight_quantizer_has_numpy_bits(dev, K, N, block, dtype)
     assert torch.equal(qh, want_q) and torch.equal(bits(sh), bits(want_s)) and torch.equal(zh, want_z)
 
 
+def test_device_grouped_weight_quantizer_at_rounding_boundaries(dev):
+    # The device kernel takes rint(x / scale) from x * (1 / scale) unless that product lies next to a
+    # half-integer, where it divides.  Every weight here sits on such a boundary or within a few
+    # float32 steps of one -- (m + 1/2) * scale for the levels m of its group, moved by -4 ... +4
+    # ulps -- with scales and minima that differ from column to column, so both the test for
+    # "next to" and the division behind it decide the integers.  Bit for bit against the numpy path.
+    import numpy as np
+
+    block, N, G = 128, 1024, 4
+    rng = np.random.default_rng(5)
+    span = rng.uniform(0.01, 3.0, size=N).astype(np.float32)         # max - min of a group, per column
+    lo = np.where(np.arange(N) % 3 == 0, 0.0, -rng.uniform(0.0, 1.0, size=N) * span).astype(np.float32)
+    hi = (lo + span).astype(np.float32)
+    scale = ((hi - lo) + np.float32(1e-7)) / np.float32(15.0)         # the scale numpy will find
+    m_lo = np.ceil(lo.astype(np.float64) / scale)                     # half-integers m + 1/2 inside (lo, hi)
+    m_hi = np.floor(hi.astype(np.float64) / scale) - 1
+    w = np.empty((G * block, N), dtype=np.float32)
+    for row in range(G * block):
+        r = row % block
+        if r == 0:
+            w[row] = lo
+        elif r == 1:
+            w[row] = hi
+        else:
+            m = m_lo + (row * 5) % np.maximum(m_hi - m_lo + 1, 1)
+            x = ((m + 0.5) * scale.astype(np.float64)).astype(np.float32)
+            steps = (row * 7) % 9 - 4
+            for _ in range(abs(steps)):
+                x = np.nextafter(x, np.float32(np.inf if steps > 0 else -np.inf))
+            w[row] = np.minimum(np.maximum(x, lo), hi)
+    w = torch.from_numpy(w)
+    want_q, want_s, want_z = ref.abs_max_quantize_grouped_with_zero_point(w, block)
+    assert torch.equal(bits(want_s), bits(torch.from_numpy(np.tile(scale, (G, 1)))))  # the scales aimed at
+    q, s, z = kq.abs_max_quantize_grouped_with_zero_point(w.to(dev), block, to_numpy=True)
+    assert torch.equal(bits(s.cpu()), bits(want_s)) and torch.equal(z.cpu(), want_z)
+    assert torch.equal(q.cpu(), want_q)
+    # the case is what it claims to be: most quotients are within 1e-5 of a half-integer
+    r = w.double().reshape(G, block, N) / want_s.double()[:, None, :]
+    near = ((r - r.floor() - 0.5).abs() < 1e-5).double().mean().item()
+    assert near > 0.5, near
+
+
 def test_device_weight_quantizers_at_llama_kernel_size(dev):
     # 4096 x 14336 (the gate / up projection of config 5): both quantizers against the oracle
     w = kernel_like((4096, 14336), 7)
