@@ -39,18 +39,51 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E, published (8 TB/s)
 # `--pmc WRITE_SIZE` (KiB per dispatch) of this same command, each scaled by what the counter
 # reads for a plain device copy of known size (FETCH_SIZE 0.50x, WRITE_SIZE 1.00x).  The
 # figures are measured offline and kept in profiles/ with the command that produced them; this
-# file reads them from there (kernel name -> bytes), so that a line never carries a number
-# from another build than the one profiled.
+# file reads them from there (kernel name -> bytes).  The file also records the SHA-256 of the
+# kernel sources it was measured on (`_sources`); a figure whose kernel source has changed since
+# is reported as null, with the file's name in `traffic_stale`, instead of being carried over.
+# `python bench.py --sources-digest` prints the digests to record after a new profile.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_bytes.json")
+CSRC = os.path.join(ROOT, "keras_amd", "csrc")
+TRAFFIC_SOURCES = {  # key prefix -> the kernel's source files (all of them include k3q_common.h)
+    "gemm_mfma": ["k3q_gemm_i8.hip"], "quantize_rows_vec": ["k3q_quantize.hip"], "gemv_w4s": ["k3q_gemv_w4s.hip"],
+    "gemv_w8s": ["k3q_gemv_w8s.hip"], "pack_int4": ["k3q_pack.hip"], "unpack_int4": ["k3q_pack.hip"],
+    "embedding_rows": ["k3q_embedding.hip"], "absmax_reduce": ["k3q_weight_quantize.hip"],
+    "grouped_zp": ["k3q_weight_quantize.hip"],
+}
+TRAFFIC_STALE = set()
+
+
+def sources_digest():
+    import hashlib
+
+    names = sorted({n for v in TRAFFIC_SOURCES.values() for n in v} | {"k3q_common.h"})
+    out = {}
+    for n in names:
+        with open(os.path.join(CSRC, n), "rb") as f:
+            out[n] = hashlib.sha256(f.read()).hexdigest()
+    return out
 
 
 def measured_traffic(key):
     try:
         with open(TRAFFIC_FILE) as f:
-            return json.load(f).get(key)
+            table = json.load(f)
     except (OSError, ValueError):
         return None
-
+    if key not in table:
+        return None
+    files = next((v for k, v in TRAFFIC_SOURCES.items() if key.startswith(k)), None)
+    recorded = table.get("_sources", {})
+    try:
+        now = sources_digest()
+    except OSError:
+        return None
+    for n in (files or []) + ["k3q_common.h"]:
+        if files is None or recorded.get(n) != now.get(n):
+            TRAFFIC_STALE.add(n if files is not None else key)
+            return None
+    return table[key]
 
 
 def gemv_algorithmic_bytes(M, K, N, grouped, block=128):
@@ -81,7 +114,12 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the end-to-end decoder measurement")
     ap.add_argument("--only", default="", help="comma list out of ceiling,sweep,einsum,gemv,gemv8,pack,wq,embed,decode,cpu: run the headline "
                     "step and only these further sections (for profiler runs); default: all")
+    ap.add_argument("--sources-digest", action="store_true",
+                    help="print the SHA-256 of the kernel sources (the `_sources` entry of profiles/hbm_traffic_bytes.json) and exit")
     args = ap.parse_args()
+    if args.sources_digest:
+        print(json.dumps(sources_digest(), indent=1))
+        return
     only = set(filter(None, args.only.split(",")))
     unknown = only - {"none", "calib", "ceiling", "sweep", "einsum", "gemv", "gemv8", "pack", "wq", "embed", "decode", "cpu"}
     if unknown:
@@ -694,6 +732,8 @@ def main():
         "llama_decode_int8": decode_int8,
         "cpu_baseline": cpu,
     }
+    if TRAFFIC_STALE:  # kernel sources that changed after their traffic figures were measured
+        out["traffic_stale"] = sorted(TRAFFIC_STALE)
     print(json.dumps(out))
 
 
